@@ -1,0 +1,216 @@
+// extern "C" entry points of libastrai_w8a8.so (declared in
+// include/astrai_w8a8.h): argument validation, kernel selection, launch check.
+// Nothing here allocates, frees or synchronises.
+#include "../../include/astrai_w8a8.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "launchers.h"
+
+namespace {
+
+thread_local char g_err[256] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_launch(const char* what) {
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess)
+        return fail(ASTRAI_W8A8_LAUNCH_FAILED, "%s: %s", what, hipGetErrorString(e));
+    return ASTRAI_W8A8_OK;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+constexpr int64_t kMaxDim = (int64_t)1 << 30;
+
+int check_gemm(const char* what, const void* a, const void* b, const void* out, int64_t m,
+               int64_t n, int64_t k) {
+    if (!a || !b || !out) return fail(ASTRAI_W8A8_BAD_ARG, "%s: null operand pointer", what);
+    if (m < 0 || n < 0 || k < 0 || m > kMaxDim || n > kMaxDim || k > kMaxDim)
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: bad dims m=%lld n=%lld k=%lld", what, (long long)m,
+                    (long long)n, (long long)k);
+    if (!aligned16(a) || !aligned16(b) || !aligned16(out))
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: operands must be 16-byte aligned", what);
+    return ASTRAI_W8A8_OK;
+}
+
+w8a8::GemmArgs pack(const void* a, const void* b, const float* sa, const float* sb,
+                    const float* out_scale, const void* bias, void* out, int64_t m, int64_t n,
+                    int64_t k, int out_kind) {
+    w8a8::GemmArgs g;
+    g.a = a;
+    g.b = b;
+    g.sa = sa;
+    g.sb = sb;
+    g.out_scale = out_scale;
+    g.bias = bias;
+    g.out = out;
+    g.m = (int)m;
+    g.n = (int)n;
+    g.k = (int)k;
+    g.out_kind = out_kind;
+    return g;
+}
+
+}  // namespace
+
+extern "C" {
+
+int astrai_w8a8_abi_version(void) { return ASTRAI_W8A8_ABI_VERSION; }
+
+const char* astrai_w8a8_last_error(void) { return g_err; }
+
+int astrai_w8a8_quantize_bf16_fp8(const void* x, void* x8, const float* scale, float* amax,
+                                  int64_t total, int fmt, void* stream) {
+    if (!x || !x8 || !scale) return fail(ASTRAI_W8A8_BAD_ARG, "quantize_bf16_fp8: null pointer");
+    if (total < 0) return fail(ASTRAI_W8A8_BAD_ARG, "quantize_bf16_fp8: negative size");
+    if (fmt != ASTRAI_W8A8_E4M3 && fmt != ASTRAI_W8A8_E5M2)
+        return fail(ASTRAI_W8A8_BAD_ARG, "quantize_bf16_fp8: fmt must be 0 (e4m3) or 1 (e5m2)");
+    if (!aligned16(x) || !aligned16(x8))
+        return fail(ASTRAI_W8A8_BAD_ARG, "quantize_bf16_fp8: pointers must be 16-byte aligned");
+    if (total == 0) return ASTRAI_W8A8_OK;
+    w8a8::launch_quantize_fp8(x, x8, scale, amax, total, fmt, static_cast<hipStream_t>(stream));
+    return check_launch("quantize_bf16_fp8");
+}
+
+int astrai_w8a8_quantize_bf16_int8_rows(const void* x, void* xq, float* s, int64_t rows,
+                                        int64_t k, void* stream) {
+    if (!x || !xq || !s) return fail(ASTRAI_W8A8_BAD_ARG, "quantize_bf16_int8_rows: null pointer");
+    if (rows < 0 || k < 0 || rows > 0x7fffffff)
+        return fail(ASTRAI_W8A8_BAD_ARG, "quantize_bf16_int8_rows: bad dims");
+    if (!aligned16(x) || !aligned16(xq))
+        return fail(ASTRAI_W8A8_BAD_ARG, "quantize_bf16_int8_rows: pointers must be 16-byte aligned");
+    if (rows == 0 || k == 0) return ASTRAI_W8A8_OK;
+    w8a8::launch_quantize_int8_rows(x, xq, s, rows, k, static_cast<hipStream_t>(stream));
+    return check_launch("quantize_bf16_int8_rows");
+}
+
+int astrai_w8a8_quantize_bf16_fp8_block128_act(const void* x, void* x8, float* sa, int64_t m,
+                                               int64_t k, void* stream) {
+    if (!x || !x8 || !sa) return fail(ASTRAI_W8A8_BAD_ARG, "quantize_block128_act: null pointer");
+    if (m < 0 || k < 0) return fail(ASTRAI_W8A8_BAD_ARG, "quantize_block128_act: bad dims");
+    if (k % 128) return fail(ASTRAI_W8A8_UNSUPPORTED, "quantize_block128_act: K must be a multiple of 128");
+    if (!aligned16(x) || !aligned16(x8))
+        return fail(ASTRAI_W8A8_BAD_ARG, "quantize_block128_act: pointers must be 16-byte aligned");
+    if (m == 0 || k == 0) return ASTRAI_W8A8_OK;
+    w8a8::launch_quantize_fp8_block128_act(x, x8, sa, m, k, static_cast<hipStream_t>(stream));
+    return check_launch("quantize_block128_act");
+}
+
+int astrai_w8a8_quantize_bf16_fp8_block128_weight(const void* w, void* w8, float* sb, int64_t n,
+                                                  int64_t k, void* stream) {
+    if (!w || !w8 || !sb) return fail(ASTRAI_W8A8_BAD_ARG, "quantize_block128_weight: null pointer");
+    if (n < 0 || k < 0) return fail(ASTRAI_W8A8_BAD_ARG, "quantize_block128_weight: bad dims");
+    if (k % 128) return fail(ASTRAI_W8A8_UNSUPPORTED, "quantize_block128_weight: K must be a multiple of 128");
+    if ((n + 127) / 128 > 65535)
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "quantize_block128_weight: N too large");
+    if (!aligned16(w) || !aligned16(w8))
+        return fail(ASTRAI_W8A8_BAD_ARG, "quantize_block128_weight: pointers must be 16-byte aligned");
+    if (n == 0 || k == 0) return ASTRAI_W8A8_OK;
+    w8a8::launch_quantize_fp8_block128_weight(w, w8, sb, n, k, static_cast<hipStream_t>(stream));
+    return check_launch("quantize_block128_weight");
+}
+
+int astrai_w8a8_gemm_fp8_pt(const void* a8, const void* b8, const float* sa, const float* sb,
+                            const float* out_scale, const void* bias, void* out, int64_t m,
+                            int64_t n, int64_t k, int fmt, int out_dtype, void* stream) {
+    if (int rc = check_gemm("gemm_fp8_pt", a8, b8, out, m, n, k)) return rc;
+    if (fmt != ASTRAI_W8A8_E4M3 && fmt != ASTRAI_W8A8_E5M2)
+        return fail(ASTRAI_W8A8_BAD_ARG, "gemm_fp8_pt: fmt must be 0 (e4m3) or 1 (e5m2)");
+    if (out_dtype < 0 || out_dtype > 2)
+        return fail(ASTRAI_W8A8_BAD_ARG, "gemm_fp8_pt: out_dtype must be 0 (bf16), 1 (e4m3) or 2 (fp32 acc)");
+    if (out_dtype != ASTRAI_W8A8_OUT_ACC && (!sa || !sb))
+        return fail(ASTRAI_W8A8_BAD_ARG, "gemm_fp8_pt: null scale pointer");
+    if (out_dtype == ASTRAI_W8A8_OUT_E4M3 && !out_scale)
+        return fail(ASTRAI_W8A8_BAD_ARG, "gemm_fp8_pt: fp8 output requires out_scale");
+    if (out_dtype == ASTRAI_W8A8_OUT_E4M3 && bias)
+        return fail(ASTRAI_W8A8_BAD_ARG, "gemm_fp8_pt: bias is not supported with fp8 output");
+    if (m == 0 || n == 0) return ASTRAI_W8A8_OK;
+    if (k == 0) return fail(ASTRAI_W8A8_UNSUPPORTED, "gemm_fp8_pt: K must be >= 1");
+    auto s = static_cast<hipStream_t>(stream);
+    const w8a8::GemmArgs g = pack(a8, b8, sa, sb, out_scale, bias, out, m, n, k, out_dtype);
+    if (!w8a8::launch_gemm_fp8_tiled(g, fmt, s))
+        w8a8::launch_gemm_generic(g, fmt ? 2 : 1, w8a8::SCALE_TENSOR, s);
+    return check_launch("gemm_fp8_pt");
+}
+
+int astrai_w8a8_gemm_fp8_block128(const void* a8, const void* b8, const float* sa,
+                                  const float* sb, const void* bias, void* out, int64_t m,
+                                  int64_t n, int64_t k, void* stream) {
+    if (int rc = check_gemm("gemm_fp8_block128", a8, b8, out, m, n, k)) return rc;
+    if (!sa || !sb) return fail(ASTRAI_W8A8_BAD_ARG, "gemm_fp8_block128: null scale pointer");
+    if (k == 0 || k % 128)
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "gemm_fp8_block128: K must be a positive multiple of 128");
+    if (m == 0 || n == 0) return ASTRAI_W8A8_OK;
+    auto s = static_cast<hipStream_t>(stream);
+    const w8a8::GemmArgs g =
+        pack(a8, b8, sa, sb, nullptr, bias, out, m, n, k, w8a8::OUT_BF16);
+    if (!w8a8::launch_gemm_fp8_block128_tiled(g, s))
+        w8a8::launch_gemm_generic(g, 1, w8a8::SCALE_BLOCK128, s);
+    return check_launch("gemm_fp8_block128");
+}
+
+static int int8_common(const char* what, const void* a, const void* b, const float* sa,
+                       const float* sb, void* out, int64_t m, int64_t n, int64_t k,
+                       int out_dtype) {
+    if (int rc = check_gemm(what, a, b, out, m, n, k)) return rc;
+    if (out_dtype != ASTRAI_W8A8_OUT_BF16 && out_dtype != ASTRAI_W8A8_OUT_ACC)
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: out_dtype must be 0 (bf16) or 2 (int32 acc)", what);
+    if (out_dtype == ASTRAI_W8A8_OUT_BF16 && (!sa || !sb))
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: null scale pointer", what);
+    if (k == 0 && m > 0 && n > 0) return fail(ASTRAI_W8A8_UNSUPPORTED, "%s: K must be >= 1", what);
+    return ASTRAI_W8A8_OK;
+}
+
+int astrai_w8a8_gemm_int8_ptpc(const void* a, const void* b, const float* sa, const float* sb,
+                               const void* bias, void* out, int64_t m, int64_t n, int64_t k,
+                               int out_dtype, void* stream) {
+    if (int rc = int8_common("gemm_int8_ptpc", a, b, sa, sb, out, m, n, k, out_dtype)) return rc;
+    if (m == 0 || n == 0) return ASTRAI_W8A8_OK;
+    auto s = static_cast<hipStream_t>(stream);
+    const w8a8::GemmArgs g = pack(a, b, sa, sb, nullptr, bias, out, m, n, k, out_dtype);
+    if (m <= 64 && w8a8::launch_gemv_int8(g, s)) return check_launch("gemv_int8_ptpc");
+    if (!w8a8::launch_gemm_int8_tiled(g, s))
+        w8a8::launch_gemm_generic(g, 0, w8a8::SCALE_ROWCOL, s);
+    return check_launch("gemm_int8_ptpc");
+}
+
+int astrai_w8a8_gemv_int8_ptpc(const void* a, const void* b, const float* sa, const float* sb,
+                               const void* bias, void* out, int64_t m, int64_t n, int64_t k,
+                               int out_dtype, void* stream) {
+    if (int rc = int8_common("gemv_int8_ptpc", a, b, sa, sb, out, m, n, k, out_dtype)) return rc;
+    if (m > 64 || k % 256 || k == 0)
+        return fail(ASTRAI_W8A8_UNSUPPORTED,
+                    "gemv_int8_ptpc: needs M <= 64 and K a positive multiple of 256 (got m=%lld k=%lld)",
+                    (long long)m, (long long)k);
+    if (m == 0 || n == 0) return ASTRAI_W8A8_OK;
+    const w8a8::GemmArgs g = pack(a, b, sa, sb, nullptr, bias, out, m, n, k, out_dtype);
+    if (!w8a8::launch_gemv_int8(g, static_cast<hipStream_t>(stream)))
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "gemv_int8_ptpc: weight matrix of 2 GiB or more");
+    return check_launch("gemv_int8_ptpc");
+}
+
+int astrai_w8a8_gemm_int8_ptpc_tiled(const void* a, const void* b, const float* sa,
+                                     const float* sb, const void* bias, void* out, int64_t m,
+                                     int64_t n, int64_t k, int out_dtype, void* stream) {
+    if (int rc = int8_common("gemm_int8_ptpc_tiled", a, b, sa, sb, out, m, n, k, out_dtype))
+        return rc;
+    if (m == 0 || n == 0) return ASTRAI_W8A8_OK;
+    const w8a8::GemmArgs g = pack(a, b, sa, sb, nullptr, bias, out, m, n, k, out_dtype);
+    if (!w8a8::launch_gemm_int8_tiled(g, static_cast<hipStream_t>(stream)))
+        return fail(ASTRAI_W8A8_UNSUPPORTED,
+                    "gemm_int8_ptpc_tiled: needs K %% 16 == 0 and operands under 2 GiB");
+    return check_launch("gemm_int8_ptpc_tiled");
+}
+
+}  // extern "C"

@@ -1,0 +1,50 @@
+// Host-side launch functions, one group per kernel family. Each launches
+// asynchronously on `stream` and returns nothing; the C ABI layer (abi.hip)
+// validates arguments first and checks hipGetLastError() afterwards.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace w8a8 {
+
+enum OutKind : int { OUT_BF16 = 0, OUT_E4M3 = 1, OUT_ACC = 2 };
+enum ScaleKind : int { SCALE_TENSOR = 0, SCALE_ROWCOL = 1, SCALE_BLOCK128 = 2 };
+
+struct GemmArgs {
+    const void* a;        // [M,K] 8-bit activations
+    const void* b;        // [N,K] 8-bit weights
+    const float* sa;      // per-tensor [1] | per-token [M] | block [M,K/128]
+    const float* sb;      // per-tensor [1] | per-channel [N] | block [ceil(N/128),K/128]
+    const float* out_scale;  // OUT_E4M3 only
+    const void* bias;     // bf16 [N] or null
+    void* out;            // [M,N]
+    int m, n, k;
+    int out_kind;
+};
+
+// quantize.hip
+void launch_quantize_fp8(const void* x, void* x8, const float* scale, float* amax,
+                         int64_t total, int fmt, hipStream_t stream);
+void launch_quantize_int8_rows(const void* x, void* xq, float* s, int64_t rows, int64_t k,
+                               hipStream_t stream);
+void launch_quantize_fp8_block128_act(const void* x, void* x8, float* sa, int64_t m,
+                                      int64_t k, hipStream_t stream);
+void launch_quantize_fp8_block128_weight(const void* w, void* w8, float* sb, int64_t n,
+                                         int64_t k, hipStream_t stream);
+
+// gemm_int8.hip / gemm_fp8.hip / gemm_fp8_block.hip: tiled MFMA kernels.
+// Require k % 16 == 0 and m*k, n*k < 2^31 bytes; return false if the shape is
+// not accepted (the caller then uses the generic kernel).
+bool launch_gemm_int8_tiled(const GemmArgs& g, hipStream_t stream);
+bool launch_gemm_fp8_tiled(const GemmArgs& g, int fmt, hipStream_t stream);
+bool launch_gemm_fp8_block128_tiled(const GemmArgs& g, hipStream_t stream);
+
+// gemm_generic.hip: any shape, guarded byte loads, one wave per 16x16 tile.
+void launch_gemm_generic(const GemmArgs& g, int op /*0=i8,1=e4m3,2=e5m2*/, int scale_kind,
+                         hipStream_t stream);
+
+// gemv_int8.hip: skinny int8 kernel, m <= 64, k % 256 == 0.
+bool launch_gemv_int8(const GemmArgs& g, hipStream_t stream);
+
+}  // namespace w8a8

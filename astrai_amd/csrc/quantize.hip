@@ -1,0 +1,257 @@
+// bf16 -> fp8 / int8 quantization kernels for gfx950.
+//
+// All kernels are bandwidth-bound elementwise passes: 16-byte loads (8 bf16 per
+// lane), IEEE fp32 division by the step (the CPU kernel's arithmetic,
+// astrai/extension/ops/fp8.py:80), hardware RNE conversion, 8-byte stores.
+#include "common.cuh"
+#include "launchers.h"
+
+namespace w8a8 {
+
+namespace {
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ void unpack8(u32x4 raw, float (&f)[8]) {
+    f[0] = __uint_as_float(raw.x << 16);
+    f[1] = __uint_as_float(raw.x & 0xffff0000u);
+    f[2] = __uint_as_float(raw.y << 16);
+    f[3] = __uint_as_float(raw.y & 0xffff0000u);
+    f[4] = __uint_as_float(raw.z << 16);
+    f[5] = __uint_as_float(raw.z & 0xffff0000u);
+    f[6] = __uint_as_float(raw.w << 16);
+    f[7] = __uint_as_float(raw.w & 0xffff0000u);
+}
+
+__device__ __forceinline__ float amax8(const float (&f)[8]) {
+    float a = fmaxf(fabsf(f[0]), fabsf(f[1]));
+    float b = fmaxf(fabsf(f[2]), fabsf(f[3]));
+    float c = fmaxf(fabsf(f[4]), fabsf(f[5]));
+    float d = fmaxf(fabsf(f[6]), fabsf(f[7]));
+    return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+
+template <int Fmt>
+__device__ __forceinline__ u32x2 quant8_fp8(const float (&f)[8], float step) {
+    u32x2 o;
+    o.x = cvt_pk_fp8<Fmt>(f[0] / step, f[1] / step) |
+          (cvt_pk_fp8<Fmt>(f[2] / step, f[3] / step) << 16);
+    o.y = cvt_pk_fp8<Fmt>(f[4] / step, f[5] / step) |
+          (cvt_pk_fp8<Fmt>(f[6] / step, f[7] / step) << 16);
+    return o;
+}
+
+__device__ __forceinline__ uint32_t quant1_int8(float f, float step) {
+    float q = rintf(f / step);
+    q = fminf(fmaxf(q, -127.0f), 127.0f);
+    return (uint32_t)(int)q & 0xffu;
+}
+
+__device__ __forceinline__ u32x2 quant8_int8(const float (&f)[8], float step) {
+    u32x2 o;
+    o.x = quant1_int8(f[0], step) | (quant1_int8(f[1], step) << 8) |
+          (quant1_int8(f[2], step) << 16) | (quant1_int8(f[3], step) << 24);
+    o.y = quant1_int8(f[4], step) | (quant1_int8(f[5], step) << 8) |
+          (quant1_int8(f[6], step) << 16) | (quant1_int8(f[7], step) << 24);
+    return o;
+}
+
+// block-wide max of a per-thread value; result valid in every thread
+__device__ __forceinline__ float block_max(float v, float* slots) {
+    v = wave_max(v);
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) slots[wave] = v;
+    __syncthreads();
+    float r = slots[0];
+#pragma unroll
+    for (int w = 1; w < kThreads / kWave; ++w) r = fmaxf(r, slots[w]);
+    __syncthreads();
+    return r;
+}
+
+// ---- per-tensor fp8 -------------------------------------------------------
+template <int Fmt>
+__global__ __launch_bounds__(kThreads) void quantize_fp8_kernel(
+    const uint16_t* __restrict__ x, uint8_t* __restrict__ x8, const float* __restrict__ scale,
+    float* __restrict__ amax, int64_t total) {
+    __shared__ float slots[kThreads / kWave];
+    const float step = *scale;
+    float local = 0.0f;
+    const int64_t nvec = total >> 3;
+    const int64_t stride = (int64_t)gridDim.x * kThreads;
+    for (int64_t v = (int64_t)blockIdx.x * kThreads + threadIdx.x; v < nvec; v += stride) {
+        float f[8];
+        unpack8(*reinterpret_cast<const u32x4*>(x + v * 8), f);
+        local = fmaxf(local, amax8(f));
+        *reinterpret_cast<u32x2*>(x8 + v * 8) = quant8_fp8<Fmt>(f, step);
+    }
+    if (blockIdx.x == 0) {  // ragged tail (< 8 elements)
+        const int64_t i = nvec * 8 + threadIdx.x;
+        if (i < total) {
+            const float f = bf16_to_f32(x[i]);
+            local = fmaxf(local, fabsf(f));
+            x8[i] = (uint8_t)cvt_pk_fp8<Fmt>(f / step, 0.0f);
+        }
+    }
+    if (amax) {
+        const float m = block_max(local, slots);
+        if (threadIdx.x == 0) atomic_max_nonneg(amax, m);
+    }
+}
+
+// ---- per-row int8 ---------------------------------------------------------
+// One workgroup per row; up to kCache 16-byte vectors per thread stay in
+// registers between the amax pass and the quantize pass (K <= 8192), longer
+// rows are re-read (they hit L2).
+constexpr int kCache = 4;
+
+__global__ __launch_bounds__(kThreads) void quantize_int8_rows_kernel(
+    const uint16_t* __restrict__ x, int8_t* __restrict__ xq, float* __restrict__ s, int64_t k) {
+    __shared__ float slots[kThreads / kWave];
+    const int64_t row = blockIdx.x;
+    const uint16_t* xr = x + row * k;
+    int8_t* qr = xq + row * k;
+    const bool vec_ok = (k & 7) == 0;
+    const int64_t nvec = vec_ok ? (k >> 3) : 0;
+    u32x4 cache[kCache];
+    float local = 0.0f;
+#pragma unroll
+    for (int c = 0; c < kCache; ++c) {
+        const int64_t v = threadIdx.x + (int64_t)c * kThreads;
+        if (v < nvec) {
+            cache[c] = *reinterpret_cast<const u32x4*>(xr + v * 8);
+            float f[8];
+            unpack8(cache[c], f);
+            local = fmaxf(local, amax8(f));
+        }
+    }
+    for (int64_t v = threadIdx.x + (int64_t)kCache * kThreads; v < nvec; v += kThreads) {
+        float f[8];
+        unpack8(*reinterpret_cast<const u32x4*>(xr + v * 8), f);
+        local = fmaxf(local, amax8(f));
+    }
+    for (int64_t i = nvec * 8 + threadIdx.x; i < k; i += kThreads)
+        local = fmaxf(local, fabsf(bf16_to_f32(xr[i])));
+
+    const float amax = fmaxf(block_max(local, slots), 1e-12f);
+    const float step = amax / 127.0f;
+    if (threadIdx.x == 0) s[row] = step;
+
+#pragma unroll
+    for (int c = 0; c < kCache; ++c) {
+        const int64_t v = threadIdx.x + (int64_t)c * kThreads;
+        if (v < nvec) {
+            float f[8];
+            unpack8(cache[c], f);
+            *reinterpret_cast<u32x2*>(qr + v * 8) = quant8_int8(f, step);
+        }
+    }
+    for (int64_t v = threadIdx.x + (int64_t)kCache * kThreads; v < nvec; v += kThreads) {
+        float f[8];
+        unpack8(*reinterpret_cast<const u32x4*>(xr + v * 8), f);
+        *reinterpret_cast<u32x2*>(qr + v * 8) = quant8_int8(f, step);
+    }
+    for (int64_t i = nvec * 8 + threadIdx.x; i < k; i += kThreads)
+        qr[i] = (int8_t)quant1_int8(bf16_to_f32(xr[i]), step);
+}
+
+// ---- 1x128 activation groups ----------------------------------------------
+// One 16-byte vector per lane; 16 consecutive lanes own one 128-wide group.
+__global__ __launch_bounds__(kThreads) void quantize_fp8_act128_kernel(
+    const uint16_t* __restrict__ x, uint8_t* __restrict__ x8, float* __restrict__ sa,
+    int64_t nvec) {
+    const int64_t v = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    float f[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    const bool live = v < nvec;  // nvec is a multiple of 16, so groups are all-or-nothing
+    if (live) unpack8(*reinterpret_cast<const u32x4*>(x + v * 8), f);
+    float a = amax8(f);
+#pragma unroll
+    for (int off = 8; off; off >>= 1) a = fmaxf(a, __shfl_xor(a, off, kWave));
+    const float step = fmaxf(a, 1e-12f) / 448.0f;
+    if (live) {
+        *reinterpret_cast<u32x2*>(x8 + v * 8) = quant8_fp8<0>(f, step);
+        if ((threadIdx.x & 15) == 0) sa[v >> 4] = step;
+    }
+}
+
+// ---- 128x128 weight blocks ------------------------------------------------
+// One workgroup per block: 128 rows x 16 vectors = 2048 vectors, 8 per thread.
+__global__ __launch_bounds__(kThreads) void quantize_fp8_weight128_kernel(
+    const uint16_t* __restrict__ w, uint8_t* __restrict__ w8, float* __restrict__ sb, int64_t n,
+    int64_t k) {
+    __shared__ float slots[kThreads / kWave];
+    const int64_t kb = blockIdx.x, nb = blockIdx.y;
+    const int64_t kblocks = gridDim.x;
+    u32x4 cache[8];
+    float local = 0.0f;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        const int q = threadIdx.x + c * kThreads;  // 0..2047
+        const int64_t row = nb * 128 + (q >> 4);
+        const int64_t col = kb * 128 + (q & 15) * 8;
+        if (row < n) {
+            cache[c] = *reinterpret_cast<const u32x4*>(w + row * k + col);
+            float f[8];
+            unpack8(cache[c], f);
+            local = fmaxf(local, amax8(f));
+        }
+    }
+    const float step = fmaxf(block_max(local, slots), 1e-12f) / 448.0f;
+    if (threadIdx.x == 0) sb[nb * kblocks + kb] = step;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        const int q = threadIdx.x + c * kThreads;
+        const int64_t row = nb * 128 + (q >> 4);
+        const int64_t col = kb * 128 + (q & 15) * 8;
+        if (row < n) {
+            float f[8];
+            unpack8(cache[c], f);
+            *reinterpret_cast<u32x2*>(w8 + row * k + col) = quant8_fp8<0>(f, step);
+        }
+    }
+}
+
+}  // namespace
+
+void launch_quantize_fp8(const void* x, void* x8, const float* scale, float* amax,
+                         int64_t total, int fmt, hipStream_t stream) {
+    if (total <= 0) return;
+    const int64_t nvec = (total + 7) / 8;
+    int64_t blocks = (nvec + kThreads - 1) / kThreads;
+    // enough workgroups to fill 256 CUs several times over, grid-stride beyond that
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    auto xs = static_cast<const uint16_t*>(x);
+    auto xo = static_cast<uint8_t*>(x8);
+    if (fmt)
+        quantize_fp8_kernel<1><<<dim3((unsigned)blocks), dim3(kThreads), 0, stream>>>(
+            xs, xo, scale, amax, total);
+    else
+        quantize_fp8_kernel<0><<<dim3((unsigned)blocks), dim3(kThreads), 0, stream>>>(
+            xs, xo, scale, amax, total);
+}
+
+void launch_quantize_int8_rows(const void* x, void* xq, float* s, int64_t rows, int64_t k,
+                               hipStream_t stream) {
+    if (rows <= 0 || k <= 0) return;
+    quantize_int8_rows_kernel<<<dim3((unsigned)rows), dim3(kThreads), 0, stream>>>(
+        static_cast<const uint16_t*>(x), static_cast<int8_t*>(xq), s, k);
+}
+
+void launch_quantize_fp8_block128_act(const void* x, void* x8, float* sa, int64_t m,
+                                      int64_t k, hipStream_t stream) {
+    const int64_t nvec = m * k / 8;
+    if (nvec <= 0) return;
+    const int64_t blocks = (nvec + kThreads - 1) / kThreads;
+    quantize_fp8_act128_kernel<<<dim3((unsigned)blocks), dim3(kThreads), 0, stream>>>(
+        static_cast<const uint16_t*>(x), static_cast<uint8_t*>(x8), sa, nvec);
+}
+
+void launch_quantize_fp8_block128_weight(const void* w, void* w8, float* sb, int64_t n,
+                                         int64_t k, hipStream_t stream) {
+    if (n <= 0 || k <= 0) return;
+    dim3 grid((unsigned)(k / 128), (unsigned)((n + 127) / 128));
+    quantize_fp8_weight128_kernel<<<grid, dim3(kThreads), 0, stream>>>(
+        static_cast<const uint16_t*>(w), static_cast<uint8_t*>(w8), sb, n, k);
+}
+
+}  // namespace w8a8

@@ -1,0 +1,440 @@
+"""ctypes binding of ``lib/libastrai_w8a8.so`` (the C ABI in include/astrai_w8a8.h)
+and the tensor-level adapters that stand where the reference's pybind module
+``fp8_mm`` stands (csrc/kernels/fp8/mm.cu:350-369).
+
+The adapters do what the reference binding does around its launches
+(mm.cu:99-234): validate devices / dtypes / shapes, make operands contiguous,
+allocate the outputs on the input's device, pass torch's current stream, and
+turn a failing status into ``RuntimeError``. There is no CPU or PyTorch fallback
+anywhere in this module: without the HIP library every call raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+import torch  # imported before the CDLL so the library binds to torch's HIP runtime
+
+_LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
+LIB_PATH = os.path.join(_LIB_DIR, "libastrai_w8a8.so")
+
+ABI_VERSION = 1
+OUT_BF16, OUT_E4M3, OUT_ACC = 0, 1, 2
+
+_P = ctypes.c_void_p
+_I64 = ctypes.c_int64
+_INT = ctypes.c_int
+
+# name -> argtypes, exactly the prototypes of include/astrai_w8a8.h
+PROTOTYPES = {
+    "astrai_w8a8_abi_version": ([], _INT),
+    "astrai_w8a8_last_error": ([], ctypes.c_char_p),
+    "astrai_w8a8_quantize_bf16_fp8": ([_P, _P, _P, _P, _I64, _INT, _P], _INT),
+    "astrai_w8a8_quantize_bf16_int8_rows": ([_P, _P, _P, _I64, _I64, _P], _INT),
+    "astrai_w8a8_quantize_bf16_fp8_block128_act": ([_P, _P, _P, _I64, _I64, _P], _INT),
+    "astrai_w8a8_quantize_bf16_fp8_block128_weight": ([_P, _P, _P, _I64, _I64, _P], _INT),
+    "astrai_w8a8_gemm_fp8_pt": ([_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _INT, _INT, _P], _INT),
+    "astrai_w8a8_gemm_fp8_block128": ([_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _INT),
+    "astrai_w8a8_gemm_int8_ptpc": ([_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _INT, _P], _INT),
+    "astrai_w8a8_gemv_int8_ptpc": ([_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _INT, _P], _INT),
+    "astrai_w8a8_gemm_int8_ptpc_tiled": ([_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _INT, _P], _INT),
+}
+
+_lib: Optional[ctypes.CDLL] = None
+_load_error: Optional[str] = None
+
+
+def load() -> Optional[ctypes.CDLL]:
+    """Load the shared library once; ``None`` (with the reason kept) if it is absent
+    or does not carry the expected ABI. Never raises: the registry reports an
+    unavailable kernel the way the reference's loader does (loader.py:36-44)."""
+    global _lib, _load_error
+    if _lib is not None or _load_error is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        _load_error = f"{LIB_PATH} not built"
+        return None
+    try:
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (argtypes, restype) in PROTOTYPES.items():
+            fn = getattr(lib, name)
+            fn.argtypes = argtypes
+            fn.restype = restype
+        got = lib.astrai_w8a8_abi_version()
+        if got != ABI_VERSION:
+            raise OSError(f"ABI version {got}, expected {ABI_VERSION}")
+    except (OSError, AttributeError) as e:
+        _load_error = f"{type(e).__name__}: {e}"
+        return None
+    _lib = lib
+    return _lib
+
+
+def load_error() -> Optional[str]:
+    return _load_error
+
+
+def _require() -> ctypes.CDLL:
+    lib = load()
+    if lib is None:
+        raise RuntimeError(
+            f"HIP library libastrai_w8a8.so is not available ({_load_error}). "
+            "Build it with `make -C astrai_amd/csrc`."
+        )
+    return lib
+
+
+def _check(rc: int, lib: ctypes.CDLL) -> None:
+    if rc != 0:
+        msg = lib.astrai_w8a8_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"astrai_w8a8 error {rc}: {msg}")
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _gpu(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name}: CUDA tensors required")  # mm.cu:104,135,192
+
+
+def _check_scale(scale: torch.Tensor, ref: torch.Tensor, name: str) -> None:
+    # mm.cu:49-54
+    if not (scale.is_cuda and scale.device == ref.device and scale.dtype == torch.float32
+            and scale.numel() == 1):
+        raise RuntimeError(f"{name} must be a CUDA float32 scalar on the input device")
+
+
+def _check_vec(s: torch.Tensor, ref: torch.Tensor, numel: int, name: str) -> torch.Tensor:
+    if not (s.is_cuda and s.device == ref.device and s.dtype == torch.float32
+            and s.numel() == numel):
+        raise RuntimeError(f"{name} must be CUDA float32 with {numel} elements on the input device")
+    return s.contiguous()
+
+
+_FP8 = (torch.float8_e4m3fn, torch.float8_e5m2)
+
+
+# ---------------------------------------------------------------------------
+# The five callables of the reference's pybind module (mm.cu:350-369)
+# ---------------------------------------------------------------------------
+
+
+def quantize_bf16(x: torch.Tensor, scale: torch.Tensor, fmt: int):
+    """bf16 -> fp8 with fused amax; returns ``(x8, amax)``. mm.cu:99-126."""
+    lib = _require()
+    _gpu(x, "quantize_bf16")
+    _gpu(scale, "quantize_bf16")
+    if x.dtype != torch.bfloat16:
+        raise RuntimeError("x must be bf16")
+    _check_scale(scale, x, "scale")
+    x_c = x.contiguous()
+    with torch.cuda.device(x.device):
+        x8 = torch.empty_like(x_c, dtype=torch.float8_e5m2 if fmt else torch.float8_e4m3fn)
+        amax = torch.zeros(1, device=x.device, dtype=torch.float32)
+        if x_c.numel():
+            _check(lib.astrai_w8a8_quantize_bf16_fp8(
+                x_c.data_ptr(), x8.data_ptr(), scale.data_ptr(), amax.data_ptr(),
+                x_c.numel(), 1 if fmt else 0, _stream(x)), lib)
+    return x8, amax
+
+
+def mm_fp8(a: torch.Tensor, b: torch.Tensor, sa: torch.Tensor, sb: torch.Tensor,
+           out_dtype: int = 0, out_scale: Optional[torch.Tensor] = None,
+           bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Pre-quantized fp8 GEMM ``a @ b^T * (sa*sb)``. mm.cu:128-184. ``bias`` (bf16
+    ``[N]``, bf16 output only) is an extension used by the fused linear forward."""
+    lib = _require()
+    _gpu(a, "mm_fp8")
+    _gpu(b, "mm_fp8")
+    if a.dtype not in _FP8:
+        raise RuntimeError("a and b must be fp8 (e4m3fn or e5m2)")
+    if a.dtype != b.dtype:
+        raise RuntimeError("a and b must share the same fp8 format")
+    if a.dim() != 2 or b.dim() != 2:
+        raise RuntimeError("a and b must be 2D")
+    if a.device != b.device:
+        raise RuntimeError("a and b must be on the same device")
+    if a.size(1) != b.size(1):
+        raise RuntimeError("inner dim mismatch")
+    _check_scale(sa, a, "sa")
+    _check_scale(sb, a, "sb")
+    if out_dtype not in (0, 1):
+        raise RuntimeError("out_dtype must be 0 (bf16) or 1 (fp8 e4m3)")
+    if out_dtype == 1:
+        if out_scale is None:
+            raise RuntimeError("fp8 output requires out_scale")
+        _check_scale(out_scale, a, "out_scale")
+    a_c, b_c = a.contiguous(), b.contiguous()
+    m, k = a_c.shape
+    n = b_c.size(0)
+    if bias is not None:
+        if not (bias.is_cuda and bias.device == a.device and bias.dtype == torch.bfloat16
+                and bias.numel() == n):
+            raise RuntimeError("bias must be CUDA bf16 with shape [N]")
+        bias = bias.contiguous()
+    with torch.cuda.device(a.device):
+        out = torch.empty((m, n), device=a.device,
+                          dtype=torch.float8_e4m3fn if out_dtype else torch.bfloat16)
+        if m and n:
+            if k == 0:
+                out.zero_()
+            else:
+                _check(lib.astrai_w8a8_gemm_fp8_pt(
+                    a_c.data_ptr(), b_c.data_ptr(), sa.data_ptr(), sb.data_ptr(),
+                    _ptr(out_scale) if out_dtype else None, _ptr(bias), out.data_ptr(),
+                    m, n, k, 1 if a.dtype == torch.float8_e5m2 else 0, out_dtype, _stream(a)), lib)
+    return out
+
+
+def mm_fp8_acc(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """Raw fp32 accumulator of the fp8 GEMM (parity surface, no scaling)."""
+    lib = _require()
+    a_c, b_c = a.contiguous(), b.contiguous()
+    m, k = a_c.shape
+    n = b_c.size(0)
+    with torch.cuda.device(a.device):
+        out = torch.empty((m, n), device=a.device, dtype=torch.float32)
+        _check(lib.astrai_w8a8_gemm_fp8_pt(
+            a_c.data_ptr(), b_c.data_ptr(), None, None, None, None, out.data_ptr(), m, n, k,
+            1 if a.dtype == torch.float8_e5m2 else 0, OUT_ACC, _stream(a)), lib)
+    return out
+
+
+def linear_forward_fp8(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor,
+                       sx: torch.Tensor, sw: torch.Tensor):
+    """bf16 linear forward through e4m3: returns ``(out, amax_x, amax_w)``.
+    mm.cu:186-234. The reference re-quantizes both operands inside its GEMM at
+    every K step (gemm.cuh:296-326); here each operand is quantized once by the
+    prologue kernel (which also yields its amax) and the pre-quantized MFMA GEMM
+    applies ``sx*sw`` and the bias in its epilogue -- the same arithmetic."""
+    _gpu(x, "linear_forward_fp8")
+    _gpu(w, "linear_forward_fp8")
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise RuntimeError("x and w must be bf16")
+    if x.device != w.device:
+        raise RuntimeError("x and w must be on the same device")
+    _check_scale(sx, x, "sx")
+    _check_scale(sw, x, "sw")
+    if w.dim() != 2 or x.size(-1) != w.size(1):
+        raise RuntimeError("inner dim mismatch")
+    k, n = w.size(1), w.size(0)
+    x2 = x.reshape(-1, k)
+    has_bias = bias is not None and bias.numel() > 0
+    if has_bias and not (bias.is_cuda and bias.device == x.device
+                         and bias.dtype == torch.bfloat16 and bias.numel() == n):
+        raise RuntimeError("bias must be CUDA bf16 with shape [N]")
+    x8, amax_x = quantize_bf16(x2, sx, 0)
+    w8, amax_w = quantize_bf16(w, sw, 0)
+    out = mm_fp8(x8, w8, sx, sw, 0, None, bias if has_bias else None)
+    return out.reshape(*x.shape[:-1], n), amax_x, amax_w
+
+
+def fp8_mm(a: torch.Tensor, b: torch.Tensor, sx: torch.Tensor, sw: torch.Tensor) -> torch.Tensor:
+    """bf16-in fused fp8 GEMM primitive (no bias, no amax). mm.cu:322-348."""
+    _gpu(a, "fp8_mm")
+    _gpu(b, "fp8_mm")
+    if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16:
+        raise RuntimeError("a and b must be bf16")
+    if a.dim() != 2 or b.dim() != 2:
+        raise RuntimeError("a and b must be 2D")
+    if a.device != b.device:
+        raise RuntimeError("a and b must be on the same device")
+    if a.size(1) != b.size(1):
+        raise RuntimeError("inner dim mismatch")
+    out, _, _ = linear_forward_fp8(a, b, None, sx, sw)
+    return out
+
+
+def linear_backward_fp8(g, x, w, masks, sg, sw, sx, fmt: int):
+    """FP8 linear backward ``(grad_input, grad_weight, grad_bias, amax_g)``.
+    mm.cu:236-320: the gradient is quantized once, ``dX = g8 @ w8`` and
+    ``dW = g8^T @ x8`` run as NT GEMMs on transposed-contiguous copies."""
+    _gpu(g, "linear_backward_fp8")
+    if not (g.dtype == x.dtype == w.dtype == torch.bfloat16):
+        raise RuntimeError("g, x, and w must be bf16")
+    if not (g.device == x.device == w.device):
+        raise RuntimeError("g, x, and w must be on the same device")
+    masks = list(masks)
+    if len(masks) != 3:
+        raise RuntimeError("masks must contain three values")
+    n, k = w.shape
+    g_c = g.reshape(-1, n).contiguous()
+    x_c = x.reshape(-1, x.size(-1)).contiguous()
+    m = g_c.size(0)
+    if x_c.size(0) != m or x_c.size(1) != k:
+        raise RuntimeError("backward shape mismatch")
+    grad_input = torch.empty_like(x)
+    grad_weight = torch.empty_like(w)
+    grad_bias = torch.empty(0, device=g.device, dtype=g.dtype)
+    amax_g = torch.zeros(1, device=g.device, dtype=torch.float32)
+    if masks[0]:
+        g8, amax_g = quantize_bf16(g_c, sg, fmt)
+        w8_t, _ = quantize_bf16(w.t().contiguous(), sw, fmt)  # [K, N]
+        grad_input.copy_(mm_fp8(g8, w8_t, sg, sw).reshape(x.shape))
+    if masks[1]:
+        g8_t, _ = quantize_bf16(g_c.t().contiguous(), sg, fmt)  # [N, M]
+        x8_t, _ = quantize_bf16(x_c.t().contiguous(), sx, fmt)  # [K, M]
+        grad_weight.copy_(mm_fp8(g8_t, x8_t, sg, sx))
+    if not masks[0] and not masks[1]:
+        amax_g = g_c.abs().amax().to(torch.float32).reshape(1)
+    if masks[2]:
+        grad_bias = g_c.sum(0).to(g.dtype)
+    return grad_input, grad_weight, grad_bias, amax_g
+
+
+# ---------------------------------------------------------------------------
+# int8 per-token x per-channel and 128-block fp8 (not in the reference)
+# ---------------------------------------------------------------------------
+
+
+def quantize_int8_rows(x: torch.Tensor):
+    """bf16 ``[..., K]`` -> ``(xq int8 [R,K], s fp32 [R,1])``, one symmetric scale per row."""
+    lib = _require()
+    _gpu(x, "quantize_int8_rows")
+    if x.dtype != torch.bfloat16:
+        raise RuntimeError("x must be bf16")
+    if x.dim() < 1:
+        raise RuntimeError("x must have at least one dimension")
+    k = x.size(-1)
+    x2 = x.reshape(-1, k).contiguous()
+    rows = x2.size(0)
+    with torch.cuda.device(x.device):
+        xq = torch.empty((rows, k), device=x.device, dtype=torch.int8)
+        s = torch.empty((rows, 1), device=x.device, dtype=torch.float32)
+        if rows and k:
+            _check(lib.astrai_w8a8_quantize_bf16_int8_rows(
+                x2.data_ptr(), xq.data_ptr(), s.data_ptr(), rows, k, _stream(x)), lib)
+        elif rows:
+            s.fill_(1e-12 / 127.0)
+    return xq, s
+
+
+_INT8_ENTRY = {
+    "auto": "astrai_w8a8_gemm_int8_ptpc",
+    "gemv": "astrai_w8a8_gemv_int8_ptpc",
+    "tiled": "astrai_w8a8_gemm_int8_ptpc_tiled",
+}
+
+
+def mm_int8(a: torch.Tensor, b: torch.Tensor, sa: Optional[torch.Tensor],
+            sb: Optional[torch.Tensor], bias: Optional[torch.Tensor] = None,
+            out_dtype: int = 0, kernel: str = "auto") -> torch.Tensor:
+    """int8 NT GEMM. ``out_dtype`` 0: ``bf16(acc*sa[m]*sb[n] (+bias))``; 2: raw int32
+    accumulator. ``kernel`` names the entry point: auto / gemv / tiled."""
+    lib = _require()
+    _gpu(a, "mm_int8")
+    _gpu(b, "mm_int8")
+    if a.dtype != torch.int8 or b.dtype != torch.int8:
+        raise RuntimeError("a and b must be int8")
+    if a.dim() != 2 or b.dim() != 2:
+        raise RuntimeError("a and b must be 2D")
+    if a.device != b.device:
+        raise RuntimeError("a and b must be on the same device")
+    if a.size(1) != b.size(1):
+        raise RuntimeError("inner dim mismatch")
+    if out_dtype not in (OUT_BF16, OUT_ACC):
+        raise RuntimeError("out_dtype must be 0 (bf16) or 2 (int32 accumulator)")
+    a_c, b_c = a.contiguous(), b.contiguous()
+    m, k = a_c.shape
+    n = b_c.size(0)
+    if out_dtype == OUT_BF16:
+        if sa is None or sb is None:
+            raise RuntimeError("bf16 output requires sa and sb")
+        sa = _check_vec(sa, a, m, "sa")
+        sb = _check_vec(sb, a, n, "sb")
+    if bias is not None:
+        if not (bias.is_cuda and bias.device == a.device and bias.dtype == torch.bfloat16
+                and bias.numel() == n):
+            raise RuntimeError("bias must be CUDA bf16 with shape [N]")
+        bias = bias.contiguous()
+    fn = getattr(lib, _INT8_ENTRY[kernel])
+    with torch.cuda.device(a.device):
+        out = torch.empty((m, n), device=a.device,
+                          dtype=torch.int32 if out_dtype == OUT_ACC else torch.bfloat16)
+        if m and n:
+            if k == 0:
+                out.zero_()
+            else:
+                _check(fn(a_c.data_ptr(), b_c.data_ptr(), _ptr(sa), _ptr(sb), _ptr(bias),
+                          out.data_ptr(), m, n, k, out_dtype, _stream(a)), lib)
+    return out
+
+
+def quantize_fp8_block128_act(x: torch.Tensor):
+    """bf16 ``[M,K]`` -> ``(x8 e4m3fn [M,K], sa fp32 [M,K/128])``."""
+    lib = _require()
+    _gpu(x, "quantize_fp8_block128_act")
+    if x.dtype != torch.bfloat16 or x.dim() != 2:
+        raise RuntimeError("x must be 2D bf16")
+    m, k = x.shape
+    if k % 128:
+        raise RuntimeError("K must be a multiple of 128")
+    x_c = x.contiguous()
+    with torch.cuda.device(x.device):
+        x8 = torch.empty((m, k), device=x.device, dtype=torch.float8_e4m3fn)
+        sa = torch.empty((m, k // 128), device=x.device, dtype=torch.float32)
+        if m and k:
+            _check(lib.astrai_w8a8_quantize_bf16_fp8_block128_act(
+                x_c.data_ptr(), x8.data_ptr(), sa.data_ptr(), m, k, _stream(x)), lib)
+    return x8, sa
+
+
+def quantize_fp8_block128_weight(w: torch.Tensor):
+    """bf16 ``[N,K]`` -> ``(w8 e4m3fn [N,K], sb fp32 [ceil(N/128),K/128])``."""
+    lib = _require()
+    _gpu(w, "quantize_fp8_block128_weight")
+    if w.dtype != torch.bfloat16 or w.dim() != 2:
+        raise RuntimeError("w must be 2D bf16")
+    n, k = w.shape
+    if k % 128:
+        raise RuntimeError("K must be a multiple of 128")
+    w_c = w.contiguous()
+    with torch.cuda.device(w.device):
+        w8 = torch.empty((n, k), device=w.device, dtype=torch.float8_e4m3fn)
+        sb = torch.empty(((n + 127) // 128, k // 128), device=w.device, dtype=torch.float32)
+        if n and k:
+            _check(lib.astrai_w8a8_quantize_bf16_fp8_block128_weight(
+                w_c.data_ptr(), w8.data_ptr(), sb.data_ptr(), n, k, _stream(w)), lib)
+    return w8, sb
+
+
+def mm_fp8_block128(a: torch.Tensor, b: torch.Tensor, sa: torch.Tensor, sb: torch.Tensor,
+                    bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """e4m3fn NT GEMM with ``sa [M,K/128]`` and ``sb [ceil(N/128),K/128]`` block scales."""
+    lib = _require()
+    _gpu(a, "mm_fp8_block128")
+    _gpu(b, "mm_fp8_block128")
+    if a.dtype != torch.float8_e4m3fn or b.dtype != torch.float8_e4m3fn:
+        raise RuntimeError("a and b must be fp8 e4m3fn")
+    if a.dim() != 2 or b.dim() != 2 or a.size(1) != b.size(1):
+        raise RuntimeError("a and b must be 2D with matching inner dim")
+    if a.device != b.device:
+        raise RuntimeError("a and b must be on the same device")
+    a_c, b_c = a.contiguous(), b.contiguous()
+    m, k = a_c.shape
+    n = b_c.size(0)
+    if k % 128 or k == 0:
+        raise RuntimeError("K must be a positive multiple of 128")
+    kb = k // 128
+    sa = _check_vec(sa, a, m * kb, "sa")
+    sb = _check_vec(sb, a, ((n + 127) // 128) * kb, "sb")
+    if bias is not None:
+        if not (bias.is_cuda and bias.device == a.device and bias.dtype == torch.bfloat16
+                and bias.numel() == n):
+            raise RuntimeError("bias must be CUDA bf16 with shape [N]")
+        bias = bias.contiguous()
+    with torch.cuda.device(a.device):
+        out = torch.empty((m, n), device=a.device, dtype=torch.bfloat16)
+        if m and n:
+            _check(lib.astrai_w8a8_gemm_fp8_block128(
+                a_c.data_ptr(), b_c.data_ptr(), sa.data_ptr(), sb.data_ptr(), _ptr(bias),
+                out.data_ptr(), m, n, k, _stream(a)), lib)
+    return out

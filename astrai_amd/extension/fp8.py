@@ -1,0 +1,309 @@
+"""FP8 scaling policy and ``aten::linear`` integration -- the counterpart of the
+reference's ``astrai/extension/fp8.py`` with the same public names:
+
+``FP8_MAX``, ``FP8Format``, ``FP8Recipe``, ``DelayedScaling``, ``DynamicScaling``,
+``FP8TensorMeta``, ``FP8State``, ``fp8_state``, ``fp8_autocast``,
+``fp8_linear_forward``, ``fp8_linear_backward``, ``fp8_linear_enable``,
+``fp8_linear_enabled``.
+
+Usage (unchanged from the reference)::
+
+    from astrai_amd.extension.fp8 import fp8_autocast
+    with fp8_autocast(enabled=True, fp8_format="hybrid"):
+        logits = model(input_ids)      # every F.linear on bf16 GPU tensors -> fp8 kernels
+
+Scales are quantization steps derived from amax: ``scale = amax / FP8_MAX[fmt] /
+2**margin``, floored at 1e-12 (fp8.py:87-89,103-105). All policy arithmetic
+stays on the device as tiny tensor ops; nothing here reads a value back to the
+host, so the path stays stream-ordered and graph-capturable.
+"""
+
+from contextlib import contextmanager
+from dataclasses import dataclass
+from enum import Enum
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from astrai_amd.extension import dispatch
+from astrai_amd.extension.ops.fp8 import (
+    linear_backward_fp8,
+    linear_forward_fp8,
+    mm_fp8,
+    quantize_bf16,
+)
+
+FP8_MAX = {"e4m3": 448.0, "e5m2": 57344.0}
+E4M3_MAX = FP8_MAX["e4m3"]
+_FLOOR = 1e-12
+
+
+class FP8Format(str, Enum):
+    """Format per direction; HYBRID = E4M3 forward, E5M2 backward (fp8.py:47-58)."""
+
+    E4M3 = "e4m3"
+    E5M2 = "e5m2"
+    HYBRID = "hybrid"
+
+    def fwd(self) -> str:
+        return "e4m3" if self is FP8Format.HYBRID else self.value
+
+    def bwd(self) -> str:
+        return "e5m2" if self is FP8Format.HYBRID else self.value
+
+
+def _step(peak: torch.Tensor, fmt: str, margin: int) -> torch.Tensor:
+    return ((peak / FP8_MAX[fmt]) / (2**margin)).clamp_min(_FLOOR)
+
+
+class FP8Recipe:
+    """Maps an amax window to a quantization step (fp8.py:61-76)."""
+
+    history_len: int = 16
+    margin: int = 0
+
+    def scale_from_history(self, amax: torch.Tensor, fmt: str) -> torch.Tensor:
+        raise NotImplementedError
+
+
+@dataclass
+class DelayedScaling(FP8Recipe):
+    """Max over the last ``history_len`` recorded amax values (fp8.py:79-92)."""
+
+    history_len: int = 16
+    margin: int = 0
+
+    def scale_from_history(self, amax: torch.Tensor, fmt: str) -> torch.Tensor:
+        return _step(amax.max(), fmt, self.margin)
+
+
+@dataclass
+class DynamicScaling(FP8Recipe):
+    """Scale from the amax of the tensor being quantized right now (fp8.py:95-108)."""
+
+    history_len: int = 1
+    margin: int = 0
+
+    def scale_from_history(self, amax: torch.Tensor, fmt: str) -> torch.Tensor:
+        return _step(amax.max(), fmt, self.margin)
+
+
+class _AmaxRing:
+    """One operand's amax history, write cursor, derived step and seeded flag."""
+
+    __slots__ = ("hist", "idx", "scale", "seeded")
+
+    def __init__(self, device: torch.device, n: int):
+        self.hist = torch.ones(n, device=device, dtype=torch.float32)
+        self.scale = torch.ones(1, device=device, dtype=torch.float32)
+        self.idx = 0
+        self.seeded = False
+
+    def push(self, amax: torch.Tensor, recipe: FP8Recipe, fmt: str) -> None:
+        # record first, then refresh: the step used next reflects amax seen so far
+        self.hist[self.idx] = amax.reshape(())
+        self.idx = (self.idx + 1) % self.hist.numel()
+        self.scale.copy_(recipe.scale_from_history(self.hist, fmt))
+
+    def seed(self, t: torch.Tensor, recipe: FP8Recipe, fmt: str) -> None:
+        self.hist.fill_(t.abs().amax().to(torch.float32).clamp_min(_FLOOR))
+        self.scale.copy_(recipe.scale_from_history(self.hist, fmt))
+        self.seeded = True
+
+
+def _ring_property(ring: str, field: str):
+    def fget(self):
+        return getattr(getattr(self, ring), field)
+
+    def fset(self, value):
+        setattr(getattr(self, ring), field, value)
+
+    return property(fget, fset)
+
+
+class FP8TensorMeta:
+    """Per-weight scaling state: rings for weight / activation / gradient
+    (fp8.py:111-190). Attribute names match the reference
+    (``w_hist, w_idx, w_scale, w_init`` and the x_/g_ twins)."""
+
+    def __init__(self, device: torch.device, recipe: FP8Recipe):
+        self.recipe = recipe
+        n = recipe.history_len
+        self._w = _AmaxRing(device, n)
+        self._x = _AmaxRing(device, n)
+        self._g = _AmaxRing(device, n)
+
+    w_hist, w_idx = _ring_property("_w", "hist"), _ring_property("_w", "idx")
+    w_scale, w_init = _ring_property("_w", "scale"), _ring_property("_w", "seeded")
+    x_hist, x_idx = _ring_property("_x", "hist"), _ring_property("_x", "idx")
+    x_scale, x_init = _ring_property("_x", "scale"), _ring_property("_x", "seeded")
+    g_hist, g_idx = _ring_property("_g", "hist"), _ring_property("_g", "idx")
+    g_scale, g_init = _ring_property("_g", "scale"), _ring_property("_g", "seeded")
+
+    def update_w(self, amax: torch.Tensor, fmt: str) -> None:
+        self._w.push(amax, self.recipe, fmt)
+
+    def update_x(self, amax: torch.Tensor, fmt: str) -> None:
+        self._x.push(amax, self.recipe, fmt)
+
+    def update_g(self, amax: torch.Tensor, fmt: str) -> None:
+        self._g.push(amax, self.recipe, fmt)
+
+    def init_w(self, w: torch.Tensor, fmt: str) -> None:
+        self._w.seed(w, self.recipe, fmt)
+
+    def init_x(self, x: torch.Tensor, fmt: str) -> None:
+        self._x.seed(x, self.recipe, fmt)
+
+    def init_g(self, g: torch.Tensor, fmt: str) -> None:
+        self._g.seed(g, self.recipe, fmt)
+
+
+class FP8State:
+    """Process-global switch, recipe, format and the per-weight metas (fp8.py:193-213).
+    Global rather than thread-local because autograd's backward runs on engine threads."""
+
+    def __init__(self):
+        self.enabled = False
+        self.recipe: FP8Recipe = DelayedScaling()
+        self.fp8_format: FP8Format = FP8Format.HYBRID
+        self._metas: Dict[Tuple, FP8TensorMeta] = {}
+        self._last_device: Optional[torch.device] = None
+
+    def get_weight_meta(self, w: torch.Tensor) -> FP8TensorMeta:
+        key = (w.data_ptr(), w.shape, w.dtype)
+        meta = self._metas.get(key)
+        if meta is None:
+            if self._last_device is None:
+                self._last_device = w.device
+            meta = self._metas[key] = FP8TensorMeta(w.device, self.recipe)
+        return meta
+
+    def reset(self) -> None:
+        self.enabled = False
+        self._metas.clear()
+        self._last_device = None
+
+
+_state = FP8State()
+
+
+def fp8_state() -> FP8State:
+    return _state
+
+
+@contextmanager
+def fp8_autocast(
+    enabled: bool = True,
+    update_interval: int = 16,
+    recipe: Optional[FP8Recipe] = None,
+    fp8_format: str = "hybrid",
+    margin: int = 0,
+):
+    """Route ``aten::linear`` through the fp8 kernels inside the block; the
+    previous (enabled, recipe, format) triple is restored on exit (fp8.py:226-262).
+    ``update_interval`` / ``margin`` parametrise the default delayed recipe."""
+    st = fp8_state()
+    saved = (st.enabled, st.recipe, st.fp8_format)
+    st.enabled = enabled
+    st.recipe = recipe if recipe is not None else DelayedScaling(update_interval, margin)
+    st.fp8_format = FP8Format(fp8_format)
+    try:
+        yield
+    finally:
+        st.enabled, st.recipe, st.fp8_format = saved
+
+
+def _dynamic_scale(t: torch.Tensor, recipe: FP8Recipe, fmt: str) -> torch.Tensor:
+    amax = t.abs().amax().to(torch.float32).clamp_min(_FLOOR)
+    return recipe.scale_from_history(amax, fmt)
+
+
+def fp8_linear_forward(x: torch.Tensor, w: torch.Tensor, bias=None):
+    """Scaled fp8 linear forward (fp8.py:275-305).
+
+    Dynamic scaling: measure both operands, quantize, pre-quantized GEMM to bf16,
+    then add the bias in bf16 (two roundings, as the reference does). Delayed
+    scaling: quantize with the rings' current steps inside the fused forward,
+    then push the returned amax values."""
+    st = fp8_state()
+    fmt = st.fp8_format.fwd()
+    meta = st.get_weight_meta(w)
+    if not meta.w_init:
+        meta.init_w(w, fmt)
+    if isinstance(st.recipe, DynamicScaling):
+        x2 = x.reshape(-1, w.size(1))
+        sx = _dynamic_scale(x2, st.recipe, fmt)
+        sw = _dynamic_scale(w, st.recipe, fmt)
+        x8, _ = quantize_bf16(x2, sx, fmt)
+        w8, _ = quantize_bf16(w, sw, fmt)
+        out = mm_fp8(x8, w8, sx, sw).reshape(*x.shape[:-1], w.size(0))
+        if bias is not None and bias.numel():
+            out = out + bias
+        return out
+    if not meta.x_init:
+        meta.init_x(x, fmt)
+    out, amax_x, amax_w = linear_forward_fp8(x, w, bias, meta.x_scale, meta.w_scale)
+    meta.update_x(amax_x, fmt)
+    meta.update_w(amax_w, fmt)
+    return out
+
+
+def fp8_linear_backward(g: torch.Tensor, x: torch.Tensor, w: torch.Tensor, masks):
+    """Scaled fp8 linear backward (fp8.py:308-330): gradient quantized once in the
+    backward format, dX and dW GEMMs share it."""
+    st = fp8_state()
+    fmt = st.fp8_format.bwd()
+    meta = st.get_weight_meta(w)
+    dynamic = isinstance(st.recipe, DynamicScaling)
+    if dynamic:
+        sg = _dynamic_scale(g, st.recipe, fmt)
+        sw = _dynamic_scale(w, st.recipe, fmt)
+        sx = _dynamic_scale(x, st.recipe, fmt)
+    else:
+        if not meta.g_init:
+            meta.init_g(g, fmt)
+        sg, sw, sx = meta.g_scale, meta.w_scale, meta.x_scale
+    gx, gw, gb, amax_g = linear_backward_fp8(g, x, w, masks, sg, sw, sx, fmt)
+    if not dynamic:
+        meta.update_g(amax_g, fmt)
+    return gx, gw, gb
+
+
+def fp8_linear_enable(enabled: bool = True) -> None:
+    fp8_state().enabled = enabled
+
+
+def fp8_linear_enabled() -> bool:
+    return fp8_state().enabled
+
+
+def _fp8_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Only the contraction must line up; ragged M / N are handled by the kernels
+    (fp8.py:348-356)."""
+    return x.dim() >= 2 and w.dim() == 2 and x.size(-1) == w.size(1)
+
+
+def _fp8_handler(x, w, bias):
+    if (
+        fp8_linear_enabled()
+        and x.dtype == torch.bfloat16
+        and w.dtype == torch.bfloat16
+        and _fp8_supported(x, w)
+    ):
+        return fp8_linear_forward(x, w, bias)
+    return None
+
+
+def _fp8_backward_handler(input_tensor, grad_output, weight, output_mask):
+    if (
+        fp8_linear_enabled()
+        and weight.dtype == torch.bfloat16
+        and _fp8_supported(grad_output, weight)
+    ):
+        return fp8_linear_backward(grad_output, input_tensor, weight, list(output_mask))
+    return None
+
+
+# importing this module installs the aten::linear override (fp8.py:404-406)
+dispatch.register_handler(_fp8_handler, _fp8_backward_handler)

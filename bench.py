@@ -1,0 +1,281 @@
+"""Benchmark of the quantized linear GEMM path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one launch of the pre-quantized fp8 e4m3fn per-tensor GEMM of
+BASELINE config 1 (A[4096,4096] . B[4096,4096]^T, fp32 accumulate, bf16 out),
+operands already resident in HBM. Prints ONE JSON line: the headline value is
+that GEMM's TFLOP/s; `roofline` prices the same kernel against the dense fp8
+MFMA peak; `cpu_baseline` is the CPU oracle timed on this host in the same run;
+`extra` carries the other BASELINE shapes (int8 GEMM, decode GEMV GB/s, block
+fp8, config 0 latency).
+"""
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP8_TFLOPS = 5000.0   # MI355X dense fp8 MFMA
+PEAK_INT8_TOPS = 5000.0    # MI355X dense int8 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+
+def _event_time_ms(fn, iters, warmup):
+    """Average duration of `fn` (launches on torch's current stream) over `iters`
+    back-to-back launches, by HIP events on that stream."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def _graph_time_ms(launch, n_launch, replays, warm_replays=2):
+    """Average per-launch duration with the launches captured in one HIP graph
+    (removes host launch overhead for kernels of a few microseconds)."""
+    import torch
+
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        for i in range(min(n_launch, 3)):
+            launch(i)
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for i in range(n_launch):
+            launch(i)
+    for _ in range(warm_replays):
+        g.replay()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(replays):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / (replays * n_launch)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-extra", action="store_true", help="headline kernel only")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU's share of the path: run with --gpus 1 "
+                 "(no multi-GPU leg exists; the sharding is described in DESIGN.md)")
+
+    import torch
+
+    from astrai_amd.extension import _cabi
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs the MI355X (no CPU fallback exists)")
+    lib = _cabi.load()
+    if lib is None:
+        sys.exit(f"HIP library missing: {_cabi.load_error()}")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def check(rc):
+        if rc:
+            raise RuntimeError(lib.astrai_w8a8_last_error().decode())
+
+    # ---------------- headline: config 1, fp8 per-tensor 4096^3 ----------------
+    M = N = K = 4096
+    g = torch.Generator().manual_seed(1)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    b = torch.randn(N, K, generator=g).to(torch.bfloat16)
+    sa = (a.abs().amax().float() / 448.0).reshape(1)
+    sb = (b.abs().amax().float() / 448.0).reshape(1)
+    a8_cpu = (a.float() / sa).to(torch.float8_e4m3fn)
+    b8_cpu = (b.float() / sb).to(torch.float8_e4m3fn)
+    a8, b8 = a8_cpu.to(dev), b8_cpu.to(dev)
+    sa_d, sb_d = sa.to(dev), sb.to(dev)
+    out = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
+
+    def step():
+        check(lib.astrai_w8a8_gemm_fp8_pt(a8.data_ptr(), b8.data_ptr(), sa_d.data_ptr(),
+                                          sb_d.data_ptr(), None, None, out.data_ptr(),
+                                          M, N, K, 0, 0, stream))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    flop = 2.0 * M * N * K
+    value = flop / (ms_per_step * 1e-3) / 1e12
+
+    kern_ms = _event_time_ms(step, args.steps, 5)
+    achieved = flop / (kern_ms * 1e-3) / 1e12
+    roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP8_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP8_TFLOPS, 4),
+                "traffic": None, "kernel": "gemm_tiled_kernel<OpF8<e4m3>,256x256,per-tensor>",
+                "avg_launch_us": round(kern_ms * 1e3, 2)}
+
+    # ---------------- CPU baseline: the oracle on this host ----------------
+    cpu_baseline = None
+    if not args.no_cpu:
+        from oracle import w8a8_oracle as O
+
+        cores = min(os.cpu_count() or 1, 16)
+        torch.set_num_threads(cores)
+        O.fp8_gemm(a8_cpu[:256], b8_cpu, sa, sb)  # warm-up
+        trials = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            O.fp8_gemm(a8_cpu, b8_cpu, sa, sb)
+            trials.append(time.perf_counter() - t0)
+        med = sorted(trials)[1]
+        cpu_baseline = {"value": round(flop / med / 1e12, 4), "unit": "TFLOP/s", "cores": cores,
+                        "kind": "port",
+                        "sample": "full config-1 GEMM (4096^3, fp8 upcast + fp32 matmul + scale -> bf16), "
+                                  "median of 3 after 1 warm-up", "ms": round(med * 1e3, 1)}
+
+    extra = {}
+    if not args.no_extra:
+        # ---- int8 4096^3 through the tiled kernel
+        ai = torch.randint(-127, 128, (M, K), dtype=torch.int8).to(dev)
+        bi = torch.randint(-127, 128, (N, K), dtype=torch.int8).to(dev)
+        sxi = torch.rand(M, device=dev) + 0.5
+        swi = torch.rand(N, device=dev) + 0.5
+
+        def step_i8():
+            check(lib.astrai_w8a8_gemm_int8_ptpc_tiled(ai.data_ptr(), bi.data_ptr(), sxi.data_ptr(),
+                                                       swi.data_ptr(), None, out.data_ptr(),
+                                                       M, N, K, 0, stream))
+
+        ms = _event_time_ms(step_i8, 100, 10)
+        tops = flop / (ms * 1e-3) / 1e12
+        extra["int8_gemm_4096"] = {"us": round(ms * 1e3, 2), "TOP/s": round(tops, 1),
+                                   "frac_mfma_peak": round(tops / PEAK_INT8_TOPS, 4)}
+
+        # ---- fp8 per-tensor with bias epilogue
+        bias = (torch.randn(N) * 0.1).to(torch.bfloat16).to(dev)
+
+        def step_bias():
+            check(lib.astrai_w8a8_gemm_fp8_pt(a8.data_ptr(), b8.data_ptr(), sa_d.data_ptr(),
+                                              sb_d.data_ptr(), None, bias.data_ptr(), out.data_ptr(),
+                                              M, N, K, 0, 0, stream))
+
+        ms = _event_time_ms(step_bias, 100, 10)
+        extra["fp8_gemm_4096_bias"] = {"us": round(ms * 1e3, 2),
+                                       "TFLOP/s": round(flop / (ms * 1e-3) / 1e12, 1)}
+        del ai, bi
+
+        # ---- config 3: block-scaled fp8 8192 x 2048 x 7168
+        M3, N3, K3 = 8192, 2048, 7168
+        a3 = torch.randn(M3, K3, device=dev).clamp(-3, 3).to(torch.float8_e4m3fn)
+        b3 = torch.randn(N3, K3, device=dev).clamp(-3, 3).to(torch.float8_e4m3fn)
+        sa3 = torch.rand(M3, K3 // 128, device=dev) + 0.5
+        sb3 = torch.rand(N3 // 128, K3 // 128, device=dev) + 0.5
+        out3 = torch.empty(M3, N3, device=dev, dtype=torch.bfloat16)
+
+        def step_blk():
+            check(lib.astrai_w8a8_gemm_fp8_block128(a3.data_ptr(), b3.data_ptr(), sa3.data_ptr(),
+                                                    sb3.data_ptr(), None, out3.data_ptr(),
+                                                    M3, N3, K3, stream))
+
+        ms = _event_time_ms(step_blk, 50, 5)
+        f3 = 2.0 * M3 * N3 * K3
+        extra["fp8_block128_8192x2048x7168"] = {
+            "us": round(ms * 1e3, 2), "TFLOP/s": round(f3 / (ms * 1e-3) / 1e12, 1),
+            "frac_mfma_peak": round(f3 / (ms * 1e-3) / 1e12 / PEAK_FP8_TFLOPS, 4)}
+        del a3, b3, out3
+
+        # ---- config 2: decode GEMV, weights rotated through a ring larger than the
+        # 256 MB Infinity Cache so that every launch streams from HBM
+        N2, K2 = 11008, 4096
+        ring = [torch.randint(-127, 128, (N2, K2), dtype=torch.int8, device=dev) for _ in range(10)]
+        sw2 = torch.rand(N2, device=dev) + 0.5
+        gemv = {}
+        for m in (1, 4, 16, 64):
+            x2 = torch.randint(-127, 128, (m, K2), dtype=torch.int8, device=dev)
+            sx2 = torch.rand(m, device=dev) + 0.5
+            y2 = torch.empty(m, N2, device=dev, dtype=torch.bfloat16)
+
+            def launch(i, x2=x2, sx2=sx2, y2=y2, m=m):
+                w = ring[i % len(ring)]
+                check(lib.astrai_w8a8_gemm_int8_ptpc(
+                    x2.data_ptr(), w.data_ptr(), sx2.data_ptr(), sw2.data_ptr(), None,
+                    y2.data_ptr(), m, N2, K2, 0, torch.cuda.current_stream().cuda_stream))
+
+            ms = _graph_time_ms(launch, 40, 10)
+            nbytes = N2 * K2 + m * K2 + 2 * m * N2 + 4 * N2 + 4 * m
+            gbs = nbytes / (ms * 1e-3) / 1e9
+            ms1 = _graph_time_ms(lambda i: launch(0), 40, 10)
+            gemv[f"M{m}"] = {"us": round(ms * 1e3, 2), "GB/s": round(gbs, 0),
+                             "frac_hbm_peak": round(gbs / PEAK_HBM_GBS, 4),
+                             "single_buffer_cache_resident_us": round(ms1 * 1e3, 2)}
+        extra["int8_gemv_11008x4096_hbm_ring"] = gemv
+        del ring
+
+        # ---- config 0: 16 x 2048 x 2048 int8 linear (launch-latency bound)
+        x0 = torch.randint(-127, 128, (16, 2048), dtype=torch.int8, device=dev)
+        w0 = torch.randint(-127, 128, (2048, 2048), dtype=torch.int8, device=dev)
+        s0 = torch.rand(16, device=dev)
+        s1 = torch.rand(2048, device=dev)
+        y0 = torch.empty(16, 2048, device=dev, dtype=torch.bfloat16)
+
+        def launch0(i):
+            check(lib.astrai_w8a8_gemm_int8_ptpc(x0.data_ptr(), w0.data_ptr(), s0.data_ptr(),
+                                                 s1.data_ptr(), None, y0.data_ptr(), 16, 2048, 2048,
+                                                 0, torch.cuda.current_stream().cuda_stream))
+
+        ms = _graph_time_ms(launch0, 40, 10)
+        extra["int8_config0_16x2048x2048"] = {"us": round(ms * 1e3, 2)}
+        if not args.no_cpu:
+            from oracle import w8a8_oracle as O
+
+            xc, wc, _ = O.make_inputs(0, 16, 2048, 2048)
+            wq, sw = O.int8_quantize_rows(wc)
+            O.int8_linear(xc, wq, sw)
+            ts = []
+            for _ in range(5):
+                t0 = time.perf_counter()
+                O.int8_linear(xc, wq, sw)
+                ts.append(time.perf_counter() - t0)
+            extra["int8_config0_16x2048x2048"]["cpu_oracle_ms"] = round(sorted(ts)[2] * 1e3, 2)
+
+    line = {
+        "metric": "W8A8 GEMM TFLOPS/TOPS + % MFMA peak; decode GEMV GB/s + % HBM peak (1 GPU)",
+        "value": round(value, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3fn", "data": "synthetic",
+        "config": {"workload": "BASELINE config 1: fp8 e4m3fn per-tensor GEMM, M=N=K=4096, "
+                               "fp32 accumulate, bf16 out, seed 1"},
+        "roofline": roofline, "cpu_baseline": cpu_baseline, "extra": extra,
+        "host": {"cpu_count": os.cpu_count(), "torch": torch.__version__},
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

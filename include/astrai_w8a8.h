@@ -1,0 +1,151 @@
+/*
+ * astrai_w8a8 -- C ABI of the gfx950 (MI355X) backend for AstrAI's quantized
+ * linear-layer GEMM path.
+ *
+ * These entry points are what the reference's `fp8_mm` pybind module
+ * (csrc/kernels/fp8/mm.cu:350-369) binds, restated as a plain C ABI: raw device
+ * pointers, sizes, a HIP stream, an int status. The host adapter
+ * (astrai_amd/extension/_cabi.py) owns tensor checks and output allocation, as
+ * the reference binding does (mm.cu:99-126,128-184,186-234).
+ *
+ * Conventions shared by every call
+ *   - All pointers are device pointers on the current HIP device, 16-byte
+ *     aligned, into contiguous row-major storage. Nothing is allocated, freed,
+ *     or synchronised; every launch is asynchronous on `stream` (a hipStream_t
+ *     passed as void*; NULL = the default stream) and reads its scales on the
+ *     device, so the calls are HIP-graph capturable
+ *     (reference: at::cuda::getCurrentCUDAStream(), mm.cu:108-109,147-148).
+ *   - A scale is the quantization STEP: q = x / scale, dequantization multiplies
+ *     by it (astrai/extension/ops/fp8.py:10-13).
+ *   - GEMMs are "NT": A is [M,K], B is [N,K] (the weight layout, no transpose),
+ *     both K-contiguous; out is [M,N] (mm.cu:150-152).
+ *   - Return value: ASTRAI_W8A8_OK or an error code; the message for the calling
+ *     thread's last error is available from astrai_w8a8_last_error().
+ */
+#ifndef ASTRAI_W8A8_H
+#define ASTRAI_W8A8_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ASTRAI_W8A8_ABI_VERSION 1
+
+/* status codes */
+#define ASTRAI_W8A8_OK 0
+#define ASTRAI_W8A8_BAD_ARG 1       /* null pointer, negative size, bad enum  */
+#define ASTRAI_W8A8_UNSUPPORTED 2   /* shape outside what the kernels accept  */
+#define ASTRAI_W8A8_LAUNCH_FAILED 3 /* hipGetLastError() after the launch     */
+
+/* fp8 formats: FP8Format in csrc/kernels/fp8/common.h:10-13 */
+#define ASTRAI_W8A8_E4M3 0 /* OCP e4m3fn, max 448 */
+#define ASTRAI_W8A8_E5M2 1 /* OCP e5m2, max 57344 */
+
+/* output element types */
+#define ASTRAI_W8A8_OUT_BF16 0
+#define ASTRAI_W8A8_OUT_E4M3 1 /* fp8 GEMM only; needs out_scale (mm.cu:152-161) */
+#define ASTRAI_W8A8_OUT_ACC 2  /* raw accumulator: int32 (int8 GEMM) / fp32 (fp8 GEMM) */
+
+/* ABI version of the loaded library (== ASTRAI_W8A8_ABI_VERSION at build time). */
+int astrai_w8a8_abi_version(void);
+
+/* Message of the calling thread's most recent failing call ("" if none). */
+const char* astrai_w8a8_last_error(void);
+
+/*
+ * bf16 -> fp8 quantize with fused amax.
+ * Replaces quantize_bf16 (csrc/kernels/fp8/mm.cu:99-126) and
+ * fp8_quantize_kernel (csrc/kernels/fp8/gemm.cuh:128-158).
+ *   x8[i]  = sat_fp8(float(x[i]) / *scale)   (true division, as the CPU kernel
+ *            astrai/extension/ops/fp8.py:80; saturating like the device kernel)
+ *   *amax  = max(*amax, max_i |x[i]|) over the raw values. The caller zeroes
+ *            *amax beforehand (the reference binding does, mm.cu:115); NULL skips it.
+ */
+int astrai_w8a8_quantize_bf16_fp8(const void* x_bf16, void* x8, const float* scale,
+                                  float* amax, int64_t total, int fmt, void* stream);
+
+/*
+ * bf16 -> int8, symmetric, one scale per row (per token for activations, per
+ * output channel for weights). No counterpart in the reference (it has no int8
+ * path); same conventions as the fp8 quantizer.
+ *   s[r]    = max(max_k |x[r,k]|, 1e-12) / 127
+ *   xq[r,k] = clamp(round_half_even(float(x[r,k]) / s[r]), -127, 127)
+ */
+int astrai_w8a8_quantize_bf16_int8_rows(const void* x_bf16, void* xq, float* s,
+                                        int64_t rows, int64_t k, void* stream);
+
+/*
+ * bf16 -> e4m3fn with one scale per 1x128 K-group (activations) or per 128x128
+ * block (weights). No counterpart in the reference. K must be a multiple of 128.
+ *   act:    sa[m,kb]  = max(max |x[m,128kb..128kb+127]|, 1e-12) / 448,   sa is [M, K/128]
+ *   weight: sb[nb,kb] = max(max |w[128nb.., 128kb..]|, 1e-12) / 448,     sb is [ceil(N/128), K/128]
+ */
+int astrai_w8a8_quantize_bf16_fp8_block128_act(const void* x_bf16, void* x8, float* sa,
+                                               int64_t m, int64_t k, void* stream);
+int astrai_w8a8_quantize_bf16_fp8_block128_weight(const void* w_bf16, void* w8, float* sb,
+                                                  int64_t n, int64_t k, void* stream);
+
+/*
+ * Pre-quantized fp8 GEMM with per-tensor scales.
+ * Replaces mm_fp8 (csrc/kernels/fp8/mm.cu:128-184), fp8_pq_gemm_kernel
+ * (gemm.cuh:447-619) and, with `bias`, the epilogue of fp8_fused_gemm_kernel
+ * (gemm.cuh:405-435).
+ *   acc[m,n] = sum_k a8[m,k] * b8[n,k]            fp32 accumulation
+ *   OUT_BF16: out = bf16(acc * *sa * *sb + bias[n])   (bias bf16 [N] or NULL; one rounding)
+ *   OUT_E4M3: out = sat_e4m3(acc * *sa * *sb * *out_scale)   (bias must be NULL)
+ *   OUT_ACC : out = acc as fp32 (parity/debug surface; scales ignored)
+ * a8 and b8 share `fmt`. Any M, N, K >= 1 is accepted.
+ */
+int astrai_w8a8_gemm_fp8_pt(const void* a8, const void* b8, const float* sa,
+                            const float* sb, const float* out_scale, const void* bias_bf16,
+                            void* out, int64_t m, int64_t n, int64_t k, int fmt,
+                            int out_dtype, void* stream);
+
+/*
+ * Pre-quantized e4m3fn GEMM with 128-block scales. No counterpart in the
+ * reference. K must be a multiple of 128.
+ *   out[m,n] = bf16( sum_kb (sum_{k in kb} a8[m,k]*b8[n,k]) * sa[m,kb] * sb[n/128,kb] + bias[n] )
+ */
+int astrai_w8a8_gemm_fp8_block128(const void* a8, const void* b8, const float* sa,
+                                  const float* sb, const void* bias_bf16, void* out,
+                                  int64_t m, int64_t n, int64_t k, void* stream);
+
+/*
+ * int8 W8A8 GEMM, per-token x per-channel scales. No counterpart in the
+ * reference; same NT layout and epilogue order as the fp8 path.
+ *   acc[m,n] = sum_k a[m,k] * b[n,k]              exact int32
+ *   OUT_BF16: out = bf16(float(acc) * sa[m] * sb[n] + bias[n])
+ *   OUT_ACC : out = acc as int32 (bit-exact parity surface)
+ * Picks the skinny kernel for M <= 64 when the shape allows it, the tiled MFMA
+ * kernel otherwise.
+ */
+int astrai_w8a8_gemm_int8_ptpc(const void* a, const void* b, const float* sa,
+                               const float* sb, const void* bias_bf16, void* out,
+                               int64_t m, int64_t n, int64_t k, int out_dtype,
+                               void* stream);
+
+/*
+ * The skinny (decode) int8 kernel on its own: same contract as
+ * astrai_w8a8_gemm_int8_ptpc but requires M <= 64 and K % 256 == 0, and
+ * returns ASTRAI_W8A8_UNSUPPORTED otherwise.
+ */
+int astrai_w8a8_gemv_int8_ptpc(const void* a, const void* b, const float* sa,
+                               const float* sb, const void* bias_bf16, void* out,
+                               int64_t m, int64_t n, int64_t k, int out_dtype,
+                               void* stream);
+
+/*
+ * The tiled MFMA int8 kernel on its own (no skinny dispatch), for tests and
+ * benchmarks that must name the kernel they measure.
+ */
+int astrai_w8a8_gemm_int8_ptpc_tiled(const void* a, const void* b, const float* sa,
+                                     const float* sb, const void* bias_bf16, void* out,
+                                     int64_t m, int64_t n, int64_t k, int out_dtype,
+                                     void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ASTRAI_W8A8_H */

@@ -1,0 +1,232 @@
+"""fp8 kernels vs the oracle with the reference's own shapes and tolerances
+(tests/extension/test_fp8_mma.py:42-198), plus 128-block scaling."""
+
+import pytest
+import torch
+
+from oracle import w8a8_oracle as O
+from tests.helpers import assert_bf16_close
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from astrai_amd.extension import get_module, is_available
+    from astrai_amd.extension.ops import fp8
+    assert is_available("fp8_mm")
+    return fp8
+
+
+def _scale(t):
+    return (t.abs().amax().float() / 448.0).clamp_min(1e-12).reshape(1)
+
+
+@pytest.mark.parametrize("m,n,k", [(16, 8, 32), (17, 9, 33), (31, 15, 64), (32, 48, 96)])
+def test_fused_fp8_mm_matches_explicit_quantization(ops, m, n, k):
+    # test_fp8_mma.py:42-61 (same seeds, same tolerance), expectation from the oracle
+    from astrai_amd.extension import get_module
+    print(f"case m={m} n={n} k={k}", flush=True)
+    torch.manual_seed(m + n + k)
+    a = torch.randn(m, k).to(torch.bfloat16)
+    b = torch.randn(n, k).to(torch.bfloat16)
+    sa, sb = _scale(a), _scale(b)
+    out = get_module("fp8_mm").fp8_mm(a.to(DEV), b.to(DEV), sa.to(DEV), sb.to(DEV))
+    a8, _ = O.fp8_quantize(a, sa, 0)
+    b8, _ = O.fp8_quantize(b, sb, 0)
+    expected = O.fp8_gemm(a8, b8, sa, sb)
+    assert out.dtype == torch.bfloat16 and out.shape == (m, n)
+    torch.testing.assert_close(out.cpu(), expected, atol=0.125, rtol=0.01)
+    assert_bf16_close(out, expected, what="fp8_mm")
+
+
+def test_linear_forward_with_bias_and_amax(ops):
+    # test_fp8_mma.py:88-116 forward half: seed 7, 19x13x37, bias, amax equalities
+    torch.manual_seed(7)
+    m, n, k = 19, 13, 37
+    x = torch.randn(m, k).to(torch.bfloat16)
+    w = torch.randn(n, k).to(torch.bfloat16)
+    _ = torch.randn(m, n)
+    bias = torch.randn(n).to(torch.bfloat16)
+    sx, sw = _scale(x), _scale(w)
+    out, ax, aw = ops.linear_forward_fp8(x.to(DEV), w.to(DEV), bias.to(DEV), sx.to(DEV), sw.to(DEV))
+    want, wax, waw = O.linear_forward_fp8(x, w, bias, sx, sw)
+    torch.testing.assert_close(out.cpu(), want, atol=0.125, rtol=0.01)
+    assert_bf16_close(out, want, what="linear_forward_fp8")
+    assert ax.item() == wax.item() and aw.item() == waw.item()
+    out3, _, _ = ops.linear_forward_fp8(x.reshape(1, m, k).to(DEV), w.to(DEV), None, sx.to(DEV), sw.to(DEV))
+    assert out3.shape == (1, m, n)
+
+
+def test_linear_backward_fp8_both_formats(ops):
+    # test_fp8_mma.py:88-145 backward halves
+    for seed, (m, n, k), fmt, gmul, tol in [(7, (19, 13, 37), "e4m3", 1.0, (0.125, 0.01)),
+                                            (5, (32, 16, 64), "e5m2", 10.0, (0.5, 0.05))]:
+        torch.manual_seed(seed)
+        x = torch.randn(m, k).to(torch.bfloat16)
+        w = torch.randn(n, k).to(torch.bfloat16)
+        g = (torch.randn(m, n) * gmul).to(torch.bfloat16)
+        sx, sw, sg = _scale(x), _scale(w), _scale(g)
+        if fmt == "e5m2":
+            sx, sw, sg = sx * 448 / 57344, sw * 448 / 57344, sg * 448 / 57344
+        gx, gw, gb, amax_g = ops.linear_backward_fp8(
+            g.to(DEV), x.to(DEV), w.to(DEV), [1, 1, 1], sg.to(DEV), sw.to(DEV), sx.to(DEV), fmt)
+        f = 1 if fmt == "e5m2" else 0
+        qg = O.fp8_quantize(g, sg, f)[0].float()
+        qw = O.fp8_quantize(w, sw, f)[0].float()
+        qx = O.fp8_quantize(x, sx, f)[0].float()
+        torch.testing.assert_close(gx.cpu(), (qg @ qw * sg * sw).to(torch.bfloat16), atol=tol[0], rtol=tol[1])
+        torch.testing.assert_close(gw.cpu(), (qg.t() @ qx * sg * sx).to(torch.bfloat16), atol=tol[0], rtol=tol[1])
+        torch.testing.assert_close(gb.cpu(), g.sum(0).to(torch.bfloat16))
+        assert amax_g.item() == g.abs().max().item()
+
+
+def test_mm_fp8_k4096_vs_float64_and_oracle(ops):
+    # test_fp8_mma.py:149-174: seed 11, 512x4096x4096, sa 2.5, sb 1.5, atol 6 / rtol .05 vs fp64
+    torch.manual_seed(11)
+    m, n, k = 512, 4096, 4096
+    a = torch.randn(m, k).to(torch.bfloat16)
+    b = torch.randn(n, k).to(torch.bfloat16)
+    sa, sb = torch.tensor([2.5]), torch.tensor([1.5])
+    a8, _ = ops.quantize_bf16(a.to(DEV), sa.to(DEV), "e4m3")
+    b8, _ = ops.quantize_bf16(b.to(DEV), sb.to(DEV), "e4m3")
+    out = ops.mm_fp8(a8, b8, sa.to(DEV), sb.to(DEV))
+    assert out.dtype == torch.bfloat16 and out.shape == (m, n)
+    ra8, _ = O.fp8_quantize(a, sa, 0)
+    rb8, _ = O.fp8_quantize(b, sb, 0)
+    assert torch.equal(a8.cpu().view(torch.uint8), ra8.view(torch.uint8))
+    ref64 = (ra8.double() @ rb8.double().t() * 2.5 * 1.5).to(torch.bfloat16)
+    torch.testing.assert_close(out.cpu(), ref64, atol=6.0, rtol=0.05)
+    assert_bf16_close(out, O.fp8_gemm(ra8, rb8, sa, sb), what="mm_fp8 k4096")
+
+
+def test_mm_fp8_fp8_output(ops):
+    # test_fp8_mma.py:177-198: seed 12, 256x128x64, scales 2 / 1 / .5
+    torch.manual_seed(12)
+    m, n, k = 256, 128, 64
+    a = torch.randn(m, k).to(torch.bfloat16)
+    b = torch.randn(n, k).to(torch.bfloat16)
+    sa, sb, os_ = torch.tensor([2.0]), torch.tensor([1.0]), torch.tensor([0.5])
+    a8, _ = O.fp8_quantize(a, sa, 0)
+    b8, _ = O.fp8_quantize(b, sb, 0)
+    out8 = ops.mm_fp8(a8.to(DEV), b8.to(DEV), sa.to(DEV), sb.to(DEV), out_dtype="e4m3", out_scale=os_.to(DEV))
+    assert out8.dtype == torch.float8_e4m3fn and out8.shape == (m, n)
+    want = O.fp8_gemm(a8, b8, sa, sb, 1, os_)
+    ref64 = (a8.double() @ b8.double().t() * 2.0 * 1.0 * 0.5).to(torch.bfloat16)
+    torch.testing.assert_close(out8.float().cpu().to(torch.bfloat16), ref64, atol=6.0, rtol=0.05)
+    # codes agree with the oracle except where the fp32 sum sits on an e4m3 rounding
+    # boundary (the MFMA's summation order differs from sgemm's): never more than one
+    # code step apart, and rarely
+    got_c, want_c = out8.cpu().view(torch.uint8).int(), want.view(torch.uint8).int()
+    diff = (got_c - want_c).abs()
+    assert diff.max().item() <= 1
+    assert (diff != 0).float().mean().item() < 0.01
+
+
+def test_reference_hand_vectors_on_device(ops, golden):
+    kat = golden("reference_kats.json")
+    k1, k2 = kat["mm_fp8_cpu"], kat["mm_fp8_fp8_out_cpu"]
+    a8 = torch.tensor(k1["a8"]).to(torch.float8_e4m3fn).to(DEV)
+    b8 = torch.tensor(k1["b8"]).to(torch.float8_e4m3fn).to(DEV)
+    sa, sb = torch.tensor([k1["sa"]], device=DEV), torch.tensor([k1["sb"]], device=DEV)
+    assert ops.mm_fp8(a8, b8, sa, sb).cpu().tolist() == k1["out_bf16"]
+    os_ = torch.tensor([k2["out_scale"]], device=DEV)
+    assert ops.mm_fp8(a8, b8, sa, sb, "e4m3", os_).float().cpu().tolist() == k2["out_e4m3"]
+
+
+@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("m,n,k", [(64, 64, 128), (129, 257, 272), (256, 256, 512), (300, 500, 1040)])
+def test_mm_fp8_both_formats_tile_edges(ops, fmt, m, n, k):
+    print(f"case fmt={fmt} m={m} n={n} k={k}", flush=True)
+    a, b, _ = O.make_inputs(1, m, n, k, w_std=1.0)
+    name = "e5m2" if fmt else "e4m3"
+    sa, sb = O.dynamic_scale(a, name).reshape(1), O.dynamic_scale(b, name).reshape(1)
+    a8, _ = O.fp8_quantize(a, sa, fmt)
+    b8, _ = O.fp8_quantize(b, sb, fmt)
+    out = ops.mm_fp8(a8.to(DEV), b8.to(DEV), sa.to(DEV), sb.to(DEV))
+    assert_bf16_close(out, O.fp8_gemm(a8, b8, sa, sb), what=f"mm_fp8 {name}")
+
+
+def test_mm_fp8_rejects_bad_arguments(ops):
+    a8 = torch.zeros(4, 16, dtype=torch.float8_e4m3fn, device=DEV)
+    b5 = torch.zeros(4, 16, dtype=torch.float8_e5m2, device=DEV)
+    one = torch.ones(1, device=DEV)
+    with pytest.raises(TypeError, match="matching fp8"):
+        ops.mm_fp8(a8, b5, one, one)                       # ops/fp8.py:109-112
+    with pytest.raises(RuntimeError, match="out_scale"):
+        ops.mm_fp8(a8, a8, one, one, out_dtype="e4m3")     # mm.cu:158
+    with pytest.raises(RuntimeError, match="float32 scalar"):
+        ops.mm_fp8(a8, a8, torch.ones(2, device=DEV), one)  # mm.cu:49-54
+    with pytest.raises(RuntimeError, match="inner dim"):
+        ops.mm_fp8(a8, a8[:, :8].contiguous(), one, one)
+    with pytest.raises(TypeError, match="bf16 input"):
+        ops.quantize_bf16(torch.zeros(4, device=DEV), one)
+
+
+def test_config1_sampled_rows_at_full_size(ops):
+    """BASELINE config 1 at 4096^3 with bias (seed 1): full-size launch, checked
+    against the oracle on a block of rows (the oracle's full sgemm is the CPU
+    baseline's job, not the test suite's)."""
+    a, b, bias = O.make_inputs(1, 4096, 4096, 4096, w_std=1.0, bias=True)
+    sa, sb = O.dynamic_scale(a).reshape(1), O.dynamic_scale(b).reshape(1)
+    a8, _ = O.fp8_quantize(a, sa, 0)
+    b8, _ = O.fp8_quantize(b, sb, 0)
+    from astrai_amd.extension import _cabi
+    out = _cabi.mm_fp8(a8.to(DEV), b8.to(DEV), sa.to(DEV), sb.to(DEV), 0, None, bias.to(DEV))
+    rows = torch.cat([torch.arange(0, 8), torch.arange(2040, 2056), torch.arange(4088, 4096)])
+    want = O.fp8_gemm_bias(a8[rows], b8, sa, sb, bias)
+    assert_bf16_close(out[rows], want, what="config1 rows")
+
+
+# ---- 128-block scaled ----
+
+@pytest.mark.parametrize("m,n,k", [(3, 130, 256), (64, 128, 128), (130, 200, 384), (257, 513, 1024)])
+def test_block128_gemm_small(m, n, k):
+    from astrai_amd.extension.ops import fp8_block as blk
+    print(f"case m={m} n={n} k={k}", flush=True)
+    x, w, _ = O.make_inputs(3, m, n, k, outlier_p=0.01)
+    x8, sa = O.fp8_quantize_act_block128(x)
+    w8, sb = O.fp8_quantize_weight_block128(w)
+    out = blk.mm_fp8_blockscaled(x8.to(DEV), w8.to(DEV), sa.to(DEV), sb.to(DEV))
+    assert_bf16_close(out, O.fp8_gemm_blockscaled(x8, w8, sa, sb), what="block128")
+
+
+def test_block128_golden_exact_rationals(golden):
+    from astrai_amd.extension.ops import fp8_block as blk
+    for c in golden("fp8_gemm_small.json")["block128"]:
+        a8 = torch.tensor(c["a"], dtype=torch.uint8).view(torch.float8_e4m3fn)
+        b8 = torch.tensor(c["b"], dtype=torch.uint8).view(torch.float8_e4m3fn)
+        sa, sb = torch.tensor(c["sa"]), torch.tensor(c["sb"])
+        exact = torch.tensor(c["exact"], dtype=torch.float64)
+        out = blk.mm_fp8_blockscaled(a8.to(DEV), b8.to(DEV), sa.to(DEV), sb.to(DEV))
+        assert_bf16_close(out, exact.to(torch.bfloat16), what="block128 exact")
+
+
+def test_block128_reduces_to_per_tensor(ops):
+    from astrai_amd.extension.ops import fp8_block as blk
+    x, w, _ = O.make_inputs(4, 96, 300, 512, w_std=1.0)
+    s = torch.tensor([0.03125])
+    a8, _ = O.fp8_quantize_saturating(x, s, 0)
+    b8, _ = O.fp8_quantize_saturating(w, s, 0)
+    sa = torch.full((96, 4), 0.03125)
+    sb = torch.full((3, 4), 0.03125)
+    got = blk.mm_fp8_blockscaled(a8.to(DEV), b8.to(DEV), sa.to(DEV), sb.to(DEV))
+    want = ops.mm_fp8(a8.to(DEV), b8.to(DEV), s.to(DEV), s.to(DEV))
+    assert_bf16_close(got, want.cpu(), what="block==tensor")
+
+
+def test_config3_shape_sampled_rows():
+    """BASELINE config 3 (seed 3): A[8192,7168], B[2048,7168] with 1% x20 outliers,
+    quantized on the device, GEMM on the device, checked on sampled rows."""
+    from astrai_amd.extension.ops import fp8_block as blk
+    x, w, _ = O.make_inputs(3, 8192, 2048, 7168, outlier_p=0.01)
+    x8, sa = blk.quantize_act_block128(x.to(DEV))
+    w8, sb = blk.quantize_weight_block128(w.to(DEV))
+    out = blk.mm_fp8_blockscaled(x8, w8, sa, sb)
+    rows = torch.cat([torch.arange(0, 4), torch.arange(4094, 4098), torch.arange(8188, 8192)])
+    rx8, rsa = O.fp8_quantize_act_block128(x[rows])
+    rw8, rsb = O.fp8_quantize_weight_block128(w)
+    assert torch.equal(x8[rows].cpu().view(torch.uint8), rx8.view(torch.uint8))
+    assert torch.equal(sb.cpu(), rsb)
+    assert_bf16_close(out[rows], O.fp8_gemm_blockscaled(rx8, rw8, rsa, rsb), what="config3 rows")

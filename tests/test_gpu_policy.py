@@ -1,0 +1,109 @@
+"""Policy level on the device: F.linear on bf16 GPU tensors is taken over by the
+fp8 / int8 handlers while enabled, and left to the stock kernel otherwise."""
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import w8a8_oracle as O
+from tests.helpers import assert_bf16_close
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def test_dynamic_scaling_linear_matches_oracle():
+    from astrai_amd.extension.fp8 import DynamicScaling, fp8_autocast, fp8_state
+    x, w, b = O.make_inputs(21, 24, 96, 160, w_std=1.0, bias=True)
+    x3 = x.reshape(2, 12, 160)
+    fp8_state().reset()
+    with fp8_autocast(enabled=True, recipe=DynamicScaling(), fp8_format="e4m3"):
+        y = F.linear(x3.to(DEV), w.to(DEV), b.to(DEV))
+    want = O.fp8_linear_dynamic(x3, w, b)
+    assert y.shape == (2, 12, 96) and y.dtype == torch.bfloat16
+    assert_bf16_close(y, want, what="dynamic fp8 linear")
+    # outside the context the stock kernel runs: result differs from the fp8 one
+    y_stock = F.linear(x3.to(DEV), w.to(DEV), b.to(DEV))
+    torch.testing.assert_close(y_stock.cpu().float(), (x3.float() @ w.float().t() + b.float()), atol=0.5, rtol=0.02)
+    assert not torch.equal(y_stock, y)
+
+
+def test_delayed_scaling_linear_seeds_then_tracks_amax():
+    from astrai_amd.extension.fp8 import fp8_autocast, fp8_state
+    x, w, _ = O.make_inputs(22, 32, 64, 128, w_std=1.0)
+    xd, wd = x.to(DEV), w.to(DEV)
+    st = fp8_state()
+    st.reset()
+    with fp8_autocast(enabled=True, update_interval=4, fp8_format="hybrid"):
+        y = F.linear(xd, wd)
+        meta = st.get_weight_meta(wd)
+        assert meta.w_init and meta.x_init
+        torch.testing.assert_close(meta.w_scale.cpu(), (w.abs().amax().float() / 448).reshape(1))
+        # first call: seeded scales == dynamic scales, so the result equals the dynamic path
+        want = O.fp8_linear_dynamic(x, w, None)
+        assert_bf16_close(y, want, what="delayed first step")
+        y2 = F.linear(xd * 4, wd)   # uses the step-1 scale for x: saturates, then ring picks up 4x
+        assert torch.isfinite(y2.float()).all()
+        torch.testing.assert_close(meta.x_scale.cpu(), ((x.float() * 4).abs().amax() / 448).reshape(1).to(torch.float32), rtol=1e-2, atol=0)
+    st.reset()
+
+
+def test_int8_autocast_linear_matches_oracle_and_caches_weights():
+    from astrai_amd.extension import w8a8
+    x, w, b = O.make_inputs(23, 10, 200, 512, bias=True)
+    wd = w.to(DEV)
+    w8a8.int8_state().reset()
+    with w8a8.int8_autocast(True):
+        y = F.linear(x.to(DEV), wd, b.to(DEV))
+        y2 = F.linear(x.to(DEV), wd)
+        assert len(w8a8.int8_state()._weights) == 1
+    wq, sw = O.int8_quantize_rows(w)
+    assert torch.equal(y.cpu().view(torch.int16), O.int8_linear(x, wq, sw, b).view(torch.int16))
+    assert torch.equal(y2.cpu().view(torch.int16), O.int8_linear(x, wq, sw, None).view(torch.int16))
+    # in-place weight update invalidates the cached quantization
+    with w8a8.int8_autocast(True):
+        wd.mul_(2)
+        y3 = F.linear(x.to(DEV), wd)
+    wq2, sw2 = O.int8_quantize_rows(w * 2)
+    assert torch.equal(y3.cpu().view(torch.int16), O.int8_linear(x, wq2, sw2, None).view(torch.int16))
+    w8a8.int8_state().reset()
+
+
+def test_guard_falls_through_for_other_dtypes():
+    from astrai_amd.extension import w8a8
+    x = torch.randn(4, 32, device=DEV)
+    w = torch.randn(8, 32, device=DEV)
+    with w8a8.int8_autocast(True):
+        y = F.linear(x, w)
+    torch.testing.assert_close(y, x @ w.t(), atol=1e-4, rtol=1e-4)
+
+
+def test_graph_capture_of_int8_linear_replays_correctly():
+    """The launches are stream-ordered and allocation-free on the C side, so a
+    linear call can be captured; every replay must equal the eager result."""
+    from astrai_amd.extension import w8a8
+    x, w, _ = O.make_inputs(24, 8, 1024, 1024)
+    xd, wd = x.to(DEV), w.to(DEV)
+    static_x = xd.clone()
+    w8a8.int8_state().reset()
+    with w8a8.int8_autocast(True):
+        eager = F.linear(static_x, wd).clone()
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            for _ in range(2):
+                F.linear(static_x, wd)
+        torch.cuda.current_stream().wait_stream(s)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_y = F.linear(static_x, wd)
+    for i in range(3):
+        static_x.copy_(xd * (i + 1))
+        graph.replay()
+        torch.cuda.synchronize()
+        with w8a8.int8_autocast(True):
+            want = F.linear(static_x, wd)
+        assert torch.equal(static_y, want), i
+    assert torch.equal(eager.cpu().view(torch.int16),
+                       O.int8_linear(x, *O.int8_quantize_rows(w)).view(torch.int16))
+    w8a8.int8_state().reset()

@@ -1,0 +1,121 @@
+"""Quantize kernels vs the oracle, bit-exact on codes (HIP path through the C ABI)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import w8a8_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+def _codes(t):
+    return t.cpu().contiguous().view(torch.uint8)
+
+
+@pytest.fixture(scope="module")
+def C():
+    from astrai_amd.extension import _cabi
+    assert _cabi.load() is not None, _cabi.load_error()
+    return _cabi
+
+
+@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("scale", [0.5, 0.0123, 3.0, 1e-3])
+def test_fp8_quantize_every_bf16_value(C, fmt, scale):
+    """All 65536 bf16 bit patterns: codes equal the saturating oracle wherever the
+    input is finite (RNE, subnormals, ties, saturation at the finite max)."""
+    print(f"case fmt={fmt} scale={scale}", flush=True)
+    bits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    x = torch.from_numpy(bits.view(np.int16).copy()).view(torch.bfloat16)
+    finite = torch.isfinite(x.float())
+    x = torch.where(finite, x, torch.zeros_like(x))
+    s = torch.tensor([scale])
+    want, want_amax = O.fp8_quantize_saturating(x, s, fmt)
+    got, amax = C.quantize_bf16(x.to(DEV), s.to(DEV), fmt)
+    assert got.dtype == want.dtype and got.shape == x.shape
+    assert torch.equal(_codes(got), _codes(want))
+    assert amax.shape == (1,) and amax.item() == want_amax.item()
+
+
+def test_fp8_quantize_reference_vector_scale_half(C, golden):
+    # tests/extension/test_fp8_mma.py:65-77
+    torch.manual_seed(3)
+    x = torch.randn(64, 128).to(torch.bfloat16)
+    scale = torch.tensor([golden("reference_kats.json")["quantize_scale"]])
+    from astrai_amd.extension.ops.fp8 import quantize_bf16
+    x8, amax = quantize_bf16(x.to(DEV), scale.to(DEV), "e4m3")
+    assert x8.dtype == torch.float8_e4m3fn and x8.shape == x.shape and amax.shape == (1,)
+    torch.testing.assert_close(amax.cpu(), x.abs().amax().float().reshape(1))
+    ref = (x.float() / 0.5).to(torch.float8_e4m3fn)
+    assert torch.equal(_codes(x8), _codes(ref))
+
+
+@pytest.mark.parametrize("shape", [(1,), (7,), (8,), (3, 5), (257, 33), (0, 16), (4096, 4096)])
+def test_fp8_quantize_shapes_tails_and_amax(C, shape):
+    print(f"case shape={shape}", flush=True)
+    g = torch.Generator().manual_seed(sum(shape))
+    x = (torch.randn(*shape, generator=g) * 2).to(torch.bfloat16)
+    s = O.dynamic_scale(x) if x.numel() else torch.tensor(1.0)
+    s = s.reshape(1)
+    got, amax = C.quantize_bf16(x.to(DEV), s.to(DEV), 0)
+    want, _ = O.fp8_quantize(x, s, 0)
+    assert torch.equal(_codes(got), _codes(want))
+    assert amax.item() == (x.abs().max().item() if x.numel() else 0.0)
+
+
+def test_fp8_quantize_noncontiguous_input(C):
+    x = torch.randn(64, 96).to(torch.bfloat16)
+    xt = x.to(DEV).t()
+    s = torch.tensor([0.25])
+    got, _ = C.quantize_bf16(xt, s.to(DEV), 0)
+    want, _ = O.fp8_quantize(x.t(), s, 0)
+    assert got.shape == (96, 64) and torch.equal(_codes(got), _codes(want))
+
+
+@pytest.mark.parametrize("rows,k", [(1, 8), (3, 24), (16, 2048), (5, 33), (2, 9000), (7, 16384), (64, 4096), (0, 32)])
+def test_int8_rows_bit_exact(C, rows, k):
+    print(f"case rows={rows} k={k}", flush=True)
+    g = torch.Generator().manual_seed(rows * 31 + k)
+    x = torch.randn(rows, k, generator=g).to(torch.bfloat16)
+    if rows > 1:
+        x[1].zero_()  # all-zero row: step = 1e-12/127, codes 0
+    got_q, got_s = C.quantize_int8_rows(x.to(DEV))
+    want_q, want_s = O.int8_quantize_rows(x)
+    assert got_q.shape == (rows, k) and got_s.shape == (rows, 1)
+    assert torch.equal(got_s.cpu(), want_s)
+    assert torch.equal(got_q.cpu(), want_q)
+
+
+def test_int8_rows_golden_ties(C, golden):
+    for c in golden("int8_small.json")["quantize_rows"]:
+        x = torch.tensor([c["x"]], dtype=torch.float32).to(torch.bfloat16)
+        q, s = C.quantize_int8_rows(x.to(DEV))
+        assert q.cpu()[0].tolist() == c["q"]
+        assert s.cpu().view(torch.int32).item() == c["scale_bits"]
+
+
+def test_int8_rows_3d_input_flattens_tokens(C):
+    x = torch.randn(2, 5, 64).to(torch.bfloat16)
+    q, s = C.quantize_int8_rows(x.to(DEV))
+    wq, ws = O.int8_quantize_rows(x.reshape(-1, 64))
+    assert q.shape == (10, 64) and torch.equal(q.cpu(), wq) and torch.equal(s.cpu(), ws)
+
+
+@pytest.mark.parametrize("m,k", [(1, 128), (5, 256), (130, 1024)])
+def test_block128_act_quantize(C, m, k):
+    x, _, _ = O.make_inputs(3, m, 8, k)
+    x8, sa = C.quantize_fp8_block128_act(x.to(DEV))
+    w8, ws = O.fp8_quantize_act_block128(x)
+    assert torch.equal(sa.cpu(), ws) and torch.equal(_codes(x8), _codes(w8))
+
+
+@pytest.mark.parametrize("n,k", [(128, 128), (200, 256), (1, 128), (257, 384)])
+def test_block128_weight_quantize(C, n, k):
+    _, w, _ = O.make_inputs(3, 4, n, k, outlier_p=0.01)
+    w8, sb = C.quantize_fp8_block128_weight(w.to(DEV))
+    r8, rs = O.fp8_quantize_weight_block128(w)
+    assert sb.shape == rs.shape and torch.equal(sb.cpu(), rs)
+    assert torch.equal(_codes(w8), _codes(r8))

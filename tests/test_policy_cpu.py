@@ -1,0 +1,142 @@
+"""Host logic that needs no GPU: registry, scaling recipes, autocast context,
+per-tensor meta, op-level argument errors -- the CPU-verifiable half of the
+reference's tests/extension/test_fp8_mma.py:206-259, against this backend."""
+
+import pytest
+import torch
+
+import astrai_amd.extension as ext
+from astrai_amd.extension import w8a8
+from astrai_amd.extension.fp8 import (
+    DelayedScaling,
+    DynamicScaling,
+    FP8Format,
+    FP8TensorMeta,
+    fp8_autocast,
+    fp8_state,
+)
+from astrai_amd.extension.ops import fp8 as ops_fp8
+from astrai_amd.extension.ops import fp8_block as ops_blk
+from astrai_amd.extension.ops import int8 as ops_int8
+
+
+def test_registry_names_and_modules():
+    assert "fp8_mm" in ext.KERNEL_NAMES and "int8_mm" in ext.KERNEL_NAMES
+    assert ext.is_available("fp8_mm")
+    assert not ext.is_available("no_such_kernel") and ext.get_module("no_such_kernel") is None
+    mod = ext.get_module("fp8_mm")
+    for name in ("fp8_mm", "quantize_bf16", "mm_fp8", "linear_forward_fp8", "linear_backward_fp8"):
+        assert callable(getattr(mod, name))  # csrc/kernels/fp8/mm.cu:350-369
+
+
+def test_recipe_scale_from_history(golden):
+    for r in golden("reference_kats.json")["recipe"]:
+        hist = torch.tensor(r["hist"])
+        rec = (DelayedScaling(history_len=len(r["hist"]), margin=r["margin"])
+               if len(r["hist"]) > 1 else DynamicScaling())
+        assert torch.allclose(rec.scale_from_history(hist, r["fmt"]), torch.tensor(r["scale"]))
+
+
+def test_fp8_format_enum():
+    assert FP8Format.HYBRID.fwd() == "e4m3" and FP8Format.HYBRID.bwd() == "e5m2"
+    assert FP8Format.E4M3.fwd() == FP8Format.E4M3.bwd() == "e4m3"
+    assert FP8Format.E5M2.fwd() == FP8Format.E5M2.bwd() == "e5m2"
+
+
+def test_fp8_autocast_context_nests_and_restores():
+    state = fp8_state()
+    prev = (state.enabled, state.recipe, state.fp8_format)
+    try:
+        with fp8_autocast(enabled=True, fp8_format="hybrid", update_interval=8):
+            assert state.enabled
+            assert isinstance(state.recipe, DelayedScaling) and state.recipe.history_len == 8
+            assert state.fp8_format is FP8Format.HYBRID
+            with fp8_autocast(enabled=True, recipe=DynamicScaling(), fp8_format="e4m3"):
+                assert isinstance(state.recipe, DynamicScaling)
+                assert state.fp8_format is FP8Format.E4M3
+            assert state.fp8_format is FP8Format.HYBRID
+        assert not state.enabled
+    finally:
+        state.enabled, state.recipe, state.fp8_format = prev
+
+
+def test_fp8_tensor_meta_delayed_update(golden):
+    kat = golden("reference_kats.json")["meta_update"]
+    meta = FP8TensorMeta(torch.device("cpu"), DelayedScaling(history_len=4, margin=0))
+    w = torch.randn(8, 8)
+    meta.init_w(w, "e4m3")
+    assert meta.w_init and not meta.x_init
+    torch.testing.assert_close(meta.w_scale, (w.abs().amax() / 448.0).reshape(1))
+    meta.update_w(torch.tensor([kat["amax"]]), "e4m3")
+    torch.testing.assert_close(meta.w_scale, torch.tensor(kat["scale"]).reshape(1))
+    assert meta.w_idx == 1 and meta.w_hist[0].item() == kat["amax"]
+
+
+def test_ring_wraps_and_forgets_old_peaks():
+    meta = FP8TensorMeta(torch.device("cpu"), DelayedScaling(history_len=2))
+    meta.init_x(torch.tensor([1.0]), "e4m3")
+    for a in (8.0, 2.0, 1.0):
+        meta.update_x(torch.tensor([a]), "e4m3")
+    # window now holds (1.0, 2.0): the 8.0 peak has rotated out
+    torch.testing.assert_close(meta.x_scale, torch.tensor([2.0 / 448.0]))
+
+
+def test_ops_have_no_cpu_arithmetic():
+    x = torch.randn(4, 8).to(torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        ops_fp8.quantize_bf16(x, torch.tensor([0.5]))
+    a8 = torch.zeros(2, 2, dtype=torch.float8_e4m3fn)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        ops_fp8.mm_fp8(a8, a8, torch.ones(1), torch.ones(1))
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        ops_int8.quantize_int8_per_token(x)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        ops_blk.mm_fp8_blockscaled(a8, a8, torch.ones(2, 1), torch.ones(1, 1))
+
+
+def test_argument_errors_match_the_reference_types():
+    x = torch.randn(2, 2).to(torch.bfloat16)
+    with pytest.raises(ValueError, match="unsupported fp8 format"):
+        ops_fp8.quantize_bf16(x, torch.tensor([1.0]), "e3m4")   # ops/fp8.py:44-48
+    a8 = torch.zeros(2, 2, dtype=torch.float8_e4m3fn)
+    with pytest.raises(ValueError, match="unsupported out_dtype"):
+        ops_fp8.mm_fp8(a8, a8, torch.ones(1), torch.ones(1), out_dtype="fp16")  # :150-153
+    with pytest.raises(TypeError, match="bf16 inputs"):
+        ops_fp8.linear_forward_fp8(x.float(), x, None, torch.ones(1), torch.ones(1))  # :162-163
+
+
+def test_fake_kernels_give_shapes_for_tracing():
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    with FakeTensorMode():
+        x = torch.empty(6, 32, dtype=torch.bfloat16)
+        x8, amax = torch.ops.custom.fp8_quantize(x, torch.empty(1), 1)
+        assert x8.dtype == torch.float8_e5m2 and x8.shape == (6, 32) and amax.shape == (1,)
+        a = torch.empty(6, 32, dtype=torch.float8_e4m3fn)
+        b = torch.empty(10, 32, dtype=torch.float8_e4m3fn)
+        assert torch.ops.custom.fp8_gemm(a, b, torch.empty(1), torch.empty(1)).shape == (6, 10)
+        assert torch.ops.custom.fp8_gemm(a, b, torch.empty(1), torch.empty(1), 1, torch.empty(1)).dtype == torch.float8_e4m3fn
+        xq, s = torch.ops.custom.int8_quantize_per_token(torch.empty(2, 3, 32, dtype=torch.bfloat16))
+        assert xq.shape == (6, 32) and s.shape == (6, 1)
+        ai = torch.empty(6, 32, dtype=torch.int8)
+        bi = torch.empty(10, 32, dtype=torch.int8)
+        out = torch.ops.custom.int8_gemm(ai, bi, torch.empty(6, 1), torch.empty(10))
+        assert out.shape == (6, 10) and out.dtype == torch.bfloat16
+
+
+def test_linear_override_leaves_cpu_and_disabled_calls_alone():
+    x, w = torch.randn(3, 8), torch.randn(5, 8)
+    with fp8_autocast(enabled=True), w8a8.int8_autocast(True):
+        y = torch.nn.functional.linear(x, w)     # CPU tensors never reach the CUDA-key hook
+    torch.testing.assert_close(y, x @ w.t())
+    assert not w8a8.int8_linear_enabled() and not fp8_state().enabled
+
+
+def test_int8_autocast_restores():
+    assert not w8a8.int8_linear_enabled()
+    with w8a8.int8_autocast(True):
+        assert w8a8.int8_linear_enabled()
+        with w8a8.int8_autocast(False):
+            assert not w8a8.int8_linear_enabled()
+        assert w8a8.int8_linear_enabled()
+    assert not w8a8.int8_linear_enabled()
