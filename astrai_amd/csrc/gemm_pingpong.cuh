@@ -206,6 +206,7 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
     const i32x4 rld_raw = raw_rsrc(ld_ptr, ld_bytes);
     uint32_t pf_reg = 0;
     auto prefetch = [&](int kstep) {
+        if constexpr (ScaleKind == SCALE_BLOCK128) return;  // registers are needed elsewhere
         const uint32_t k0 = (uint32_t)kstep << 7;
         asm volatile("buffer_load_dword %0, %1, %2, %3 offen"
                      : "+v"(pf_reg) : "v"(pf_off), "s"(rld_raw), "s"(k0) : "memory");
@@ -258,6 +259,51 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
                     acc[ni][mi] = Op::mma_step(st, wf[ni], xf[mi], acc[ni][mi]);
     };
 
+    // ---- 128-block scales (SCALE_BLOCK128 only). The promotion
+    //   out += P_kb * sa[m,kb] * sb[n/128,kb]
+    // is run in place on the accumulator: it is kept divided by the current
+    // block's scale s_kb = sa*sb, i.e. before slab kb's MFMAs the accumulator is
+    // multiplied by s_{kb-1}/s_kb and after the last slab by s_last. That needs no
+    // second register tile for P_kb. Scales below 1e-20 are taken as 1e-20.
+    // A lane owns one m per 32-row sub-tile (4 values) and one weight block.
+    [[maybe_unused]] float blk_s[MI] = {1.0f, 1.0f, 1.0f, 1.0f};   // scale the accumulators are divided by
+    [[maybe_unused]] float blk_next[MI] = {1.0f, 1.0f, 1.0f, 1.0f}; // scale of the slab computed next
+    [[maybe_unused]] const int kblocks = ksteps;
+    // activation scales through a buffer resource: one 32-bit row offset per lane,
+    // rows past M read as zero (and are clamped like any tiny scale)
+    [[maybe_unused]] const __amdgpu_buffer_rsrc_t rsa =
+        make_rsrc(g.sa, (ScaleKind == SCALE_BLOCK128) ? (uint32_t)g.m * (uint32_t)kblocks * 4u : 0u);
+    [[maybe_unused]] const uint32_t sa_off =
+        (uint32_t)(m0 + wave_m * 128 + lrow) * (uint32_t)kblocks * 4u;
+    [[maybe_unused]] auto load_block_scales = [&](int kb) {
+        if constexpr (ScaleKind == SCALE_BLOCK128) {
+            const int nb = (n0 + wave_n * 64) >> 7;
+            const float sbv = g.sb[(size_t)nb * kblocks + kb];
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi) {
+                const float sav = __builtin_bit_cast(
+                    float, __builtin_amdgcn_raw_buffer_load_b32(
+                               rsa, sa_off + (uint32_t)(mi * 32) * (uint32_t)kblocks * 4u,
+                               (uint32_t)kb * 4u, 0));
+                blk_next[mi] = fmaxf(sav * sbv, 1e-20f);
+            }
+        }
+    };
+    // multiply the accumulators by s_prev / s_cur and make s_cur the current scale
+    [[maybe_unused]] auto rescale = [&](bool first) {
+        if constexpr (ScaleKind == SCALE_BLOCK128) {
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi) {
+                const float r = first ? 1.0f : blk_s[mi] / blk_next[mi];
+                blk_s[mi] = blk_next[mi];
+                if (!first) {
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni) acc[ni][mi] *= r;
+                }
+            }
+        }
+    };
+
     // ---- prologue: slabs 0 and 1 of both operands in flight, then visible
     PP_STAMP();
     issue_loads(0, 0);
@@ -282,7 +328,9 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
     if (group == 0) {
         int xs = 0;  // k % 3
         for (int k = 0; k < ksteps; ++k) {
+            load_block_scales(k);  // lands while the operand reads are in flight
             read_frags(xs, k & 1);
+            rescale(k == 0);       // accumulators now relative to slab k's scale
             if (k >= 1 && k + 1 < ksteps) issue_loads(k + 1, (k + 1) & 1);
             // always one touch, so that "all but the last one" below means the slab
             // loads; past the end it re-touches the last slab (an L2 hit)
@@ -296,7 +344,8 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
             compute();
             __builtin_amdgcn_s_setprio(0);
             PP_STAMP();
-            wait_vmcnt<1>();  // the slab loads; the prefetch touch may stay in flight
+            // the slab loads; the prefetch touch (if any) may stay in flight
+            wait_vmcnt<(ScaleKind == SCALE_BLOCK128) ? 0 : 1>();
             PP_STAMP();
             phase_barrier();  // B_{k+1}
             PP_STAMP();
@@ -311,7 +360,9 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
             if (k > 0) compute();  // slab k-1
             __builtin_amdgcn_s_setprio(0);
             PP_STAMP();
+            load_block_scales(k);
             read_frags(xs, k & 1);
+            rescale(k == 0);      // slab k-1's MFMAs are issued; next come slab k's
             const int xs2 = (xs == 0) ? 2 : xs - 1;  // (k + 2) % 3
             const bool more = k + 2 < ksteps;
             if (more) issue_loads(k + 2, xs2);
@@ -320,8 +371,10 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
             PP_STAMP();
             // slab k+1 (issued one slab ago) must have landed; this slab's eight
             // loads and the two latest touches may stay in flight
-            if (more) wait_vmcnt<10>();
-            else wait_vmcnt<1>();
+            // (block scales: this phase's scale loads precede its slab loads and no
+            // touches exist, so the eight slab loads are the only younger ones)
+            if (more) wait_vmcnt<(ScaleKind == SCALE_BLOCK128) ? 8 : 10>();
+            else wait_vmcnt<(ScaleKind == SCALE_BLOCK128) ? 0 : 1>();
             PP_STAMP();
             phase_barrier();  // B_{k+1}
             PP_STAMP();
@@ -332,7 +385,7 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
         phase_barrier();
     }
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): no prefetch touch outlives the loop
-    asm volatile("" :: "v"(pf_reg));
+    if constexpr (ScaleKind != SCALE_BLOCK128) asm volatile("" :: "v"(pf_reg));
 
     // ---------------- epilogue ----------------
     PP_STAMP();
@@ -376,6 +429,7 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
                         float f = (float)acc[ni][mi][4 * q + j];
                         if constexpr (ScaleKind == SCALE_TENSOR) f = f * es.sa * es.sb;
                         else if constexpr (ScaleKind == SCALE_ROWCOL) f = f * sx * sw4[j];
+                        else f = f * blk_s[mi];
                         v[j] = f + b4[j];
                     }
                     u32x2 pk;

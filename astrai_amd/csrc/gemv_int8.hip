@@ -1,16 +1,14 @@
-// Skinny int8 W8A8 kernel for decode shapes (M <= 64): bandwidth-bound, the
-// weight matrix is streamed from HBM exactly once.
+// Skinny int8 W8A8 kernels for decode shapes (M <= 64): bandwidth-bound, the
+// weight matrix is streamed from HBM exactly once and the MFMA pipe is almost
+// idle -- speed is set by bytes in flight and by how whole the memory requests
+// are. The int32 partials of the waves that split K are summed through LDS
+// (integer addition is associative, so the split keeps the accumulator
+// bit-exact) and the first waves run the dequant epilogue.
 //
-// A workgroup of NW waves owns RG*16 weight rows; the waves split K into
-// 256-byte chunks (wave w takes chunks w, w+NW, ...), so that at K = 4096 every
-// wave issues all of its loads at once and the whole matrix is in flight
-// together. Per chunk a lane loads 64 contiguous bytes of one weight row (four
-// lanes cover the 256-byte chunk of that row) and the matching bytes of the
-// activation rows; the products run on v_mfma_i32_16x16x64_i8 with the weight
-// rows as the first operand, which leaves the MFMA pipe almost idle -- the
-// kernel's speed is set by bytes in flight. The int32 partials of the waves are
-// summed through LDS (integer addition is associative, so the split keeps the
-// accumulator bit-exact) and the first waves run the dequant epilogue.
+//  * M <= 32: gemv_int8_lds_kernel streams the weights through LDS with 1 KiB
+//    contiguous row pieces per instruction (see the comment on the kernel).
+//  * 32 < M <= 64: gemv_int8_kernel loads MFMA-shaped operands straight into
+//    registers (64 contiguous bytes of 16 rows per instruction).
 #include "gemm_tile.cuh"
 
 namespace w8a8 {
@@ -30,17 +28,16 @@ __global__ __launch_bounds__(NW * 64) void gemv_int8_kernel(GemmArgs g) {
     const __amdgpu_buffer_rsrc_t rw = make_rsrc(g.b, (uint32_t)g.n * (uint32_t)K);
     const __amdgpu_buffer_rsrc_t rx = make_rsrc(g.a, (uint32_t)g.m * (uint32_t)K);
 
+    // Lane (row r, K-group q) takes bytes [64j + 16q, +16) of each 256-byte chunk
+    // for j = 0..3: one instruction touches 64 contiguous bytes of each of its 16
+    // rows, two instructions a whole 128-byte line. Rows past N / M read as zero
+    // (their offset is past the buffer's num_records).
     uint32_t w_off[RG], x_off[MB];
 #pragma unroll
-    for (int r = 0; r < RG; ++r) {
-        const int n = n0 + r * 16 + lrow;
-        w_off[r] = (n < g.n) ? (uint32_t)n * (uint32_t)K + lgrp * 64 : kOutOfRange;
-    }
+    for (int r = 0; r < RG; ++r)
+        w_off[r] = (uint32_t)(n0 + r * 16 + lrow) * (uint32_t)K + lgrp * 16;
 #pragma unroll
-    for (int b = 0; b < MB; ++b) {
-        const int m = b * 16 + lrow;
-        x_off[b] = (m < g.m) ? (uint32_t)m * (uint32_t)K + lgrp * 64 : kOutOfRange;
-    }
+    for (int b = 0; b < MB; ++b) x_off[b] = (uint32_t)(b * 16 + lrow) * (uint32_t)K + lgrp * 16;
 
     i32x4 acc[RG][MB];
 #pragma unroll
@@ -54,11 +51,11 @@ __global__ __launch_bounds__(NW * 64) void gemv_int8_kernel(GemmArgs g) {
 #pragma unroll
         for (int r = 0; r < RG; ++r)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) wf[r][j] = buf_load16(rw, w_off[r] + j * 16, k0);
+            for (int j = 0; j < 4; ++j) wf[r][j] = buf_load16(rw, w_off[r] + j * 64, k0);
 #pragma unroll
         for (int b = 0; b < MB; ++b)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) xf[b][j] = buf_load16(rx, x_off[b] + j * 16, k0);
+            for (int j = 0; j < 4; ++j) xf[b][j] = buf_load16(rx, x_off[b] + j * 64, k0);
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -85,6 +82,131 @@ __global__ __launch_bounds__(NW * 64) void gemv_int8_kernel(GemmArgs g) {
     }
 }
 
+// Variant that streams the weights through LDS: every load instruction moves
+// 1 KiB of ONE weight row (64 lanes x 16 contiguous bytes) straight into LDS, so
+// HBM, L2 and the address coalescer all see whole 128-byte lines in order; the
+// MFMA operands (16 rows x 16 bytes per K-group) are then cut out of LDS, where
+// the strided access is free. A workgroup of four waves owns 16 weight rows, wave
+// w takes the 1 KiB K-steps w, w+4, ...; rows are laid down 1040 bytes apart so
+// that the 16 rows of an operand read fall in distinct banks.
+constexpr int kLdsRow = 1040;
+
+template <int MB>
+__global__ __launch_bounds__(256) void gemv_int8_lds_kernel(GemmArgs g) {
+    __shared__ __attribute__((aligned(16))) uint8_t wbuf[4][16 * kLdsRow];
+    __shared__ i32x4 red[4][MB][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lrow = lane & 15, lgrp = lane >> 4;
+    const int K = g.k;
+    const int nsteps = (K + 1023) >> 10;
+    const int n0 = blockIdx.x * 16;
+
+    const __amdgpu_buffer_rsrc_t rw = make_rsrc(g.b, (uint32_t)g.n * (uint32_t)K);
+    const __amdgpu_buffer_rsrc_t rx = make_rsrc(g.a, (uint32_t)g.m * (uint32_t)K);
+
+    // epilogue operands first: their latency hides under the weight stream
+    const int en = n0 + lgrp * 4;
+    f32x4 sw4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    float sxv[MB];
+    if (g.out_kind != OUT_ACC && wave < MB) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (en + j < g.n) sw4[j] = g.sb[en + j];
+    }
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+        const int m = b * 16 + lrow;
+        sxv[b] = (g.out_kind != OUT_ACC && m < g.m) ? g.sa[m] : 0.0f;
+    }
+
+    i32x4 acc[MB];
+#pragma unroll
+    for (int b = 0; b < MB; ++b) acc[b] = i32x4{0, 0, 0, 0};
+    uint8_t* const mine = wbuf[wave];
+
+    for (int s = wave; s < nsteps; s += 4) {
+        const uint32_t k0 = (uint32_t)s << 10;
+        // weights: 16 rows x 1 KiB, one instruction per row
+        const bool k_in = (int)(k0 + lane * 16) < K;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const uint32_t off = (uint32_t)(n0 + r) * (uint32_t)K + lane * 16;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                rw, (__attribute__((address_space(3))) void*)(mine + r * kLdsRow), 16,
+                k_in ? off : kOutOfRange, k0, 0, 0);
+        }
+        // activations: MFMA layout straight from L2 (they are a few KiB, shared by
+        // every workgroup)
+        u32x4 xf[MB][16];
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+            const uint32_t xo = (uint32_t)(b * 16 + lrow) * (uint32_t)K + lgrp * 16;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const bool in = (int)(k0 + j * 64 + lgrp * 16) < K;
+                xf[b][j] = buf_load16(rx, in ? xo + j * 64 : kOutOfRange, k0);
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the wave's own rows are in LDS
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const u32x4 wf = *reinterpret_cast<const u32x4*>(mine + lrow * kLdsRow + j * 64 + lgrp * 16);
+#pragma unroll
+            for (int b = 0; b < MB; ++b)
+                acc[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8((i32x4)wf, (i32x4)xf[b][j], acc[b], 0, 0, 0);
+        }
+    }
+
+#pragma unroll
+    for (int b = 0; b < MB; ++b) red[wave][b][lane] = acc[b];
+    __syncthreads();
+    if (wave < MB) {
+        const int b = wave;
+        const i32x4 sum = red[0][b][lane] + red[1][b][lane] + red[2][b][lane] + red[3][b][lane];
+        const int m = b * 16 + lrow;
+        if (m < g.m && en < g.n) {
+            const size_t o = (size_t)m * g.n + en;
+            if (g.out_kind == OUT_ACC) {
+                int* out = static_cast<int*>(g.out);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (en + j < g.n) out[o + j] = sum[j];
+            } else {
+                const uint16_t* bias = static_cast<const uint16_t*>(g.bias);
+                float sx = 0.0f;
+#pragma unroll
+                for (int bb = 0; bb < MB; ++bb)
+                    if (bb == b) sx = sxv[bb];
+                float v[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float f = (float)sum[j] * sx * sw4[j];
+                    if (bias && en + j < g.n) f += bf16_to_f32(bias[en + j]);
+                    v[j] = f;
+                }
+                uint16_t* out = static_cast<uint16_t*>(g.out);
+                if ((g.n & 3) == 0) {
+                    u32x2 pk;
+                    pk.x = pack_bf16x2(v[0], v[1]);
+                    pk.y = pack_bf16x2(v[2], v[3]);
+                    *reinterpret_cast<u32x2*>(out + o) = pk;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (en + j < g.n) out[o + j] = f32_to_bf16(v[j]);
+                }
+            }
+        }
+    }
+}
+
+template <int MB>
+void launch_lds(const GemmArgs& g, hipStream_t stream) {
+    const int blocks = (g.n + 15) / 16;
+    gemv_int8_lds_kernel<MB><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(g);
+}
+
 template <int RG, int MB, int NW>
 void launch(const GemmArgs& g, hipStream_t stream) {
     const int blocks = (g.n + RG * 16 - 1) / (RG * 16);
@@ -107,8 +229,8 @@ bool launch_gemv_int8(const GemmArgs& g, hipStream_t stream) {
     if ((int64_t)g.n * g.k >= lim) return false;
     const int mb = (g.m + 15) / 16;
     switch (mb) {
-        case 1: launch_nw<2, 1>(g, stream); break;
-        case 2: launch_nw<1, 2>(g, stream); break;
+        case 1: launch_lds<1>(g, stream); break;
+        case 2: launch_lds<2>(g, stream); break;
         case 3: launch_nw<1, 3>(g, stream); break;
         default: launch_nw<1, 4>(g, stream); break;
     }
