@@ -1,0 +1,12 @@
+"""The decoder the quantized Linear layers sit in (the unchanged caller of the
+GEMM path): same modules, parameter names and math as the reference's
+``astrai/model`` for a dense GQA + SwiGLU decoder, with a dense KV cache."""
+
+from astrai_amd.model.decoder import (
+    AutoRegressiveLM,
+    AutoRegressiveLMConfig,
+    DenseKVCache,
+    greedy_generate,
+)
+
+__all__ = ["AutoRegressiveLM", "AutoRegressiveLMConfig", "DenseKVCache", "greedy_generate"]

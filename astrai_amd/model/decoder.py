@@ -1,0 +1,272 @@
+"""Dense decoder whose every projection is ``Linear -> F.linear``, so that the
+``aten::linear`` hook of ``astrai_amd.extension`` routes it through the W8A8
+kernels without the model knowing.
+
+Module structure, parameter names, initialisation and arithmetic follow the
+reference: ``AutoRegressiveLM`` (astrai/model/transformer.py:29-152),
+``DecoderBlock`` (components/decoder_block.py:19-76), ``GQA``
+(components/attention.py:19-85), ``MLP`` (components/mlp.py:32-43), ``Linear``
+(components/linear.py:7-24), ``RMSNorm`` (components/norm.py:7-15), ``Embedding``
+(components/embedding.py:9-26), rotary tables and their application
+(components/rope.py:8-76, extension/backend/rotary.py:25-33), GQA head expansion
+and causal SDPA (extension/backend/attention.py:244-253,443-470).
+
+The reference's inference path packs requests and walks a paged cache per request
+with host reads; here requests form a dense ``[batch, seq]`` block over a dense
+``[layer, batch, kv_head, position, head_dim]`` cache, which is the same
+arithmetic for equal-length prompts and keeps the decode step free of host
+synchronisation, hence HIP-graph capturable.
+"""
+
+from dataclasses import dataclass
+from typing import Dict, Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+from torch import Tensor
+
+
+@dataclass
+class AutoRegressiveLMConfig:
+    """The fields of the reference's config (config/model_config.py:38-101) that a
+    dense GQA decoder uses."""
+
+    vocab_size: int = 32000
+    hidden_size: int = 2048
+    num_hidden_layers: int = 24
+    num_attention_heads: int = 16
+    num_key_value_heads: int = 4
+    intermediate_size: int = 5632
+    rms_norm_eps: float = 1e-5
+    rope_theta: float = 10000.0
+    max_position_embeddings: int = 2048
+    tie_word_embeddings: bool = False
+
+
+class Linear(nn.Module):
+    def __init__(self, in_dim: int, out_dim: int, bias: bool = False, init_std: float = 0.02):
+        super().__init__()
+        self.weight = nn.Parameter(torch.empty((out_dim, in_dim)))
+        self.bias = nn.Parameter(torch.zeros(out_dim)) if bias else None
+        self.init_std = init_std
+
+    def reset_parameters(self):
+        nn.init.normal_(self.weight, mean=0.0, std=self.init_std)
+        if self.bias is not None:
+            bound = 1 / (self.weight.size(1) ** 0.5)
+            nn.init.uniform_(self.bias, -bound, bound)
+
+    def forward(self, x: Tensor) -> Tensor:
+        return F.linear(x, self.weight, self.bias)
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, dim: int, norm_eps: float):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(dim))
+        self.normalized_shape = (dim,)
+        self.norm_eps = norm_eps
+
+    def forward(self, x: Tensor) -> Tensor:
+        return F.rms_norm(x, self.normalized_shape, self.weight, self.norm_eps)
+
+
+class Embedding(nn.Module):
+    def __init__(self, vocab_size: int, embedding_dim: int):
+        super().__init__()
+        self.weight = nn.Parameter(torch.empty((vocab_size, embedding_dim)))
+
+    def reset_parameters(self):
+        nn.init.normal_(self.weight, mean=0.0, std=0.02)
+
+    def forward(self, x: Tensor) -> Tensor:
+        return F.embedding(x, self.weight)
+
+
+def get_rotary_emb(dim: int, max_len: int, base: float = 10000.0) -> Tensor:
+    """``[max_len, dim/2, 2]`` fp32 table of (cos, sin), angles computed in fp64."""
+    theta = base ** (-torch.arange(0, dim, 2, dtype=torch.float64) / dim)
+    t = torch.arange(0, max_len, dtype=torch.float64)
+    freqs = torch.outer(t, theta).float()
+    return torch.stack([torch.cos(freqs), torch.sin(freqs)], dim=-1)
+
+
+def apply_rotary_emb(x: Tensor, freqs_cis: Tensor) -> Tensor:
+    """Rotate adjacent (even, odd) pairs of the head dimension; fp32 math, cast back.
+    ``x`` is ``[batch, seq, heads, head_dim]``, ``freqs_cis`` ``[batch|1, seq, head_dim/2, 2]``."""
+    cos, sin = freqs_cis[..., 0].unsqueeze(-2), freqs_cis[..., 1].unsqueeze(-2)
+    x_ = x.float().reshape(*x.shape[:-1], -1, 2)
+    xe, xo = x_[..., 0], x_[..., 1]
+    out = torch.stack([xe * cos - xo * sin, xe * sin + xo * cos], dim=-1)
+    return out.flatten(-2).to(x.dtype)
+
+
+def repeat_kv(x: Tensor, n_rep: int) -> Tensor:
+    """``[B, H_kv, S, D] -> [B, H_kv*n_rep, S, D]``, each KV head repeated n_rep times in place order."""
+    if n_rep == 1:
+        return x
+    b, h, s, d = x.shape
+    return x.unsqueeze(2).expand(b, h, n_rep, s, d).reshape(b, h * n_rep, s, d)
+
+
+class DenseKVCache:
+    """``k``/``v``: ``[layers, batch, kv_heads, max_len, head_dim]``."""
+
+    def __init__(self, config: AutoRegressiveLMConfig, batch: int, max_len: int, device, dtype):
+        hd = config.hidden_size // config.num_attention_heads
+        shape = (config.num_hidden_layers, batch, config.num_key_value_heads, max_len, hd)
+        self.k = torch.zeros(shape, device=device, dtype=dtype)
+        self.v = torch.zeros(shape, device=device, dtype=dtype)
+        self.max_len = max_len
+
+
+class GQA(nn.Module):
+    def __init__(self, dim: int, n_heads: int, n_kv_heads: int, layer_id: int, n_layers: int):
+        super().__init__()
+        assert dim % n_heads == 0 and n_heads % n_kv_heads == 0
+        self.head_dim = dim // n_heads
+        self.layer_id = layer_id
+        self.dim, self.n_heads, self.n_kv_heads = dim, n_heads, n_kv_heads
+        self.n_rep = n_heads // n_kv_heads
+        self.q_proj = Linear(dim, n_heads * self.head_dim)
+        self.k_proj = Linear(dim, n_kv_heads * self.head_dim)
+        self.v_proj = Linear(dim, n_kv_heads * self.head_dim)
+        self.o_proj = Linear(dim, dim, init_std=0.02 / (2 * n_layers) ** 0.5)
+
+    def forward(self, x: Tensor, rotary_emb: Tensor, kv_cache: Optional[DenseKVCache],
+                positions: Optional[Tensor], key_mask: Optional[Tensor]) -> Tensor:
+        b, s, _ = x.shape
+        q = self.q_proj(x).reshape(b, s, self.n_heads, self.head_dim)
+        k = self.k_proj(x).reshape(b, s, self.n_kv_heads, self.head_dim)
+        v = self.v_proj(x).reshape(b, s, self.n_kv_heads, self.head_dim)
+        q, k = apply_rotary_emb(q, rotary_emb), apply_rotary_emb(k, rotary_emb)
+        q, k, v = q.permute(0, 2, 1, 3), k.permute(0, 2, 1, 3), v.permute(0, 2, 1, 3)
+        if kv_cache is None:
+            out = F.scaled_dot_product_attention(q, repeat_kv(k, self.n_rep), repeat_kv(v, self.n_rep),
+                                                 is_causal=True)
+        else:
+            # write the new keys / values at `positions` (a device index tensor: no
+            # host read), then attend over the cache under `key_mask`
+            kv_cache.k[self.layer_id].index_copy_(2, positions, k)
+            kv_cache.v[self.layer_id].index_copy_(2, positions, v)
+            # the n_rep query heads that share a KV head are folded into the query
+            # axis ([B, H_kv, n_rep*S, D]) instead of copying the cache n_rep times:
+            # the same dot products and softmax rows as after repeat_kv
+            qf = q.reshape(b, self.n_kv_heads, self.n_rep * s, self.head_dim)
+            mask = key_mask if self.n_rep == 1 else key_mask.repeat(1, 1, self.n_rep, 1)
+            out = F.scaled_dot_product_attention(qf, kv_cache.k[self.layer_id],
+                                                 kv_cache.v[self.layer_id], attn_mask=mask)
+            out = out.reshape(b, self.n_heads, s, self.head_dim)
+        out = out.permute(0, 2, 1, 3).reshape(b, s, self.dim)
+        return self.o_proj(out)
+
+
+class MLP(nn.Module):
+    def __init__(self, dim: int, dim_ffn: int, down_init_std: float = 0.02):
+        super().__init__()
+        self.up = Linear(dim, dim_ffn)
+        self.gate = Linear(dim, dim_ffn)
+        self.down = Linear(dim_ffn, dim, init_std=down_init_std)
+
+    def forward(self, x: Tensor) -> Tensor:
+        return self.down(self.up(x) * F.silu(self.gate(x)))
+
+
+class DecoderBlock(nn.Module):
+    def __init__(self, config: AutoRegressiveLMConfig, layer_id: int):
+        super().__init__()
+        n = config.num_hidden_layers
+        self.attention = GQA(config.hidden_size, config.num_attention_heads,
+                             config.num_key_value_heads, layer_id, n)
+        self.input_norm = RMSNorm(config.hidden_size, config.rms_norm_eps)
+        self.post_attention_norm = RMSNorm(config.hidden_size, config.rms_norm_eps)
+        self.mlp = MLP(config.hidden_size, config.intermediate_size,
+                       down_init_std=0.02 / (2 * n) ** 0.5)
+
+    def forward(self, x, rotary_emb, kv_cache, positions, key_mask):
+        x = self.attention(self.input_norm(x), rotary_emb, kv_cache, positions, key_mask) + x
+        return self.mlp(self.post_attention_norm(x)) + x
+
+
+class AutoRegressiveLM(nn.Module):
+    def __init__(self, config: AutoRegressiveLMConfig):
+        super().__init__()
+        self.config = config
+        rope_dim = config.hidden_size // config.num_attention_heads
+        self.register_buffer(
+            "freqs_cis", get_rotary_emb(rope_dim, config.max_position_embeddings, config.rope_theta),
+            persistent=False)
+        self.embed_tokens = Embedding(config.vocab_size, config.hidden_size)
+        self.layers = nn.ModuleList(
+            [DecoderBlock(config, i) for i in range(config.num_hidden_layers)])
+        self.norm = RMSNorm(config.hidden_size, config.rms_norm_eps)
+        self.lm_head = Linear(config.hidden_size, config.vocab_size)
+        if config.tie_word_embeddings:
+            self.lm_head.weight = self.embed_tokens.weight
+        self.apply(lambda m: m.reset_parameters() if hasattr(m, "reset_parameters") else None)
+
+    def forward(self, input_ids: Tensor, kv_cache: Optional[DenseKVCache] = None,
+                positions: Optional[Tensor] = None) -> Dict[str, Tensor]:
+        """``input_ids [batch, seq]``. Without a cache: causal forward over the block.
+        With a cache: the block's tokens sit at ``positions`` (``[seq]`` int64, on the
+        device), keys/values are written there and every query attends to cache
+        entries at positions <= its own."""
+        if input_ids.ndim != 2:
+            raise ValueError("input_ids must be [batch, seq_len]")
+        b, s = input_ids.shape
+        x = self.embed_tokens(input_ids)
+        if positions is None:
+            positions = torch.arange(s, device=input_ids.device)
+        rotary = self.freqs_cis.index_select(0, positions).unsqueeze(0).float()
+        key_mask = None
+        if kv_cache is not None:
+            key_pos = torch.arange(kv_cache.max_len, device=input_ids.device)
+            key_mask = (key_pos[None, :] <= positions[:, None])[None, None]  # [1,1,seq,max_len]
+        for layer in self.layers:
+            x = layer(x, rotary, kv_cache, positions, key_mask)
+        hidden = self.norm(x)
+        return {"logits": self.lm_head(hidden), "hidden_states": hidden}
+
+
+@torch.no_grad()
+def greedy_generate(model: AutoRegressiveLM, prompt_ids: Tensor, steps: int,
+                    use_graph: bool = False, warmup_steps: int = 2) -> Tensor:
+    """Prefill ``prompt_ids [batch, prompt_len]`` then ``steps`` greedy (argmax) decode
+    steps; returns the generated ids ``[batch, steps]``. With ``use_graph`` the decode
+    step is captured after ``warmup_steps`` eager steps and replayed
+    (the reference's warm -> capture -> replay pattern, inference/runtime/graph.py:86-100)."""
+    b, p = prompt_ids.shape
+    dev = prompt_ids.device
+    dtype = model.embed_tokens.weight.dtype
+    cache = DenseKVCache(model.config, b, p + steps, dev, dtype)
+    logits = model(prompt_ids, cache, torch.arange(p, device=dev))["logits"]
+    tok = logits[:, -1].argmax(-1)
+    out = torch.empty(b, steps, dtype=torch.long, device=dev)
+    cur = tok.clone().reshape(b, 1)
+    pos = torch.full((1,), p, dtype=torch.long, device=dev)
+
+    def step():
+        lg = model(cur, cache, pos)["logits"]
+        return lg[:, -1].argmax(-1)
+
+    graph = None
+    nxt_static = None
+    for i in range(steps):
+        out[:, i] = cur[:, 0]
+        if i + 1 == steps:
+            break
+        if use_graph and graph is None and i >= warmup_steps:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                nxt_static = step()
+            graph.replay()  # capture records the step without running it
+            nxt = nxt_static
+        elif graph is not None:
+            graph.replay()
+            nxt = nxt_static
+        else:
+            nxt = step()
+        cur.copy_(nxt.reshape(b, 1))
+        pos.add_(1)
+    return out

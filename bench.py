@@ -77,6 +77,63 @@ def _graph_time_ms(launch, n_launch, replays, warm_replays=2):
     return e0.elapsed_time(e1) / (replays * n_launch)
 
 
+def _bench_decoder(dev):
+    """BASELINE config 4: 24-layer GQA/SwiGLU decoder (hidden 2048, 16/4 heads, FFN 5632, vocab 32000),
+    random-init bf16 weights quantized to int8 per channel, every Linear through the int8 kernels;
+    batch 32 x 512-token prefill, then 128 greedy decode steps (eager and as a replayed HIP graph)."""
+    import torch
+
+    from astrai_amd.extension import w8a8
+    from astrai_amd.model import AutoRegressiveLM, AutoRegressiveLMConfig, DenseKVCache, greedy_generate
+
+    cfg = AutoRegressiveLMConfig()
+    torch.manual_seed(4)
+    with torch.device(dev):
+        model = AutoRegressiveLM(cfg).to(torch.bfloat16).eval()
+    batch, prompt, steps = 32, 512, 128
+    ids = torch.randint(0, cfg.vocab_size, (batch, prompt), generator=torch.Generator().manual_seed(4)).to(dev)
+    w8a8.int8_state().reset()
+    n_lin = w8a8.prepare_int8_weights(model)
+    res = {"linears": n_lin, "batch": batch, "prompt_len": prompt, "decode_steps": steps}
+    with torch.no_grad(), w8a8.int8_autocast(True):
+        def prefill():
+            cache = DenseKVCache(cfg, batch, prompt + steps, dev, torch.bfloat16)
+            return model(ids, cache, torch.arange(prompt, device=dev))["logits"][:, -1].argmax(-1)
+
+        for _ in range(2):
+            prefill()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(3):
+            prefill()
+        torch.cuda.synchronize()
+        t_pre = (time.perf_counter() - t0) / 3
+        res["prefill_ms"] = round(t_pre * 1e3, 2)
+        res["prefill_tokens_per_s"] = round(batch * prompt / t_pre)
+        for name, graph in (("eager", False), ("graph", True)):
+            greedy_generate(model, ids, 8, use_graph=graph)  # warm
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            greedy_generate(model, ids, steps, use_graph=graph)
+            torch.cuda.synchronize()
+            t_all = time.perf_counter() - t0
+            t_dec = max(t_all - t_pre, 1e-9)
+            res[f"decode_{name}_ms_per_step"] = round(t_dec * 1e3 / (steps - 1), 3)
+            res[f"decode_{name}_tokens_per_s"] = round(batch * (steps - 1) / t_dec)
+        # the same model with the stock bf16 kernels, for scale
+    w8a8.int8_state().reset()
+    with torch.no_grad():
+        greedy_generate(model, ids, 8, use_graph=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        greedy_generate(model, ids, steps, use_graph=True)
+        torch.cuda.synchronize()
+        res["bf16_stock_total_ms_graph"] = round((time.perf_counter() - t0) * 1e3, 1)
+    del model
+    torch.cuda.empty_cache()
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -84,6 +141,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=300)
     ap.add_argument("--no-extra", action="store_true", help="headline kernel only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-model", action="store_true", help="skip the config-4 decoder leg")
+    ap.add_argument("--decoder-trace", action="store_true",
+                    help="tracing mode: build the config-4 decoder, one prefill + 19 eager decode steps, nothing else")
     ap.add_argument("--pmc", action="store_true",
                     help="counter-collection mode: a few launches of the headline kernel and of a "
                          "plain 256 MiB device copy (the calibration kernel), nothing else")
@@ -108,6 +168,22 @@ def main():
     def check(rc):
         if rc:
             raise RuntimeError(lib.astrai_w8a8_last_error().decode())
+
+    if args.decoder_trace:
+        from astrai_amd.extension import w8a8
+        from astrai_amd.model import AutoRegressiveLM, AutoRegressiveLMConfig, greedy_generate
+
+        cfg = AutoRegressiveLMConfig()
+        torch.manual_seed(4)
+        with torch.device(dev):
+            model = AutoRegressiveLM(cfg).to(torch.bfloat16).eval()
+        ids = torch.randint(0, cfg.vocab_size, (32, 512), generator=torch.Generator().manual_seed(4)).to(dev)
+        w8a8.prepare_int8_weights(model)
+        with torch.no_grad(), w8a8.int8_autocast(True):
+            greedy_generate(model, ids, 20, use_graph=False)
+        torch.cuda.synchronize()
+        print(json.dumps({"decoder_trace": True, "prefill_tokens": 32 * 512, "decode_steps": 19}))
+        return
 
     # ---------------- headline: config 1, fp8 per-tensor 4096^3 ----------------
     M = N = K = 4096
@@ -284,6 +360,9 @@ def main():
                 O.int8_linear(xc, wq, sw)
                 ts.append(time.perf_counter() - t0)
             extra["int8_config0_16x2048x2048"]["cpu_oracle_ms"] = round(sorted(ts)[2] * 1e3, 2)
+
+    if not args.no_extra and not args.no_model:
+        extra["decoder_config4_int8"] = _bench_decoder(dev)
 
     line = {
         "metric": "W8A8 GEMM TFLOPS/TOPS + % MFMA peak; decode GEMV GB/s + % HBM peak (1 GPU)",

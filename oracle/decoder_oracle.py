@@ -1,0 +1,90 @@
+"""CPU restatement of the reference decoder forward with every Linear computed by
+the W8A8 oracle. TEST INFRASTRUCTURE ONLY (see oracle/__init__.py).
+
+Works on a plain ``state_dict`` (parameter names of astrai/model/transformer.py:43-62)
+so that it shares no code with the product's modules. Arithmetic followed:
+  embed -> blocks -> final RMSNorm -> lm_head over all tokens   transformer.py:126-146
+  x = attn(input_norm(x)) + x ; x = mlp(post_attention_norm(x)) + x   decoder_block.py:59-70
+  q/k/v projections, rotary on q and k, SDPA, o_proj             components/attention.py:69-84
+  rotary = complex multiply of adjacent pairs in fp32, cast back extension/backend/rotary.py:25-33
+  cos/sin tables, angles in fp64                                  components/rope.py:8-24
+  KV heads expanded by repeating each head n_rep times            extension/backend/attention.py:244-253
+  causal SDPA                                                     extension/backend/attention.py:443-470
+  MLP = down(up(x) * silu(gate(x)))                               components/mlp.py:40-43
+  RMSNorm = F.rms_norm                                            components/norm.py:14-15
+"""
+
+from __future__ import annotations
+
+from typing import Callable, Dict
+
+import torch
+import torch.nn.functional as F
+
+from oracle import w8a8_oracle as O
+
+
+def rotary_table(dim: int, max_len: int, base: float) -> torch.Tensor:
+    theta = base ** (-torch.arange(0, dim, 2, dtype=torch.float64) / dim)
+    t = torch.arange(0, max_len, dtype=torch.float64)
+    freqs = torch.outer(t, theta).float()
+    return torch.stack([torch.cos(freqs), torch.sin(freqs)], dim=-1)
+
+
+def apply_rotary(x: torch.Tensor, freqs_cis: torch.Tensor) -> torch.Tensor:
+    cos, sin = freqs_cis[..., 0], freqs_cis[..., 1]
+    xc = torch.view_as_complex(x.float().reshape(*x.shape[:-1], -1, 2))
+    rot = xc * torch.complex(cos, sin).unsqueeze(-2)
+    return torch.view_as_real(rot).flatten(-2).to(x.dtype)
+
+
+def repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:
+    # x: [B, S, H_kv, D] -> [B, S, H_kv*n_rep, D]
+    if n_rep == 1:
+        return x
+    h, d = x.shape[-2:]
+    return x.unsqueeze(-2).expand(*x.shape[:-2], h, n_rep, d).reshape(*x.shape[:-2], h * n_rep, d)
+
+
+def int8_linear_fn(sd: Dict[str, torch.Tensor]) -> Callable[[torch.Tensor, str], torch.Tensor]:
+    """Quantize every 2-D projection weight per output channel once; activations per token per call."""
+    q = {k: O.int8_quantize_rows(v) for k, v in sd.items()
+         if v.dim() == 2 and not k.startswith("embed_tokens")}
+
+    def lin(x: torch.Tensor, name: str) -> torch.Tensor:
+        wq, sw = q[name]
+        return O.int8_linear(x, wq, sw)
+
+    return lin
+
+
+def bf16_linear_fn(sd: Dict[str, torch.Tensor]) -> Callable[[torch.Tensor, str], torch.Tensor]:
+    return lambda x, name: F.linear(x, sd[name])
+
+
+def forward(sd: Dict[str, torch.Tensor], cfg, input_ids: torch.Tensor,
+            lin: Callable[[torch.Tensor, str], torch.Tensor]) -> torch.Tensor:
+    """Causal forward over ``input_ids [B, S]``; returns logits ``[B, S, vocab]`` (bf16)."""
+    b, s = input_ids.shape
+    nh, nkv = cfg.num_attention_heads, cfg.num_key_value_heads
+    hd = cfg.hidden_size // nh
+    x = F.embedding(input_ids, sd["embed_tokens.weight"])
+    fc = rotary_table(hd, s, cfg.rope_theta).unsqueeze(0)  # [1, S, hd/2, 2]
+    for i in range(cfg.num_hidden_layers):
+        p = f"layers.{i}."
+        h = F.rms_norm(x, (cfg.hidden_size,), sd[p + "input_norm.weight"], cfg.rms_norm_eps)
+        q = lin(h, p + "attention.q_proj.weight").reshape(b, s, nh, hd)
+        k = lin(h, p + "attention.k_proj.weight").reshape(b, s, nkv, hd)
+        v = lin(h, p + "attention.v_proj.weight").reshape(b, s, nkv, hd)
+        q, k = apply_rotary(q, fc), apply_rotary(k, fc)
+        k, v = repeat_kv(k, nh // nkv), repeat_kv(v, nh // nkv)
+        a = F.scaled_dot_product_attention(q.permute(0, 2, 1, 3), k.permute(0, 2, 1, 3),
+                                           v.permute(0, 2, 1, 3), is_causal=True)
+        a = a.permute(0, 2, 1, 3).reshape(b, s, cfg.hidden_size)
+        x = lin(a, p + "attention.o_proj.weight") + x
+        h = F.rms_norm(x, (cfg.hidden_size,), sd[p + "post_attention_norm.weight"], cfg.rms_norm_eps)
+        up = lin(h, p + "mlp.up.weight")
+        gate = lin(h, p + "mlp.gate.weight")
+        x = lin(up * F.silu(gate), p + "mlp.down.weight") + x
+    hidden = F.rms_norm(x, (cfg.hidden_size,), sd["norm.weight"], cfg.rms_norm_eps)
+    return lin(hidden, "lm_head.weight")
