@@ -74,16 +74,18 @@ __device__ __forceinline__ float bf16_to_f32(uint16_t h) {
     return __uint_as_float((uint32_t)h << 16);
 }
 
-// round-to-nearest-even fp32 -> bf16 (NaN kept quiet)
-__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
-}
+// round-to-nearest-even fp32 -> bf16 on the hardware converter
+// (v_cvt_pk_bf16_f32; NaN stays NaN)
+typedef __bf16 bf16x2_hw __attribute__((ext_vector_type(2)));
+typedef float f32x2_hw __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-    return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+    const f32x2_hw v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_hw));
+}
+
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+    return (uint16_t)(pack_bf16x2(f, 0.0f) & 0xffffu);
 }
 
 // Saturating fp32 -> fp8 pair (low 16 bits of the result). The hardware

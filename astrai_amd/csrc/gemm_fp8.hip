@@ -1,21 +1,28 @@
 // fp8 (OCP e4m3fn / e5m2) MFMA GEMMs, per-tensor scales, optional bias, bf16 /
-// e4m3 / fp32 output: the 256x256 ping-pong kernel (v_mfma_f32_32x32x64_f8f6f4)
-// for large shapes, the generic tiled kernel otherwise.
-#include "gemm_pingpong.cuh"
+// e4m3 / fp32 output. Large shapes run v_mfma_f32_32x32x64_f8f6f4 on 256x256
+// tiles: the four-wave 128x128-register-tile kernel for bf16 output, the
+// eight-wave ping-pong kernel for the other outputs; the generic tiled kernel
+// takes everything else.
+#include "gemm_wave128.cuh"
 #include "gemm_tile.cuh"
 
 namespace w8a8 {
 
+namespace {
+template <int Fmt>
+void launch_for(const GemmArgs& g, hipStream_t stream) {
+#ifndef W8A8_NO_WAVE128
+    if (wave128_shape_ok(g)) return launch_wave128<Op32F8<Fmt>, SCALE_TENSOR>(g, stream);
+#endif
+    if (pingpong_shape_ok(g)) return launch_pingpong<Op32F8<Fmt>, SCALE_TENSOR>(g, stream);
+    launch_tiled_auto<OpF8<Fmt>, SCALE_TENSOR>(g, stream);
+}
+}  // namespace
+
 bool launch_gemm_fp8_tiled(const GemmArgs& g, int fmt, hipStream_t stream) {
     if (!tiled_shape_ok(g)) return false;
-    const bool big = pingpong_shape_ok(g);
-    if (fmt) {
-        if (big) launch_pingpong<Op32F8<1>, SCALE_TENSOR>(g, stream);
-        else launch_tiled_auto<OpF8<1>, SCALE_TENSOR>(g, stream);
-    } else {
-        if (big) launch_pingpong<Op32F8<0>, SCALE_TENSOR>(g, stream);
-        else launch_tiled_auto<OpF8<0>, SCALE_TENSOR>(g, stream);
-    }
+    if (fmt) launch_for<1>(g, stream);
+    else launch_for<0>(g, stream);
     return true;
 }
 

@@ -1,13 +1,19 @@
-// int8 x int8 -> int32 MFMA GEMMs, per-token x per-channel dequant epilogue:
-// the 256x256 ping-pong kernel (v_mfma_i32_32x32x32_i8) for large shapes, the
-// generic tiled kernel otherwise.
-#include "gemm_pingpong.cuh"
+// int8 x int8 -> int32 MFMA GEMMs, per-token x per-channel dequant epilogue.
+// Large shapes run v_mfma_i32_32x32x32_i8 on 256x256 tiles: the four-wave
+// 128x128-register-tile kernel for bf16 output, the eight-wave ping-pong kernel
+// for int32 output; the generic tiled kernel takes everything else.
+#include "gemm_wave128.cuh"
 #include "gemm_tile.cuh"
 
 namespace w8a8 {
 
 bool launch_gemm_int8_tiled(const GemmArgs& g, hipStream_t stream) {
     if (!tiled_shape_ok(g)) return false;
+#ifndef W8A8_NO_WAVE128
+    if (wave128_shape_ok(g))
+        launch_wave128<Op32I8, SCALE_ROWCOL>(g, stream);
+    else
+#endif
     if (pingpong_shape_ok(g))
         launch_pingpong<Op32I8, SCALE_ROWCOL>(g, stream);
     else

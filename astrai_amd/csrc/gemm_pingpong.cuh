@@ -48,6 +48,11 @@ struct Op32I8 {
     static __device__ __forceinline__ Acc mma_step(int q, const u32x4 (&w)[4], const u32x4 (&x)[4], Acc c) {
         return __builtin_amdgcn_mfma_i32_32x32x32_i8((i32x4)w[q], (i32x4)x[q], c, 0, 0, 0);
     }
+    // half a slab (two chunks per row) is two K=32 steps; step s uses chunk s
+    static constexpr int HALF_STEPS = 2;
+    static __device__ __forceinline__ Acc mma_half(int s, const u32x4 (&w)[2], const u32x4 (&x)[2], Acc c) {
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8((i32x4)w[s], (i32x4)x[s], c, 0, 0, 0);
+    }
 };
 
 template <int Fmt>
@@ -63,6 +68,15 @@ struct Op32F8 {
                    (int)w1.x, (int)w1.y, (int)w1.z, (int)w1.w};
         i32x8 b = {(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w,
                    (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
+        return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, Fmt, Fmt, 0, 0, 0, 0);
+    }
+    // half a slab (two chunks per row) is one K=64 step
+    static constexpr int HALF_STEPS = 1;
+    static __device__ __forceinline__ Acc mma_half(int, const u32x4 (&w)[2], const u32x4 (&x)[2], Acc c) {
+        i32x8 a = {(int)w[0].x, (int)w[0].y, (int)w[0].z, (int)w[0].w,
+                   (int)w[1].x, (int)w[1].y, (int)w[1].z, (int)w[1].w};
+        i32x8 b = {(int)x[0].x, (int)x[0].y, (int)x[0].z, (int)x[0].w,
+                   (int)x[1].x, (int)x[1].y, (int)x[1].z, (int)x[1].w};
         return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, Fmt, Fmt, 0, 0, 0, 0);
     }
 };
@@ -427,7 +441,7 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         float f = (float)acc[ni][mi][4 * q + j];
-                        if constexpr (ScaleKind == SCALE_TENSOR) f = f * es.sa * es.sb;
+                        if constexpr (ScaleKind == SCALE_TENSOR) f = f * (es.sa * es.sb);
                         else if constexpr (ScaleKind == SCALE_ROWCOL) f = f * sx * sw4[j];
                         else f = f * blk_s[mi];
                         v[j] = f + b4[j];

@@ -82,7 +82,7 @@ __device__ __forceinline__ void store_subtile(const GemmArgs& g, const EpilogueS
     for (int j = 0; j < 4; ++j) {
         float f = (float)a[j];
         if constexpr (ScaleKind == SCALE_TENSOR) {
-            f = f * es.sa * es.sb;
+            f = f * (es.sa * es.sb);  // one combined output scale, as csrc/kernels/fp8/gemm.cuh:583
         } else if constexpr (ScaleKind == SCALE_ROWCOL) {
             const float sw = (n + j < g.n) ? g.sb[n + j] : 0.0f;
             f = f * sx * sw;

@@ -1,0 +1,336 @@
+// 256x256x128 8-bit NT GEMM for gfx950 with four waves and 128x128 register
+// tiles, software-pipelined inside each wave.
+//
+// Why. With 32x32 MFMAs a 128(m) x 128(n) wave tile reads (128+128) x 128 bytes
+// of operands from LDS per K slab for 2048 MFMA cycles: 128 KiB per workgroup
+// and slab against the 192 KiB of eight 128x64 wave tiles. LDS serves both the
+// operand reads and the incoming direct-to-LDS loads (64 KiB a slab), so that
+// third less read traffic is what lets the MFMA pipe stay busy. The price: the
+// 256 accumulator registers of a wave leave room for one wave per SIMD only, so
+// nothing can hide one wave's memory phase behind another wave's MFMAs -- each
+// wave interleaves its own LDS reads and loads between its own MFMAs instead.
+//
+// Pipeline of one wave, K slab k (two register sets F0, F1 of half a slab each;
+// a slab's half h is chunks 2h, 2h+1 of every row, 64 bytes of K):
+//   first half:   MFMAs on F0 = (k, half 0)   | LDS reads (k, half 1)   -> F1
+//                                             | loads: activation rows of slab k+2
+//   -- own loads of slab k+1 landed, own reads of slab k done; barrier --
+//   second half:  MFMAs on F1 = (k, half 1)   | LDS reads (k+1, half 0) -> F0
+//                                             | loads: weight rows of slab k+2
+// The instruction order is written out and pinned (one MFMA, then at most two
+// LDS reads and one load) so that the MFMA pipe always has the next instruction
+// waiting. Three activation stages and two weight stages (all 160 KiB): the
+// activation rows of slab k+2 may be fetched before the barrier that retires
+// slab k, which spreads the loads evenly over the slab -- the CU's single load
+// path is the scarce resource, see the comment at the main loop. No L2 prefetch
+// touches here: a touch pulls its whole line through that same path a second
+// time, which costs more than the L2 misses it saves.
+//
+// LDS layout of a stage, operand roles and accumulator layout are those of the
+// ping-pong kernel: 256 activation rows then 256 weight rows of 128 bytes, chunk
+// c of row r at position c ^ (r & 7) ^ ((r >> 3) & 1); weight rows are the
+// first MFMA operand.
+#pragma once
+
+#include "gemm_pingpong.cuh"
+
+namespace w8a8 {
+
+struct Wave128Cfg {
+    static constexpr int BM = 256, BN = 256, BK = 128;
+    static constexpr int THREADS = 256;
+    static constexpr int MI = 4, NI = 4;  // 32-row sub-tiles per wave: 128 m x 128 n
+    static constexpr int OPERAND_BYTES = 256 * BK;       // one operand's slab: 32 KiB
+    static constexpr int X_STAGES = 3, W_STAGES = 2;
+    static constexpr int W_BASE = X_STAGES * OPERAND_BYTES;  // weights after activations
+    static constexpr int EPI_ROW_BYTES = 144;            // 64 bf16 + 16 bytes of padding
+    static constexpr int EPI_WAVE_BYTES = 128 * EPI_ROW_BYTES;
+    static constexpr int LDS_BYTES = (X_STAGES + W_STAGES) * OPERAND_BYTES;  // all 160 KiB
+    static_assert(4 * EPI_WAVE_BYTES <= LDS_BYTES, "epilogue staging must fit");
+};
+
+// order in which a half slab's sixteen 16-byte operand pieces are read from LDS:
+// the first MFMAs need weight sub-tile 0 and activation sub-tile 0, then the
+// other weight sub-tiles, then the other activation sub-tiles (m is the outer
+// MFMA loop)
+__device__ constexpr int kReadIsW[8] = {1, 0, 1, 1, 1, 0, 0, 0};
+__device__ constexpr int kReadSub[8] = {0, 0, 1, 2, 3, 1, 2, 3};
+
+template <class Op, int ScaleKind>
+__global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmArgs g) {
+    static_assert(ScaleKind != SCALE_BLOCK128, "block scales run on the ping-pong kernel");
+    PP_STAMP_INIT();
+    using Cfg = Wave128Cfg;
+    using Acc = typename Op::Acc;
+    constexpr int MI = Cfg::MI, NI = Cfg::NI;
+    constexpr int HS = Op::HALF_STEPS;
+    constexpr int NM = HS * MI * NI;  // MFMAs per half slab
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave & 1;
+    const int wave_n = wave >> 1;
+    const int lrow = lane & 31;
+    const int lgrp = lane >> 5;
+
+    const int tiles_m = (g.m + Cfg::BM - 1) / Cfg::BM;
+    const int tiles_n = (g.n + Cfg::BN - 1) / Cfg::BN;
+    const TileCoord tc = map_tile(tiles_m, tiles_n);
+    const int m0 = tc.tm * Cfg::BM, n0 = tc.tn * Cfg::BN;
+    const int K = g.k;
+    const int ksteps = K >> 7;
+
+    // ---- direct-to-LDS load plan: wave w fills rows 64w..64w+63 of both
+    // operands, 8 rows per instruction, 8 + 8 instructions per slab. Lane l lands
+    // at row (l>>3), position (l&7) of its 1 KiB block and so fetches logical chunk
+    // (l&7) ^ f(row): c0 = (l&7)^(l>>3) for even instructions, c0 ^ 1 for odd ones.
+    // Rows past M / N are past the buffer's num_records and read as zero; a slab
+    // past K is switched off by a zero-length descriptor.
+    const uint32_t x_bytes = (uint32_t)g.m * (uint32_t)K, w_bytes = (uint32_t)g.n * (uint32_t)K;
+    uint32_t x_off[2], w_off[2];
+    {
+        const int c0 = (lane & 7) ^ (lane >> 3);
+        const uint32_t xr = (uint32_t)(m0 + wave * 64 + (lane >> 3)) * (uint32_t)K;
+        const uint32_t wr = (uint32_t)(n0 + wave * 64 + (lane >> 3)) * (uint32_t)K;
+        x_off[0] = xr + (uint32_t)c0 * 16;
+        x_off[1] = xr + (uint32_t)(c0 ^ 1) * 16;
+        w_off[0] = wr + (uint32_t)c0 * 16;
+        w_off[1] = wr + (uint32_t)(c0 ^ 1) * 16;
+    }
+    const uint32_t row8 = 8u * (uint32_t)K;
+    uint8_t* const dma_base = lds + wave * (64 * 128);
+
+    // instruction r of 8 of one operand's slab
+    auto dma_x = [&](int r, __amdgpu_buffer_rsrc_t rx, int xstage, uint32_t k0) {
+        lds_dma16(rx, dma_base + xstage * Cfg::OPERAND_BYTES + r * 1024,
+                  x_off[r & 1] + (uint32_t)r * row8, k0);
+    };
+    auto dma_w = [&](int r, __amdgpu_buffer_rsrc_t rw, int wstage, uint32_t k0) {
+        lds_dma16(rw, dma_base + Cfg::W_BASE + wstage * Cfg::OPERAND_BYTES + r * 1024,
+                  w_off[r & 1] + (uint32_t)r * row8, k0);
+    };
+
+    // ---- operand read plan
+    int frag_off[4];
+    {
+        const int sw = (lrow & 7) ^ ((lrow >> 3) & 1);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) frag_off[j] = lrow * 128 + (((4 * lgrp + j) ^ sw) << 4);
+    }
+    const int x_rd = (wave_m * 128) * 128;
+    const int w_rd = Cfg::W_BASE + (wave_n * 128) * 128;
+
+    // piece r of 16 of half h of the slab in activation stage xs / weight stage ws
+    auto read_one = [&](int r, int xs, int ws, int h, u32x4 (&xf)[MI][2], u32x4 (&wf)[NI][2]) {
+        const int which = r >> 1, c = r & 1, sub = kReadSub[which];
+        if (kReadIsW[which])
+            wf[sub][c] = *reinterpret_cast<const u32x4*>(
+                lds + w_rd + ws * Cfg::OPERAND_BYTES + sub * 4096 + frag_off[2 * h + c]);
+        else
+            xf[sub][c] = *reinterpret_cast<const u32x4*>(
+                lds + x_rd + xs * Cfg::OPERAND_BYTES + sub * 4096 + frag_off[2 * h + c]);
+    };
+
+    Acc acc[NI][MI];
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) acc[ni][mi][j] = 0;
+
+    u32x4 xf0[MI][2], wf0[NI][2], xf1[MI][2], wf1[NI][2];
+
+    // MFMA number i of a half slab: K step outermost, then m, then n -- sixteen
+    // accumulators in turn, never two MFMAs in a row on the same one
+    auto mfma_one = [&](int i, const u32x4 (&xf)[MI][2], const u32x4 (&wf)[NI][2]) {
+        const int s = i / (MI * NI), mi = (i / NI) % MI, ni = i % NI;
+        acc[ni][mi] = Op::mma_half(s, wf[ni], xf[mi], acc[ni][mi]);
+    };
+
+    // ---- prologue: slabs 0 and 1 in flight; slab 0 visible; first half of slab 0 in F0
+    PP_STAMP();
+    {
+        const __amdgpu_buffer_rsrc_t rx = make_rsrc(g.a, x_bytes), rw = make_rsrc(g.b, w_bytes);
+        const __amdgpu_buffer_rsrc_t rx1 = make_rsrc(g.a, ksteps > 1 ? x_bytes : 0u);
+        const __amdgpu_buffer_rsrc_t rw1 = make_rsrc(g.b, ksteps > 1 ? w_bytes : 0u);
+#pragma unroll
+        for (int r = 0; r < 8; ++r) dma_x(r, rx, 0, 0u);
+#pragma unroll
+        for (int r = 0; r < 8; ++r) dma_w(r, rw, 0, 0u);
+#pragma unroll
+        for (int r = 0; r < 8; ++r) dma_x(r, rx1, 1, 128u);
+#pragma unroll
+        for (int r = 0; r < 8; ++r) dma_w(r, rw1, 1, 128u);
+        wait_vmcnt<16>();  // slab 0
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < 16; ++r) read_one(r, 0, 0, 0, xf0, wf0);
+    }
+
+    // reads are spread over the first three quarters of a half's MFMAs so that the
+    // last one has returned by the time the half ends; the eight loads of a half
+    // over all of them, one every other MFMA -- the CU's one load path takes a
+    // 1 KiB instruction every 16 cycles, so four waves issuing one per 64-cycle
+    // MFMA would saturate it and stall their own instruction streams
+    constexpr int kReadSpan = (3 * NM) / 4;
+
+    int xs = 0;  // k % 3
+    const __amdgpu_buffer_rsrc_t rx = make_rsrc(g.a, x_bytes), rw = make_rsrc(g.b, w_bytes);
+
+    // one K slab; LOADS: slab k+2 exists and is fetched during this one
+    auto slab = [&](auto loads_c, int k) {
+        constexpr bool LOADS = decltype(loads_c)::value;
+        const int ws = k & 1;
+        const int xs1 = (xs == 2) ? 0 : xs + 1;   // (k + 1) % 3
+        const int xs2 = (xs == 0) ? 2 : xs - 1;   // (k + 2) % 3
+        const uint32_t k2 = (uint32_t)(k + 2) << 7;
+
+        // first half: MFMAs on F0, reads of (k, half 1) into F1, activation rows
+        // of slab k+2 into the stage slab k-1 left at the previous barrier
+        PP_STAMP();
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < NM; ++i) {
+            mfma_one(i, xf0, wf0);
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                if ((r * kReadSpan) / 16 == i) read_one(r, xs, ws, 1, xf1, wf1);
+            if constexpr (LOADS) {
+#pragma unroll
+                for (int d = 0; d < 8; ++d)
+                    if ((d * NM) / 8 == i) dma_x(d, rx, xs2, k2);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+
+        // Slab k+1 has landed for this wave -- all but this half's eight loads are
+        // older -- and this wave is done reading slab k; after the barrier both
+        // hold for every wave.
+        PP_STAMP();
+        wait_vmcnt<LOADS ? 8 : 0>();
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+        PP_STAMP();
+        phase_barrier();
+        PP_STAMP();
+
+        // second half: MFMAs on F1, reads of (k+1, half 0) into F0 (stale bytes
+        // after the last slab, never used), weight rows of slab k+2 into the stage
+        // slab k occupied
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < NM; ++i) {
+            mfma_one(i, xf1, wf1);
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                if ((r * kReadSpan) / 16 == i) read_one(r, xs1, ws ^ 1, 0, xf0, wf0);
+            if constexpr (LOADS) {
+#pragma unroll
+                for (int d = 0; d < 8; ++d)
+                    if ((d * NM) / 8 == i) dma_w(d, rw, ws, k2);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        xs = xs1;
+    };
+
+    int k = 0;
+    for (; k + 2 < ksteps; ++k) slab(std::true_type{}, k);
+    for (; k < ksteps; ++k) slab(std::false_type{}, k);
+    // no load outlives the loop; the stages are dead for every wave
+    PP_STAMP();
+    __builtin_amdgcn_s_waitcnt(0x0070);
+    phase_barrier();
+
+    // ---------------- epilogue ----------------
+    const EpilogueScalars es = load_epilogue_scalars<ScaleKind>(g);
+    {
+        // bf16 only, N % 8 == 0 (the launcher sends everything else to the ping-pong
+        // kernel). Through LDS, 64 columns at a time: the wave lays 128(m) x 64(n)
+        // values down row-major (144-byte rows) in its private region and streams
+        // them out as full 128-byte lines, 16 bytes a lane. LDS operations of one
+        // wave complete in order, so the second pass may overwrite the first.
+        uint8_t* const mine = lds + wave * Cfg::EPI_WAVE_BYTES;
+        const uint16_t* bias = static_cast<const uint16_t*>(g.bias);
+        uint16_t* out = static_cast<uint16_t*>(g.out);
+        const int rr = lane >> 3, cc = lane & 7;
+        [[maybe_unused]] const float s_tensor = es.sa * es.sb;
+#pragma unroll
+        for (int p = 0; p < NI / 2; ++p) {
+            const int nw = n0 + wave_n * 128 + p * 64;
+#pragma unroll
+            for (int nj = 0; nj < 2; ++nj) {
+                const int ni = 2 * p + nj;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int nl = nj * 32 + q * 8 + lgrp * 4;  // first of this lane's four n
+                    const int n = nw + nl;
+                    f32x4 sw4 = {1.0f, 1.0f, 1.0f, 1.0f};
+                    f32x4 b4 = {0.0f, 0.0f, 0.0f, 0.0f};
+                    if (n < g.n) {  // N % 8 == 0: the four are in range together
+                        if constexpr (ScaleKind == SCALE_ROWCOL)
+                            sw4 = *reinterpret_cast<const f32x4*>(g.sb + n);
+                        if (bias) {
+                            const u32x2 raw = *reinterpret_cast<const u32x2*>(bias + n);
+                            b4 = f32x4{__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u),
+                                       __uint_as_float(raw.y << 16), __uint_as_float(raw.y & 0xffff0000u)};
+                        }
+                    }
+#pragma unroll
+                    for (int mi = 0; mi < MI; ++mi) {
+                        const int ml = mi * 32 + lrow;
+                        const int m = m0 + wave_m * 128 + ml;
+                        float sx = 1.0f;
+                        if constexpr (ScaleKind == SCALE_ROWCOL) sx = (m < g.m) ? g.sa[m] : 0.0f;
+                        float v[4];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            float f = (float)acc[ni][mi][4 * q + j];
+                            if constexpr (ScaleKind == SCALE_TENSOR) f = f * s_tensor;
+                            else f = f * sx * sw4[j];
+                            v[j] = f + b4[j];
+                        }
+                        u32x2 pk;
+                        pk.x = pack_bf16x2(v[0], v[1]);
+                        pk.y = pack_bf16x2(v[2], v[3]);
+                        *reinterpret_cast<u32x2*>(mine + ml * Cfg::EPI_ROW_BYTES + nl * 2) = pk;
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int ml = i * 8 + rr;
+                const u32x4 v = *reinterpret_cast<const u32x4*>(mine + ml * Cfg::EPI_ROW_BYTES + cc * 16);
+                const int m = m0 + wave_m * 128 + ml;
+                const int n = nw + cc * 8;
+                if (m < g.m && n < g.n) *reinterpret_cast<u32x4*>(out + (size_t)m * g.n + n) = v;
+            }
+        }
+    }
+    PP_STAMP();
+}
+
+// bf16 output with whole 16-byte output pieces only; other outputs keep the
+// ping-pong kernel, whose epilogue handles every case
+inline bool wave128_shape_ok(const GemmArgs& g) {
+    return pingpong_shape_ok(g) && g.out_kind == OUT_BF16 && (g.n & 7) == 0;
+}
+
+template <class Op, int ScaleKind>
+inline void launch_wave128(const GemmArgs& g, hipStream_t stream) {
+    using Cfg = Wave128Cfg;
+    const int tiles = ((g.m + Cfg::BM - 1) / Cfg::BM) * ((g.n + Cfg::BN - 1) / Cfg::BN);
+    auto kern = gemm_wave128_kernel<Op, ScaleKind>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+        attr_set = true;
+    }
+    kern<<<dim3((unsigned)tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(g);
+}
+
+}  // namespace w8a8
