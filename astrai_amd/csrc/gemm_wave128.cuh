@@ -31,6 +31,9 @@
 // c of row r at position c ^ (r & 7) ^ ((r >> 3) & 1); weight rows are the
 // first MFMA operand.
 #pragma once
+#ifndef W128_STORE_COND
+#define W128_STORE_COND
+#endif
 
 #include "gemm_pingpong.cuh"
 
@@ -81,6 +84,9 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
     const int m0 = tc.tm * Cfg::BM, n0 = tc.tn * Cfg::BN;
     const int K = g.k;
     const int ksteps = K >> 7;
+    // requested now, used in the epilogue: the latency hides under the main loop
+    const EpilogueScalars es = load_epilogue_scalars<ScaleKind>(g);
+    [[maybe_unused]] const float s_tensor = es.sa * es.sb;
 
     // ---- direct-to-LDS load plan: wave w fills rows 64w..64w+63 of both
     // operands, 8 rows per instruction, 8 + 8 instructions per slab. Lane l lands
@@ -246,51 +252,70 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
     phase_barrier();
 
     // ---------------- epilogue ----------------
-    const EpilogueScalars es = load_epilogue_scalars<ScaleKind>(g);
+    // bf16 only, N % 8 == 0 (the launcher sends everything else to the ping-pong
+    // kernel). Through LDS, 64 columns at a time: the wave lays 128(m) x 64(n)
+    // values down row-major (144-byte rows) in its private region and streams
+    // them out as full 128-byte lines, 16 bytes a lane. LDS operations of one
+    // wave complete in order, so the second pass may overwrite the first.
+    // Every per-column / per-row operand of a pass is requested before the first
+    // one is used, so the pass pays one memory latency, not one per use.
     {
-        // bf16 only, N % 8 == 0 (the launcher sends everything else to the ping-pong
-        // kernel). Through LDS, 64 columns at a time: the wave lays 128(m) x 64(n)
-        // values down row-major (144-byte rows) in its private region and streams
-        // them out as full 128-byte lines, 16 bytes a lane. LDS operations of one
-        // wave complete in order, so the second pass may overwrite the first.
         uint8_t* const mine = lds + wave * Cfg::EPI_WAVE_BYTES;
         const uint16_t* bias = static_cast<const uint16_t*>(g.bias);
-        uint16_t* out = static_cast<uint16_t*>(g.out);
         const int rr = lane >> 3, cc = lane & 7;
-        [[maybe_unused]] const float s_tensor = es.sa * es.sb;
+        // output rows of this tile through a buffer descriptor: rows past M and
+        // (by the offset chosen below) columns past N are dropped by the bounds
+        // check, no predicates, no 64-bit address arithmetic per store
+        const int rows_here = min(Cfg::BM, g.m - m0);
+        const uint32_t row_bytes = (uint32_t)g.n * 2u;
+        const __amdgpu_buffer_rsrc_t rout =
+            make_rsrc(static_cast<uint16_t*>(g.out) + (size_t)m0 * g.n, (uint32_t)rows_here * row_bytes);
+
+        float sx[MI];
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi) {
+            sx[mi] = 1.0f;
+            if constexpr (ScaleKind == SCALE_ROWCOL) {
+                const int m = m0 + wave_m * 128 + mi * 32 + lrow;
+                sx[mi] = (m < g.m) ? g.sa[m] : 0.0f;
+            }
+        }
 #pragma unroll
         for (int p = 0; p < NI / 2; ++p) {
             const int nw = n0 + wave_n * 128 + p * 64;
+            f32x4 sw4[2][4];
+            u32x2 braw[2][4];
+#pragma unroll
+            for (int nj = 0; nj < 2; ++nj)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int n = nw + nj * 32 + q * 8 + lgrp * 4;  // first of this lane's four n
+                    sw4[nj][q] = f32x4{1.0f, 1.0f, 1.0f, 1.0f};
+                    braw[nj][q] = u32x2{0u, 0u};
+                    if (n < g.n) {  // N % 8 == 0: the four are in range together
+                        if constexpr (ScaleKind == SCALE_ROWCOL)
+                            sw4[nj][q] = *reinterpret_cast<const f32x4*>(g.sb + n);
+                        if (bias) braw[nj][q] = *reinterpret_cast<const u32x2*>(bias + n);
+                    }
+                }
 #pragma unroll
             for (int nj = 0; nj < 2; ++nj) {
                 const int ni = 2 * p + nj;
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    const int nl = nj * 32 + q * 8 + lgrp * 4;  // first of this lane's four n
-                    const int n = nw + nl;
-                    f32x4 sw4 = {1.0f, 1.0f, 1.0f, 1.0f};
-                    f32x4 b4 = {0.0f, 0.0f, 0.0f, 0.0f};
-                    if (n < g.n) {  // N % 8 == 0: the four are in range together
-                        if constexpr (ScaleKind == SCALE_ROWCOL)
-                            sw4 = *reinterpret_cast<const f32x4*>(g.sb + n);
-                        if (bias) {
-                            const u32x2 raw = *reinterpret_cast<const u32x2*>(bias + n);
-                            b4 = f32x4{__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u),
-                                       __uint_as_float(raw.y << 16), __uint_as_float(raw.y & 0xffff0000u)};
-                        }
-                    }
+                    const int nl = nj * 32 + q * 8 + lgrp * 4;
+                    const u32x2 raw = braw[nj][q];
+                    const f32x4 b4 = {__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u),
+                                      __uint_as_float(raw.y << 16), __uint_as_float(raw.y & 0xffff0000u)};
 #pragma unroll
                     for (int mi = 0; mi < MI; ++mi) {
                         const int ml = mi * 32 + lrow;
-                        const int m = m0 + wave_m * 128 + ml;
-                        float sx = 1.0f;
-                        if constexpr (ScaleKind == SCALE_ROWCOL) sx = (m < g.m) ? g.sa[m] : 0.0f;
                         float v[4];
 #pragma unroll
                         for (int j = 0; j < 4; ++j) {
                             float f = (float)acc[ni][mi][4 * q + j];
                             if constexpr (ScaleKind == SCALE_TENSOR) f = f * s_tensor;
-                            else f = f * sx * sw4[j];
+                            else f = f * sx[mi] * sw4[nj][q][j];
                             v[j] = f + b4[j];
                         }
                         u32x2 pk;
@@ -300,13 +325,17 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
                     }
                 }
             }
+            const int n = nw + cc * 8;
+            const uint32_t lane_off = (n < g.n)
+                ? (uint32_t)(wave_m * 128 + rr) * row_bytes + (uint32_t)n * 2u
+                : kOutOfRange;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int ml = i * 8 + rr;
                 const u32x4 v = *reinterpret_cast<const u32x4*>(mine + ml * Cfg::EPI_ROW_BYTES + cc * 16);
-                const int m = m0 + wave_m * 128 + ml;
-                const int n = nw + cc * 8;
-                if (m < g.m && n < g.n) *reinterpret_cast<u32x4*>(out + (size_t)m * g.n + n) = v;
+                // the row step goes into the checked (vector) offset: the scalar
+                // offset of a buffer instruction takes no part in the bounds check
+                __builtin_amdgcn_raw_buffer_store_b128(v, rout, lane_off + (uint32_t)(i * 8) * row_bytes, 0, 0);
             }
         }
     }
@@ -316,7 +345,8 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
 // bf16 output with whole 16-byte output pieces only; other outputs keep the
 // ping-pong kernel, whose epilogue handles every case
 inline bool wave128_shape_ok(const GemmArgs& g) {
-    return pingpong_shape_ok(g) && g.out_kind == OUT_BF16 && (g.n & 7) == 0;
+    // (a tile's 256 output rows are addressed with 32-bit byte offsets)
+    return pingpong_shape_ok(g) && g.out_kind == OUT_BF16 && (g.n & 7) == 0 && g.n <= (1 << 22);
 }
 
 template <class Op, int ScaleKind>

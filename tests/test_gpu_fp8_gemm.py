@@ -230,3 +230,38 @@ def test_config3_shape_sampled_rows():
     assert torch.equal(x8[rows].cpu().view(torch.uint8), rx8.view(torch.uint8))
     assert torch.equal(sb.cpu(), rsb)
     assert_bf16_close(out[rows], O.fp8_gemm_blockscaled(rx8, rw8, rsa, rsb), what="config3 rows")
+
+
+# ---- large ragged shapes: the 256x256-tile kernels with partial edge tiles ----
+
+@pytest.mark.parametrize("m,n,k,bias", [(3900, 4104, 1152, True),    # N % 8 == 0: four-wave kernel
+                                        (3841, 4100, 640, False),   # N % 8 != 0: ping-pong kernel
+                                        (4096, 3848, 256, False)])  # shortest K the big kernels take
+def test_large_ragged_tiles_with_guard_rows(m, n, k, bias):
+    """Edge tiles of the large-shape kernels: rows past M / columns past N must
+    read as zero and must not be written. The call goes through the C ABI into
+    an output buffer with sentinel rows behind row M-1."""
+    from astrai_amd.extension import _cabi
+    print(f"case m={m} n={n} k={k} bias={bias}", flush=True)
+    lib = _cabi.load()
+    g = torch.Generator().manual_seed(m + n + k)
+    a8 = (torch.randn(m, k, generator=g) * 0.5).to(torch.float8_e4m3fn)
+    b8 = (torch.randn(n, k, generator=g) * 0.5).to(torch.float8_e4m3fn)
+    bvec = torch.randn(n, generator=g).to(torch.bfloat16) if bias else None
+    sa, sb = torch.tensor([0.75]), torch.tensor([1.25])
+    guard = 8
+    out = torch.full((m + guard, n), -777.0, dtype=torch.bfloat16, device=DEV)
+    da, db, dsa, dsb = a8.to(DEV), b8.to(DEV), sa.to(DEV), sb.to(DEV)
+    dbias = bvec.to(DEV) if bias else None
+    rc = lib.astrai_w8a8_gemm_fp8_pt(da.data_ptr(), db.data_ptr(), dsa.data_ptr(), dsb.data_ptr(), None,
+                                     dbias.data_ptr() if bias else None, out.data_ptr(), m, n, k, 0, 0,
+                                     torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, lib.astrai_w8a8_last_error()
+    torch.cuda.synchronize()
+    assert torch.all(out[m:] == -777.0), "rows past M were written"
+    rows = torch.cat([torch.arange(0, 3), torch.arange(255, 258), torch.arange(m - 3, m)])
+    want = O.fp8_gemm_bias(a8[rows], b8, sa, sb, bvec)
+    assert_bf16_close(out[rows], want, what="ragged rows")
+    cols = torch.cat([torch.arange(0, 2), torch.arange(n - 9, n)])
+    want_c = O.fp8_gemm_bias(a8, b8[cols], sa, sb, bvec[cols] if bias else None)
+    assert_bf16_close(out[:m, cols], want_c, what="ragged columns")

@@ -120,3 +120,39 @@ def test_full_size_linearity_property(C):
     assert torch.equal(s, p1 + p2)
     rows = torch.tensor([0, 1, 255, 256, 2047, 4095])
     assert torch.equal(p1.cpu()[rows], O.int8_acc(a1[rows], b))
+
+
+@pytest.mark.parametrize("m,n,k,out_dtype", [(3900, 4104, 1152, 0),   # bf16, N % 8 == 0: four-wave kernel
+                                             (3841, 4100, 640, 0),    # bf16, N % 8 != 0: ping-pong kernel
+                                             (3900, 4104, 384, 2)])   # int32 accumulator: ping-pong kernel
+def test_large_ragged_tiles_with_guard_rows(C, m, n, k, out_dtype):
+    """Edge tiles of the large-shape kernels: bit-exact int32 (or the bf16
+    epilogue of it) on the first / tile-boundary / last rows and the last columns,
+    and nothing written behind row M-1 (sentinel rows after the output)."""
+    print(f"case m={m} n={n} k={k} out_dtype={out_dtype}", flush=True)
+    lib = C.load()
+    g = torch.Generator().manual_seed(m + n + k)
+    a = _rand_i8(g, m, k)
+    b = _rand_i8(g, n, k)
+    sa = torch.rand(m, generator=g) * 0.02 + 0.001
+    sb = torch.rand(n, generator=g) * 0.02 + 0.001
+    guard = 8
+    if out_dtype == 2:
+        out = torch.full((m + guard, n), -777, dtype=torch.int32, device=DEV)
+    else:
+        out = torch.full((m + guard, n), -777.0, dtype=torch.bfloat16, device=DEV)
+    da, db, dsa, dsb = a.to(DEV), b.to(DEV), sa.to(DEV), sb.to(DEV)
+    rc = lib.astrai_w8a8_gemm_int8_ptpc(da.data_ptr(), db.data_ptr(), dsa.data_ptr(), dsb.data_ptr(), None,
+                                        out.data_ptr(), m, n, k, out_dtype,
+                                        torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, lib.astrai_w8a8_last_error()
+    torch.cuda.synchronize()
+    assert torch.all(out[m:] == -777), "rows past M were written"
+    rows = torch.cat([torch.arange(0, 3), torch.arange(255, 258), torch.arange(m - 3, m)])
+    cols = torch.cat([torch.arange(0, 2), torch.arange(n - 9, n)])
+    if out_dtype == 2:
+        assert torch.equal(out[rows].cpu(), O.int8_acc(a[rows], b))
+        assert torch.equal(out[:m, cols].cpu(), O.int8_acc(a, b[cols]))
+    else:
+        assert torch.equal(out[rows].cpu(), O.int8_gemm(a[rows], b, sa[rows], sb))
+        assert torch.equal(out[:m, cols].cpu(), O.int8_gemm(a, b[cols], sa, sb[cols]))
