@@ -313,10 +313,16 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
                         float v[4];
 #pragma unroll
                         for (int j = 0; j < 4; ++j) {
-                            float f = (float)acc[ni][mi][4 * q + j];
-                            if constexpr (ScaleKind == SCALE_TENSOR) f = f * s_tensor;
-                            else f = f * sx[mi] * sw4[nj][q][j];
-                            v[j] = f + b4[j];
+                            const float f = (float)acc[ni][mi][4 * q + j];
+                            if constexpr (ScaleKind == SCALE_TENSOR) {
+                                v[j] = f * s_tensor + b4[j];
+                            } else {
+                                // int8: product and bias add rounded separately, the
+                                // epilogue is elementwise fp32 on the exact integer
+#pragma clang fp contract(off)
+                                const float scaled = f * sx[mi] * sw4[nj][q][j];
+                                v[j] = scaled + b4[j];
+                            }
                         }
                         u32x2 pk;
                         pk.x = pack_bf16x2(v[0], v[1]);

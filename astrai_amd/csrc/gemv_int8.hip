@@ -5,7 +5,10 @@
 // (integer addition is associative, so the split keeps the accumulator
 // bit-exact) and the first waves run the dequant epilogue.
 //
-//  * M <= 32: gemv_int8_lds_kernel streams the weights through LDS with 1 KiB
+//  * M = 1: gemv_int8_dot_kernel, one wave per four weight rows, whole 1 KiB row
+//    pieces straight into registers and v_dot4 on the vector ALU -- no LDS, no
+//    barrier, every wave of the launch resident and loading at once.
+//  * 1 < M <= 32: gemv_int8_lds_kernel streams the weights through LDS with 1 KiB
 //    contiguous row pieces per instruction (see the comment on the kernel).
 //  * 32 < M <= 64: gemv_int8_kernel loads MFMA-shaped operands straight into
 //    registers (64 contiguous bytes of 16 rows per instruction).
@@ -79,6 +82,82 @@ __global__ __launch_bounds__(NW * 64) void gemv_int8_kernel(GemmArgs g) {
         for (int w = 1; w < NW; ++w) sum += red[w][t][lane];
         const int r = t / MB, b = t % MB;
         store_subtile<OpI8, SCALE_ROWCOL>(g, es, sum, b * 16 + lrow, n0 + r * 16 + lgrp * 4);
+    }
+}
+
+// Single-token kernel (M = 1). A workgroup is one wave and owns R = 4 weight
+// rows; lane l holds bytes [16 l, 16 l + 16) of every 1 KiB K-step of its rows and
+// of the token, so each load instruction moves one whole 1 KiB row piece (the
+// request pattern HBM and the address coalescer like best) and the matching
+// activation bytes sit in the same lane. The dot products run on the vector ALU
+// (v_dot4_i32_i8, exact int32), which frees the kernel of LDS, barriers and
+// operand shuffles: a wave needs ~60 registers, so the ~2750 waves of an
+// 11008-row matrix are all resident at once and the whole matrix is requested in
+// the first microsecond. Lane partials are summed across the wave at the end
+// (integer addition: the split over lanes keeps the accumulator bit-exact). The
+// vector ALU's dot4 rate carries one token comfortably, not several: from two
+// tokens on the MFMA kernel below is faster.
+__global__ __launch_bounds__(64) void gemv_int8_dot_kernel(GemmArgs g) {
+    constexpr int R = 4;
+    const int lane = threadIdx.x;
+    const int n0 = blockIdx.x * R;
+    const int K = g.k;
+    const __amdgpu_buffer_rsrc_t rw = make_rsrc(g.b, (uint32_t)g.n * (uint32_t)K);
+    const __amdgpu_buffer_rsrc_t rx = make_rsrc(g.a, (uint32_t)K);
+
+    // rows past N start past the buffer's num_records: zeros
+    uint32_t w_off[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) w_off[r] = (uint32_t)(n0 + r) * (uint32_t)K + lane * 16;
+
+    // epilogue operands of the lane that will write row n0 + lane, requested
+    // first so that their latency hides under the weight stream
+    const int en = n0 + lane;
+    const bool writer = lane < R && en < g.n;
+    float e_sx = 0.0f, e_sw = 0.0f, e_b = 0.0f;
+    if (writer && g.out_kind != OUT_ACC) {
+        e_sx = g.sa[0];
+        e_sw = g.sb[en];
+        if (g.bias) e_b = bf16_to_f32(static_cast<const uint16_t*>(g.bias)[en]);
+    }
+
+    int acc[R] = {0, 0, 0, 0};
+#pragma unroll 2
+    for (int k0 = 0; k0 < K; k0 += 1024) {
+        const bool in = k0 + lane * 16 < K;
+        u32x4 wv[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) wv[r] = buf_load16(rw, in ? w_off[r] : kOutOfRange, (uint32_t)k0);
+        const u32x4 xv = buf_load16(rx, in ? (uint32_t)(lane * 16) : kOutOfRange, (uint32_t)k0);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int a = acc[r];
+            a = __builtin_amdgcn_sdot4((int)wv[r].x, (int)xv.x, a, false);
+            a = __builtin_amdgcn_sdot4((int)wv[r].y, (int)xv.y, a, false);
+            a = __builtin_amdgcn_sdot4((int)wv[r].z, (int)xv.z, a, false);
+            a = __builtin_amdgcn_sdot4((int)wv[r].w, (int)xv.w, a, false);
+            acc[r] = a;
+        }
+    }
+
+    int mine = 0;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        int v = acc[r];
+#pragma unroll
+        for (int off = 32; off; off >>= 1) v += __shfl_xor(v, off, kWave);
+        if (lane == r) mine = v;
+    }
+    if (writer) {
+        if (g.out_kind == OUT_ACC) {
+            static_cast<int*>(g.out)[en] = mine;
+        } else {
+            // product and bias add rounded separately (no fused multiply-add): the
+            // int8 epilogue is specified as elementwise fp32 on the exact integer
+#pragma clang fp contract(off)
+            const float scaled = (float)mine * e_sx * e_sw;
+            static_cast<uint16_t*>(g.out)[en] = f32_to_bf16(scaled + e_b);
+        }
     }
 }
 
@@ -201,6 +280,11 @@ __global__ __launch_bounds__(256) void gemv_int8_lds_kernel(GemmArgs g) {
     }
 }
 
+void launch_dot(const GemmArgs& g, hipStream_t stream) {
+    const int blocks = (g.n + 3) / 4;
+    gemv_int8_dot_kernel<<<dim3((unsigned)blocks), dim3(64), 0, stream>>>(g);
+}
+
 template <int MB>
 void launch_lds(const GemmArgs& g, hipStream_t stream) {
     const int blocks = (g.n + 15) / 16;
@@ -227,6 +311,10 @@ bool launch_gemv_int8(const GemmArgs& g, hipStream_t stream) {
     if (g.m <= 0 || g.m > 64 || g.n <= 0 || g.k <= 0 || (g.k & 255) != 0) return false;
     const int64_t lim = (int64_t)1 << 31;
     if ((int64_t)g.n * g.k >= lim) return false;
+    if (g.m == 1) {
+        launch_dot(g, stream);
+        return true;
+    }
     const int mb = (g.m + 15) / 16;
     switch (mb) {
         case 1: launch_lds<1>(g, stream); break;

@@ -27,7 +27,7 @@ PEAK_INT8_TOPS = 5000.0    # MI355X dense int8 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM-side bytes per launch of the headline kernel from two counter passes
 # (reads 101.0 MB + writes 33.6 MB); algorithmic bytes are 67.1 MB
-HEADLINE_TRAFFIC_MB = 134.6
+HEADLINE_TRAFFIC_MB = 135.5
 
 
 def _event_time_ms(fn, iters, warmup):
@@ -233,8 +233,8 @@ def main():
     roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP8_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP8_TFLOPS, 4),
                 "traffic": HEADLINE_TRAFFIC_MB, "traffic_unit": "MB per launch (rocprofv3 FETCH_SIZE + "
-                "WRITE_SIZE, calibrated on a plain copy; summary in profiles/gemm_fp8_pingpong_4096cubed.txt)",
-                "kernel": "gemm_pingpong_kernel<Op32F8<e4m3>,per-tensor> (256x256x128)",
+                "WRITE_SIZE, calibrated on a plain copy; summary in profiles/gemm_fp8_wave128_4096cubed.txt)",
+                "kernel": "gemm_wave128_kernel<Op32F8<e4m3>,per-tensor> (256x256x128, 4 waves)",
                 "avg_launch_us": round(kern_ms * 1e3, 2)}
 
     # ---------------- CPU baseline: the oracle on this host ----------------
