@@ -31,8 +31,12 @@
 // c of row r at position c ^ (r & 7) ^ ((r >> 3) & 1); weight rows are the
 // first MFMA operand.
 #pragma once
-#ifndef W128_STORE_COND
-#define W128_STORE_COND
+// per-phase timestamps inside the main loop perturb it (~100 cycles each): off
+// unless asked for; the stamps around the loop are always taken when timing is on
+#ifdef W128_INNER_STAMPS
+#define PP_STAMP_INNER() PP_STAMP()
+#else
+#define PP_STAMP_INNER()
 #endif
 
 #include "gemm_pingpong.cuh"
@@ -87,6 +91,15 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
     // requested now, used in the epilogue: the latency hides under the main loop
     const EpilogueScalars es = load_epilogue_scalars<ScaleKind>(g);
     [[maybe_unused]] const float s_tensor = es.sa * es.sb;
+    float sx[Cfg::MI];  // per-row scales of this lane's four rows (SCALE_ROWCOL)
+#pragma unroll
+    for (int mi = 0; mi < Cfg::MI; ++mi) {
+        sx[mi] = 1.0f;
+        if constexpr (ScaleKind == SCALE_ROWCOL) {
+            const int m = m0 + wave_m * 128 + mi * 32 + lrow;
+            sx[mi] = (m < g.m) ? g.sa[m] : 0.0f;
+        }
+    }
 
     // ---- direct-to-LDS load plan: wave w fills rows 64w..64w+63 of both
     // operands, 8 rows per instruction, 8 + 8 instructions per slab. Lane l lands
@@ -197,7 +210,7 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
 
         // first half: MFMAs on F0, reads of (k, half 1) into F1, activation rows
         // of slab k+2 into the stage slab k-1 left at the previous barrier
-        PP_STAMP();
+        PP_STAMP_INNER();
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < NM; ++i) {
@@ -216,12 +229,12 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
         // Slab k+1 has landed for this wave -- all but this half's eight loads are
         // older -- and this wave is done reading slab k; after the barrier both
         // hold for every wave.
-        PP_STAMP();
+        PP_STAMP_INNER();
         wait_vmcnt<LOADS ? 8 : 0>();
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
-        PP_STAMP();
+        PP_STAMP_INNER();
         phase_barrier();
-        PP_STAMP();
+        PP_STAMP_INNER();
 
         // second half: MFMAs on F1, reads of (k+1, half 0) into F0 (stale bytes
         // after the last slab, never used), weight rows of slab k+2 into the stage
@@ -244,6 +257,7 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
     };
 
     int k = 0;
+    PP_STAMP();
     for (; k + 2 < ksteps; ++k) slab(std::true_type{}, k);
     for (; k < ksteps; ++k) slab(std::false_type{}, k);
     // no load outlives the loop; the stages are dead for every wave
@@ -271,15 +285,6 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
         const __amdgpu_buffer_rsrc_t rout =
             make_rsrc(static_cast<uint16_t*>(g.out) + (size_t)m0 * g.n, (uint32_t)rows_here * row_bytes);
 
-        float sx[MI];
-#pragma unroll
-        for (int mi = 0; mi < MI; ++mi) {
-            sx[mi] = 1.0f;
-            if constexpr (ScaleKind == SCALE_ROWCOL) {
-                const int m = m0 + wave_m * 128 + mi * 32 + lrow;
-                sx[mi] = (m < g.m) ? g.sa[m] : 0.0f;
-            }
-        }
 #pragma unroll
         for (int p = 0; p < NI / 2; ++p) {
             const int nw = n0 + wave_n * 128 + p * 64;
