@@ -95,6 +95,44 @@ int astrai_w8a8_quantize_bf16_int8_rows(const void* x, void* xq, float* s, int64
     return check_launch("quantize_bf16_int8_rows");
 }
 
+int astrai_w8a8_add_rmsnorm_quantize_int8_rows(const void* x, const void* res, const void* weight,
+                                               float eps, void* sum_out, void* y_out, void* xq,
+                                               float* s, int64_t rows, int64_t k, void* stream) {
+    if (!x || !weight || !xq || !s)
+        return fail(ASTRAI_W8A8_BAD_ARG, "add_rmsnorm_quantize_int8_rows: null pointer");
+    if (rows < 0 || k < 0 || rows > 0x7fffffff)
+        return fail(ASTRAI_W8A8_BAD_ARG, "add_rmsnorm_quantize_int8_rows: bad dims");
+    if (!(eps >= 0.0f)) return fail(ASTRAI_W8A8_BAD_ARG, "add_rmsnorm_quantize_int8_rows: eps must be >= 0");
+    if ((k & 7) != 0 || k > w8a8::kFusedRowMax)
+        return fail(ASTRAI_W8A8_UNSUPPORTED,
+                    "add_rmsnorm_quantize_int8_rows: K must be a multiple of 8 and at most 8192");
+    if (!aligned16(x) || !aligned16(weight) || !aligned16(xq) || (res && !aligned16(res)) ||
+        (sum_out && !aligned16(sum_out)) || (y_out && !aligned16(y_out)))
+        return fail(ASTRAI_W8A8_BAD_ARG, "add_rmsnorm_quantize_int8_rows: pointers must be 16-byte aligned");
+    if (rows == 0 || k == 0) return ASTRAI_W8A8_OK;
+    w8a8::launch_add_rmsnorm_quantize_int8_rows(x, res, weight, eps, sum_out, y_out, xq, s, rows, k,
+                                                static_cast<hipStream_t>(stream));
+    return check_launch("add_rmsnorm_quantize_int8_rows");
+}
+
+int astrai_w8a8_silu_mul_quantize_int8_rows(const void* gate, const void* up, int64_t ld, void* h_out,
+                                            void* hq, float* s, int64_t rows, int64_t width,
+                                            void* stream) {
+    if (!gate || !up || !hq || !s)
+        return fail(ASTRAI_W8A8_BAD_ARG, "silu_mul_quantize_int8_rows: null pointer");
+    if (rows < 0 || width < 0 || rows > 0x7fffffff || ld < width)
+        return fail(ASTRAI_W8A8_BAD_ARG, "silu_mul_quantize_int8_rows: bad dims");
+    if ((width & 7) != 0 || (ld & 7) != 0 || width > w8a8::kFusedRowMax)
+        return fail(ASTRAI_W8A8_UNSUPPORTED,
+                    "silu_mul_quantize_int8_rows: width and ld must be multiples of 8, width at most 8192");
+    if (!aligned16(gate) || !aligned16(up) || !aligned16(hq) || (h_out && !aligned16(h_out)))
+        return fail(ASTRAI_W8A8_BAD_ARG, "silu_mul_quantize_int8_rows: pointers must be 16-byte aligned");
+    if (rows == 0 || width == 0) return ASTRAI_W8A8_OK;
+    w8a8::launch_silu_mul_quantize_int8_rows(gate, up, ld, h_out, hq, s, rows, width,
+                                             static_cast<hipStream_t>(stream));
+    return check_launch("silu_mul_quantize_int8_rows");
+}
+
 int astrai_w8a8_quantize_bf16_fp8_block128_act(const void* x, void* x8, float* sa, int64_t m,
                                                int64_t k, void* stream) {
     if (!x || !x8 || !sa) return fail(ASTRAI_W8A8_BAD_ARG, "quantize_block128_act: null pointer");

@@ -28,6 +28,15 @@ void launch_quantize_fp8(const void* x, void* x8, const float* scale, float* ama
                          int64_t total, int fmt, hipStream_t stream);
 void launch_quantize_int8_rows(const void* x, void* xq, float* s, int64_t rows, int64_t k,
                                hipStream_t stream);
+// fused producers: (residual add +) RMSNorm + per-row int8; SwiGLU product + per-row
+// int8. Row width must be a multiple of 8 and at most kFusedRowMax.
+constexpr int64_t kFusedRowMax = 8192;
+void launch_add_rmsnorm_quantize_int8_rows(const void* x, const void* res, const void* w, float eps,
+                                           void* sum_out, void* y_out, void* xq, float* s,
+                                           int64_t rows, int64_t k, hipStream_t stream);
+void launch_silu_mul_quantize_int8_rows(const void* gate, const void* up, int64_t ld, void* h_out,
+                                        void* hq, float* s, int64_t rows, int64_t width,
+                                        hipStream_t stream);
 void launch_quantize_fp8_block128_act(const void* x, void* x8, float* sa, int64_t m,
                                       int64_t k, hipStream_t stream);
 void launch_quantize_fp8_block128_weight(const void* w, void* w8, float* sb, int64_t n,

@@ -155,6 +155,125 @@ __global__ __launch_bounds__(kThreads) void quantize_int8_rows_kernel(
         qr[i] = (int8_t)quant1_int8(bf16_to_f32(xr[i]), step);
 }
 
+// ---- producers fused with the per-row int8 quantizer -------------------------
+// The activation of every int8 Linear in the decoder comes out of an RMSNorm
+// (after a residual add) or out of the SwiGLU product. Fusing the per-token
+// quantizer into those removes a write and a read of the bf16 activation and a
+// launch per Linear. One workgroup per row, the row stays in registers
+// (width <= kCache * kThreads * 8 = 8192, a multiple of 8).
+
+// block-wide sum of a per-thread value; result valid in every thread
+__device__ __forceinline__ float block_sum(float v, float* slots) {
+#pragma unroll
+    for (int off = 32; off; off >>= 1) v += __shfl_xor(v, off, kWave);
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) slots[wave] = v;
+    __syncthreads();
+    float r = slots[0];
+#pragma unroll
+    for (int w = 1; w < kThreads / kWave; ++w) r += slots[w];
+    __syncthreads();
+    return r;
+}
+
+__device__ __forceinline__ float round_bf16(float f) { return bf16_to_f32(f32_to_bf16(f)); }
+
+__device__ __forceinline__ u32x4 pack8(const float (&f)[8]) {
+    u32x4 o;
+    o.x = pack_bf16x2(f[0], f[1]);
+    o.y = pack_bf16x2(f[2], f[3]);
+    o.z = pack_bf16x2(f[4], f[5]);
+    o.w = pack_bf16x2(f[6], f[7]);
+    return o;
+}
+
+// s = bf16(x + res) (when res is given; written to sum_out), y = bf16(w * (rstd * s))
+// with rstd = rsqrt(mean(s^2) + eps) in fp32 -- one rounding, the arithmetic of
+// F.rms_norm on a bf16 tensor (model/components/norm.py:7-15) -- then the per-row
+// int8 quantizer on y.
+__global__ __launch_bounds__(kThreads) void add_rmsnorm_quantize_int8_rows_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ res,
+    const uint16_t* __restrict__ w, float eps, uint16_t* __restrict__ sum_out,
+    uint16_t* __restrict__ y_out, int8_t* __restrict__ xq, float* __restrict__ s, int64_t k) {
+    __shared__ float slots[kThreads / kWave];
+    const int64_t row = blockIdx.x;
+    const int64_t nvec = k >> 3;
+    float v[kCache][8];
+    float ss = 0.0f;
+#pragma unroll
+    for (int c = 0; c < kCache; ++c) {
+        const int64_t i = threadIdx.x + (int64_t)c * kThreads;
+        if (i < nvec) {
+            unpack8(*reinterpret_cast<const u32x4*>(x + row * k + i * 8), v[c]);
+            if (res) {
+                float r[8];
+                unpack8(*reinterpret_cast<const u32x4*>(res + row * k + i * 8), r);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[c][j] = round_bf16(v[c][j] + r[j]);
+                if (sum_out) *reinterpret_cast<u32x4*>(sum_out + row * k + i * 8) = pack8(v[c]);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) ss += v[c][j] * v[c][j];
+        }
+    }
+    const float rstd = rsqrtf(block_sum(ss, slots) / (float)k + eps);
+    float local = 0.0f;
+#pragma unroll
+    for (int c = 0; c < kCache; ++c) {
+        const int64_t i = threadIdx.x + (int64_t)c * kThreads;
+        if (i < nvec) {
+            float g[8];
+            unpack8(*reinterpret_cast<const u32x4*>(w + i * 8), g);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[c][j] = round_bf16(g[j] * (rstd * v[c][j]));
+            local = fmaxf(local, amax8(v[c]));
+            if (y_out) *reinterpret_cast<u32x4*>(y_out + row * k + i * 8) = pack8(v[c]);
+        }
+    }
+    const float step = fmaxf(block_max(local, slots), 1e-12f) / 127.0f;
+    if (threadIdx.x == 0) s[row] = step;
+#pragma unroll
+    for (int c = 0; c < kCache; ++c) {
+        const int64_t i = threadIdx.x + (int64_t)c * kThreads;
+        if (i < nvec) *reinterpret_cast<u32x2*>(xq + row * k + i * 8) = quant8_int8(v[c], step);
+    }
+}
+
+// h = bf16(up * bf16(silu(gate))), silu(g) = g / (1 + exp(-g)) in fp32: the bf16
+// arithmetic of ``up(x) * F.silu(gate(x))`` (model/components/mlp.py:41); then the
+// per-row int8 quantizer on h. gate and up rows are `ld` elements apart (they may
+// be the two halves of one fused gate|up GEMM output).
+__global__ __launch_bounds__(kThreads) void silu_mul_quantize_int8_rows_kernel(
+    const uint16_t* __restrict__ gate, const uint16_t* __restrict__ up, int64_t ld,
+    uint16_t* __restrict__ h_out, int8_t* __restrict__ hq, float* __restrict__ s, int64_t width) {
+    __shared__ float slots[kThreads / kWave];
+    const int64_t row = blockIdx.x;
+    const int64_t nvec = width >> 3;
+    float v[kCache][8];
+    float local = 0.0f;
+#pragma unroll
+    for (int c = 0; c < kCache; ++c) {
+        const int64_t i = threadIdx.x + (int64_t)c * kThreads;
+        if (i < nvec) {
+            float g[8];
+            unpack8(*reinterpret_cast<const u32x4*>(gate + row * ld + i * 8), g);
+            unpack8(*reinterpret_cast<const u32x4*>(up + row * ld + i * 8), v[c]);
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                v[c][j] = round_bf16(v[c][j] * round_bf16(g[j] / (1.0f + expf(-g[j]))));
+            local = fmaxf(local, amax8(v[c]));
+            if (h_out) *reinterpret_cast<u32x4*>(h_out + row * width + i * 8) = pack8(v[c]);
+        }
+    }
+    const float step = fmaxf(block_max(local, slots), 1e-12f) / 127.0f;
+    if (threadIdx.x == 0) s[row] = step;
+#pragma unroll
+    for (int c = 0; c < kCache; ++c) {
+        const int64_t i = threadIdx.x + (int64_t)c * kThreads;
+        if (i < nvec) *reinterpret_cast<u32x2*>(hq + row * width + i * 8) = quant8_int8(v[c], step);
+    }
+}
+
 // ---- 1x128 activation groups ----------------------------------------------
 // One 16-byte vector per lane; 16 consecutive lanes own one 128-wide group.
 __global__ __launch_bounds__(kThreads) void quantize_fp8_act128_kernel(
@@ -235,6 +354,25 @@ void launch_quantize_int8_rows(const void* x, void* xq, float* s, int64_t rows, 
     if (rows <= 0 || k <= 0) return;
     quantize_int8_rows_kernel<<<dim3((unsigned)rows), dim3(kThreads), 0, stream>>>(
         static_cast<const uint16_t*>(x), static_cast<int8_t*>(xq), s, k);
+}
+
+void launch_add_rmsnorm_quantize_int8_rows(const void* x, const void* res, const void* w, float eps,
+                                           void* sum_out, void* y_out, void* xq, float* s,
+                                           int64_t rows, int64_t k, hipStream_t stream) {
+    if (rows <= 0 || k <= 0) return;
+    add_rmsnorm_quantize_int8_rows_kernel<<<dim3((unsigned)rows), dim3(kThreads), 0, stream>>>(
+        static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(res),
+        static_cast<const uint16_t*>(w), eps, static_cast<uint16_t*>(sum_out),
+        static_cast<uint16_t*>(y_out), static_cast<int8_t*>(xq), s, k);
+}
+
+void launch_silu_mul_quantize_int8_rows(const void* gate, const void* up, int64_t ld, void* h_out,
+                                        void* hq, float* s, int64_t rows, int64_t width,
+                                        hipStream_t stream) {
+    if (rows <= 0 || width <= 0) return;
+    silu_mul_quantize_int8_rows_kernel<<<dim3((unsigned)rows), dim3(kThreads), 0, stream>>>(
+        static_cast<const uint16_t*>(gate), static_cast<const uint16_t*>(up), ld,
+        static_cast<uint16_t*>(h_out), static_cast<int8_t*>(hq), s, width);
 }
 
 void launch_quantize_fp8_block128_act(const void* x, void* x8, float* sa, int64_t m,

@@ -33,6 +33,9 @@ PROTOTYPES = {
     "astrai_w8a8_last_error": ([], ctypes.c_char_p),
     "astrai_w8a8_quantize_bf16_fp8": ([_P, _P, _P, _P, _I64, _INT, _P], _INT),
     "astrai_w8a8_quantize_bf16_int8_rows": ([_P, _P, _P, _I64, _I64, _P], _INT),
+    "astrai_w8a8_add_rmsnorm_quantize_int8_rows": (
+        [_P, _P, _P, ctypes.c_float, _P, _P, _P, _P, _I64, _I64, _P], _INT),
+    "astrai_w8a8_silu_mul_quantize_int8_rows": ([_P, _P, _I64, _P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_quantize_bf16_fp8_block128_act": ([_P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_quantize_bf16_fp8_block128_weight": ([_P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_gemm_fp8_pt": ([_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _INT, _INT, _P], _INT),
@@ -315,6 +318,62 @@ def quantize_int8_rows(x: torch.Tensor):
         elif rows:
             s.fill_(1e-12 / 127.0)
     return xq, s
+
+
+def add_rmsnorm_quantize_int8(x: torch.Tensor, weight: torch.Tensor, eps: float,
+                              res: Optional[torch.Tensor] = None, want_y: bool = False):
+    """``t = x + res`` (bf16, when ``res`` is given), ``y = rms_norm(t) * weight``, per-row
+    int8 of ``y`` in one kernel. Returns ``(xq [R,K], s [R,1], t or None, y or None)``."""
+    lib = _require()
+    _gpu(x, "add_rmsnorm_quantize_int8")
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise RuntimeError("x and weight must be bf16")
+    k = x.size(-1)
+    if weight.numel() != k or weight.device != x.device:
+        raise RuntimeError("weight must be [K] on x's device")
+    x2 = x.reshape(-1, k).contiguous()
+    rows = x2.size(0)
+    r2 = None
+    if res is not None:
+        if res.shape != x.shape or res.dtype != torch.bfloat16 or res.device != x.device:
+            raise RuntimeError("res must match x in shape, dtype and device")
+        r2 = res.reshape(-1, k).contiguous()
+    with torch.cuda.device(x.device):
+        xq = torch.empty((rows, k), device=x.device, dtype=torch.int8)
+        s = torch.empty((rows, 1), device=x.device, dtype=torch.float32)
+        t = torch.empty_like(x2) if r2 is not None else None
+        y = torch.empty_like(x2) if want_y else None
+        _check(lib.astrai_w8a8_add_rmsnorm_quantize_int8_rows(
+            x2.data_ptr(), _ptr(r2), weight.contiguous().data_ptr(), float(eps), _ptr(t), _ptr(y),
+            xq.data_ptr(), s.data_ptr(), rows, k, _stream(x)), lib)
+    return (xq, s, None if t is None else t.reshape(x.shape), None if y is None else y.reshape(x.shape))
+
+
+def silu_mul_quantize_int8(gate: torch.Tensor, up: torch.Tensor, want_h: bool = False):
+    """``h = up * silu(gate)`` (bf16 arithmetic) and per-row int8 of ``h`` in one kernel.
+    ``gate`` / ``up`` are ``[..., W]`` views whose last dimension is contiguous and whose
+    rows are equally spaced (e.g. the two halves of a ``[R, 2W]`` tensor).
+    Returns ``(hq [R,W], s [R,1], h or None)``."""
+    lib = _require()
+    _gpu(gate, "silu_mul_quantize_int8")
+    if gate.dtype != torch.bfloat16 or up.dtype != torch.bfloat16:
+        raise RuntimeError("gate and up must be bf16")
+    if gate.shape != up.shape or gate.device != up.device:
+        raise RuntimeError("gate and up must match in shape and device")
+    w = gate.size(-1)
+    g2, u2 = gate.reshape(-1, w), up.reshape(-1, w)
+    if g2.stride(1) != 1 or u2.stride(1) != 1 or g2.stride(0) != u2.stride(0):
+        g2, u2 = g2.contiguous(), u2.contiguous()
+    rows = g2.size(0)
+    ld = g2.stride(0) if rows > 1 else max(w, g2.stride(0))
+    with torch.cuda.device(gate.device):
+        hq = torch.empty((rows, w), device=gate.device, dtype=torch.int8)
+        s = torch.empty((rows, 1), device=gate.device, dtype=torch.float32)
+        h = torch.empty((rows, w), device=gate.device, dtype=torch.bfloat16) if want_h else None
+        _check(lib.astrai_w8a8_silu_mul_quantize_int8_rows(
+            g2.data_ptr(), u2.data_ptr(), ld, _ptr(h), hq.data_ptr(), s.data_ptr(), rows, w,
+            _stream(gate)), lib)
+    return hq, s, None if h is None else h.reshape(gate.shape)
 
 
 _INT8_ENTRY = {

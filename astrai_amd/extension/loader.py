@@ -36,6 +36,8 @@ def _int8_mm_module() -> SimpleNamespace:
     return SimpleNamespace(
         quantize_int8_rows=_cabi.quantize_int8_rows,
         mm_int8=_cabi.mm_int8,
+        add_rmsnorm_quantize_int8=_cabi.add_rmsnorm_quantize_int8,
+        silu_mul_quantize_int8=_cabi.silu_mul_quantize_int8,
     )
 
 

@@ -7,6 +7,10 @@ scales as quantization steps.
 - ``mm_int8(xq, wq, sx, sw, bias=None) -> bf16 [M,N]``  (``xq @ wq^T * sx[m] * sw[n] + bias``)
 - ``mm_int8_acc(xq, wq) -> int32 [M,N]``  (raw accumulator, the bit-exact parity surface)
 - ``linear_forward_int8(x, wq, sw, bias=None) -> bf16 [..., N]``
+- ``rmsnorm_quantize_int8(x, weight, eps, res=None) -> (xq, sx, x + res | None)``: the
+  residual add, ``F.rms_norm`` and the per-token quantizer in one kernel
+- ``silu_mul_quantize_int8(gate, up) -> (hq, sh)``: ``up * silu(gate)`` and the
+  per-token quantizer in one kernel
 """
 
 from typing import Optional
@@ -114,3 +118,70 @@ def linear_forward_int8(x, wq, sw, bias: Optional[torch.Tensor] = None) -> torch
     xq, sx = int8_quantize_per_token(x)
     out = int8_gemm(xq, wq, sx, sw, bias)
     return out.reshape(*x.shape[:-1], wq.size(0))
+
+
+@custom_op("custom::int8_add_rmsnorm_quantize", mutates_args=())
+def int8_add_rmsnorm_quantize(
+    x: torch.Tensor, weight: torch.Tensor, eps: float, res: Optional[torch.Tensor] = None
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``t = x + res`` (``x`` itself without ``res``), ``y = rms_norm(t) * weight``,
+    per-token int8 of ``y``. Returns ``(xq int8 [R,K], s fp32 [R,1], t)``."""
+    _no_cpu("custom::int8_add_rmsnorm_quantize")
+
+
+@int8_add_rmsnorm_quantize.register_fake
+def _int8_add_rmsnorm_quantize_fake(x, weight, eps, res=None):
+    k = x.shape[-1]
+    rows = x.numel() // k if k else 0
+    return (
+        torch.empty((rows, k), device=x.device, dtype=torch.int8),
+        torch.empty((rows, 1), device=x.device, dtype=torch.float32),
+        torch.empty_like(x),
+    )
+
+
+@int8_add_rmsnorm_quantize.register_kernel("cuda")
+def _int8_add_rmsnorm_quantize_cuda(x, weight, eps, res=None):
+    if x.dtype != torch.bfloat16:
+        raise TypeError(f"int8 rmsnorm-quantize requires bf16 input, got {x.dtype}")
+    xq, s, t, _ = _mod().add_rmsnorm_quantize_int8(x, weight, eps, res, False)
+    # a custom op may not return an input: without a residual the sum is a copy of x
+    return xq, s, (t if t is not None else x.clone())
+
+
+@custom_op("custom::int8_silu_mul_quantize", mutates_args=())
+def int8_silu_mul_quantize(gate: torch.Tensor, up: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """``h = up * silu(gate)`` in bf16 arithmetic, per-token int8 of ``h``:
+    ``(hq int8 [R,W], s fp32 [R,1])``."""
+    _no_cpu("custom::int8_silu_mul_quantize")
+
+
+@int8_silu_mul_quantize.register_fake
+def _int8_silu_mul_quantize_fake(gate, up):
+    w = gate.shape[-1]
+    rows = gate.numel() // w if w else 0
+    return (
+        torch.empty((rows, w), device=gate.device, dtype=torch.int8),
+        torch.empty((rows, 1), device=gate.device, dtype=torch.float32),
+    )
+
+
+@int8_silu_mul_quantize.register_kernel("cuda")
+def _int8_silu_mul_quantize_cuda(gate, up):
+    if gate.dtype != torch.bfloat16 or up.dtype != torch.bfloat16:
+        raise TypeError(f"int8 silu-mul-quantize requires bf16 inputs, got {gate.dtype}/{up.dtype}")
+    hq, s, _ = _mod().silu_mul_quantize_int8(gate, up, False)
+    return hq, s
+
+
+def rmsnorm_quantize_int8(x, weight, eps: float, res: Optional[torch.Tensor] = None):
+    """Fused (residual add +) RMSNorm + per-token int8. Returns ``(xq, sx, t)`` with
+    ``t = x + res`` when ``res`` is given, else ``None`` (no copy is made)."""
+    if x.dtype != torch.bfloat16:
+        raise TypeError(f"int8 rmsnorm-quantize requires bf16 input, got {x.dtype}")
+    xq, s, t, _ = _mod().add_rmsnorm_quantize_int8(x, weight, eps, res, False)
+    return xq, s, t
+
+
+def silu_mul_quantize_int8(gate, up):
+    return int8_silu_mul_quantize(gate, up)

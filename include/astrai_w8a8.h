@@ -77,6 +77,35 @@ int astrai_w8a8_quantize_bf16_int8_rows(const void* x_bf16, void* xq, float* s,
                                         int64_t rows, int64_t k, void* stream);
 
 /*
+ * Producers fused with the per-row int8 quantizer: the activation of every int8
+ * Linear in the decoder comes out of an RMSNorm (after a residual add) or out of
+ * the SwiGLU product, and is read by nothing but the quantizer.
+ *
+ * add_rmsnorm: replaces the residual add of DecoderBlock.forward
+ * (astrai/model/components/decoder_block.py:59-70), RMSNorm.forward = F.rms_norm
+ * (astrai/model/components/norm.py:7-15) and quantize_bf16_int8_rows above.
+ *   t[r,:]  = res ? bf16(x[r,:] + res[r,:]) : x[r,:]          (written to sum_out when res and sum_out are given)
+ *   y[r,k]  = bf16(weight[k] * (t[r,k] * rsqrt(mean_k t[r,k]^2 + eps)))   fp32 arithmetic, one rounding
+ *   s[r], xq[r,:] = the per-row int8 quantizer applied to y[r,:]
+ * res, sum_out, y_out may be NULL (y_out receives y when given). K % 8 == 0, K <= 8192.
+ *
+ * silu_mul: replaces ``up(x) * F.silu(gate(x))`` of MLP.forward
+ * (astrai/model/components/mlp.py:41) and the quantizer in front of ``down``.
+ *   h[r,j]  = bf16(up[r,j] * bf16(gate[r,j] / (1 + exp(-gate[r,j]))))
+ *   s[r], hq[r,:] = the per-row int8 quantizer applied to h[r,:]
+ * gate and up rows are ld elements apart (the two halves of one [rows, 2*width]
+ * gate|up GEMM output, or two separate tensors with ld = width); hq and h_out
+ * (optional) are dense [rows, width]. width % 8 == 0, ld % 8 == 0, width <= 8192.
+ */
+int astrai_w8a8_add_rmsnorm_quantize_int8_rows(const void* x_bf16, const void* res_bf16,
+                                               const void* weight_bf16, float eps,
+                                               void* sum_out_bf16, void* y_out_bf16, void* xq,
+                                               float* s, int64_t rows, int64_t k, void* stream);
+int astrai_w8a8_silu_mul_quantize_int8_rows(const void* gate_bf16, const void* up_bf16, int64_t ld,
+                                            void* h_out_bf16, void* hq, float* s, int64_t rows,
+                                            int64_t width, void* stream);
+
+/*
  * bf16 -> e4m3fn with one scale per 1x128 K-group (activations) or per 128x128
  * block (weights). No counterpart in the reference. K must be a multiple of 128.
  *   act:    sa[m,kb]  = max(max |x[m,128kb..128kb+127]|, 1e-12) / 448,   sa is [M, K/128]

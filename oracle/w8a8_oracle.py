@@ -231,6 +231,26 @@ def fp8_gemm_blockscaled(a8, b8, sa, sb, bias=None):
     return acc.to(torch.bfloat16)
 
 
+def add_rmsnorm_quantize_int8(x, weight, eps, res=None):
+    """Residual add, RMSNorm and per-token int8 as the decoder computes them one
+    after the other: ``t = x + res`` in bf16 (astrai/model/components/
+    decoder_block.py:59-70), ``y = F.rms_norm(t, (K,), weight, eps)``
+    (components/norm.py:7-15), then :func:`int8_quantize_rows`. Returns
+    ``(xq, s, t, y)``."""
+    t = x if res is None else x + res
+    y = torch.nn.functional.rms_norm(t, (t.size(-1),), weight, eps)
+    xq, s = int8_quantize_rows(y.reshape(-1, y.size(-1)))
+    return xq, s, t, y
+
+
+def silu_mul_quantize_int8(gate, up):
+    """``h = up * F.silu(gate)`` in bf16 (astrai/model/components/mlp.py:41), then
+    :func:`int8_quantize_rows`. Returns ``(hq, s, h)``."""
+    h = up * torch.nn.functional.silu(gate)
+    hq, s = int8_quantize_rows(h.reshape(-1, h.size(-1)))
+    return hq, s, h
+
+
 # ---------------------------------------------------------------------------
 # Seeded workload generators shared by tests and bench (activation, weight,
 # bias, outlier mask drawn in that order from one CPU generator)

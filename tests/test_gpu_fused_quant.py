@@ -1,0 +1,80 @@
+"""Producers fused with the per-token int8 quantizer (residual add + RMSNorm,
+SwiGLU product) against the oracle's unfused chain. The float part carries the
+bf16 tolerance; the quantizer part is checked bit-exactly on the kernel's own
+bf16 output."""
+
+import pytest
+import torch
+
+from oracle import w8a8_oracle as O
+from tests.helpers import assert_bf16_close
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module")
+def C():
+    from astrai_amd.extension import _cabi
+    assert _cabi.load() is not None, _cabi.load_error()
+    return _cabi
+
+
+def _codes_close(got, want, s_got, s_want):
+    """codes within one step and >= 98% equal; steps within one bf16 ulp of the row maximum"""
+    d = (got.cpu().int() - want.int()).abs()
+    assert d.max().item() <= 1, d.max().item()
+    assert (d == 0).float().mean().item() >= 0.98
+    torch.testing.assert_close(s_got.cpu().reshape(-1), s_want.reshape(-1), rtol=2.0 ** -7, atol=0)
+
+
+@pytest.mark.parametrize("rows,k,with_res", [(32, 2048, True), (32, 2048, False), (1, 2048, True),
+                                             (5, 8, True), (3, 8192, False), (17, 5632, True)])
+def test_add_rmsnorm_quantize(C, rows, k, with_res):
+    print(f"case rows={rows} k={k} res={with_res}", flush=True)
+    g = torch.Generator().manual_seed(rows * 131 + k)
+    x = torch.randn(rows, k, generator=g).to(torch.bfloat16)
+    res = (torch.randn(rows, k, generator=g) * 0.5).to(torch.bfloat16) if with_res else None
+    w = (1.0 + 0.1 * torch.randn(k, generator=g)).to(torch.bfloat16)
+    eps = 1e-5
+    xq, s, t, y = C.add_rmsnorm_quantize_int8(x.to(DEV), w.to(DEV), eps, res.to(DEV) if with_res else None,
+                                              want_y=True)
+    wq, ws, wt, wy = O.add_rmsnorm_quantize_int8(x, w, eps, res)
+    if with_res:
+        assert torch.equal(t.cpu().view(torch.int16), wt.view(torch.int16))  # one bf16 add: exact
+    else:
+        assert t is None
+    assert_bf16_close(y, wy, what="rmsnorm y")
+    # the quantizer on the kernel's own y: bit-exact
+    oq, os_ = O.int8_quantize_rows(y.cpu())
+    assert torch.equal(xq.cpu(), oq) and torch.equal(s.cpu(), os_)
+    _codes_close(xq, wq, s, ws)
+
+
+@pytest.mark.parametrize("rows,width,fused_buffer", [(32, 5632, True), (32, 5632, False), (1, 5632, True),
+                                                     (7, 8, False), (3, 8192, True)])
+def test_silu_mul_quantize(C, rows, width, fused_buffer):
+    print(f"case rows={rows} width={width} fused={fused_buffer}", flush=True)
+    g = torch.Generator().manual_seed(rows * 17 + width)
+    gu = (torch.randn(rows, 2 * width, generator=g) * 2.0).to(torch.bfloat16)
+    gate, up = gu[:, :width], gu[:, width:]
+    d = gu.to(DEV)
+    if fused_buffer:
+        hq, s, h = C.silu_mul_quantize_int8(d[:, :width], d[:, width:], want_h=True)
+    else:
+        hq, s, h = C.silu_mul_quantize_int8(d[:, :width].contiguous(), d[:, width:].contiguous(), want_h=True)
+    wq, ws, wh = O.silu_mul_quantize_int8(gate, up)
+    assert_bf16_close(h, wh, what="silu*up")
+    oq, os_ = O.int8_quantize_rows(h.cpu())
+    assert torch.equal(hq.cpu(), oq) and torch.equal(s.cpu(), os_)
+    _codes_close(hq, wq, s, ws)
+
+
+def test_fused_entry_points_reject_unsupported(C):
+    x = torch.zeros(2, 12, device=DEV, dtype=torch.bfloat16)   # K % 8 != 0
+    w = torch.ones(12, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        C.add_rmsnorm_quantize_int8(x, w, 1e-5)
+    big = torch.zeros(1, 8200, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="8192"):
+        C.silu_mul_quantize_int8(big, big)
