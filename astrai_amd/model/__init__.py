@@ -6,7 +6,10 @@ from astrai_amd.model.decoder import (
     AutoRegressiveLM,
     AutoRegressiveLMConfig,
     DenseKVCache,
+    fuse_int8_weights,
     greedy_generate,
+    unfuse_int8_weights,
 )
 
-__all__ = ["AutoRegressiveLM", "AutoRegressiveLMConfig", "DenseKVCache", "greedy_generate"]
+__all__ = ["AutoRegressiveLM", "AutoRegressiveLMConfig", "DenseKVCache", "greedy_generate",
+           "fuse_int8_weights", "unfuse_int8_weights"]

@@ -16,9 +16,18 @@ with host reads; here requests form a dense ``[batch, seq]`` block over a dense
 ``[layer, batch, kv_head, position, head_dim]`` cache, which is the same
 arithmetic for equal-length prompts and keeps the decode step free of host
 synchronisation, hence HIP-graph capturable.
+
+``fuse_int8_weights(model)`` adds a second way through the same blocks for int8
+inference: q|k|v and gate|up weights concatenated into one int8 matrix each, the
+residual add + RMSNorm and the SwiGLU product fused with the per-token quantizer,
+so a block issues 4 GEMMs and 4 producer kernels around its attention core
+instead of 7 GEMMs, 7 quantizers, 2 norms, 2 adds and a product. The arithmetic
+per element is that of the modular path (concatenating per-channel quantized rows
+changes no row; the fused producers round where the separate ops round).
 """
 
 from dataclasses import dataclass
+from types import SimpleNamespace
 from typing import Dict, Optional
 
 import torch
@@ -136,10 +145,19 @@ class GQA(nn.Module):
 
     def forward(self, x: Tensor, rotary_emb: Tensor, kv_cache: Optional[DenseKVCache],
                 positions: Optional[Tensor], key_mask: Optional[Tensor]) -> Tensor:
-        b, s, _ = x.shape
-        q = self.q_proj(x).reshape(b, s, self.n_heads, self.head_dim)
-        k = self.k_proj(x).reshape(b, s, self.n_kv_heads, self.head_dim)
-        v = self.v_proj(x).reshape(b, s, self.n_kv_heads, self.head_dim)
+        out = self.core(self.q_proj(x), self.k_proj(x), self.v_proj(x), rotary_emb, kv_cache,
+                        positions, key_mask)
+        return self.o_proj(out)
+
+    def core(self, q: Tensor, k: Tensor, v: Tensor, rotary_emb: Tensor,
+             kv_cache: Optional[DenseKVCache], positions: Optional[Tensor],
+             key_mask: Optional[Tensor]) -> Tensor:
+        """Everything between the q/k/v projections and ``o_proj``: ``[B, S, *]`` in,
+        ``[B, S, dim]`` out."""
+        b, s = q.shape[0], q.shape[1]
+        q = q.reshape(b, s, self.n_heads, self.head_dim)
+        k = k.reshape(b, s, self.n_kv_heads, self.head_dim)
+        v = v.reshape(b, s, self.n_kv_heads, self.head_dim)
         q, k = apply_rotary_emb(q, rotary_emb), apply_rotary_emb(k, rotary_emb)
         q, k, v = q.permute(0, 2, 1, 3), k.permute(0, 2, 1, 3), v.permute(0, 2, 1, 3)
         if kv_cache is None:
@@ -158,8 +176,7 @@ class GQA(nn.Module):
             out = F.scaled_dot_product_attention(qf, kv_cache.k[self.layer_id],
                                                  kv_cache.v[self.layer_id], attn_mask=mask)
             out = out.reshape(b, self.n_heads, s, self.head_dim)
-        out = out.permute(0, 2, 1, 3).reshape(b, s, self.dim)
-        return self.o_proj(out)
+        return out.permute(0, 2, 1, 3).reshape(b, s, self.dim)
 
 
 class MLP(nn.Module):
@@ -184,9 +201,32 @@ class DecoderBlock(nn.Module):
         self.mlp = MLP(config.hidden_size, config.intermediate_size,
                        down_init_std=0.02 / (2 * n) ** 0.5)
 
+        self.fused_int8 = None  # set by fuse_int8_weights
+
     def forward(self, x, rotary_emb, kv_cache, positions, key_mask):
+        if self.fused_int8 is not None and _fused_int8_active(x):
+            return self._forward_fused_int8(x, rotary_emb, kv_cache, positions, key_mask)
         x = self.attention(self.input_norm(x), rotary_emb, kv_cache, positions, key_mask) + x
         return self.mlp(self.post_attention_norm(x)) + x
+
+    def _forward_fused_int8(self, x, rotary_emb, kv_cache, positions, key_mask):
+        from astrai_amd.extension.ops import int8 as I
+        f, att = self.fused_int8, self.attention
+        b, s, d = x.shape
+        xq, sx, _ = I.rmsnorm_quantize_int8(x, self.input_norm.weight, self.input_norm.norm_eps)
+        qkv = I.mm_int8(xq, f.wqkv, sx, f.sqkv).reshape(b, s, -1)
+        nq, nkv = att.n_heads * att.head_dim, att.n_kv_heads * att.head_dim
+        a = att.core(qkv[..., :nq], qkv[..., nq:nq + nkv], qkv[..., nq + nkv:], rotary_emb, kv_cache,
+                     positions, key_mask)
+        aq, sa = I.quantize_int8_per_token(a)
+        o = I.mm_int8(aq, f.wo, sa, f.so).reshape(b, s, d)
+        # h = attention + x, then its norm, quantized: one kernel
+        hq, sh, h = I.rmsnorm_quantize_int8(o, self.post_attention_norm.weight,
+                                            self.post_attention_norm.norm_eps, res=x)
+        gu = I.mm_int8(hq, f.wgu, sh, f.sgu)                 # [B*S, gate | up]
+        w = f.wgu.size(0) // 2
+        mq, sm = I.silu_mul_quantize_int8(gu[:, :w], gu[:, w:])
+        return I.mm_int8(mq, f.wdown, sm, f.sdown).reshape(b, s, d) + h
 
 
 class AutoRegressiveLM(nn.Module):
@@ -205,6 +245,7 @@ class AutoRegressiveLM(nn.Module):
         if config.tie_word_embeddings:
             self.lm_head.weight = self.embed_tokens.weight
         self.apply(lambda m: m.reset_parameters() if hasattr(m, "reset_parameters") else None)
+        self.fused_int8 = None  # set by fuse_int8_weights
 
     def forward(self, input_ids: Tensor, kv_cache: Optional[DenseKVCache] = None,
                 positions: Optional[Tensor] = None) -> Dict[str, Tensor]:
@@ -225,8 +266,54 @@ class AutoRegressiveLM(nn.Module):
             key_mask = (key_pos[None, :] <= positions[:, None])[None, None]  # [1,1,seq,max_len]
         for layer in self.layers:
             x = layer(x, rotary, kv_cache, positions, key_mask)
+        if self.fused_int8 is not None and _fused_int8_active(x):
+            from astrai_amd.extension import _cabi
+            from astrai_amd.extension.ops import int8 as I
+            hq, sh, _, hidden = _cabi.add_rmsnorm_quantize_int8(x, self.norm.weight, self.norm.norm_eps,
+                                                                None, True)
+            logits = I.mm_int8(hq, self.fused_int8.wlm, sh, self.fused_int8.slm).reshape(b, s, -1)
+            return {"logits": logits, "hidden_states": hidden}
         hidden = self.norm(x)
         return {"logits": self.lm_head(hidden), "hidden_states": hidden}
+
+
+def _fused_int8_active(x: Tensor) -> bool:
+    from astrai_amd.extension import w8a8
+    return w8a8.int8_linear_enabled() and x.is_cuda and x.dtype == torch.bfloat16
+
+
+@torch.no_grad()
+def fuse_int8_weights(model: AutoRegressiveLM) -> int:
+    """Quantize every projection per output channel (the per-row quantizer on the
+    weight, as ``w8a8.prepare_int8_weights`` does) and store q|k|v and gate|up as one
+    int8 matrix each on the block. While ``w8a8.int8_autocast`` is on, blocks then take
+    the fused path. Returns the number of int8 matrices held. Call again after
+    changing weights."""
+    from astrai_amd.extension.ops.int8 import quantize_int8_per_channel as qpc
+
+    def cat(*linears):
+        parts = [qpc(l.weight.detach()) for l in linears]
+        return torch.cat([p[0] for p in parts]).contiguous(), torch.cat([p[1] for p in parts]).contiguous()
+
+    n = 0
+    for blk in model.layers:
+        att, mlp = blk.attention, blk.mlp
+        wqkv, sqkv = cat(att.q_proj, att.k_proj, att.v_proj)
+        wo, so = cat(att.o_proj)
+        wgu, sgu = cat(mlp.gate, mlp.up)
+        wdown, sdown = cat(mlp.down)
+        blk.fused_int8 = SimpleNamespace(wqkv=wqkv, sqkv=sqkv, wo=wo, so=so, wgu=wgu, sgu=sgu,
+                                         wdown=wdown, sdown=sdown)
+        n += 4
+    wlm, slm = cat(model.lm_head)
+    model.fused_int8 = SimpleNamespace(wlm=wlm, slm=slm)
+    return n + 1
+
+
+def unfuse_int8_weights(model: AutoRegressiveLM) -> None:
+    for blk in model.layers:
+        blk.fused_int8 = None
+    model.fused_int8 = None
 
 
 @torch.no_grad()

@@ -84,7 +84,8 @@ def _bench_decoder(dev):
     import torch
 
     from astrai_amd.extension import w8a8
-    from astrai_amd.model import AutoRegressiveLM, AutoRegressiveLMConfig, DenseKVCache, greedy_generate
+    from astrai_amd.model import (AutoRegressiveLM, AutoRegressiveLMConfig, DenseKVCache, fuse_int8_weights,
+                                  greedy_generate, unfuse_int8_weights)
 
     cfg = AutoRegressiveLMConfig()
     torch.manual_seed(4)
@@ -110,16 +111,34 @@ def _bench_decoder(dev):
         t_pre = (time.perf_counter() - t0) / 3
         res["prefill_ms"] = round(t_pre * 1e3, 2)
         res["prefill_tokens_per_s"] = round(batch * prompt / t_pre)
-        for name, graph in (("eager", False), ("graph", True)):
-            greedy_generate(model, ids, 8, use_graph=graph)  # warm
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            greedy_generate(model, ids, steps, use_graph=graph)
-            torch.cuda.synchronize()
-            t_all = time.perf_counter() - t0
-            t_dec = max(t_all - t_pre, 1e-9)
-            res[f"decode_{name}_ms_per_step"] = round(t_dec * 1e3 / (steps - 1), 3)
-            res[f"decode_{name}_tokens_per_s"] = round(batch * (steps - 1) / t_dec)
+        def decode_legs(prefix, t_prefill):
+            for name, graph in (("eager", False), ("graph", True)):
+                greedy_generate(model, ids, 8, use_graph=graph)  # warm
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                greedy_generate(model, ids, steps, use_graph=graph)
+                torch.cuda.synchronize()
+                t_all = time.perf_counter() - t0
+                t_dec = max(t_all - t_prefill, 1e-9)
+                res[f"{prefix}decode_{name}_ms_per_step"] = round(t_dec * 1e3 / (steps - 1), 3)
+                res[f"{prefix}decode_{name}_tokens_per_s"] = round(batch * (steps - 1) / t_dec)
+
+        decode_legs("", t_pre)
+        # the same blocks with q|k|v and gate|up concatenated and the norm / SwiGLU
+        # producers fused with the per-token quantizer
+        res["fused_int8_matrices"] = fuse_int8_weights(model)
+        for _ in range(2):
+            prefill()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(3):
+            prefill()
+        torch.cuda.synchronize()
+        t_pre_f = (time.perf_counter() - t0) / 3
+        res["fused_prefill_ms"] = round(t_pre_f * 1e3, 2)
+        res["fused_prefill_tokens_per_s"] = round(batch * prompt / t_pre_f)
+        decode_legs("fused_", t_pre_f)
+        unfuse_int8_weights(model)
         # the same model with the stock bf16 kernels, for scale
     w8a8.int8_state().reset()
     with torch.no_grad():
@@ -142,8 +161,9 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="headline kernel only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-model", action="store_true", help="skip the config-4 decoder leg")
-    ap.add_argument("--decoder-trace", action="store_true",
-                    help="tracing mode: build the config-4 decoder, one prefill + 19 eager decode steps, nothing else")
+    ap.add_argument("--decoder-trace", choices=["modular", "fused"], default=None,
+                    help="tracing mode: build the config-4 decoder (Linear-by-Linear int8 path, or the fused "
+                         "one), one prefill + 19 eager decode steps, nothing else")
     ap.add_argument("--pmc", action="store_true",
                     help="counter-collection mode: a few launches of the headline kernel and of a "
                          "plain 256 MiB device copy (the calibration kernel), nothing else")
@@ -171,18 +191,21 @@ def main():
 
     if args.decoder_trace:
         from astrai_amd.extension import w8a8
-        from astrai_amd.model import AutoRegressiveLM, AutoRegressiveLMConfig, greedy_generate
+        from astrai_amd.model import AutoRegressiveLM, AutoRegressiveLMConfig, fuse_int8_weights, greedy_generate
 
         cfg = AutoRegressiveLMConfig()
         torch.manual_seed(4)
         with torch.device(dev):
             model = AutoRegressiveLM(cfg).to(torch.bfloat16).eval()
         ids = torch.randint(0, cfg.vocab_size, (32, 512), generator=torch.Generator().manual_seed(4)).to(dev)
-        w8a8.prepare_int8_weights(model)
+        if args.decoder_trace == "fused":
+            fuse_int8_weights(model)
+        else:
+            w8a8.prepare_int8_weights(model)
         with torch.no_grad(), w8a8.int8_autocast(True):
             greedy_generate(model, ids, 20, use_graph=False)
         torch.cuda.synchronize()
-        print(json.dumps({"decoder_trace": True, "prefill_tokens": 32 * 512, "decode_steps": 19}))
+        print(json.dumps({"decoder_trace": args.decoder_trace, "prefill_tokens": 32 * 512, "decode_steps": 19}))
         return
 
     # ---------------- headline: config 1, fp8 per-tensor 4096^3 ----------------
@@ -269,7 +292,7 @@ def main():
                                                        swi.data_ptr(), None, out.data_ptr(),
                                                        M, N, K, 0, stream))
 
-        ms = _event_time_ms(step_i8, 100, 10)
+        ms = _event_time_ms(step_i8, 500, 300)
         tops = flop / (ms * 1e-3) / 1e12
         extra["int8_gemm_4096"] = {"us": round(ms * 1e3, 2), "TOP/s": round(tops, 1),
                                    "frac_mfma_peak": round(tops / PEAK_INT8_TOPS, 4)}
@@ -282,7 +305,7 @@ def main():
                                               sb_d.data_ptr(), None, bias.data_ptr(), out.data_ptr(),
                                               M, N, K, 0, 0, stream))
 
-        ms = _event_time_ms(step_bias, 100, 10)
+        ms = _event_time_ms(step_bias, 500, 300)
         extra["fp8_gemm_4096_bias"] = {"us": round(ms * 1e3, 2),
                                        "TFLOP/s": round(flop / (ms * 1e-3) / 1e12, 1)}
         del ai, bi
@@ -300,7 +323,7 @@ def main():
                                                     sb3.data_ptr(), None, out3.data_ptr(),
                                                     M3, N3, K3, stream))
 
-        ms = _event_time_ms(step_blk, 50, 5)
+        ms = _event_time_ms(step_blk, 300, 150)
         f3 = 2.0 * M3 * N3 * K3
         extra["fp8_block128_8192x2048x7168"] = {
             "us": round(ms * 1e3, 2), "TFLOP/s": round(f3 / (ms * 1e-3) / 1e12, 1),

@@ -62,3 +62,43 @@ def test_prefill_then_decode_equals_full_forward_and_graph_replay_equals_eager()
     w8a8.int8_state().reset()
     assert torch.equal(eager, graph)
     assert eager.shape == (4, 10)
+
+
+def test_fused_int8_path_matches_modular_path_and_oracle():
+    """q|k|v and gate|up concatenated, norms / SwiGLU fused with the quantizer: same
+    logits as the Linear-by-Linear int8 path up to the bf16 rounding of the norm
+    (both paths round once; the device library's rms_norm and the fused kernel may
+    differ in the last bit), same greedy tokens, graph replay equals eager."""
+    from astrai_amd.extension import w8a8
+    from astrai_amd.model import DenseKVCache, fuse_int8_weights, greedy_generate, unfuse_int8_weights
+    cfg, model = _model(6, vocab_size=512, hidden_size=256, num_hidden_layers=3, num_attention_heads=4,
+                        num_key_value_heads=2, intermediate_size=512, max_position_embeddings=64)
+    sd = {k: v.detach().clone() for k, v in model.state_dict().items()}
+    ids = torch.randint(0, cfg.vocab_size, (3, 16), generator=torch.Generator().manual_seed(6))
+    want = D.forward(sd, cfg, ids, D.int8_linear_fn(sd)).float()
+    gm = model.to(DEV)
+    w8a8.int8_state().reset()
+    w8a8.prepare_int8_weights(gm)
+    with torch.no_grad(), w8a8.int8_autocast(True):
+        modular = gm(ids.to(DEV))
+        assert fuse_int8_weights(gm) == 3 * 4 + 1
+        fused = gm(ids.to(DEV))
+        cache = DenseKVCache(cfg, 3, 16, DEV, torch.bfloat16)
+        pre = gm(ids[:, :10].to(DEV), cache, torch.arange(10, device=DEV))["logits"]
+        dec = [gm(ids[:, t:t + 1].to(DEV), cache, torch.tensor([t], device=DEV))["logits"] for t in range(10, 16)]
+        eager = greedy_generate(gm, ids[:, :8].to(DEV), 8, use_graph=False)
+        graph = greedy_generate(gm, ids[:, :8].to(DEV), 8, use_graph=True)
+        unfuse_int8_weights(gm)
+        eager_modular = greedy_generate(gm, ids[:, :8].to(DEV), 8, use_graph=False)
+    w8a8.int8_state().reset()
+    lf, lm = fused["logits"].float().cpu(), modular["logits"].float().cpu()
+    scale = lm.abs().max().item()
+    assert (lf - lm).abs().max().item() <= 0.03 * scale
+    assert torch.nn.functional.cosine_similarity(lf.flatten(), lm.flatten(), dim=0).item() > 0.9995
+    assert torch.nn.functional.cosine_similarity(lf.flatten(), want.flatten(), dim=0).item() > 0.999
+    hf, hm = fused["hidden_states"].float().cpu(), modular["hidden_states"].float().cpu()
+    assert (hf - hm).abs().max().item() <= 0.03 * hm.abs().max().item()
+    inc = torch.cat([pre] + dec, 1).float().cpu()
+    assert (inc - lf).abs().max().item() <= 0.03 * scale
+    assert torch.equal(eager, graph)
+    assert (eager == eager_modular).float().mean().item() >= 0.9
