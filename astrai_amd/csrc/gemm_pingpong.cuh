@@ -462,8 +462,10 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
             const u32x4 v = *reinterpret_cast<const u32x4*>(mine + ml * Cfg::EPI_ROW_BYTES + cc * 16);
             const int m = m0 + wave_m * 128 + ml;
             const int n = nw + cc * 8;
+            // non-temporal: the output streams to memory during the epilogue instead of
+            // sitting dirty in L2 until the end-of-kernel write-back
             if (m < g.m && n < g.n)
-                *reinterpret_cast<u32x4*>(out + (size_t)m * g.n + n) = v;
+                __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(out + (size_t)m * g.n + n));
         }
     } else {
 #pragma unroll

@@ -345,8 +345,11 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
                 const int ml = i * 8 + rr;
                 const u32x4 v = *reinterpret_cast<const u32x4*>(mine + ml * Cfg::EPI_ROW_BYTES + cc * 16);
                 // the row step goes into the checked (vector) offset: the scalar
-                // offset of a buffer instruction takes no part in the bounds check
-                __builtin_amdgcn_raw_buffer_store_b128(v, rout, lane_off + (uint32_t)(i * 8) * row_bytes, 0, 0);
+                // offset of a buffer instruction takes no part in the bounds check.
+                // Non-temporal (aux bit 1): the 2·M·N output bytes stream to memory
+                // while the epilogue still computes instead of sitting dirty in L2
+                // until the end-of-kernel write-back (measured -1.5 us at 4096^3).
+                __builtin_amdgcn_raw_buffer_store_b128(v, rout, lane_off + (uint32_t)(i * 8) * row_bytes, 0, 2);
             }
         }
     }
