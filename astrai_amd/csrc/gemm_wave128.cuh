@@ -50,10 +50,10 @@ struct Wave128Cfg {
     static constexpr int OPERAND_BYTES = 256 * BK;       // one operand's slab: 32 KiB
     static constexpr int X_STAGES = 3, W_STAGES = 2;
     static constexpr int W_BASE = X_STAGES * OPERAND_BYTES;  // weights after activations
-    static constexpr int EPI_ROW_BYTES = 144;            // 64 bf16 + 16 bytes of padding
-    static constexpr int EPI_WAVE_BYTES = 128 * EPI_ROW_BYTES;
+    static constexpr int EPI_ROW_BYTES = 272;            // 128 bf16 + 16 bytes of padding
+    static constexpr int EPI_PASS_BYTES = 32 * EPI_ROW_BYTES;  // one 32-row pass of a wave
     static constexpr int LDS_BYTES = (X_STAGES + W_STAGES) * OPERAND_BYTES;  // all 160 KiB
-    static_assert(4 * EPI_WAVE_BYTES <= LDS_BYTES, "epilogue staging must fit");
+    static_assert(4 * 2 * EPI_PASS_BYTES <= LDS_BYTES, "epilogue staging must fit");
 };
 
 // order in which a half slab's sixteen 16-byte operand pieces are read from LDS:
@@ -267,89 +267,80 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
 
     // ---------------- epilogue ----------------
     // bf16 only, N % 8 == 0 (the launcher sends everything else to the ping-pong
-    // kernel). Through LDS, 64 columns at a time: the wave lays 128(m) x 64(n)
-    // values down row-major (144-byte rows) in its private region and streams
-    // them out as full 128-byte lines, 16 bytes a lane. LDS operations of one
-    // wave complete in order, so the second pass may overwrite the first.
-    // Every per-column / per-row operand of a pass is requested before the first
-    // one is used, so the pass pays one memory latency, not one per use.
+    // kernel). Through LDS: the wave lays 32(m) x 128(n) values down row-major
+    // (272-byte rows) in a private staging buffer and streams them out as full
+    // 128-byte lines, 16 bytes a lane; four such passes over two buffers in turn, so
+    // the first stores leave after a quarter of the conversions. Per-column operands
+    // are all requested before the first one is used: one memory latency, not one
+    // per use. Output rows go through a buffer descriptor: rows past M and (by the
+    // offset chosen below) columns past N are dropped by the bounds check -- no
+    // predicates, no 64-bit address arithmetic per store; the row step goes into the
+    // checked (vector) offset because the scalar offset of a buffer instruction
+    // takes no part in the check. The stores are non-temporal (aux bit 1): the
+    // 2 M N output bytes stream to memory while the epilogue still computes instead
+    // of sitting dirty in L2 until the end-of-kernel write-back (-1.5 us at 4096^3).
     {
-        uint8_t* const mine = lds + wave * Cfg::EPI_WAVE_BYTES;
+        constexpr int ROWB = Cfg::EPI_ROW_BYTES, PASS_BYTES = Cfg::EPI_PASS_BYTES;
+        uint8_t* const mine = lds + wave * (2 * PASS_BYTES);
         const uint16_t* bias = static_cast<const uint16_t*>(g.bias);
-        const int rr = lane >> 3, cc = lane & 7;
-        // output rows of this tile through a buffer descriptor: rows past M and
-        // (by the offset chosen below) columns past N are dropped by the bounds
-        // check, no predicates, no 64-bit address arithmetic per store
         const int rows_here = min(Cfg::BM, g.m - m0);
         const uint32_t row_bytes = (uint32_t)g.n * 2u;
         const __amdgpu_buffer_rsrc_t rout =
             make_rsrc(static_cast<uint16_t*>(g.out) + (size_t)m0 * g.n, (uint32_t)rows_here * row_bytes);
-
+        const int nwv = n0 + wave_n * 128;
+        f32x4 sw4[NI][4];
+        u32x2 braw[NI][4];
 #pragma unroll
-        for (int p = 0; p < NI / 2; ++p) {
-            const int nw = n0 + wave_n * 128 + p * 64;
-            f32x4 sw4[2][4];
-            u32x2 braw[2][4];
+        for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
-            for (int nj = 0; nj < 2; ++nj)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int n = nw + nj * 32 + q * 8 + lgrp * 4;  // first of this lane's four n
-                    sw4[nj][q] = f32x4{1.0f, 1.0f, 1.0f, 1.0f};
-                    braw[nj][q] = u32x2{0u, 0u};
-                    if (n < g.n) {  // N % 8 == 0: the four are in range together
-                        if constexpr (ScaleKind == SCALE_ROWCOL)
-                            sw4[nj][q] = *reinterpret_cast<const f32x4*>(g.sb + n);
-                        if (bias) braw[nj][q] = *reinterpret_cast<const u32x2*>(bias + n);
-                    }
-                }
-#pragma unroll
-            for (int nj = 0; nj < 2; ++nj) {
-                const int ni = 2 * p + nj;
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int nl = nj * 32 + q * 8 + lgrp * 4;
-                    const u32x2 raw = braw[nj][q];
-                    const f32x4 b4 = {__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u),
-                                      __uint_as_float(raw.y << 16), __uint_as_float(raw.y & 0xffff0000u)};
-#pragma unroll
-                    for (int mi = 0; mi < MI; ++mi) {
-                        const int ml = mi * 32 + lrow;
-                        float v[4];
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            const float f = (float)acc[ni][mi][4 * q + j];
-                            if constexpr (ScaleKind == SCALE_TENSOR) {
-                                v[j] = f * s_tensor + b4[j];
-                            } else {
-                                // int8: product and bias add rounded separately, the
-                                // epilogue is elementwise fp32 on the exact integer
-#pragma clang fp contract(off)
-                                const float scaled = f * sx[mi] * sw4[nj][q][j];
-                                v[j] = scaled + b4[j];
-                            }
-                        }
-                        u32x2 pk;
-                        pk.x = pack_bf16x2(v[0], v[1]);
-                        pk.y = pack_bf16x2(v[2], v[3]);
-                        *reinterpret_cast<u32x2*>(mine + ml * Cfg::EPI_ROW_BYTES + nl * 2) = pk;
-                    }
+            for (int q = 0; q < 4; ++q) {
+                const int n = nwv + ni * 32 + q * 8 + lgrp * 4;
+                sw4[ni][q] = f32x4{1.0f, 1.0f, 1.0f, 1.0f};
+                braw[ni][q] = u32x2{0u, 0u};
+                if (n < g.n) {
+                    if constexpr (ScaleKind == SCALE_ROWCOL)
+                        sw4[ni][q] = *reinterpret_cast<const f32x4*>(g.sb + n);
+                    if (bias) braw[ni][q] = *reinterpret_cast<const u32x2*>(bias + n);
                 }
             }
-            const int n = nw + cc * 8;
-            const uint32_t lane_off = (n < g.n)
-                ? (uint32_t)(wave_m * 128 + rr) * row_bytes + (uint32_t)n * 2u
-                : kOutOfRange;
+        const int r4 = lane >> 4, c16 = lane & 15;
+        const int nst = nwv + c16 * 8;
+        const uint32_t lane_off = (nst < g.n)
+            ? (uint32_t)(wave_m * 128 + r4) * row_bytes + (uint32_t)nst * 2u
+            : kOutOfRange;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int ml = i * 8 + rr;
-                const u32x4 v = *reinterpret_cast<const u32x4*>(mine + ml * Cfg::EPI_ROW_BYTES + cc * 16);
-                // the row step goes into the checked (vector) offset: the scalar
-                // offset of a buffer instruction takes no part in the bounds check.
-                // Non-temporal (aux bit 1): the 2·M·N output bytes stream to memory
-                // while the epilogue still computes instead of sitting dirty in L2
-                // until the end-of-kernel write-back (measured -1.5 us at 4096^3).
-                __builtin_amdgcn_raw_buffer_store_b128(v, rout, lane_off + (uint32_t)(i * 8) * row_bytes, 0, 2);
+        for (int mi = 0; mi < MI; ++mi) {
+            uint8_t* const buf = mine + (mi & 1) * PASS_BYTES;
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int nl = ni * 32 + q * 8 + lgrp * 4;
+                    const u32x2 raw = braw[ni][q];
+                    const f32x4 b4 = {__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u),
+                                      __uint_as_float(raw.y << 16), __uint_as_float(raw.y & 0xffff0000u)};
+                    float v[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float f = (float)acc[ni][mi][4 * q + j];
+                        if constexpr (ScaleKind == SCALE_TENSOR) {
+                            v[j] = f * s_tensor + b4[j];
+                        } else {
+#pragma clang fp contract(off)
+                            const float scaled = f * sx[mi] * sw4[ni][q][j];
+                            v[j] = scaled + b4[j];
+                        }
+                    }
+                    u32x2 pk;
+                    pk.x = pack_bf16x2(v[0], v[1]);
+                    pk.y = pack_bf16x2(v[2], v[3]);
+                    *reinterpret_cast<u32x2*>(buf + lrow * ROWB + nl * 2) = pk;
+                }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const u32x4 v = *reinterpret_cast<const u32x4*>(buf + (i * 4 + r4) * ROWB + c16 * 16);
+                __builtin_amdgcn_raw_buffer_store_b128(
+                    v, rout, lane_off + (uint32_t)(mi * 32 + i * 4) * row_bytes, 0, 2);
             }
         }
     }
