@@ -27,7 +27,7 @@ PEAK_INT8_TOPS = 5000.0    # MI355X dense int8 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM-side bytes per launch of the headline kernel from two counter passes
 # (reads 101.0 MB + writes 33.6 MB); algorithmic bytes are 67.1 MB
-HEADLINE_TRAFFIC_MB = 135.5
+HEADLINE_TRAFFIC_MB = 134.5
 
 
 def _event_time_ms(fn, iters, warmup):
@@ -233,10 +233,26 @@ def main():
             step()
         for _ in range(3):
             dst.copy_(src)
+        # decode GEMV (config 2 shape) over four distinct weight buffers, after the
+        # 512 MiB of copy traffic above has pushed everything else out of the caches
+        gn, gk = 11008, 4096
+        ring = [torch.randint(-127, 128, (gn, gk), dtype=torch.int8, device=dev) for _ in range(4)]
+        gsw = torch.rand(gn, device=dev) + 0.5
+        dst.copy_(src)
+        for gm in (1, 16):
+            gx = torch.randint(-127, 128, (gm, gk), dtype=torch.int8, device=dev)
+            gsx = torch.rand(gm, device=dev) + 0.5
+            gy = torch.empty(gm, gn, device=dev, dtype=torch.bfloat16)
+            for w in ring:
+                check(lib.astrai_w8a8_gemv_int8_ptpc(gx.data_ptr(), w.data_ptr(), gsx.data_ptr(), gsw.data_ptr(),
+                                                     None, gy.data_ptr(), gm, gn, gk, 0, stream))
         torch.cuda.synchronize()
-        print(json.dumps({"pmc_mode": True, "gemm_launches": 5, "copy_launches": 3,
+        print(json.dumps({"pmc_mode": True, "gemm_launches": 5, "copy_launches": 4,
                           "copy_bytes_each_way": 256 << 20,
-                          "gemm_algorithmic_bytes": 2 * M * K + 2 * M * N}))
+                          "gemm_algorithmic_bytes": 2 * M * K + 2 * M * N,
+                          "gemv_launches": "4 at M=1 (dot kernel), then 4 at M=16 (LDS kernel), 11008x4096",
+                          "gemv_algorithmic_bytes": {"M1": gn * gk + gk + 2 * gn + 4 * gn + 4,
+                                                     "M16": gn * gk + 16 * gk + 32 * gn + 4 * gn + 64}}))
         return
 
     for _ in range(args.warmup):
