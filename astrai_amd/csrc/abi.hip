@@ -217,7 +217,7 @@ int astrai_w8a8_gemm_int8_ptpc(const void* a, const void* b, const float* sa, co
     if (m == 0 || n == 0) return ASTRAI_W8A8_OK;
     auto s = static_cast<hipStream_t>(stream);
     const w8a8::GemmArgs g = pack(a, b, sa, sb, nullptr, bias, out, m, n, k, out_dtype);
-    if (m <= 64 && w8a8::launch_gemv_int8(g, s)) return check_launch("gemv_int8_ptpc");
+    if (m <= 128 && w8a8::launch_gemv_int8(g, s)) return check_launch("gemv_int8_ptpc");
     if (!w8a8::launch_gemm_int8_tiled(g, s))
         w8a8::launch_gemm_generic(g, 0, w8a8::SCALE_ROWCOL, s);
     return check_launch("gemm_int8_ptpc");
@@ -227,9 +227,9 @@ int astrai_w8a8_gemv_int8_ptpc(const void* a, const void* b, const float* sa, co
                                const void* bias, void* out, int64_t m, int64_t n, int64_t k,
                                int out_dtype, void* stream) {
     if (int rc = int8_common("gemv_int8_ptpc", a, b, sa, sb, out, m, n, k, out_dtype)) return rc;
-    if (m > 64 || k % 256 || k == 0)
+    if (m > 128 || k % 256 || k == 0)
         return fail(ASTRAI_W8A8_UNSUPPORTED,
-                    "gemv_int8_ptpc: needs M <= 64 and K a positive multiple of 256 (got m=%lld k=%lld)",
+                    "gemv_int8_ptpc: needs M <= 128 and K a positive multiple of 256 (got m=%lld k=%lld)",
                     (long long)m, (long long)k);
     if (m == 0 || n == 0) return ASTRAI_W8A8_OK;
     const w8a8::GemmArgs g = pack(a, b, sa, sb, nullptr, bias, out, m, n, k, out_dtype);

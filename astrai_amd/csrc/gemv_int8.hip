@@ -1,4 +1,4 @@
-// Skinny int8 W8A8 kernels for decode shapes (M <= 64): bandwidth-bound, the
+// Skinny int8 W8A8 kernels for decode shapes (M <= 128): bandwidth-bound, the
 // weight matrix is streamed from HBM exactly once and the MFMA pipe is almost
 // idle -- speed is set by bytes in flight and by how whole the memory requests
 // are. The int32 partials of the waves that split K are summed through LDS
@@ -8,82 +8,17 @@
 //  * M = 1: gemv_int8_dot_kernel, one wave per four weight rows, whole 1 KiB row
 //    pieces straight into registers and v_dot4 on the vector ALU -- no LDS, no
 //    barrier, every wave of the launch resident and loading at once.
-//  * 1 < M <= 32: gemv_int8_lds_kernel streams the weights through LDS with 1 KiB
-//    contiguous row pieces per instruction (see the comment on the kernel).
-//  * 32 < M <= 64: gemv_int8_kernel loads MFMA-shaped operands straight into
-//    registers (64 contiguous bytes of 16 rows per instruction).
+//  * 2 <= M <= 16: gemv_int8_lds_kernel, 16 rows per workgroup, weights through
+//    LDS in 1 KiB row pieces, every load of the workgroup issued at once.
+//  * 17 <= M <= 128: skinny_int8_kernel, up to 48 rows per workgroup so that the
+//    activation block is pulled from L2 by as few workgroups as possible.
+// Measured at N=11008, K=4096 (weights from HBM): M=1 10.4 us, M=2..16 11.0-13.4,
+// M=32 16.6, M=64 21.2 (the tiled GEMM kernel needs 29 us for any M <= 128).
 #include "gemm_tile.cuh"
 
 namespace w8a8 {
 
 namespace {
-
-template <int RG, int MB, int NW>
-__global__ __launch_bounds__(NW * 64) void gemv_int8_kernel(GemmArgs g) {
-    __shared__ i32x4 red[NW][RG * MB][64];
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int lrow = lane & 15, lgrp = lane >> 4;
-    const int K = g.k;
-    const int nchunks = K >> 8;
-    const int n0 = blockIdx.x * (RG * 16);
-
-    const __amdgpu_buffer_rsrc_t rw = make_rsrc(g.b, (uint32_t)g.n * (uint32_t)K);
-    const __amdgpu_buffer_rsrc_t rx = make_rsrc(g.a, (uint32_t)g.m * (uint32_t)K);
-
-    // Lane (row r, K-group q) takes bytes [64j + 16q, +16) of each 256-byte chunk
-    // for j = 0..3: one instruction touches 64 contiguous bytes of each of its 16
-    // rows, two instructions a whole 128-byte line. Rows past N / M read as zero
-    // (their offset is past the buffer's num_records).
-    uint32_t w_off[RG], x_off[MB];
-#pragma unroll
-    for (int r = 0; r < RG; ++r)
-        w_off[r] = (uint32_t)(n0 + r * 16 + lrow) * (uint32_t)K + lgrp * 16;
-#pragma unroll
-    for (int b = 0; b < MB; ++b) x_off[b] = (uint32_t)(b * 16 + lrow) * (uint32_t)K + lgrp * 16;
-
-    i32x4 acc[RG][MB];
-#pragma unroll
-    for (int r = 0; r < RG; ++r)
-#pragma unroll
-        for (int b = 0; b < MB; ++b) acc[r][b] = i32x4{0, 0, 0, 0};
-
-    for (int c = wave; c < nchunks; c += NW) {
-        const uint32_t k0 = (uint32_t)c << 8;
-        u32x4 wf[RG][4], xf[MB][4];
-#pragma unroll
-        for (int r = 0; r < RG; ++r)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) wf[r][j] = buf_load16(rw, w_off[r] + j * 64, k0);
-#pragma unroll
-        for (int b = 0; b < MB; ++b)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) xf[b][j] = buf_load16(rx, x_off[b] + j * 64, k0);
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int r = 0; r < RG; ++r)
-#pragma unroll
-                for (int b = 0; b < MB; ++b)
-                    acc[r][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
-                        (i32x4)wf[r][j], (i32x4)xf[b][j], acc[r][b], 0, 0, 0);
-    }
-
-#pragma unroll
-    for (int r = 0; r < RG; ++r)
-#pragma unroll
-        for (int b = 0; b < MB; ++b) red[wave][r * MB + b][lane] = acc[r][b];
-    __syncthreads();
-
-    const EpilogueScalars es = load_epilogue_scalars<SCALE_ROWCOL>(g);
-    for (int t = wave; t < RG * MB; t += NW) {
-        i32x4 sum = red[0][t][lane];
-#pragma unroll
-        for (int w = 1; w < NW; ++w) sum += red[w][t][lane];
-        const int r = t / MB, b = t % MB;
-        store_subtile<OpI8, SCALE_ROWCOL>(g, es, sum, b * 16 + lrow, n0 + r * 16 + lgrp * 4);
-    }
-}
 
 // Single-token kernel (M = 1). A workgroup is one wave and owns R = 4 weight
 // rows; lane l holds bytes [16 l, 16 l + 16) of every 1 KiB K-step of its rows and
@@ -285,43 +220,202 @@ void launch_dot(const GemmArgs& g, hipStream_t stream) {
     gemv_int8_dot_kernel<<<dim3((unsigned)blocks), dim3(64), 0, stream>>>(g);
 }
 
+// Skinny kernel for 2 <= M <= 128 (batched decode). The weight matrix is streamed
+// once; what limits such shapes besides HBM is how often the activation block
+// X[M,K] is pulled from L2 again: every workgroup needs all of it. So a
+// workgroup takes as many weight rows as still leaves ~200 workgroups (RG groups
+// of 16 rows, RG = 1..3) and keeps all M tokens of its rows.
+//   * Four waves split K in 512-byte steps (wave w takes steps w, w+4, ...): a
+//     2048-wide K already keeps all four busy.
+//   * Weights go straight to LDS, one instruction per 2 rows x 512 bytes (whole
+//     lines, in order). Rows are 512 bytes apart; the lane that lands at 16-byte
+//     position p of row r fetches logical chunk p ^ (r & 15), which makes the
+//     16-rows-per-instruction operand reads conflict-free without padding.
+//   * Activations come from L2 in MFMA layout, at most four token groups (64
+//     tokens, 128 registers) at a time; with more tokens the weight operands are
+//     cut out of LDS again for the next four groups.
+//   * int32 partials of the four waves are summed through LDS (exact), then the
+//     dequant epilogue.
+template <int RG, int MB, int NW>
+__global__ __launch_bounds__(NW * 64) void skinny_int8_kernel(GemmArgs g) {
+    constexpr int R = RG * 16;
+    constexpr int XB = MB < 4 ? MB : 4;
+    constexpr int PASSES = (MB + XB - 1) / XB;
+    constexpr int WAVE_BYTES = R * 512;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lrow = lane & 15, lgrp = lane >> 4;
+    const int K = g.k;
+    const int nsteps = (K + 511) >> 9;
+    const int n0 = blockIdx.x * R;
+
+    const __amdgpu_buffer_rsrc_t rw = make_rsrc(g.b, (uint32_t)g.n * (uint32_t)K);
+    const __amdgpu_buffer_rsrc_t rx = make_rsrc(g.a, (uint32_t)g.m * (uint32_t)K);
+
+    i32x4 acc[RG][MB];
+#pragma unroll
+    for (int r = 0; r < RG; ++r)
+#pragma unroll
+        for (int b = 0; b < MB; ++b) acc[r][b] = i32x4{0, 0, 0, 0};
+
+    uint8_t* const mine = smem + wave * WAVE_BYTES;
+    // load plan: instruction i covers rows 2i, 2i+1; lane -> row 2i + (lane>>5),
+    // position lane&31, logical chunk (lane&31) ^ ((2i + (lane>>5)) & 15)
+    const int r2 = lane >> 5;
+    const uint32_t w_row_off = (uint32_t)(n0 + r2) * (uint32_t)K;  // rows past N: past num_records, zeros
+    const int cx = (lane & 31) ^ r2;
+    // operand plan: lane (lrow, lgrp) of row group rg reads chunk 4j+lgrp of row 16rg+lrow
+    const uint32_t x_row_off = (uint32_t)lrow * (uint32_t)K + lgrp * 16;
+
+    for (int s = wave; s < nsteps; s += NW) {
+        const uint32_t k0 = (uint32_t)s << 9;
+#pragma unroll
+        for (int i = 0; i < R / 2; ++i) {
+            const int chunk = cx ^ ((2 * i) & 15);
+            const bool in = (int)(k0 + chunk * 16) < K;
+            const uint32_t off = w_row_off + (uint32_t)(2 * i) * (uint32_t)K + (uint32_t)chunk * 16;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                rw, (__attribute__((address_space(3))) void*)(mine + i * 1024), 16,
+                in ? off : kOutOfRange, k0, 0, 0);
+        }
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p) {
+            u32x4 xf[XB][8];
+#pragma unroll
+            for (int b = 0; b < XB; ++b) {
+                // tokens past M start past num_records: zeros
+                const uint32_t xo = x_row_off + (uint32_t)((p * XB + b) * 16) * (uint32_t)K;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const bool in = (int)(k0 + j * 64 + lgrp * 16) < K;
+                    xf[b][j] = (p * XB + b < MB) ? buf_load16(rx, in ? xo + j * 64 : kOutOfRange, k0)
+                                                 : u32x4{0, 0, 0, 0};
+                }
+            }
+            __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): own rows in LDS, activations in registers
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+#pragma unroll
+                for (int r = 0; r < RG; ++r) {
+                    const u32x4 wf = *reinterpret_cast<const u32x4*>(
+                        mine + (r * 16 + lrow) * 512 + (((4 * j + lgrp) ^ lrow) << 4));
+#pragma unroll
+                    for (int b = 0; b < XB; ++b)
+                        if (p * XB + b < MB)
+                            acc[r][p * XB + b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
+                                (i32x4)wf, (i32x4)xf[b][j], acc[r][p * XB + b], 0, 0, 0);
+                }
+        }
+        __builtin_amdgcn_sched_barrier(0);  // the next step's loads overwrite what was just read
+    }
+
+    // sum the four waves' partials through LDS (the staging space is free now)
+    __syncthreads();
+    i32x4* const red = reinterpret_cast<i32x4*>(smem);  // [NW][RG * MB][64]
+#pragma unroll
+    for (int r = 0; r < RG; ++r)
+#pragma unroll
+        for (int b = 0; b < MB; ++b) red[(wave * RG * MB + r * MB + b) * 64 + lane] = acc[r][b];
+    __syncthreads();
+    const uint16_t* bias = static_cast<const uint16_t*>(g.bias);
+    for (int t = wave; t < RG * MB; t += NW) {
+        i32x4 sum = red[t * 64 + lane];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) sum += red[(w * RG * MB + t) * 64 + lane];
+        const int r = t / MB, b = t % MB;
+        const int m = b * 16 + lrow;
+        const int en = n0 + r * 16 + lgrp * 4;
+        if (m >= g.m || en >= g.n) continue;
+        const size_t o = (size_t)m * g.n + en;
+        if (g.out_kind == OUT_ACC) {
+            int* out = static_cast<int*>(g.out);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (en + j < g.n) out[o + j] = sum[j];
+            continue;
+        }
+        const float sx = g.sa[m];
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            // product and bias add rounded separately (no fused multiply-add): the
+            // int8 epilogue is specified as elementwise fp32 on the exact integer
+#pragma clang fp contract(off)
+            const float sw = (en + j < g.n) ? g.sb[en + j] : 0.0f;
+            float f = (float)sum[j] * sx * sw;
+            if (bias && en + j < g.n) f = f + bf16_to_f32(bias[en + j]);
+            v[j] = f;
+        }
+        uint16_t* out = static_cast<uint16_t*>(g.out);
+        if ((g.n & 3) == 0) {
+            u32x2 pk;
+            pk.x = pack_bf16x2(v[0], v[1]);
+            pk.y = pack_bf16x2(v[2], v[3]);
+            *reinterpret_cast<u32x2*>(out + o) = pk;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (en + j < g.n) out[o + j] = f32_to_bf16(v[j]);
+        }
+    }
+}
+
+template <int RG, int MB>
+void launch_skinny(const GemmArgs& g, hipStream_t stream) {
+    constexpr int NW = 4;
+    constexpr int lds_bytes = NW * RG * 16 * 512;
+    static_assert(MB <= 8, "the reduction re-uses the staging space: NW * RG * MB KiB must fit");
+    auto kern = skinny_int8_kernel<RG, MB, NW>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        attr_set = true;
+    }
+    const int blocks = (g.n + RG * 16 - 1) / (RG * 16);
+    kern<<<dim3((unsigned)blocks), dim3(NW * 64), lds_bytes, stream>>>(g);
+}
+
+template <int RG>
+void launch_skinny_mb(const GemmArgs& g, hipStream_t stream) {
+    switch ((g.m + 15) / 16) {
+        case 1: launch_skinny<RG, 1>(g, stream); break;
+        case 2: launch_skinny<RG, 2>(g, stream); break;
+        case 3: launch_skinny<RG, 3>(g, stream); break;
+        case 4: launch_skinny<RG, 4>(g, stream); break;
+        case 5: launch_skinny<RG, 5>(g, stream); break;
+        case 6: launch_skinny<RG, 6>(g, stream); break;
+        case 7: launch_skinny<RG, 7>(g, stream); break;
+        default: launch_skinny<RG, 8>(g, stream); break;
+    }
+}
+
+// as many rows per workgroup as still leaves ~200 workgroups
+void launch_skinny_auto(const GemmArgs& g, hipStream_t stream) {
+    if ((g.n + 47) / 48 >= 192) launch_skinny_mb<3>(g, stream);
+    else if ((g.n + 31) / 32 >= 192) launch_skinny_mb<2>(g, stream);
+    else launch_skinny_mb<1>(g, stream);
+}
+
 template <int MB>
 void launch_lds(const GemmArgs& g, hipStream_t stream) {
     const int blocks = (g.n + 15) / 16;
     gemv_int8_lds_kernel<MB><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(g);
 }
 
-template <int RG, int MB, int NW>
-void launch(const GemmArgs& g, hipStream_t stream) {
-    const int blocks = (g.n + RG * 16 - 1) / (RG * 16);
-    gemv_int8_kernel<RG, MB, NW><<<dim3((unsigned)blocks), dim3(NW * 64), 0, stream>>>(g);
-}
-
-template <int RG, int MB>
-void launch_nw(const GemmArgs& g, hipStream_t stream) {
-    if ((g.k >> 8) >= 16)
-        launch<RG, MB, 16>(g, stream);
-    else
-        launch<RG, MB, 4>(g, stream);
-}
-
 }  // namespace
 
 bool launch_gemv_int8(const GemmArgs& g, hipStream_t stream) {
-    if (g.m <= 0 || g.m > 64 || g.n <= 0 || g.k <= 0 || (g.k & 255) != 0) return false;
+    if (g.m <= 0 || g.m > 128 || g.n <= 0 || g.k <= 0 || (g.k & 255) != 0) return false;
     const int64_t lim = (int64_t)1 << 31;
     if ((int64_t)g.n * g.k >= lim) return false;
-    if (g.m == 1) {
+    if (g.m == 1)
         launch_dot(g, stream);
-        return true;
-    }
-    const int mb = (g.m + 15) / 16;
-    switch (mb) {
-        case 1: launch_lds<1>(g, stream); break;
-        case 2: launch_lds<2>(g, stream); break;
-        case 3: launch_nw<1, 3>(g, stream); break;
-        default: launch_nw<1, 4>(g, stream); break;
-    }
+    else if (g.m <= 16)
+        launch_lds<1>(g, stream);
+    else
+        launch_skinny_auto(g, stream);
     return true;
 }
 

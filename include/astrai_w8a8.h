@@ -147,7 +147,7 @@ int astrai_w8a8_gemm_fp8_block128(const void* a8, const void* b8, const float* s
  *   acc[m,n] = sum_k a[m,k] * b[n,k]              exact int32
  *   OUT_BF16: out = bf16(float(acc) * sa[m] * sb[n] + bias[n])
  *   OUT_ACC : out = acc as int32 (bit-exact parity surface)
- * Picks the skinny kernel for M <= 64 when the shape allows it, the tiled MFMA
+ * Picks the skinny kernel for M <= 128 when the shape allows it, the tiled MFMA
  * kernel otherwise.
  */
 int astrai_w8a8_gemm_int8_ptpc(const void* a, const void* b, const float* sa,
@@ -157,7 +157,7 @@ int astrai_w8a8_gemm_int8_ptpc(const void* a, const void* b, const float* sa,
 
 /*
  * The skinny (decode) int8 kernel on its own: same contract as
- * astrai_w8a8_gemm_int8_ptpc but requires M <= 64 and K % 256 == 0, and
+ * astrai_w8a8_gemm_int8_ptpc but requires M <= 128 and K % 256 == 0, and
  * returns ASTRAI_W8A8_UNSUPPORTED otherwise.
  */
 int astrai_w8a8_gemv_int8_ptpc(const void* a, const void* b, const float* sa,

@@ -41,8 +41,8 @@ def test_argument_validation_needs_no_gpu():
     assert b"null" in lib.astrai_w8a8_last_error()
     rc = lib.astrai_w8a8_quantize_bf16_fp8(16, 16, 16, None, 8, 7, None)
     assert rc == 1 and b"fmt" in lib.astrai_w8a8_last_error()
-    rc = lib.astrai_w8a8_gemv_int8_ptpc(16, 16, 16, 16, None, 16, 65, 4, 256, 0, None)
-    assert rc == 2 and b"M <= 64" in lib.astrai_w8a8_last_error()
+    rc = lib.astrai_w8a8_gemv_int8_ptpc(16, 16, 16, 16, None, 16, 129, 4, 256, 0, None)
+    assert rc == 2 and b"M <= 128" in lib.astrai_w8a8_last_error()
     rc = lib.astrai_w8a8_gemm_fp8_block128(16, 16, 16, 16, None, 16, 4, 4, 100, None)
     assert rc == 2 and b"128" in lib.astrai_w8a8_last_error()
     rc = lib.astrai_w8a8_gemm_fp8_pt(16, 16, 16, 16, None, None, 16, 4, 4, 64, 0, 1, None)

@@ -47,8 +47,8 @@ def test_golden_integer_cases_including_worst_case_magnitude(C, golden):
 
 
 @pytest.mark.parametrize("kernel", ["tiled", "gemv"])
-@pytest.mark.parametrize("m", [1, 4, 16, 17, 33, 64])
-@pytest.mark.parametrize("n,k", [(11008, 4096), (1000, 512), (40, 256)])
+@pytest.mark.parametrize("m", [1, 2, 4, 16, 17, 33, 64, 65, 100, 128])
+@pytest.mark.parametrize("n,k", [(11008, 4096), (1000, 512), (40, 256), (3072, 2048), (2048, 5632), (200, 11008)])
 def test_skinny_shapes_both_kernels_bit_exact(C, kernel, m, n, k):
     """Decode shapes through the wave-split skinny kernel and through the tiled
     kernel: the split-K integer sums must equal the single-pass ones."""
@@ -59,10 +59,26 @@ def test_skinny_shapes_both_kernels_bit_exact(C, kernel, m, n, k):
     assert torch.equal(got, O.int8_acc(a, b))
 
 
+@pytest.mark.parametrize("m,n,k", [(2, 11008, 4096), (32, 3072, 2048), (48, 11264, 2048), (128, 2048, 5632),
+                                   (5, 1001, 768)])
+def test_skinny_bf16_epilogue_bit_exact(C, m, n, k):
+    """The skinny kernel's dequant epilogue (scales, bias, one rounding; ragged N
+    takes the scalar stores) against the oracle's elementwise fp32 formula."""
+    print(f"case m={m} n={n} k={k}", flush=True)
+    g = torch.Generator().manual_seed(m * 7 + n + k)
+    a, b = _rand_i8(g, m, k), _rand_i8(g, n, k)
+    sa = torch.rand(m, generator=g) * 0.02 + 0.001
+    sb = torch.rand(n, generator=g) * 0.02 + 0.001
+    bias = torch.randn(n, generator=g).to(torch.bfloat16)
+    got = C.mm_int8(a.to(DEV), b.to(DEV), sa.to(DEV), sb.to(DEV), bias.to(DEV), 0, "gemv").cpu()
+    want = O.int8_gemm(a, b, sa, sb, bias)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
 def test_gemv_entry_rejects_what_it_cannot_run(C):
-    a = torch.zeros(65, 256, dtype=torch.int8, device=DEV)
+    a = torch.zeros(129, 256, dtype=torch.int8, device=DEV)
     b = torch.zeros(8, 256, dtype=torch.int8, device=DEV)
-    with pytest.raises(RuntimeError, match="M <= 64"):
+    with pytest.raises(RuntimeError, match="M <= 128"):
         C.mm_int8(a, b, None, None, None, 2, "gemv")
     with pytest.raises(RuntimeError, match="multiple of 256"):
         C.mm_int8(a[:4, :128].contiguous(), b[:, :128].contiguous(), None, None, None, 2, "gemv")
