@@ -133,6 +133,29 @@ int astrai_w8a8_silu_mul_quantize_int8_rows(const void* gate, const void* up, in
     return check_launch("silu_mul_quantize_int8_rows");
 }
 
+int astrai_w8a8_rope_cache_write_bf16(const void* qkv, int64_t ld, const float* freqs,
+                                      const int64_t* positions, void* q_out, void* k_cache,
+                                      void* v_cache, int64_t batch, int64_t seq, int64_t n_heads,
+                                      int64_t n_kv_heads, int64_t head_dim, int64_t max_len,
+                                      void* stream) {
+    if (!qkv || !freqs || !positions || !q_out || !k_cache || !v_cache)
+        return fail(ASTRAI_W8A8_BAD_ARG, "rope_cache_write_bf16: null pointer");
+    if (batch < 0 || seq < 0 || n_heads <= 0 || n_kv_heads <= 0 || head_dim <= 0 || max_len <= 0 ||
+        batch > 0x7fffffff || seq > 0x7fffffff || n_heads > 65535 || n_kv_heads > 65535)
+        return fail(ASTRAI_W8A8_BAD_ARG, "rope_cache_write_bf16: bad dims");
+    if (head_dim % 8 || head_dim > 65536)
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "rope_cache_write_bf16: head_dim must be a multiple of 8");
+    if (ld < (n_heads + 2 * n_kv_heads) * head_dim || ld % 8)
+        return fail(ASTRAI_W8A8_BAD_ARG, "rope_cache_write_bf16: ld must cover q|k|v and be a multiple of 8");
+    if (!aligned16(qkv) || !aligned16(freqs) || !aligned16(q_out) || !aligned16(k_cache) || !aligned16(v_cache))
+        return fail(ASTRAI_W8A8_BAD_ARG, "rope_cache_write_bf16: pointers must be 16-byte aligned");
+    if (batch == 0 || seq == 0) return ASTRAI_W8A8_OK;
+    w8a8::RopeCacheArgs a{qkv, ld, freqs, positions, q_out, k_cache, v_cache,
+                          (int)batch, (int)seq, (int)n_heads, (int)n_kv_heads, (int)head_dim, max_len};
+    w8a8::launch_rope_cache_write(a, static_cast<hipStream_t>(stream));
+    return check_launch("rope_cache_write_bf16");
+}
+
 int astrai_w8a8_quantize_bf16_fp8_block128_act(const void* x, void* x8, float* sa, int64_t m,
                                                int64_t k, void* stream) {
     if (!x || !x8 || !sa) return fail(ASTRAI_W8A8_BAD_ARG, "quantize_block128_act: null pointer");

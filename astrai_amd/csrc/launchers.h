@@ -42,6 +42,21 @@ void launch_quantize_fp8_block128_act(const void* x, void* x8, float* sa, int64_
 void launch_quantize_fp8_block128_weight(const void* w, void* w8, float* sb, int64_t n,
                                          int64_t k, hipStream_t stream);
 
+// rope_cache.hip: rotary embedding of q / k and the KV-cache write, one pass over
+// the fused q|k|v projection output
+struct RopeCacheArgs {
+    const void* qkv;          // bf16 [batch*seq, ld], columns q heads | k heads | v heads
+    int64_t ld;               // row pitch of qkv in elements
+    const float* freqs;       // fp32 [seq, head_dim/2, 2] (cos, sin) of the tokens' positions
+    const int64_t* positions; // int64 [seq]: cache slot of each token
+    void* q_out;              // bf16 [batch, n_heads, seq, head_dim]
+    void* k_cache;            // bf16 [batch, n_kv_heads, max_len, head_dim]
+    void* v_cache;            // same
+    int batch, seq, n_heads, n_kv_heads, head_dim;
+    int64_t max_len;
+};
+void launch_rope_cache_write(const RopeCacheArgs& a, hipStream_t stream);
+
 // gemm_int8.hip / gemm_fp8.hip / gemm_fp8_block.hip: tiled MFMA kernels.
 // Require k % 16 == 0 and m*k, n*k < 2^31 bytes; return false if the shape is
 // not accepted (the caller then uses the generic kernel).

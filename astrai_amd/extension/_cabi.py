@@ -36,6 +36,8 @@ PROTOTYPES = {
     "astrai_w8a8_add_rmsnorm_quantize_int8_rows": (
         [_P, _P, _P, ctypes.c_float, _P, _P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_silu_mul_quantize_int8_rows": ([_P, _P, _I64, _P, _P, _P, _I64, _I64, _P], _INT),
+    "astrai_w8a8_rope_cache_write_bf16": (
+        [_P, _I64, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _P], _INT),
     "astrai_w8a8_quantize_bf16_fp8_block128_act": ([_P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_quantize_bf16_fp8_block128_weight": ([_P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_gemm_fp8_pt": ([_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _INT, _INT, _P], _INT),
@@ -374,6 +376,47 @@ def silu_mul_quantize_int8(gate: torch.Tensor, up: torch.Tensor, want_h: bool = 
             g2.data_ptr(), u2.data_ptr(), ld, _ptr(h), hq.data_ptr(), s.data_ptr(), rows, w,
             _stream(gate)), lib)
     return hq, s, None if h is None else h.reshape(gate.shape)
+
+
+def rope_cache_write(qkv: torch.Tensor, freqs: torch.Tensor, positions: torch.Tensor,
+                     k_cache: torch.Tensor, v_cache: torch.Tensor, n_heads: int, n_kv_heads: int,
+                     head_dim: int) -> torch.Tensor:
+    """Rotate q and k of ``qkv [batch, seq, (n_heads + 2 n_kv_heads) * head_dim]`` (a view whose
+    last dimension is contiguous and whose tokens are equally spaced), write k and v into
+    ``k_cache`` / ``v_cache`` ``[batch, n_kv_heads, max_len, head_dim]`` at ``positions [seq]``
+    and return q as ``[batch, n_heads, seq, head_dim]``. ``freqs`` is fp32
+    ``[seq, head_dim/2, 2]`` (cos, sin)."""
+    lib = _require()
+    _gpu(qkv, "rope_cache_write")
+    if qkv.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
+        raise RuntimeError("qkv and the caches must be bf16")
+    if qkv.dim() != 3:
+        raise RuntimeError("qkv must be [batch, seq, features]")
+    b, s, feat = qkv.shape
+    if feat != (n_heads + 2 * n_kv_heads) * head_dim:
+        raise RuntimeError("qkv features must be (n_heads + 2 n_kv_heads) * head_dim")
+    q2 = qkv.reshape(b * s, feat)
+    if q2.stride(1) != 1:
+        q2 = q2.contiguous()
+    ld = q2.stride(0) if b * s > 1 else max(feat, q2.stride(0))
+    if freqs.dtype != torch.float32 or tuple(freqs.shape[-3:]) != (s, head_dim // 2, 2):
+        raise RuntimeError("freqs must be fp32 [seq, head_dim/2, 2]")
+    if positions.dtype != torch.int64 or positions.numel() != s:
+        raise RuntimeError("positions must be int64 [seq]")
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous()) or k_cache.shape != v_cache.shape:
+        raise RuntimeError("caches must be contiguous and of one shape")
+    if k_cache.dim() != 4 or k_cache.size(0) != b or k_cache.size(1) != n_kv_heads or k_cache.size(3) != head_dim:
+        raise RuntimeError("caches must be [batch, n_kv_heads, max_len, head_dim]")
+    for t in (freqs, positions, k_cache, v_cache):
+        if t.device != qkv.device:
+            raise RuntimeError("all tensors must be on qkv's device")
+    with torch.cuda.device(qkv.device):
+        q_out = torch.empty((b, n_heads, s, head_dim), device=qkv.device, dtype=torch.bfloat16)
+        _check(lib.astrai_w8a8_rope_cache_write_bf16(
+            q2.data_ptr(), ld, freqs.contiguous().data_ptr(), positions.contiguous().data_ptr(),
+            q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), b, s, n_heads, n_kv_heads,
+            head_dim, k_cache.size(2), _stream(qkv)), lib)
+    return q_out
 
 
 _INT8_ENTRY = {

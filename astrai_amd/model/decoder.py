@@ -171,11 +171,28 @@ class GQA(nn.Module):
             # the n_rep query heads that share a KV head are folded into the query
             # axis ([B, H_kv, n_rep*S, D]) instead of copying the cache n_rep times:
             # the same dot products and softmax rows as after repeat_kv
-            qf = q.reshape(b, self.n_kv_heads, self.n_rep * s, self.head_dim)
-            mask = key_mask if self.n_rep == 1 else key_mask.repeat(1, 1, self.n_rep, 1)
-            out = F.scaled_dot_product_attention(qf, kv_cache.k[self.layer_id],
-                                                 kv_cache.v[self.layer_id], attn_mask=mask)
-            out = out.reshape(b, self.n_heads, s, self.head_dim)
+            out = self._attend_cache(q, kv_cache, key_mask)
+        return out.permute(0, 2, 1, 3).reshape(b, s, self.dim)
+
+    def _attend_cache(self, q: Tensor, kv_cache: DenseKVCache, key_mask: Tensor) -> Tensor:
+        """``q [B, H, S, D]`` against the layer's cache; ``key_mask`` is ``[1, 1, n_rep*S, max_len]``
+        (the block's mask repeated once per query head of a KV group)."""
+        b, _, s, _ = q.shape
+        qf = q.reshape(b, self.n_kv_heads, self.n_rep * s, self.head_dim)
+        out = F.scaled_dot_product_attention(qf, kv_cache.k[self.layer_id],
+                                             kv_cache.v[self.layer_id], attn_mask=key_mask)
+        return out.reshape(b, self.n_heads, s, self.head_dim)
+
+    def core_fused_qkv(self, qkv: Tensor, rotary_emb: Tensor, kv_cache: DenseKVCache,
+                       positions: Tensor, key_mask: Tensor) -> Tensor:
+        """Same as :meth:`core` for a fused ``q|k|v`` projection ``[B, S, (H + 2 H_kv) D]`` with a
+        cache: rotation, permutes and the cache write are one kernel."""
+        from astrai_amd.extension import _cabi
+        b, s, _ = qkv.shape
+        q = _cabi.rope_cache_write(qkv, rotary_emb[0], positions, kv_cache.k[self.layer_id],
+                                   kv_cache.v[self.layer_id], self.n_heads, self.n_kv_heads,
+                                   self.head_dim)
+        out = self._attend_cache(q, kv_cache, key_mask)
         return out.permute(0, 2, 1, 3).reshape(b, s, self.dim)
 
 
@@ -216,8 +233,11 @@ class DecoderBlock(nn.Module):
         xq, sx, _ = I.rmsnorm_quantize_int8(x, self.input_norm.weight, self.input_norm.norm_eps)
         qkv = I.mm_int8(xq, f.wqkv, sx, f.sqkv).reshape(b, s, -1)
         nq, nkv = att.n_heads * att.head_dim, att.n_kv_heads * att.head_dim
-        a = att.core(qkv[..., :nq], qkv[..., nq:nq + nkv], qkv[..., nq + nkv:], rotary_emb, kv_cache,
-                     positions, key_mask)
+        if kv_cache is not None:
+            a = att.core_fused_qkv(qkv, rotary_emb, kv_cache, positions, key_mask)
+        else:
+            a = att.core(qkv[..., :nq], qkv[..., nq:nq + nkv], qkv[..., nq + nkv:], rotary_emb, None,
+                         positions, key_mask)
         aq, sa = I.quantize_int8_per_token(a)
         o = I.mm_int8(aq, f.wo, sa, f.so).reshape(b, s, d)
         # h = attention + x, then its norm, quantized: one kernel
@@ -264,6 +284,9 @@ class AutoRegressiveLM(nn.Module):
         if kv_cache is not None:
             key_pos = torch.arange(kv_cache.max_len, device=input_ids.device)
             key_mask = (key_pos[None, :] <= positions[:, None])[None, None]  # [1,1,seq,max_len]
+            n_rep = self.config.num_attention_heads // self.config.num_key_value_heads
+            if n_rep > 1:  # one copy per query head of a KV group, made once for all layers
+                key_mask = key_mask.repeat(1, 1, n_rep, 1)
         for layer in self.layers:
             x = layer(x, rotary, kv_cache, positions, key_mask)
         if self.fused_int8 is not None and _fused_int8_active(x):

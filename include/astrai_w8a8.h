@@ -106,6 +106,28 @@ int astrai_w8a8_silu_mul_quantize_int8_rows(const void* gate_bf16, const void* u
                                             int64_t width, void* stream);
 
 /*
+ * Rotary embedding of q and k plus the KV-cache write of one decoder layer, one
+ * pass over the (fused) q|k|v projection output. Replaces, between the
+ * projections and the attention call of GQA.forward
+ * (astrai/model/components/attention.py:19-85): the reshape/permute of q, k, v,
+ * the rotation of adjacent pairs in fp32 with one cast back
+ * (astrai/extension/backend/rotary.py:25-33) and the cache update.
+ *   qkv        bf16 [batch*seq, ld]: per token  q (n_heads*head_dim) | k (n_kv_heads*head_dim) | v (same)
+ *   freqs      fp32 [seq, head_dim/2, 2]: (cos, sin) of each token's position
+ *   positions  int64 [seq] (device): cache slot of each token; a slot outside [0, max_len) is skipped
+ *   q_out      bf16 [batch, n_heads, seq, head_dim]
+ *   k_cache, v_cache  bf16 [batch, n_kv_heads, max_len, head_dim], written at positions[s]
+ *   rope(x)[2i] = x[2i] cos_i - x[2i+1] sin_i;  rope(x)[2i+1] = x[2i] sin_i + x[2i+1] cos_i
+ *   (every product and sum rounded in fp32, one rounding to bf16: identical to the tensor ops)
+ * head_dim % 8 == 0, ld % 8 == 0.
+ */
+int astrai_w8a8_rope_cache_write_bf16(const void* qkv_bf16, int64_t ld, const float* freqs,
+                                      const int64_t* positions, void* q_out_bf16,
+                                      void* k_cache_bf16, void* v_cache_bf16, int64_t batch,
+                                      int64_t seq, int64_t n_heads, int64_t n_kv_heads,
+                                      int64_t head_dim, int64_t max_len, void* stream);
+
+/*
  * bf16 -> e4m3fn with one scale per 1x128 K-group (activations) or per 128x128
  * block (weights). No counterpart in the reference. K must be a multiple of 128.
  *   act:    sa[m,kb]  = max(max |x[m,128kb..128kb+127]|, 1e-12) / 448,   sa is [M, K/128]

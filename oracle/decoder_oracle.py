@@ -38,6 +38,24 @@ def apply_rotary(x: torch.Tensor, freqs_cis: torch.Tensor) -> torch.Tensor:
     return torch.view_as_real(rot).flatten(-2).to(x.dtype)
 
 
+def rope_cache_write(qkv: torch.Tensor, freqs_cis: torch.Tensor, positions: torch.Tensor,
+                     k_cache: torch.Tensor, v_cache: torch.Tensor, n_heads: int, n_kv_heads: int,
+                     head_dim: int) -> torch.Tensor:
+    """What sits between the q/k/v projections and the attention call with a cache
+    (components/attention.py:19-85): split ``qkv [B, S, (H + 2 H_kv) D]``, rotate q and k
+    (:func:`apply_rotary`), permute to ``[B, heads, S, D]``, write k and v into the caches
+    ``[B, H_kv, max_len, D]`` at ``positions [S]`` (in place) and return q."""
+    b, s, _ = qkv.shape
+    nq, nkv = n_heads * head_dim, n_kv_heads * head_dim
+    q = qkv[..., :nq].reshape(b, s, n_heads, head_dim)
+    k = qkv[..., nq:nq + nkv].reshape(b, s, n_kv_heads, head_dim)
+    v = qkv[..., nq + nkv:].reshape(b, s, n_kv_heads, head_dim)
+    q, k = apply_rotary(q, freqs_cis), apply_rotary(k, freqs_cis)
+    k_cache.index_copy_(2, positions, k.permute(0, 2, 1, 3))
+    v_cache.index_copy_(2, positions, v.permute(0, 2, 1, 3))
+    return q.permute(0, 2, 1, 3).contiguous()
+
+
 def repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:
     # x: [B, S, H_kv, D] -> [B, S, H_kv*n_rep, D]
     if n_rep == 1:
