@@ -156,6 +156,42 @@ int astrai_w8a8_rope_cache_write_bf16(const void* qkv, int64_t ld, const float* 
     return check_launch("rope_cache_write_bf16");
 }
 
+int64_t astrai_w8a8_attn_decode_workspace_floats(int64_t batch, int64_t n_kv_heads, int64_t nsplit,
+                                                 int64_t n_query_rows) {
+    if (batch <= 0 || n_kv_heads <= 0 || nsplit <= 0 || n_query_rows <= 0 || n_query_rows > 8) return 0;
+    return w8a8::attn_decode_workspace_floats((int)batch, (int)n_kv_heads, (int)nsplit, (int)n_query_rows);
+}
+
+int astrai_w8a8_attn_decode_bf16(const void* q, const void* k_cache, const void* v_cache,
+                                 const int64_t* positions, float* workspace, int64_t workspace_floats,
+                                 void* out, int64_t batch, int64_t seq, int64_t n_heads,
+                                 int64_t n_kv_heads, int64_t head_dim, int64_t max_len,
+                                 int64_t nsplit, float scale, void* stream) {
+    if (!q || !k_cache || !v_cache || !positions || !workspace || !out)
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_decode_bf16: null pointer");
+    if (batch < 0 || seq < 0 || n_heads <= 0 || n_kv_heads <= 0 || max_len <= 0 || nsplit <= 0 ||
+        nsplit > 64 || batch > 65535 || n_heads % n_kv_heads)
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_decode_bf16: bad dims");
+    if (head_dim != 128 || (n_heads / n_kv_heads) * seq > 8)
+        return fail(ASTRAI_W8A8_UNSUPPORTED,
+                    "attn_decode_bf16: needs head_dim 128 and (n_heads / n_kv_heads) * seq <= 8");
+    if (max_len * 256 >= ((int64_t)1 << 32))
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "attn_decode_bf16: one head of the cache must stay under 4 GiB");
+    if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out))
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_decode_bf16: pointers must be 16-byte aligned");
+    if (batch == 0 || seq == 0) return ASTRAI_W8A8_OK;
+    const int64_t need = w8a8::attn_decode_workspace_floats((int)batch, (int)n_kv_heads, (int)nsplit,
+                                                            (int)((n_heads / n_kv_heads) * seq));
+    if (workspace_floats < need)
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_decode_bf16: workspace too small (%lld floats needed)",
+                    (long long)need);
+    w8a8::AttnDecodeArgs a{q, k_cache, v_cache, positions, workspace, out, (int)batch, (int)seq,
+                           (int)n_heads, (int)n_kv_heads, (int)head_dim, max_len, (int)nsplit, scale};
+    if (!w8a8::launch_attn_decode(a, static_cast<hipStream_t>(stream)))
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "attn_decode_bf16: shape not supported");
+    return check_launch("attn_decode_bf16");
+}
+
 int astrai_w8a8_quantize_bf16_fp8_block128_act(const void* x, void* x8, float* sa, int64_t m,
                                                int64_t k, void* stream) {
     if (!x || !x8 || !sa) return fail(ASTRAI_W8A8_BAD_ARG, "quantize_block128_act: null pointer");

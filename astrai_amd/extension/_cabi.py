@@ -38,6 +38,9 @@ PROTOTYPES = {
     "astrai_w8a8_silu_mul_quantize_int8_rows": ([_P, _P, _I64, _P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_rope_cache_write_bf16": (
         [_P, _I64, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _P], _INT),
+    "astrai_w8a8_attn_decode_workspace_floats": ([_I64, _I64, _I64, _I64], _I64),
+    "astrai_w8a8_attn_decode_bf16": (
+        [_P, _P, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, ctypes.c_float, _P], _INT),
     "astrai_w8a8_quantize_bf16_fp8_block128_act": ([_P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_quantize_bf16_fp8_block128_weight": ([_P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_gemm_fp8_pt": ([_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _INT, _INT, _P], _INT),
@@ -417,6 +420,47 @@ def rope_cache_write(qkv: torch.Tensor, freqs: torch.Tensor, positions: torch.Te
             q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), b, s, n_heads, n_kv_heads,
             head_dim, k_cache.size(2), _stream(qkv)), lib)
     return q_out
+
+
+def attn_decode_supported(n_heads: int, n_kv_heads: int, seq: int, head_dim: int) -> bool:
+    return head_dim == 128 and n_heads % n_kv_heads == 0 and (n_heads // n_kv_heads) * seq <= 8
+
+
+def attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, positions: torch.Tensor,
+                scale: Optional[float] = None, nsplit: int = 0) -> torch.Tensor:
+    """``q [batch, n_heads, seq, 128]`` (bf16) against the dense caches
+    ``[batch, n_kv_heads, max_len, 128]``; token ``s`` attends keys ``0..positions[s]``.
+    Returns ``[batch, seq, n_heads * 128]``. ``nsplit`` 0 picks a split count that fills the chip."""
+    lib = _require()
+    _gpu(q, "attn_decode")
+    if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
+        raise RuntimeError("q and the caches must be bf16")
+    if q.dim() != 4 or k_cache.dim() != 4 or k_cache.shape != v_cache.shape:
+        raise RuntimeError("q must be [B, H, S, D] and the caches [B, H_kv, max_len, D]")
+    b, h, s, d = q.shape
+    hkv, max_len = k_cache.size(1), k_cache.size(2)
+    if k_cache.size(0) != b or k_cache.size(3) != d:
+        raise RuntimeError("cache batch / head_dim do not match q")
+    if not (q.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise RuntimeError("q and the caches must be contiguous")
+    if positions.dtype != torch.int64 or positions.numel() != s or positions.device != q.device:
+        raise RuntimeError("positions must be int64 [seq] on q's device")
+    if h % hkv:
+        raise RuntimeError("n_heads must be a multiple of n_kv_heads")
+    if scale is None:
+        scale = d ** -0.5
+    if nsplit <= 0:
+        nsplit = max(1, min(16, 1024 // max(1, b * hkv)))
+    nq = (h // hkv) * s
+    with torch.cuda.device(q.device):
+        need = lib.astrai_w8a8_attn_decode_workspace_floats(b, hkv, nsplit, nq)
+        ws = torch.empty(max(need, 1), device=q.device, dtype=torch.float32)
+        out = torch.empty((b, s, h * d), device=q.device, dtype=torch.bfloat16)
+        _check(lib.astrai_w8a8_attn_decode_bf16(
+            q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), positions.contiguous().data_ptr(),
+            ws.data_ptr(), ws.numel(), out.data_ptr(), b, s, h, hkv, d, max_len, nsplit, float(scale),
+            _stream(q)), lib)
+    return out
 
 
 _INT8_ENTRY = {

@@ -192,6 +192,9 @@ class GQA(nn.Module):
         q = _cabi.rope_cache_write(qkv, rotary_emb[0], positions, kv_cache.k[self.layer_id],
                                    kv_cache.v[self.layer_id], self.n_heads, self.n_kv_heads,
                                    self.head_dim)
+        if _cabi.attn_decode_supported(self.n_heads, self.n_kv_heads, s, self.head_dim):
+            # a few new tokens: the split-context kernel (mask from `positions`, token-major output)
+            return _cabi.attn_decode(q, kv_cache.k[self.layer_id], kv_cache.v[self.layer_id], positions)
         out = self._attend_cache(q, kv_cache, key_mask)
         return out.permute(0, 2, 1, 3).reshape(b, s, self.dim)
 

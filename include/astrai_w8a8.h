@@ -128,6 +128,32 @@ int astrai_w8a8_rope_cache_write_bf16(const void* qkv_bf16, int64_t ld, const fl
                                       int64_t head_dim, int64_t max_len, void* stream);
 
 /*
+ * Grouped-query attention of the `seq` newest tokens of every sequence against the
+ * dense KV cache (decode step; split over the context and merged). Replaces the
+ * cached branch of GQA.forward / the decode attention backend
+ * (astrai/model/components/attention.py:19-85,
+ * astrai/extension/backend/attention.py:244-253,443-498): head expansion, mask and
+ * softmax(q k^T * scale) v, with the permute back to token-major folded in.
+ *   q          bf16 [batch, n_heads, seq, 128] (as written by rope_cache_write)
+ *   k_cache, v_cache  bf16 [batch, n_kv_heads, max_len, 128]; entries at positions
+ *              <= the largest positions[s] must have been written
+ *   positions  int64 [seq] (device): token s attends keys 0..positions[s]
+ *   workspace  fp32, at least astrai_w8a8_attn_decode_workspace_floats(batch,
+ *              n_kv_heads, nsplit, (n_heads / n_kv_heads) * seq) floats (caller-owned scratch)
+ *   out        bf16 [batch, seq, n_heads * 128]
+ *   nsplit     number of context splits (1..64): batch * n_kv_heads * nsplit workgroups
+ * fp32 scores and softmax, fp32 accumulation of p*v, one rounding to bf16.
+ * head_dim == 128 and (n_heads / n_kv_heads) * seq <= 8.
+ */
+int64_t astrai_w8a8_attn_decode_workspace_floats(int64_t batch, int64_t n_kv_heads, int64_t nsplit,
+                                                 int64_t n_query_rows);
+int astrai_w8a8_attn_decode_bf16(const void* q_bf16, const void* k_cache_bf16, const void* v_cache_bf16,
+                                 const int64_t* positions, float* workspace, int64_t workspace_floats,
+                                 void* out_bf16, int64_t batch, int64_t seq, int64_t n_heads,
+                                 int64_t n_kv_heads, int64_t head_dim, int64_t max_len,
+                                 int64_t nsplit, float scale, void* stream);
+
+/*
  * bf16 -> e4m3fn with one scale per 1x128 K-group (activations) or per 128x128
  * block (weights). No counterpart in the reference. K must be a multiple of 128.
  *   act:    sa[m,kb]  = max(max |x[m,128kb..128kb+127]|, 1e-12) / 448,   sa is [M, K/128]

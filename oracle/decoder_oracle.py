@@ -56,6 +56,25 @@ def rope_cache_write(qkv: torch.Tensor, freqs_cis: torch.Tensor, positions: torc
     return q.permute(0, 2, 1, 3).contiguous()
 
 
+def attn_cached(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                positions: torch.Tensor) -> torch.Tensor:
+    """Attention of ``q [B, H, S, D]`` over the caches ``[B, H_kv, max_len, D]`` where token ``s``
+    sees keys ``0..positions[s]``: head expansion (extension/backend/attention.py:244-253) and
+    ``softmax(q k^T / sqrt(D)) v`` in float32 (:443-498), returned token-major ``[B, S, H*D]`` in
+    the input dtype, as the cached branch of components/attention.py:19-85 hands it to ``o_proj``."""
+    b, h, s, d = q.shape
+    n_rep = h // k_cache.size(1)
+    # repeat_kv works on [B, S, H_kv, D]; the caches are [B, H_kv, max_len, D]
+    k = repeat_kv(k_cache.transpose(1, 2), n_rep).transpose(1, 2).float()
+    v = repeat_kv(v_cache.transpose(1, 2), n_rep).transpose(1, 2).float()
+    scores = q.float() @ k.transpose(-1, -2) / (d ** 0.5)          # [B, H, S, max_len]
+    key_pos = torch.arange(k_cache.size(2))
+    visible = key_pos[None, :] <= positions[:, None]                 # [S, max_len]
+    scores = scores.masked_fill(~visible[None, None], float("-inf"))
+    out = torch.softmax(scores, dim=-1) @ v                          # [B, H, S, D]
+    return out.permute(0, 2, 1, 3).reshape(b, s, h * d).to(q.dtype)
+
+
 def repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:
     # x: [B, S, H_kv, D] -> [B, S, H_kv*n_rep, D]
     if n_rep == 1:

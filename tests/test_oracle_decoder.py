@@ -83,3 +83,46 @@ def test_int8_path_tracks_bf16_path():
     a = D.forward(sd, CFG, ids, D.int8_linear_fn(sd)).float().flatten()
     b = D.forward(sd, CFG, ids, D.bf16_linear_fn(sd)).float().flatten()
     assert torch.nn.functional.cosine_similarity(a, b, dim=0).item() > 0.99
+
+
+def test_attn_cached_closed_forms():
+    """Pins the oracle's cached attention: one visible key returns that key's value row;
+    equal scores return the mean of the visible value rows; KV heads are shared by
+    consecutive query heads."""
+    b, h, hkv, s, max_len, d = 2, 4, 2, 2, 6, 8
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(b, h, s, d, generator=g)
+    kc = torch.randn(b, hkv, max_len, d, generator=g)
+    vc = torch.randn(b, hkv, max_len, d, generator=g)
+    pos = torch.tensor([0, 3])
+    out = D.attn_cached(q, kc, vc, pos).reshape(b, s, h, d)
+    for head in range(h):
+        torch.testing.assert_close(out[:, 0, head], vc[:, head // 2, 0])          # token 0 sees key 0 only
+    kc0 = torch.zeros_like(kc)                                                    # all scores equal
+    out0 = D.attn_cached(q, kc0, vc, pos).reshape(b, s, h, d)
+    for head in range(h):
+        torch.testing.assert_close(out0[:, 1, head], vc[:, head // 2, :4].mean(1))
+    # brute force over one (batch, head, token)
+    sc = (q[1, 3, 1] @ kc[1, 1, :4].T) / d ** 0.5
+    want = torch.softmax(sc, 0) @ vc[1, 1, :4]
+    torch.testing.assert_close(out[1, 1, 3], want)
+
+
+def test_rope_cache_write_is_the_tensor_op_chain():
+    """Pins the oracle's rope + cache write: rotation by 90 degrees swaps and negates the pair;
+    caches change only at the written positions."""
+    b, s, h, hkv, d, max_len = 1, 2, 2, 1, 4, 5
+    qkv = torch.arange(b * s * (h + 2 * hkv) * d, dtype=torch.float32).reshape(b, s, -1)
+    freqs = torch.zeros(1, s, d // 2, 2)
+    freqs[..., 0] = 0.0   # cos
+    freqs[..., 1] = 1.0   # sin: rotate every pair by 90 degrees: (e, o) -> (-o, e)
+    kc = torch.full((b, hkv, max_len, d), -1.0)
+    vc = torch.full((b, hkv, max_len, d), -1.0)
+    pos = torch.tensor([1, 4])
+    q = D.rope_cache_write(qkv, freqs, pos, kc, vc, h, hkv, d)
+    x = qkv[0, 0, :d]
+    torch.testing.assert_close(q[0, 0, 0], torch.stack([-x[1], x[0], -x[3], x[2]]))
+    kx = qkv[0, 1, h * d:h * d + d]
+    torch.testing.assert_close(kc[0, 0, 4], torch.stack([-kx[1], kx[0], -kx[3], kx[2]]))
+    torch.testing.assert_close(vc[0, 0, 1], qkv[0, 0, (h + hkv) * d:])
+    assert (kc[0, 0, [0, 2, 3]] == -1).all() and (vc[0, 0, [0, 2, 3]] == -1).all()
