@@ -259,6 +259,25 @@ __global__ __launch_bounds__(NW * 64) void skinny_int8_kernel(GemmArgs g) {
 #pragma unroll
         for (int b = 0; b < MB; ++b) acc[r][b] = i32x4{0, 0, 0, 0};
 
+    // epilogue operands of the (row group, token group) tasks this wave will write,
+    // requested now so that their latency hides under the weight stream
+    constexpr int TASKS = (RG * MB + NW - 1) / NW;
+    float e_sx[TASKS], e_sw[TASKS][4], e_b[TASKS][4];
+#pragma unroll
+    for (int ti = 0; ti < TASKS; ++ti) {
+        const int t = wave + ti * NW;
+        const int m = (t % MB) * 16 + lrow;
+        const int en = n0 + (t / MB) * 16 + lgrp * 4;
+        const bool live = t < RG * MB && g.out_kind != OUT_ACC;
+        e_sx[ti] = (live && m < g.m) ? g.sa[m] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const bool in = live && en + j < g.n;
+            e_sw[ti][j] = in ? g.sb[en + j] : 0.0f;
+            e_b[ti][j] = (in && g.bias) ? bf16_to_f32(static_cast<const uint16_t*>(g.bias)[en + j]) : 0.0f;
+        }
+    }
+
     uint8_t* const mine = smem + wave * WAVE_BYTES;
     // load plan: instruction i covers rows 2i, 2i+1; lane -> row 2i + (lane>>5),
     // position lane&31, logical chunk (lane&31) ^ ((2i + (lane>>5)) & 15)
@@ -310,7 +329,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_int8_kernel(GemmArgs g) {
         __builtin_amdgcn_sched_barrier(0);  // the next step's loads overwrite what was just read
     }
 
-    // sum the four waves' partials through LDS (the staging space is free now)
+    // sum the waves' partials through LDS (the staging space is free now)
     __syncthreads();
     i32x4* const red = reinterpret_cast<i32x4*>(smem);  // [NW][RG * MB][64]
 #pragma unroll
@@ -318,8 +337,10 @@ __global__ __launch_bounds__(NW * 64) void skinny_int8_kernel(GemmArgs g) {
 #pragma unroll
         for (int b = 0; b < MB; ++b) red[(wave * RG * MB + r * MB + b) * 64 + lane] = acc[r][b];
     __syncthreads();
-    const uint16_t* bias = static_cast<const uint16_t*>(g.bias);
-    for (int t = wave; t < RG * MB; t += NW) {
+#pragma unroll
+    for (int ti = 0; ti < TASKS; ++ti) {
+        const int t = wave + ti * NW;
+        if (t >= RG * MB) break;
         i32x4 sum = red[t * 64 + lane];
 #pragma unroll
         for (int w = 1; w < NW; ++w) sum += red[(w * RG * MB + t) * 64 + lane];
@@ -335,17 +356,14 @@ __global__ __launch_bounds__(NW * 64) void skinny_int8_kernel(GemmArgs g) {
                 if (en + j < g.n) out[o + j] = sum[j];
             continue;
         }
-        const float sx = g.sa[m];
         float v[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             // product and bias add rounded separately (no fused multiply-add): the
             // int8 epilogue is specified as elementwise fp32 on the exact integer
 #pragma clang fp contract(off)
-            const float sw = (en + j < g.n) ? g.sb[en + j] : 0.0f;
-            float f = (float)sum[j] * sx * sw;
-            if (bias && en + j < g.n) f = f + bf16_to_f32(bias[en + j]);
-            v[j] = f;
+            const float f = (float)sum[j] * e_sx[ti] * e_sw[ti][j];
+            v[j] = f + e_b[ti][j];
         }
         uint16_t* out = static_cast<uint16_t*>(g.out);
         if ((g.n & 3) == 0) {
@@ -361,11 +379,11 @@ __global__ __launch_bounds__(NW * 64) void skinny_int8_kernel(GemmArgs g) {
     }
 }
 
-template <int RG, int MB>
+template <int RG, int MB, int NW>
 void launch_skinny(const GemmArgs& g, hipStream_t stream) {
-    constexpr int NW = 4;
     constexpr int lds_bytes = NW * RG * 16 * 512;
     static_assert(MB <= 8, "the reduction re-uses the staging space: NW * RG * MB KiB must fit");
+    static_assert(lds_bytes <= 160 * 1024, "staging space of all waves must fit in LDS");
     auto kern = skinny_int8_kernel<RG, MB, NW>;
     static bool attr_set = false;
     if (!attr_set) {
@@ -377,25 +395,31 @@ void launch_skinny(const GemmArgs& g, hipStream_t stream) {
     kern<<<dim3((unsigned)blocks), dim3(NW * 64), lds_bytes, stream>>>(g);
 }
 
-template <int RG>
+template <int RG, int NW>
 void launch_skinny_mb(const GemmArgs& g, hipStream_t stream) {
     switch ((g.m + 15) / 16) {
-        case 1: launch_skinny<RG, 1>(g, stream); break;
-        case 2: launch_skinny<RG, 2>(g, stream); break;
-        case 3: launch_skinny<RG, 3>(g, stream); break;
-        case 4: launch_skinny<RG, 4>(g, stream); break;
-        case 5: launch_skinny<RG, 5>(g, stream); break;
-        case 6: launch_skinny<RG, 6>(g, stream); break;
-        case 7: launch_skinny<RG, 7>(g, stream); break;
-        default: launch_skinny<RG, 8>(g, stream); break;
+        case 1: launch_skinny<RG, 1, NW>(g, stream); break;
+        case 2: launch_skinny<RG, 2, NW>(g, stream); break;
+        case 3: launch_skinny<RG, 3, NW>(g, stream); break;
+        case 4: launch_skinny<RG, 4, NW>(g, stream); break;
+        case 5: launch_skinny<RG, 5, NW>(g, stream); break;
+        case 6: launch_skinny<RG, 6, NW>(g, stream); break;
+        case 7: launch_skinny<RG, 7, NW>(g, stream); break;
+        default: launch_skinny<RG, 8, NW>(g, stream); break;
     }
 }
 
-// as many rows per workgroup as still leaves ~200 workgroups
+// As many rows per workgroup as still leaves ~200 workgroups. A matrix too short
+// for that (16-row workgroups, fewer of them than CUs) makes up for it with more
+// waves per workgroup when K is long, so that every 512-byte K-step still has a
+// wave of its own and all of the matrix is requested at once.
 void launch_skinny_auto(const GemmArgs& g, hipStream_t stream) {
-    if ((g.n + 47) / 48 >= 192) launch_skinny_mb<3>(g, stream);
-    else if ((g.n + 31) / 32 >= 192) launch_skinny_mb<2>(g, stream);
-    else launch_skinny_mb<1>(g, stream);
+    const int nsteps = (g.k + 511) >> 9;
+    if ((g.n + 47) / 48 >= 192) launch_skinny_mb<3, 4>(g, stream);
+    else if ((g.n + 31) / 32 >= 192) launch_skinny_mb<2, 4>(g, stream);
+    else if (nsteps <= 4 || (g.n + 15) / 16 >= 512) launch_skinny_mb<1, 4>(g, stream);
+    else if (nsteps <= 8) launch_skinny_mb<1, 8>(g, stream);
+    else launch_skinny_mb<1, 16>(g, stream);
 }
 
 template <int MB>
