@@ -164,20 +164,22 @@ int64_t astrai_w8a8_attn_decode_workspace_floats(int64_t batch, int64_t n_kv_hea
 
 int astrai_w8a8_attn_decode_bf16(const void* q, const void* k_cache, const void* v_cache,
                                  const int64_t* positions, float* workspace, int64_t workspace_floats,
-                                 void* out, int64_t batch, int64_t seq, int64_t n_heads,
+                                 void* out, void* out_q, float* out_scale, int64_t batch,
+                                 int64_t seq, int64_t n_heads,
                                  int64_t n_kv_heads, int64_t head_dim, int64_t max_len,
                                  int64_t nsplit, float scale, void* stream) {
-    if (!q || !k_cache || !v_cache || !positions || !workspace || !out)
+    if (!q || !k_cache || !v_cache || !positions || !workspace || (!out && !out_q) || (out_q && !out_scale))
         return fail(ASTRAI_W8A8_BAD_ARG, "attn_decode_bf16: null pointer");
     if (batch < 0 || seq < 0 || n_heads <= 0 || n_kv_heads <= 0 || max_len <= 0 || nsplit <= 0 ||
         nsplit > 64 || batch > 65535 || n_heads % n_kv_heads)
         return fail(ASTRAI_W8A8_BAD_ARG, "attn_decode_bf16: bad dims");
-    if (head_dim != 128 || (n_heads / n_kv_heads) * seq > 8)
+    if (head_dim != 128 || (n_heads / n_kv_heads) * seq > 8 || n_heads > 64)
         return fail(ASTRAI_W8A8_UNSUPPORTED,
-                    "attn_decode_bf16: needs head_dim 128 and (n_heads / n_kv_heads) * seq <= 8");
+                    "attn_decode_bf16: needs head_dim 128, (n_heads / n_kv_heads) * seq <= 8, n_heads <= 64");
     if (max_len * 256 >= ((int64_t)1 << 32))
         return fail(ASTRAI_W8A8_UNSUPPORTED, "attn_decode_bf16: one head of the cache must stay under 4 GiB");
-    if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out))
+    if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || (out && !aligned16(out)) ||
+        (out_q && !aligned16(out_q)))
         return fail(ASTRAI_W8A8_BAD_ARG, "attn_decode_bf16: pointers must be 16-byte aligned");
     if (batch == 0 || seq == 0) return ASTRAI_W8A8_OK;
     const int64_t need = w8a8::attn_decode_workspace_floats((int)batch, (int)n_kv_heads, (int)nsplit,
@@ -185,7 +187,7 @@ int astrai_w8a8_attn_decode_bf16(const void* q, const void* k_cache, const void*
     if (workspace_floats < need)
         return fail(ASTRAI_W8A8_BAD_ARG, "attn_decode_bf16: workspace too small (%lld floats needed)",
                     (long long)need);
-    w8a8::AttnDecodeArgs a{q, k_cache, v_cache, positions, workspace, out, (int)batch, (int)seq,
+    w8a8::AttnDecodeArgs a{q, k_cache, v_cache, positions, workspace, out, out_q, out_scale, (int)batch, (int)seq,
                            (int)n_heads, (int)n_kv_heads, (int)head_dim, max_len, (int)nsplit, scale};
     if (!w8a8::launch_attn_decode(a, static_cast<hipStream_t>(stream)))
         return fail(ASTRAI_W8A8_UNSUPPORTED, "attn_decode_bf16: shape not supported");

@@ -196,14 +196,31 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(AttnDecodeArgs
     }
 }
 
-// one workgroup per (batch, token): all heads, 8 output values per thread
+// One workgroup per (batch, token): all heads, 8 output values per thread and
+// pass. Besides (or instead of) the bf16 row it can emit the per-token int8
+// quantization of that row -- the input of the int8 output projection -- computed
+// on the bf16-rounded values, i.e. what the separate quantizer would produce.
+constexpr int kMergeCache = 4;  // rows up to 4 * 256 * 8 = 8192 wide stay in registers
+
+__device__ __forceinline__ float merge_block_max(float v, float* slots) {
+    v = wave_max(v);
+    if ((threadIdx.x & 63) == 0) slots[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return fmaxf(fmaxf(slots[0], slots[1]), fmaxf(slots[2], slots[3]));
+}
+
 template <int NQ>
 __global__ __launch_bounds__(256) void attn_decode_merge_kernel(AttnDecodeArgs a) {
+    __shared__ float slots[4];
     const int n_rep = a.n_heads / a.n_kv_heads;
     const int b = blockIdx.x / a.seq, s = blockIdx.x % a.seq;
     const int width = a.n_heads * kD;
-    uint16_t* out = static_cast<uint16_t*>(a.out) + (int64_t)blockIdx.x * width;
-    for (int e = threadIdx.x * 8; e < width; e += 256 * 8) {
+    float keep[kMergeCache][8];
+    float local = 0.0f;
+#pragma unroll
+    for (int c = 0; c < kMergeCache; ++c) {
+        const int e = (threadIdx.x + c * 256) * 8;
+        if (e >= width) break;
         const int h = e / kD, d0 = e - h * kD;
         const int hk = h / n_rep, q = (h - hk * n_rep) * a.seq + s;
         const float* base = a.ws + ((int64_t)(b * a.n_kv_heads + hk) * a.nsplit) * NQ * kWsRow + q * kWsRow;
@@ -223,7 +240,33 @@ __global__ __launch_bounds__(256) void attn_decode_merge_kernel(AttnDecodeArgs a
         o.y = pack_bf16x2(v[2] * inv, v[3] * inv);
         o.z = pack_bf16x2(v[4] * inv, v[5] * inv);
         o.w = pack_bf16x2(v[6] * inv, v[7] * inv);
-        *reinterpret_cast<u32x4*>(out + e) = o;
+        if (a.out) *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(a.out) + (int64_t)blockIdx.x * width + e) = o;
+        keep[c][0] = __uint_as_float(o.x << 16); keep[c][1] = __uint_as_float(o.x & 0xffff0000u);
+        keep[c][2] = __uint_as_float(o.y << 16); keep[c][3] = __uint_as_float(o.y & 0xffff0000u);
+        keep[c][4] = __uint_as_float(o.z << 16); keep[c][5] = __uint_as_float(o.z & 0xffff0000u);
+        keep[c][6] = __uint_as_float(o.w << 16); keep[c][7] = __uint_as_float(o.w & 0xffff0000u);
+#pragma unroll
+        for (int d = 0; d < 8; ++d) local = fmaxf(local, fabsf(keep[c][d]));
+    }
+    if (!a.out_q) return;
+    // per-token int8: step = max(amax, 1e-12) / 127, round half to even, clamp
+    const float step = fmaxf(merge_block_max(local, slots), 1e-12f) / 127.0f;
+    if (threadIdx.x == 0) a.out_scale[blockIdx.x] = step;
+#pragma unroll
+    for (int c = 0; c < kMergeCache; ++c) {
+        const int e = (threadIdx.x + c * 256) * 8;
+        if (e >= width) break;
+        uint32_t w[2] = {0u, 0u};
+#pragma unroll
+        for (int d = 0; d < 8; ++d) {
+            float qv = rintf(keep[c][d] / step);
+            qv = fminf(fmaxf(qv, -127.0f), 127.0f);
+            w[d >> 2] |= ((uint32_t)(int)qv & 0xffu) << (8 * (d & 3));
+        }
+        u32x2 pk;
+        pk.x = w[0];
+        pk.y = w[1];
+        *reinterpret_cast<u32x2*>(static_cast<int8_t*>(a.out_q) + (int64_t)blockIdx.x * width + e) = pk;
     }
 }
 
@@ -238,6 +281,7 @@ bool launch_attn_decode(const AttnDecodeArgs& a, hipStream_t stream) {
     const int n_rep = a.n_heads / a.n_kv_heads;
     const int nq = n_rep * a.seq;
     if (a.head_dim != kD || nq > 8 || nq <= 0 || a.nsplit <= 0) return false;
+    if (a.n_heads * kD > kMergeCache * 256 * 8) return false;  // the merge kernel keeps a token's row in registers
     const unsigned grid1 = (unsigned)(a.batch * a.n_kv_heads * a.nsplit);
     const unsigned grid2 = (unsigned)(a.batch * a.seq);
     if (nq <= 4) {

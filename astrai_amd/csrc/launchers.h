@@ -65,7 +65,9 @@ struct AttnDecodeArgs {
     const void* v_cache;       // same
     const int64_t* positions;  // int64 [seq]: position of each new token (keys <= it are attended)
     float* ws;                 // attn_decode_workspace_floats(...) floats
-    void* out;                 // bf16 [batch, seq, n_heads * 128]
+    void* out;                 // bf16 [batch, seq, n_heads * 128], or null
+    void* out_q;               // int8 [batch*seq, n_heads * 128] per-token quantization of `out`, or null
+    float* out_scale;          // fp32 [batch*seq] steps of out_q
     int batch, seq, n_heads, n_kv_heads, head_dim;
     int64_t max_len;
     int nsplit;

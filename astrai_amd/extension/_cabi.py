@@ -40,7 +40,8 @@ PROTOTYPES = {
         [_P, _I64, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _P], _INT),
     "astrai_w8a8_attn_decode_workspace_floats": ([_I64, _I64, _I64, _I64], _I64),
     "astrai_w8a8_attn_decode_bf16": (
-        [_P, _P, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, ctypes.c_float, _P], _INT),
+        [_P, _P, _P, _P, _P, _I64, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, ctypes.c_float, _P],
+        _INT),
     "astrai_w8a8_quantize_bf16_fp8_block128_act": ([_P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_quantize_bf16_fp8_block128_weight": ([_P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_gemm_fp8_pt": ([_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _INT, _INT, _P], _INT),
@@ -427,10 +428,12 @@ def attn_decode_supported(n_heads: int, n_kv_heads: int, seq: int, head_dim: int
 
 
 def attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, positions: torch.Tensor,
-                scale: Optional[float] = None, nsplit: int = 0) -> torch.Tensor:
+                scale: Optional[float] = None, nsplit: int = 0, quantized: bool = False):
     """``q [batch, n_heads, seq, 128]`` (bf16) against the dense caches
     ``[batch, n_kv_heads, max_len, 128]``; token ``s`` attends keys ``0..positions[s]``.
-    Returns ``[batch, seq, n_heads * 128]``. ``nsplit`` 0 picks a split count that fills the chip."""
+    Returns ``[batch, seq, n_heads * 128]`` bf16, or with ``quantized`` the per-token int8
+    form of it ``(int8 [batch*seq, n_heads*128], fp32 [batch*seq, 1])``.
+    ``nsplit`` 0 picks a split count that fills the chip."""
     lib = _require()
     _gpu(q, "attn_decode")
     if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
@@ -455,12 +458,17 @@ def attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, p
     with torch.cuda.device(q.device):
         need = lib.astrai_w8a8_attn_decode_workspace_floats(b, hkv, nsplit, nq)
         ws = torch.empty(max(need, 1), device=q.device, dtype=torch.float32)
-        out = torch.empty((b, s, h * d), device=q.device, dtype=torch.bfloat16)
+        out = oq = os_ = None
+        if quantized:
+            oq = torch.empty((b * s, h * d), device=q.device, dtype=torch.int8)
+            os_ = torch.empty((b * s, 1), device=q.device, dtype=torch.float32)
+        else:
+            out = torch.empty((b, s, h * d), device=q.device, dtype=torch.bfloat16)
         _check(lib.astrai_w8a8_attn_decode_bf16(
             q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), positions.contiguous().data_ptr(),
-            ws.data_ptr(), ws.numel(), out.data_ptr(), b, s, h, hkv, d, max_len, nsplit, float(scale),
-            _stream(q)), lib)
-    return out
+            ws.data_ptr(), ws.numel(), _ptr(out), _ptr(oq), _ptr(os_), b, s, h, hkv, d, max_len, nsplit,
+            float(scale), _stream(q)), lib)
+    return (oq, os_) if quantized else out
 
 
 _INT8_ENTRY = {

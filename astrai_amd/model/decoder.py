@@ -184,19 +184,23 @@ class GQA(nn.Module):
         return out.reshape(b, self.n_heads, s, self.head_dim)
 
     def core_fused_qkv(self, qkv: Tensor, rotary_emb: Tensor, kv_cache: DenseKVCache,
-                       positions: Tensor, key_mask: Tensor) -> Tensor:
+                       positions: Tensor, key_mask: Tensor):
         """Same as :meth:`core` for a fused ``q|k|v`` projection ``[B, S, (H + 2 H_kv) D]`` with a
-        cache: rotation, permutes and the cache write are one kernel."""
+        cache: rotation, permutes and the cache write are one kernel. Returns the attention
+        output already quantized per token, ``(int8 [B*S, dim], fp32 [B*S, 1])``: for a few new
+        tokens straight out of the split-context attention kernel (mask from ``positions``,
+        token-major), otherwise SDPA followed by the quantizer."""
         from astrai_amd.extension import _cabi
+        from astrai_amd.extension.ops import int8 as I
         b, s, _ = qkv.shape
         q = _cabi.rope_cache_write(qkv, rotary_emb[0], positions, kv_cache.k[self.layer_id],
                                    kv_cache.v[self.layer_id], self.n_heads, self.n_kv_heads,
                                    self.head_dim)
         if _cabi.attn_decode_supported(self.n_heads, self.n_kv_heads, s, self.head_dim):
-            # a few new tokens: the split-context kernel (mask from `positions`, token-major output)
-            return _cabi.attn_decode(q, kv_cache.k[self.layer_id], kv_cache.v[self.layer_id], positions)
+            return _cabi.attn_decode(q, kv_cache.k[self.layer_id], kv_cache.v[self.layer_id], positions,
+                                     quantized=True)
         out = self._attend_cache(q, kv_cache, key_mask)
-        return out.permute(0, 2, 1, 3).reshape(b, s, self.dim)
+        return I.quantize_int8_per_token(out.permute(0, 2, 1, 3).reshape(b, s, self.dim))
 
 
 class MLP(nn.Module):
@@ -225,23 +229,30 @@ class DecoderBlock(nn.Module):
 
     def forward(self, x, rotary_emb, kv_cache, positions, key_mask):
         if self.fused_int8 is not None and _fused_int8_active(x):
-            return self._forward_fused_int8(x, rotary_emb, kv_cache, positions, key_mask)
+            h, out = self._forward_fused_int8(x, None, rotary_emb, kv_cache, positions, key_mask)
+            return h + out
         x = self.attention(self.input_norm(x), rotary_emb, kv_cache, positions, key_mask) + x
         return self.mlp(self.post_attention_norm(x)) + x
 
-    def _forward_fused_int8(self, x, rotary_emb, kv_cache, positions, key_mask):
+    def _forward_fused_int8(self, x, pending, rotary_emb, kv_cache, positions, key_mask):
+        """``x`` plus the not yet added residual branch ``pending`` (``None`` for the first
+        block) is the block input; returns ``(h, mlp_out)`` whose sum is the block output -- the
+        add is left to the next norm kernel, which also has to read both."""
         from astrai_amd.extension.ops import int8 as I
         f, att = self.fused_int8, self.attention
         b, s, d = x.shape
-        xq, sx, _ = I.rmsnorm_quantize_int8(x, self.input_norm.weight, self.input_norm.norm_eps)
+        xq, sx, xsum = I.rmsnorm_quantize_int8(x, self.input_norm.weight, self.input_norm.norm_eps,
+                                               res=pending)
+        if xsum is not None:
+            x = xsum
         qkv = I.mm_int8(xq, f.wqkv, sx, f.sqkv).reshape(b, s, -1)
-        nq, nkv = att.n_heads * att.head_dim, att.n_kv_heads * att.head_dim
         if kv_cache is not None:
-            a = att.core_fused_qkv(qkv, rotary_emb, kv_cache, positions, key_mask)
+            aq, sa = att.core_fused_qkv(qkv, rotary_emb, kv_cache, positions, key_mask)
         else:
-            a = att.core(qkv[..., :nq], qkv[..., nq:nq + nkv], qkv[..., nq + nkv:], rotary_emb, None,
-                         positions, key_mask)
-        aq, sa = I.quantize_int8_per_token(a)
+            nq, nkv = att.n_heads * att.head_dim, att.n_kv_heads * att.head_dim
+            aq, sa = I.quantize_int8_per_token(
+                att.core(qkv[..., :nq], qkv[..., nq:nq + nkv], qkv[..., nq + nkv:], rotary_emb, None,
+                         positions, key_mask))
         o = I.mm_int8(aq, f.wo, sa, f.so).reshape(b, s, d)
         # h = attention + x, then its norm, quantized: one kernel
         hq, sh, h = I.rmsnorm_quantize_int8(o, self.post_attention_norm.weight,
@@ -249,7 +260,7 @@ class DecoderBlock(nn.Module):
         gu = I.mm_int8(hq, f.wgu, sh, f.sgu)                 # [B*S, gate | up]
         w = f.wgu.size(0) // 2
         mq, sm = I.silu_mul_quantize_int8(gu[:, :w], gu[:, w:])
-        return I.mm_int8(mq, f.wdown, sm, f.sdown).reshape(b, s, d) + h
+        return h, I.mm_int8(mq, f.wdown, sm, f.sdown).reshape(b, s, d)
 
 
 class AutoRegressiveLM(nn.Module):
@@ -290,15 +301,18 @@ class AutoRegressiveLM(nn.Module):
             n_rep = self.config.num_attention_heads // self.config.num_key_value_heads
             if n_rep > 1:  # one copy per query head of a KV group, made once for all layers
                 key_mask = key_mask.repeat(1, 1, n_rep, 1)
-        for layer in self.layers:
-            x = layer(x, rotary, kv_cache, positions, key_mask)
         if self.fused_int8 is not None and _fused_int8_active(x):
             from astrai_amd.extension import _cabi
             from astrai_amd.extension.ops import int8 as I
+            pending = None  # residual branch not yet added to x: the next norm kernel adds it
+            for layer in self.layers:
+                x, pending = layer._forward_fused_int8(x, pending, rotary, kv_cache, positions, key_mask)
             hq, sh, _, hidden = _cabi.add_rmsnorm_quantize_int8(x, self.norm.weight, self.norm.norm_eps,
-                                                                None, True)
+                                                                pending, True)
             logits = I.mm_int8(hq, self.fused_int8.wlm, sh, self.fused_int8.slm).reshape(b, s, -1)
             return {"logits": logits, "hidden_states": hidden}
+        for layer in self.layers:
+            x = layer(x, rotary, kv_cache, positions, key_mask)
         hidden = self.norm(x)
         return {"logits": self.lm_head(hidden), "hidden_states": hidden}
 

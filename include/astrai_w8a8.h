@@ -140,16 +140,20 @@ int astrai_w8a8_rope_cache_write_bf16(const void* qkv_bf16, int64_t ld, const fl
  *   positions  int64 [seq] (device): token s attends keys 0..positions[s]
  *   workspace  fp32, at least astrai_w8a8_attn_decode_workspace_floats(batch,
  *              n_kv_heads, nsplit, (n_heads / n_kv_heads) * seq) floats (caller-owned scratch)
- *   out        bf16 [batch, seq, n_heads * 128]
+ *   out        bf16 [batch, seq, n_heads * 128], or NULL
+ *   out_q, out_scale  int8 [batch*seq, n_heads * 128] and fp32 [batch*seq]: the per-token int8
+ *              quantization of the bf16-rounded output rows (quantize_bf16_int8_rows applied to
+ *              `out`), or NULL; at least one of out / out_q must be given
  *   nsplit     number of context splits (1..64): batch * n_kv_heads * nsplit workgroups
  * fp32 scores and softmax, fp32 accumulation of p*v, one rounding to bf16.
- * head_dim == 128 and (n_heads / n_kv_heads) * seq <= 8.
+ * head_dim == 128, (n_heads / n_kv_heads) * seq <= 8, n_heads <= 64.
  */
 int64_t astrai_w8a8_attn_decode_workspace_floats(int64_t batch, int64_t n_kv_heads, int64_t nsplit,
                                                  int64_t n_query_rows);
 int astrai_w8a8_attn_decode_bf16(const void* q_bf16, const void* k_cache_bf16, const void* v_cache_bf16,
                                  const int64_t* positions, float* workspace, int64_t workspace_floats,
-                                 void* out_bf16, int64_t batch, int64_t seq, int64_t n_heads,
+                                 void* out_bf16, void* out_q, float* out_scale, int64_t batch,
+                                 int64_t seq, int64_t n_heads,
                                  int64_t n_kv_heads, int64_t head_dim, int64_t max_len,
                                  int64_t nsplit, float scale, void* stream);
 

@@ -77,3 +77,18 @@ def test_attn_decode_rejects_unsupported():
     kc = torch.zeros(1, 4, 8, 128, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(RuntimeError, match="<= 8"):
         _cabi.attn_decode(q, kc, kc.clone(), torch.zeros(3, dtype=torch.long, device=DEV))
+
+
+def test_quantized_output_is_the_quantizer_applied_to_the_bf16_output():
+    from astrai_amd.extension import _cabi
+    from oracle import w8a8_oracle as O
+    g = torch.Generator().manual_seed(9)
+    b, h, hkv, s, max_len, d = 4, 16, 4, 2, 80, 128
+    q = torch.randn(b, h, s, d, generator=g).to(torch.bfloat16).to(DEV)
+    kc = torch.randn(b, hkv, max_len, d, generator=g).to(torch.bfloat16).to(DEV)
+    vc = torch.randn(b, hkv, max_len, d, generator=g).to(torch.bfloat16).to(DEV)
+    pos = torch.tensor([70, 71], device=DEV)
+    out = _cabi.attn_decode(q, kc, vc, pos, nsplit=4)
+    oq, os_ = _cabi.attn_decode(q, kc, vc, pos, nsplit=4, quantized=True)
+    wq, ws = O.int8_quantize_rows(out.cpu().reshape(b * s, h * d))
+    assert torch.equal(oq.cpu(), wq) and torch.equal(os_.cpu(), ws)
