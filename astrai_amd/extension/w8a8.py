@@ -37,6 +37,13 @@ class Int8State:
         self._weights[key] = (w._version, wq, sw)
         return wq, sw
 
+    def put_weight(self, w: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor) -> None:
+        """Install an already quantized form of ``w`` (e.g. from an int8 checkpoint)."""
+        if wq.shape != w.shape or wq.dtype != torch.int8 or sw.numel() != w.size(0):
+            raise ValueError("wq must be int8 of w's shape and sw one step per output channel")
+        self._weights[(w.data_ptr(), w.shape, w.dtype)] = (
+            w._version, wq.contiguous(), sw.reshape(-1).float().contiguous())
+
     def reset(self) -> None:
         self.enabled = False
         self._weights.clear()

@@ -11,5 +11,7 @@ from astrai_amd.model.decoder import (
     unfuse_int8_weights,
 )
 
-__all__ = ["AutoRegressiveLM", "AutoRegressiveLMConfig", "DenseKVCache", "greedy_generate",
+from astrai_amd.model.checkpoint import load_int8_checkpoint, save_int8_checkpoint
+
+__all__ = ["load_int8_checkpoint", "save_int8_checkpoint", "AutoRegressiveLM", "AutoRegressiveLMConfig", "DenseKVCache", "greedy_generate",
            "fuse_int8_weights", "unfuse_int8_weights"]

@@ -324,15 +324,19 @@ def _fused_int8_active(x: Tensor) -> bool:
 
 @torch.no_grad()
 def fuse_int8_weights(model: AutoRegressiveLM) -> int:
-    """Quantize every projection per output channel (the per-row quantizer on the
-    weight, as ``w8a8.prepare_int8_weights`` does) and store q|k|v and gate|up as one
+    """Quantize every projection per output channel (through the int8 policy's weight
+    cache, as ``w8a8.prepare_int8_weights`` does) and store q|k|v and gate|up as one
     int8 matrix each on the block. While ``w8a8.int8_autocast`` is on, blocks then take
     the fused path. Returns the number of int8 matrices held. Call again after
     changing weights."""
-    from astrai_amd.extension.ops.int8 import quantize_int8_per_channel as qpc
+    from astrai_amd.extension import w8a8
+
+    state = w8a8.int8_state()
 
     def cat(*linears):
-        parts = [qpc(l.weight.detach()) for l in linears]
+        # the policy cache quantizes on first use and returns what it holds otherwise
+        # (e.g. the integers an int8 checkpoint installed)
+        parts = [state.get_weight(l.weight) for l in linears]
         return torch.cat([p[0] for p in parts]).contiguous(), torch.cat([p[1] for p in parts]).contiguous()
 
     n = 0

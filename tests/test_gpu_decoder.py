@@ -102,3 +102,31 @@ def test_fused_int8_path_matches_modular_path_and_oracle():
     assert (inc - lf).abs().max().item() <= 0.03 * scale
     assert torch.equal(eager, graph)
     assert (eager == eager_modular).float().mean().item() >= 0.9
+
+
+def test_int8_checkpoint_round_trip(tmp_path):
+    """Saved integers and steps come back unchanged, no quantization pass at load, and
+    the loaded model produces the logits of the model it was saved from."""
+    import json
+    import safetensors.torch as st
+    from astrai_amd.extension import w8a8
+    from astrai_amd.model import fuse_int8_weights, load_int8_checkpoint, save_int8_checkpoint
+    cfg, model = _model(8, vocab_size=256, hidden_size=128, num_hidden_layers=2, num_attention_heads=2,
+                        num_key_value_heads=1, intermediate_size=256, max_position_embeddings=32)
+    gm = model.to(DEV)
+    ids = torch.randint(0, cfg.vocab_size, (2, 9), generator=torch.Generator().manual_seed(8)).to(DEV)
+    w8a8.int8_state().reset()
+    fuse_int8_weights(gm)
+    with torch.no_grad(), w8a8.int8_autocast(True):
+        want = gm(ids)["logits"]
+    save_int8_checkpoint(gm, str(tmp_path))
+    names = set(st.load_file(str(tmp_path / "model.safetensors")))
+    assert "layers.0.attention.q_proj.weight_int8" in names and "layers.0.attention.q_proj.weight_scale" in names
+    assert "layers.0.attention.q_proj.weight" not in names and "embed_tokens.weight" in names
+    assert json.loads((tmp_path / "meta.json").read_text())["quantization"]["scheme"] == "int8_w8a8_per_channel"
+    w8a8.int8_state().reset()
+    loaded = load_int8_checkpoint(str(tmp_path), DEV)
+    with torch.no_grad(), w8a8.int8_autocast(True):
+        got = loaded(ids)["logits"]
+    w8a8.int8_state().reset()
+    assert torch.equal(got, want)
