@@ -83,6 +83,46 @@ int astrai_w8a8_quantize_bf16_fp8(const void* x, void* x8, const float* scale, f
     return check_launch("quantize_bf16_fp8");
 }
 
+int astrai_w8a8_amax_bf16(const void* x, float* amax, int64_t total, void* stream) {
+    if (!x || !amax) return fail(ASTRAI_W8A8_BAD_ARG, "amax_bf16: null pointer");
+    if (total < 0) return fail(ASTRAI_W8A8_BAD_ARG, "amax_bf16: negative size");
+    if (!aligned16(x)) return fail(ASTRAI_W8A8_BAD_ARG, "amax_bf16: x must be 16-byte aligned");
+    if (total == 0) return ASTRAI_W8A8_OK;
+    w8a8::launch_amax_bf16(x, amax, total, static_cast<hipStream_t>(stream));
+    return check_launch("amax_bf16");
+}
+
+int astrai_w8a8_amax_ring_push(float* hist, int n, int idx, const float* amax, float* scale,
+                               float fmax, float pow2_margin, void* stream) {
+    if (!hist || !amax || !scale) return fail(ASTRAI_W8A8_BAD_ARG, "amax_ring_push: null pointer");
+    if (n <= 0 || idx < 0 || idx >= n)
+        return fail(ASTRAI_W8A8_BAD_ARG, "amax_ring_push: idx must lie in [0, n)");
+    if (!(fmax > 0.0f) || !(pow2_margin > 0.0f))
+        return fail(ASTRAI_W8A8_BAD_ARG, "amax_ring_push: fmax and pow2_margin must be positive");
+    w8a8::launch_amax_ring_push(hist, n, idx, amax, scale, fmax, pow2_margin,
+                                static_cast<hipStream_t>(stream));
+    return check_launch("amax_ring_push");
+}
+
+int astrai_w8a8_quantize_transpose_bf16_fp8(const void* x, void* x8, void* x8t, const float* scale,
+                                            float* amax, int64_t rows, int64_t cols, int fmt,
+                                            void* stream) {
+    if (!x || !x8t || !scale)
+        return fail(ASTRAI_W8A8_BAD_ARG, "quantize_transpose_bf16_fp8: null pointer");
+    if (rows < 0 || cols < 0 || rows > (int64_t)65535 * 128 || cols > ((int64_t)1 << 31) - 64)
+        return fail(ASTRAI_W8A8_BAD_ARG, "quantize_transpose_bf16_fp8: bad dims");
+    if (fmt != ASTRAI_W8A8_E4M3 && fmt != ASTRAI_W8A8_E5M2)
+        return fail(ASTRAI_W8A8_BAD_ARG,
+                    "quantize_transpose_bf16_fp8: fmt must be 0 (e4m3) or 1 (e5m2)");
+    if (!aligned16(x) || !aligned16(x8t) || (x8 && !aligned16(x8)))
+        return fail(ASTRAI_W8A8_BAD_ARG,
+                    "quantize_transpose_bf16_fp8: pointers must be 16-byte aligned");
+    if (rows == 0 || cols == 0) return ASTRAI_W8A8_OK;
+    w8a8::launch_quantize_transpose_fp8(x, x8, x8t, scale, amax, rows, cols, fmt,
+                                        static_cast<hipStream_t>(stream));
+    return check_launch("quantize_transpose_bf16_fp8");
+}
+
 int astrai_w8a8_quantize_bf16_int8_rows(const void* x, void* xq, float* s, int64_t rows,
                                         int64_t k, void* stream) {
     if (!x || !xq || !s) return fail(ASTRAI_W8A8_BAD_ARG, "quantize_bf16_int8_rows: null pointer");

@@ -118,8 +118,14 @@ __device__ __forceinline__ int wave_sum_i32(int v) {
 }
 
 // max into a non-negative float slot through its bit pattern
+// (non-negative floats order like their bits). Device-scope atomics on one address
+// are served one at a time, about 10 ns each, so a workgroup first looks at the slot
+// and leaves it alone when its own maximum cannot raise it: thousands of workgroups
+// would otherwise queue for tens of microseconds behind one another.
 __device__ __forceinline__ void atomic_max_nonneg(float* dst, float v) {
-    atomicMax(reinterpret_cast<unsigned int*>(dst), __float_as_uint(v));
+    unsigned int* p = reinterpret_cast<unsigned int*>(dst);
+    const unsigned int bits = __float_as_uint(v);
+    if (__hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < bits) atomicMax(p, bits);
 }
 
 }  // namespace w8a8

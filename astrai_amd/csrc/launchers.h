@@ -26,6 +26,15 @@ struct GemmArgs {
 // quantize.hip
 void launch_quantize_fp8(const void* x, void* x8, const float* scale, float* amax,
                          int64_t total, int fmt, hipStream_t stream);
+// hist[idx] = *amax; *scale = max((max(hist) / fmax) / pow2_margin, 1e-12)
+void launch_amax_ring_push(float* hist, int n, int idx, const float* amax, float* scale,
+                           float fmax, float pow2_margin, hipStream_t stream);
+// *amax = max(*amax, max |x|)
+void launch_amax_bf16(const void* x, float* amax, int64_t total, hipStream_t stream);
+// codes of a [rows, cols] matrix row-major (x8, may be null) and transposed (x8t, [cols, rows])
+void launch_quantize_transpose_fp8(const void* x, void* x8, void* x8t, const float* scale,
+                                   float* amax, int64_t rows, int64_t cols, int fmt,
+                                   hipStream_t stream);
 void launch_quantize_int8_rows(const void* x, void* xq, float* s, int64_t rows, int64_t k,
                                hipStream_t stream);
 // fused producers: (residual add +) RMSNorm + per-row int8; SwiGLU product + per-row

@@ -99,6 +99,137 @@ __global__ __launch_bounds__(kThreads) void quantize_fp8_kernel(
     }
 }
 
+// ---- max |x| alone ---------------------------------------------------------
+// Dynamic scaling measures a tensor before it quantizes it
+// (astrai/extension/fp8.py:289-292: t.abs().amax()); this is that reduction as one
+// read of the tensor, without the intermediate |x| tensor.
+__global__ __launch_bounds__(kThreads) void amax_bf16_kernel(
+    const uint16_t* __restrict__ x, float* __restrict__ amax, int64_t total) {
+    __shared__ float slots[kThreads / kWave];
+    float local = 0.0f;
+    const int64_t nvec = total >> 3;
+    const int64_t stride = (int64_t)gridDim.x * kThreads;
+    for (int64_t v = (int64_t)blockIdx.x * kThreads + threadIdx.x; v < nvec; v += stride) {
+        float f[8];
+        unpack8(*reinterpret_cast<const u32x4*>(x + v * 8), f);
+        local = fmaxf(local, amax8(f));
+    }
+    if (blockIdx.x == 0) {
+        const int64_t i = nvec * 8 + threadIdx.x;
+        if (i < total) local = fmaxf(local, fabsf(bf16_to_f32(x[i])));
+    }
+    const float m = block_max(local, slots);
+    if (threadIdx.x == 0) atomic_max_nonneg(amax, m);
+}
+
+// ---- delayed scaling: record one amax, refresh the step -------------------
+// hist[idx] = amax; *scale = max((max(hist) / fmax) / pow2_margin, 1e-12), the
+// record-then-refresh of FP8TensorMeta (astrai/extension/fp8.py:147-173, formula
+// :87-89) as one single-wave launch instead of six tiny ones.
+// (amax may be the ring's own slot: dynamic scaling is a ring of length one)
+__global__ __launch_bounds__(kWave) void amax_ring_push_kernel(
+    float* hist, int n, int idx, const float* amax, float* scale, float fmax, float pow2_margin) {
+    const float fresh = *amax;
+    float peak = 0.0f;
+    for (int i = threadIdx.x; i < n; i += kWave) {
+        float h = hist[i];
+        if (i == idx) hist[i] = h = fresh;
+        peak = fmaxf(peak, h);
+    }
+    peak = wave_max(peak);
+    if (threadIdx.x == 0) *scale = fmaxf((peak / fmax) / pow2_margin, 1e-12f);
+}
+
+// ---- per-tensor fp8, row-major and transposed codes in one pass -----------
+// The backward of a Linear contracts the gradient over both of its axes
+// (dX = g.w over N, dW = g^T.x over M; csrc/kernels/fp8/mm.cu:298-312 makes
+// transposed-contiguous copies first). Here one read of a [R,C] bf16 matrix
+// yields its codes row-major (optional) and transposed [C,R]. Tile 128 x 128:
+// 256-byte runs in, 128-byte runs out in both layouts. A thread converts 4 rows
+// x 8 columns per pass, packs the four rows of each column into a dword and
+// writes it to a column-major LDS tile (pitch 132 bytes); the tile then leaves
+// as 16-byte pieces of the transposed rows.
+constexpr int kTrRows = 128, kTrCols = 128, kTrPitch = kTrRows + 4;
+
+template <int Fmt>
+__global__ __launch_bounds__(kThreads) void quantize_transpose_fp8_kernel(
+    const uint16_t* __restrict__ x, uint8_t* __restrict__ x8, uint8_t* __restrict__ x8t,
+    const float* __restrict__ scale, float* __restrict__ amax, int64_t rows, int64_t cols) {
+    __shared__ __attribute__((aligned(16))) uint8_t tile[kTrCols * kTrPitch];
+    __shared__ float slots[kThreads / kWave];
+    const int64_t r0 = (int64_t)blockIdx.y * kTrRows, c0 = (int64_t)blockIdx.x * kTrCols;
+    const int cc = threadIdx.x & 15, r4 = threadIdx.x >> 4;
+    const float step = *scale;
+    const bool vec = (cols & 7) == 0;
+    const int64_t c = c0 + cc * 8;
+    float local = 0.0f;
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        u32x2 q[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int64_t r = r0 + pass * 64 + r4 * 4 + i;
+            float f[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+            const bool whole = vec && r < rows && c < cols;
+            if (whole) {
+                unpack8(*reinterpret_cast<const u32x4*>(x + r * cols + c), f);
+            } else if (r < rows) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (c + j < cols) f[j] = bf16_to_f32(x[r * cols + c + j]);
+            }
+            local = fmaxf(local, amax8(f));
+            q[i] = quant8_fp8<Fmt>(f, step);
+            if (x8) {
+                if (whole) {
+                    *reinterpret_cast<u32x2*>(x8 + r * cols + c) = q[i];
+                } else if (r < rows) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (c + j < cols)
+                            x8[r * cols + c + j] =
+                                (uint8_t)(((j < 4 ? q[i].x : q[i].y) >> ((j & 3) * 8)) & 0xffu);
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            uint32_t d = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                d |= (((j < 4 ? q[i].x : q[i].y) >> ((j & 3) * 8)) & 0xffu) << (8 * i);
+            *reinterpret_cast<uint32_t*>(tile + (cc * 8 + j) * kTrPitch + pass * 64 + r4 * 4) = d;
+        }
+    }
+    __syncthreads();
+    const bool runs = (rows & 15) == 0;  // 16-byte pieces stay aligned and inside the matrix
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+        const int cl = (threadIdx.x >> 3) + 32 * h;
+        const int64_t ct = c0 + cl, rt = r0 + (threadIdx.x & 7) * 16;
+        if (ct >= cols || rt >= rows) continue;
+        const uint8_t* src = tile + cl * kTrPitch + (threadIdx.x & 7) * 16;
+        u32x4 v;
+        v.x = *reinterpret_cast<const uint32_t*>(src);
+        v.y = *reinterpret_cast<const uint32_t*>(src + 4);
+        v.z = *reinterpret_cast<const uint32_t*>(src + 8);
+        v.w = *reinterpret_cast<const uint32_t*>(src + 12);
+        if (runs) {
+            *reinterpret_cast<u32x4*>(x8t + ct * rows + rt) = v;
+        } else {
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int b = 0; b < 16; ++b)
+                if (rt + b < rows)
+                    x8t[ct * rows + rt + b] = (uint8_t)((w[b >> 2] >> ((b & 3) * 8)) & 0xffu);
+        }
+    }
+    if (amax) {
+        const float m = block_max(local, slots);
+        if (threadIdx.x == 0) atomic_max_nonneg(amax, m);
+    }
+}
+
 // ---- per-row int8 ---------------------------------------------------------
 // One workgroup per row; up to kCache 16-byte vectors per thread stay in
 // registers between the amax pass and the quantize pass (K <= 8192), longer
@@ -347,6 +478,34 @@ void launch_quantize_fp8(const void* x, void* x8, const float* scale, float* ama
     else
         quantize_fp8_kernel<0><<<dim3((unsigned)blocks), dim3(kThreads), 0, stream>>>(
             xs, xo, scale, amax, total);
+}
+
+void launch_amax_ring_push(float* hist, int n, int idx, const float* amax, float* scale,
+                           float fmax, float pow2_margin, hipStream_t stream) {
+    amax_ring_push_kernel<<<dim3(1), dim3(kWave), 0, stream>>>(hist, n, idx, amax, scale, fmax,
+                                                               pow2_margin);
+}
+
+void launch_amax_bf16(const void* x, float* amax, int64_t total, hipStream_t stream) {
+    if (total <= 0) return;
+    int64_t blocks = ((total + 7) / 8 + kThreads - 1) / kThreads;
+    if (blocks > 256 * 8) blocks = 256 * 8;
+    amax_bf16_kernel<<<dim3((unsigned)blocks), dim3(kThreads), 0, stream>>>(
+        static_cast<const uint16_t*>(x), amax, total);
+}
+
+void launch_quantize_transpose_fp8(const void* x, void* x8, void* x8t, const float* scale,
+                                   float* amax, int64_t rows, int64_t cols, int fmt,
+                                   hipStream_t stream) {
+    if (rows <= 0 || cols <= 0) return;
+    const dim3 grid((unsigned)((cols + kTrCols - 1) / kTrCols), (unsigned)((rows + kTrRows - 1) / kTrRows));
+    auto* xi = static_cast<const uint16_t*>(x);
+    auto* o = static_cast<uint8_t*>(x8);
+    auto* ot = static_cast<uint8_t*>(x8t);
+    if (fmt == 0)
+        quantize_transpose_fp8_kernel<0><<<grid, dim3(kThreads), 0, stream>>>(xi, o, ot, scale, amax, rows, cols);
+    else
+        quantize_transpose_fp8_kernel<1><<<grid, dim3(kThreads), 0, stream>>>(xi, o, ot, scale, amax, rows, cols);
 }
 
 void launch_quantize_int8_rows(const void* x, void* xq, float* s, int64_t rows, int64_t k,

@@ -26,12 +26,16 @@ OUT_BF16, OUT_E4M3, OUT_ACC = 0, 1, 2
 _P = ctypes.c_void_p
 _I64 = ctypes.c_int64
 _INT = ctypes.c_int
+_F32 = ctypes.c_float
 
 # name -> argtypes, exactly the prototypes of include/astrai_w8a8.h
 PROTOTYPES = {
     "astrai_w8a8_abi_version": ([], _INT),
     "astrai_w8a8_last_error": ([], ctypes.c_char_p),
     "astrai_w8a8_quantize_bf16_fp8": ([_P, _P, _P, _P, _I64, _INT, _P], _INT),
+    "astrai_w8a8_amax_bf16": ([_P, _P, _I64, _P], _INT),
+    "astrai_w8a8_amax_ring_push": ([_P, _INT, _INT, _P, _P, _F32, _F32, _P], _INT),
+    "astrai_w8a8_quantize_transpose_bf16_fp8": ([_P, _P, _P, _P, _P, _I64, _I64, _INT, _P], _INT),
     "astrai_w8a8_quantize_bf16_int8_rows": ([_P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_add_rmsnorm_quantize_int8_rows": (
         [_P, _P, _P, ctypes.c_float, _P, _P, _P, _P, _I64, _I64, _P], _INT),
@@ -262,10 +266,85 @@ def fp8_mm(a: torch.Tensor, b: torch.Tensor, sx: torch.Tensor, sw: torch.Tensor)
     return out
 
 
+def amax_bf16(x: torch.Tensor) -> torch.Tensor:
+    """``x.abs().amax()`` of a bf16 tensor as fp32 ``[1]`` from one read of ``x``
+    (the measurement of dynamic scaling, astrai/extension/fp8.py:289-292)."""
+    lib = _require()
+    _gpu(x, "amax_bf16")
+    if x.dtype != torch.bfloat16:
+        raise RuntimeError("x must be bf16")
+    x_c = x.contiguous()
+    with torch.cuda.device(x.device):
+        amax = torch.zeros(1, device=x.device, dtype=torch.float32)
+        if x_c.numel():
+            _check(lib.astrai_w8a8_amax_bf16(x_c.data_ptr(), amax.data_ptr(), x_c.numel(),
+                                            _stream(x)), lib)
+    return amax
+
+
+def amax_ring_push(hist: torch.Tensor, idx: int, amax: torch.Tensor, scale: torch.Tensor,
+                   fmax: float, pow2_margin: float) -> None:
+    """In place: ``hist[idx] = amax; scale = max((hist.max() / fmax) / pow2_margin, 1e-12)``
+    (FP8TensorMeta's record-then-refresh, astrai/extension/fp8.py:147-173)."""
+    lib = _require()
+    _gpu(hist, "amax_ring_push")
+    for t, name in ((hist, "hist"), (amax, "amax"), (scale, "scale")):
+        if not (t.is_cuda and t.device == hist.device and t.dtype == torch.float32
+                and t.is_contiguous()):
+            raise RuntimeError(f"{name} must be a contiguous float32 tensor on the ring's device")
+    if amax.numel() != 1 or scale.numel() != 1:
+        raise RuntimeError("amax and scale must have one element")
+    with torch.cuda.device(hist.device):
+        _check(lib.astrai_w8a8_amax_ring_push(hist.data_ptr(), hist.numel(), int(idx),
+                                             amax.data_ptr(), scale.data_ptr(), float(fmax),
+                                             float(pow2_margin), _stream(hist)), lib)
+
+
+def quantize_transpose_bf16(x: torch.Tensor, scale: torch.Tensor, fmt: int,
+                            want_rowmajor: bool = False, want_amax: bool = False):
+    """One pass over a bf16 ``[R, C]`` matrix -> ``(x8 [R,C] or None, x8t [C,R], amax [1])``:
+    the codes ``quantize_bf16`` gives for ``x`` and for ``x.t().contiguous()``
+    (mm.cu:276-312 makes that copy first). ``amax`` stays zero unless asked for."""
+    lib = _require()
+    _gpu(x, "quantize_transpose_bf16")
+    if x.dtype != torch.bfloat16 or x.dim() != 2:
+        raise RuntimeError("x must be a 2D bf16 tensor")
+    _check_scale(scale, x, "scale")
+    x_c = x.contiguous()
+    rows, cols = x_c.shape
+    f8 = torch.float8_e5m2 if fmt else torch.float8_e4m3fn
+    with torch.cuda.device(x.device):
+        x8 = torch.empty((rows, cols), device=x.device, dtype=f8) if want_rowmajor else None
+        x8t = torch.empty((cols, rows), device=x.device, dtype=f8)
+        amax = torch.zeros(1, device=x.device, dtype=torch.float32)
+        if rows and cols:
+            _check(lib.astrai_w8a8_quantize_transpose_bf16_fp8(
+                x_c.data_ptr(), _ptr(x8), x8t.data_ptr(), scale.data_ptr(),
+                amax.data_ptr() if want_amax else None, rows, cols, 1 if fmt else 0,
+                _stream(x)), lib)
+    return x8, x8t, amax
+
+
+def _mm_fp8_into(out: torch.Tensor, a8: torch.Tensor, b8: torch.Tensor, sa, sb, lib):
+    m, k = a8.shape
+    n = b8.size(0)
+    if not (m and n):
+        return
+    if k == 0:
+        out.zero_()
+        return
+    _check(lib.astrai_w8a8_gemm_fp8_pt(
+        a8.data_ptr(), b8.data_ptr(), sa.data_ptr(), sb.data_ptr(), None, None, out.data_ptr(),
+        m, n, k, 1 if a8.dtype == torch.float8_e5m2 else 0, 0, _stream(a8)), lib)
+
+
 def linear_backward_fp8(g, x, w, masks, sg, sw, sx, fmt: int):
     """FP8 linear backward ``(grad_input, grad_weight, grad_bias, amax_g)``.
-    mm.cu:236-320: the gradient is quantized once, ``dX = g8 @ w8`` and
-    ``dW = g8^T @ x8`` run as NT GEMMs on transposed-contiguous copies."""
+    mm.cu:236-320: ``dX = g8 @ w8`` and ``dW = g8^T @ x8`` as NT GEMMs. The
+    reference copies g, w and x transposed and quantizes each copy; here one
+    kernel per tensor reads it once and writes the codes in the layouts the two
+    GEMMs contract over (g in both), and the GEMMs write the gradients in place."""
+    lib = _require()
     _gpu(g, "linear_backward_fp8")
     if not (g.dtype == x.dtype == w.dtype == torch.bfloat16):
         raise RuntimeError("g, x, and w must be bf16")
@@ -280,22 +359,32 @@ def linear_backward_fp8(g, x, w, masks, sg, sw, sx, fmt: int):
     m = g_c.size(0)
     if x_c.size(0) != m or x_c.size(1) != k:
         raise RuntimeError("backward shape mismatch")
-    grad_input = torch.empty_like(x)
-    grad_weight = torch.empty_like(w)
-    grad_bias = torch.empty(0, device=g.device, dtype=g.dtype)
-    amax_g = torch.zeros(1, device=g.device, dtype=torch.float32)
-    if masks[0]:
-        g8, amax_g = quantize_bf16(g_c, sg, fmt)
-        w8_t, _ = quantize_bf16(w.t().contiguous(), sw, fmt)  # [K, N]
-        grad_input.copy_(mm_fp8(g8, w8_t, sg, sw).reshape(x.shape))
-    if masks[1]:
-        g8_t, _ = quantize_bf16(g_c.t().contiguous(), sg, fmt)  # [N, M]
-        x8_t, _ = quantize_bf16(x_c.t().contiguous(), sx, fmt)  # [K, M]
-        grad_weight.copy_(mm_fp8(g8_t, x8_t, sg, sx))
-    if not masks[0] and not masks[1]:
-        amax_g = g_c.abs().amax().to(torch.float32).reshape(1)
-    if masks[2]:
-        grad_bias = g_c.sum(0).to(g.dtype)
+    for t, name in ((sg, "sg"), (sw, "sw"), (sx, "sx")):
+        _check_scale(t, g, name)
+    with torch.cuda.device(g.device):
+        grad_input = torch.empty(x.shape, device=x.device, dtype=x.dtype)
+        grad_weight = torch.empty((n, k), device=w.device, dtype=w.dtype)
+        grad_bias = torch.empty(0, device=g.device, dtype=g.dtype)
+        amax_g = torch.zeros(1, device=g.device, dtype=torch.float32)
+        g8 = g8_t = None
+        if masks[1]:
+            # amax_g is measured only on the dX branch (mm.cu:293-296)
+            g8, g8_t, amax = quantize_transpose_bf16(g_c, sg, fmt, want_rowmajor=bool(masks[0]),
+                                                     want_amax=bool(masks[0]))
+            if masks[0]:
+                amax_g = amax
+        elif masks[0]:
+            g8, amax_g = quantize_bf16(g_c, sg, fmt)
+        if masks[0]:
+            _, w8_t, _ = quantize_transpose_bf16(w, sw, fmt)  # [K, N]
+            _mm_fp8_into(grad_input, g8, w8_t, sg, sw, lib)
+        if masks[1]:
+            _, x8_t, _ = quantize_transpose_bf16(x_c, sx, fmt)  # [K, M]
+            _mm_fp8_into(grad_weight, g8_t, x8_t, sg, sx, lib)
+        if not masks[0] and not masks[1]:
+            amax_g = g_c.abs().amax().to(torch.float32).reshape(1)
+        if masks[2]:
+            grad_bias = g_c.sum(0).to(g.dtype)
     return grad_input, grad_weight, grad_bias, amax_g
 
 

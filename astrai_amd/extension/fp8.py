@@ -27,9 +27,12 @@ import torch
 
 from astrai_amd.extension import dispatch
 from astrai_amd.extension.ops.fp8 import (
+    amax_bf16,
+    amax_ring_push,
     linear_backward_fp8,
     linear_forward_fp8,
     mm_fp8,
+    mm_fp8_bias,
     quantize_bf16,
 )
 
@@ -101,6 +104,13 @@ class _AmaxRing:
 
     def push(self, amax: torch.Tensor, recipe: FP8Recipe, fmt: str) -> None:
         # record first, then refresh: the step used next reflects amax seen so far
+        if self.hist.is_cuda and type(recipe) in (DelayedScaling, DynamicScaling) \
+                and amax.is_cuda and amax.dtype == torch.float32 and amax.is_contiguous():
+            # both stock recipes take the window's maximum: one launch does the lot
+            amax_ring_push(self.hist, self.idx, amax, self.scale, FP8_MAX[fmt],
+                           float(2 ** recipe.margin))
+            self.idx = (self.idx + 1) % self.hist.numel()
+            return
         self.hist[self.idx] = amax.reshape(())
         self.idx = (self.idx + 1) % self.hist.numel()
         self.scale.copy_(recipe.scale_from_history(self.hist, fmt))
@@ -132,6 +142,10 @@ class FP8TensorMeta:
         self._w = _AmaxRing(device, n)
         self._x = _AmaxRing(device, n)
         self._g = _AmaxRing(device, n)
+        # host-side bookkeeping of FP8State.cache_weights
+        self.w_version = -1   # weight._version at the last push into the weight ring
+        self.w_repeats = 0    # consecutive pushes made from that same version
+        self.w_cached = None  # (version, w8, amax_w) quantized with the settled step
 
     w_hist, w_idx = _ring_property("_w", "hist"), _ring_property("_w", "idx")
     w_scale, w_init = _ring_property("_w", "scale"), _ring_property("_w", "seeded")
@@ -151,6 +165,19 @@ class FP8TensorMeta:
 
     def init_w(self, w: torch.Tensor, fmt: str) -> None:
         self._w.seed(w, self.recipe, fmt)
+        self.w_version, self.w_repeats = w._version, self.recipe.history_len
+
+    def w_settled(self, w: torch.Tensor) -> bool:
+        """True when every slot of the weight ring holds the amax of ``w`` as it is
+        now, so that one more push would change neither the ring nor the step."""
+        return self.w_version == w._version and self.w_repeats >= self.recipe.history_len
+
+    def note_w_push(self, w: torch.Tensor) -> None:
+        self.w_cached = None  # the step may have moved with this push
+        if self.w_version == w._version:
+            self.w_repeats += 1
+        else:
+            self.w_version, self.w_repeats = w._version, 1
 
     def init_x(self, x: torch.Tensor, fmt: str) -> None:
         self._x.seed(x, self.recipe, fmt)
@@ -169,6 +196,13 @@ class FP8State:
         self.fp8_format: FP8Format = FP8Format.HYBRID
         self._metas: Dict[Tuple, FP8TensorMeta] = {}
         self._last_device: Optional[torch.device] = None
+        # Opt-in (fp8_cache_weights): keep each weight's fp8 codes between calls for as
+        # long as the tensor's version counter stands still, instead of measuring and
+        # quantizing the weight again in every forward (fp8.py:291-299 does). Outputs
+        # are unchanged; writes that bypass the version counter (``w.data`` tricks)
+        # are not seen, hence opt-in.
+        self.cache_weights = False
+        self._dyn_w: Dict[Tuple, Tuple] = {}
 
     def get_weight_meta(self, w: torch.Tensor) -> FP8TensorMeta:
         key = (w.data_ptr(), w.shape, w.dtype)
@@ -179,9 +213,22 @@ class FP8State:
             meta = self._metas[key] = FP8TensorMeta(w.device, self.recipe)
         return meta
 
+    def dynamic_weight(self, w: torch.Tensor, fmt: str):
+        """``(sw, w8)`` of dynamic scaling, reused while ``w`` is unmodified."""
+        key = (w.data_ptr(), w.shape, fmt, self.recipe.margin)
+        hit = self._dyn_w.get(key)
+        if hit is not None and hit[0] == w._version:
+            return hit[1], hit[2]
+        sw = _dynamic_scale(w, self.recipe, fmt)
+        w8, _ = quantize_bf16(w, sw, fmt)
+        self._dyn_w[key] = (w._version, sw, w8)
+        return sw, w8
+
     def reset(self) -> None:
         self.enabled = False
+        self.cache_weights = False
         self._metas.clear()
+        self._dyn_w.clear()
         self._last_device = None
 
 
@@ -215,7 +262,17 @@ def fp8_autocast(
 
 
 def _dynamic_scale(t: torch.Tensor, recipe: FP8Recipe, fmt: str) -> torch.Tensor:
-    amax = t.abs().amax().to(torch.float32).clamp_min(_FLOOR)
+    if t.is_cuda and t.dtype == torch.bfloat16:
+        amax = amax_bf16(t)  # one read, no |t| temporary
+        if type(recipe) in (DelayedScaling, DynamicScaling):
+            # a window of one: max((amax / FP8_MAX) / 2^margin, floor) in one launch
+            # (flooring amax first, as the host formula does, cannot change that)
+            scale = torch.empty_like(amax)
+            amax_ring_push(amax, 0, amax, scale, FP8_MAX[fmt], float(2 ** recipe.margin))
+            return scale
+        amax = amax.reshape(()).clamp_min(_FLOOR)
+    else:
+        amax = t.abs().amax().to(torch.float32).clamp_min(_FLOOR)
     return recipe.scale_from_history(amax, fmt)
 
 
@@ -234,18 +291,36 @@ def fp8_linear_forward(x: torch.Tensor, w: torch.Tensor, bias=None):
     if isinstance(st.recipe, DynamicScaling):
         x2 = x.reshape(-1, w.size(1))
         sx = _dynamic_scale(x2, st.recipe, fmt)
-        sw = _dynamic_scale(w, st.recipe, fmt)
         x8, _ = quantize_bf16(x2, sx, fmt)
-        w8, _ = quantize_bf16(w, sw, fmt)
+        if st.cache_weights:
+            sw, w8 = st.dynamic_weight(w, fmt)
+        else:
+            sw = _dynamic_scale(w, st.recipe, fmt)
+            w8, _ = quantize_bf16(w, sw, fmt)
         out = mm_fp8(x8, w8, sx, sw).reshape(*x.shape[:-1], w.size(0))
         if bias is not None and bias.numel():
             out = out + bias
         return out
     if not meta.x_init:
         meta.init_x(x, fmt)
+    if st.cache_weights and meta.w_settled(w):
+        # The weight ring already holds this weight's amax in every slot: pushing it
+        # again would leave ring and step as they are, so codes made with that step
+        # stay valid until the weight is written to.
+        if meta.w_cached is None or meta.w_cached[0] != w._version:
+            w8, amax_w = quantize_bf16(w, meta.w_scale, "e4m3")
+            meta.w_cached = (w._version, w8, amax_w)
+        x2 = x.reshape(-1, w.size(1))
+        x8, amax_x = quantize_bf16(x2, meta.x_scale, "e4m3")
+        has_bias = bias is not None and bias.numel() > 0
+        out = mm_fp8_bias(x8, meta.w_cached[1], meta.x_scale, meta.w_scale,
+                          bias if has_bias else None).reshape(*x.shape[:-1], w.size(0))
+        meta.update_x(amax_x, fmt)
+        return out
     out, amax_x, amax_w = linear_forward_fp8(x, w, bias, meta.x_scale, meta.w_scale)
     meta.update_x(amax_x, fmt)
     meta.update_w(amax_w, fmt)
+    meta.note_w_push(w)
     return out
 
 
@@ -272,6 +347,18 @@ def fp8_linear_backward(g: torch.Tensor, x: torch.Tensor, w: torch.Tensor, masks
 
 def fp8_linear_enable(enabled: bool = True) -> None:
     fp8_state().enabled = enabled
+
+
+def fp8_cache_weights(enabled: bool = True) -> None:
+    """Keep each weight's fp8 codes between forwards while the weight is unmodified
+    (inference, or several micro-batches per optimizer step). Off by default: the
+    reference quantizes the weight in every call (fp8.py:291-299)."""
+    st = fp8_state()
+    st.cache_weights = enabled
+    if not enabled:
+        st._dyn_w.clear()
+        for meta in st._metas.values():
+            meta.w_cached = None
 
 
 def fp8_linear_enabled() -> bool:

@@ -29,6 +29,9 @@ def _fp8_mm_module() -> SimpleNamespace:
         linear_forward_fp8=_cabi.linear_forward_fp8,
         linear_backward_fp8=_cabi.linear_backward_fp8,
         mm_fp8_acc=_cabi.mm_fp8_acc,
+        quantize_transpose_bf16=_cabi.quantize_transpose_bf16,
+        amax_bf16=_cabi.amax_bf16,
+        amax_ring_push=_cabi.amax_ring_push,
     )
 
 

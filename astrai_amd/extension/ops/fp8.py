@@ -117,6 +117,25 @@ def quantize_bf16(x: torch.Tensor, scale: torch.Tensor, fmt: str = "e4m3"):
     return fp8_quantize(x, scale, _fmt_int(fmt))
 
 
+def amax_bf16(x: torch.Tensor) -> torch.Tensor:
+    """``x.abs().amax()`` as a fresh float32 ``[1]`` tensor from one read of a bf16
+    device tensor (what dynamic scaling measures before it quantizes)."""
+    if x.dtype != torch.bfloat16:
+        raise TypeError(f"amax_bf16 requires a bf16 input, got {x.dtype}")
+    return _mod().amax_bf16(x)
+
+
+def amax_ring_push(hist, idx: int, amax, scale, fmax: float, pow2_margin: float) -> None:
+    """Delayed scaling's record-then-refresh on device rings, in place, one launch."""
+    _mod().amax_ring_push(hist, idx, amax, scale, fmax, pow2_margin)
+
+
+def mm_fp8_bias(a, b, sa, sb, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """``mm_fp8`` to bf16 with the bias added before the single rounding, the
+    epilogue of the fused forward (csrc/kernels/fp8/gemm.cuh:405-435)."""
+    return _mod().mm_fp8(a, b, sa, sb, 0, None, bias)
+
+
 def mm_fp8(
     a: torch.Tensor,
     b: torch.Tensor,

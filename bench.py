@@ -326,6 +326,46 @@ def main():
                                        "TFLOP/s": round(flop / (ms * 1e-3) / 1e12, 1)}
         del ai, bi
 
+        # ---- fp8 linear backward at 4096^3 (dX and dW GEMMs + the three transposing
+        # quantizer passes), through the module the registry hands out
+        from astrai_amd.extension import get_module
+
+        mod = get_module("fp8_mm")
+        gb16 = torch.randn(M, N, device=dev).to(torch.bfloat16)
+        xb16 = torch.randn(M, K, device=dev).to(torch.bfloat16)
+        wb16 = torch.randn(N, K, device=dev).to(torch.bfloat16)
+        s_one = torch.full((1,), 4.0 / 448.0, device=dev)
+
+        def step_bwd():
+            mod.linear_backward_fp8(gb16, xb16, wb16, [1, 1, 0], s_one, s_one, s_one, 0)
+
+        ms = _event_time_ms(step_bwd, 100, 30)
+
+        def step_qt():
+            mod.quantize_transpose_bf16(gb16, s_one, 0, True, True)
+
+        ms_qt = _event_time_ms(step_qt, 200, 50)
+        extra["fp8_linear_backward_4096"] = {
+            "us": round(ms * 1e3, 1), "TFLOP/s_two_gemms": round(2 * flop / (ms * 1e-3) / 1e12, 1),
+            "quantize_transpose_us": round(ms_qt * 1e3, 2),
+            "quantize_transpose_GB/s": round(M * N * 4 / (ms_qt * 1e-3) / 1e9, 0)}
+        # ---- the whole Linear as the dispatcher override runs it (measure / quantize /
+        # GEMM / ring update), per recipe, with and without the opt-in weight-code cache
+        import torch.nn.functional as F
+        from astrai_amd.extension import fp8 as P
+
+        e2e = {"bf16_stock_us": round(_event_time_ms(lambda: F.linear(xb16, wb16), 100, 30) * 1e3, 1)}
+        for rname, recipe in (("dynamic", P.DynamicScaling()), ("delayed", P.DelayedScaling())):
+            for cache in (False, True):
+                P.fp8_state().reset()
+                with P.fp8_autocast(True, recipe=recipe):
+                    P.fp8_cache_weights(cache)
+                    ms = _event_time_ms(lambda: F.linear(xb16, wb16), 100, 30)
+                e2e[f"{rname}{'_cached_weight' if cache else ''}_us"] = round(ms * 1e3, 1)
+        P.fp8_state().reset()
+        extra["fp8_linear_4096_through_dispatcher"] = e2e
+        del gb16, xb16, wb16
+
         # ---- config 3: block-scaled fp8 8192 x 2048 x 7168
         M3, N3, K3 = 8192, 2048, 7168
         a3 = torch.randn(M3, K3, device=dev).clamp(-3, 3).to(torch.float8_e4m3fn)

@@ -67,6 +67,36 @@ int astrai_w8a8_quantize_bf16_fp8(const void* x_bf16, void* x8, const float* sca
                                   float* amax, int64_t total, int fmt, void* stream);
 
 /*
+ * *amax = max(*amax, max_i |x[i]|) over a bf16 tensor, one read and no temporary.
+ * Replaces the t.abs().amax() with which dynamic scaling measures each operand
+ * before quantizing it (astrai/extension/fp8.py:289-292). The caller zeroes *amax.
+ */
+int astrai_w8a8_amax_bf16(const void* x_bf16, float* amax, int64_t total, void* stream);
+
+/*
+ * Delayed scaling's record-then-refresh (FP8TensorMeta.update_*,
+ * astrai/extension/fp8.py:147-173, step formula :87-89) in one launch:
+ *   hist[idx] = *amax;  *scale = max((max_i hist[i] / fmax) / pow2_margin, 1e-12)
+ * hist is the fp32 ring of n recorded amax values, fmax the format's largest
+ * finite value (448 or 57344), pow2_margin = 2^margin. True fp32 divisions, as
+ * the reference's formula evaluates on host tensors.
+ */
+int astrai_w8a8_amax_ring_push(float* hist, int n, int idx, const float* amax, float* scale,
+                               float fmax, float pow2_margin, void* stream);
+
+/*
+ * The same quantizer on a [rows, cols] matrix, writing the codes transposed
+ * ([cols, rows], x8t) and, when x8 is not NULL, row-major as well, from one read
+ * of x. Replaces the transposed-contiguous copies followed by quantize_bf16 in
+ * linear_backward_fp8 (csrc/kernels/fp8/mm.cu:276-312): dX = g.w contracts
+ * over the gradient's columns and dW = g^T.x over its rows, so the gradient is
+ * needed in both layouts and w, x transposed. amax as above.
+ */
+int astrai_w8a8_quantize_transpose_bf16_fp8(const void* x_bf16, void* x8, void* x8t,
+                                            const float* scale, float* amax, int64_t rows,
+                                            int64_t cols, int fmt, void* stream);
+
+/*
  * bf16 -> int8, symmetric, one scale per row (per token for activations, per
  * output channel for weights). No counterpart in the reference (it has no int8
  * path); same conventions as the fp8 quantizer.

@@ -82,6 +82,56 @@ def test_linear_backward_fp8_both_formats(ops):
         assert amax_g.item() == g.abs().max().item()
 
 
+@pytest.mark.parametrize("masks", [[1, 0, 0], [0, 1, 0], [0, 0, 1], [0, 0, 0], [1, 1, 0]])
+def test_linear_backward_fp8_masks(ops, masks):
+    """Each output-mask combination of mm.cu:293-319: unrequested gradients are not
+    computed, and amax_g is measured on the dX branch (or when neither GEMM runs) only."""
+    print(f"case masks={masks}", flush=True)
+    torch.manual_seed(21)
+    m, n, k = 69, 24, 40  # 3 x 23 tokens
+    x = torch.randn(3, 23, k).to(torch.bfloat16)
+    w = torch.randn(n, k).to(torch.bfloat16)
+    g = torch.randn(3, 23, n).to(torch.bfloat16)
+    sx, sw, sg = _scale(x), _scale(w), _scale(g)
+    gx, gw, gb, amax_g = ops.linear_backward_fp8(
+        g.to(DEV), x.to(DEV), w.to(DEV), masks, sg.to(DEV), sw.to(DEV), sx.to(DEV), "e4m3")
+    qg = O.fp8_quantize(g.reshape(m, n), sg, 0)[0].float()
+    qw = O.fp8_quantize(w, sw, 0)[0].float()
+    qx = O.fp8_quantize(x.reshape(m, k), sx, 0)[0].float()
+    assert gx.shape == x.shape and gw.shape == w.shape
+    if masks[0]:
+        torch.testing.assert_close(gx.cpu().reshape(m, k), (qg @ qw * sg * sw).to(torch.bfloat16),
+                                   atol=0.125, rtol=0.01)
+    if masks[1]:
+        torch.testing.assert_close(gw.cpu(), (qg.t() @ qx * sg * sx).to(torch.bfloat16),
+                                   atol=0.125, rtol=0.01)
+    if masks[2]:
+        torch.testing.assert_close(gb.cpu(), g.reshape(m, n).sum(0).to(torch.bfloat16))
+    else:
+        assert gb.numel() == 0
+    want_amax = g.abs().max().item() if (masks[0] or not masks[1]) else 0.0
+    assert amax_g.item() == want_amax
+
+
+def test_linear_backward_fp8_4096(ops):
+    """Full-size backward (4096 tokens, 4096 x 4096 weight): both GEMMs against
+    fp64 products of the oracle's codes, the tolerance of test_fp8_mma.py:149-174."""
+    torch.manual_seed(13)
+    m = n = k = 4096
+    x = torch.randn(m, k).to(torch.bfloat16)
+    w = torch.randn(n, k).to(torch.bfloat16)
+    g = torch.randn(m, n).to(torch.bfloat16)
+    sx, sw, sg = _scale(x), _scale(w), _scale(g)
+    gx, gw, gb, amax_g = ops.linear_backward_fp8(
+        g.to(DEV), x.to(DEV), w.to(DEV), [1, 1, 1], sg.to(DEV), sw.to(DEV), sx.to(DEV), "e4m3")
+    qg = O.fp8_quantize(g, sg, 0)[0].float()
+    qw = O.fp8_quantize(w, sw, 0)[0].float()
+    qx = O.fp8_quantize(x, sx, 0)[0].float()
+    assert_bf16_close(gx, (qg @ qw * sg * sw).to(torch.bfloat16), what="dX 4096")
+    assert_bf16_close(gw, (qg.t() @ qx * sg * sx).to(torch.bfloat16), what="dW 4096")
+    assert amax_g.item() == g.abs().max().item()
+
+
 def test_mm_fp8_k4096_vs_float64_and_oracle(ops):
     # test_fp8_mma.py:149-174: seed 11, 512x4096x4096, sa 2.5, sb 1.5, atol 6 / rtol .05 vs fp64
     torch.manual_seed(11)

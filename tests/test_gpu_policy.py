@@ -48,6 +48,77 @@ def test_delayed_scaling_linear_seeds_then_tracks_amax():
     st.reset()
 
 
+@pytest.mark.parametrize("shape", [(1,), (7,), (64, 128), (257, 33), (4096, 1024), (0, 8)])
+def test_amax_kernel_equals_abs_amax(shape):
+    from astrai_amd.extension.ops.fp8 import amax_bf16
+    g = torch.Generator().manual_seed(5 + sum(shape))
+    x = (torch.randn(*shape, generator=g) * 7).to(torch.bfloat16)
+    got = amax_bf16(x.to(DEV))
+    assert got.shape == (1,) and got.dtype == torch.float32
+    want = x.abs().amax().float().item() if x.numel() else 0.0
+    assert got.item() == want
+    if x.numel() > 8:  # the peak in the ragged tail / as a negative value
+        x.view(-1)[-1] = -1000.0
+        assert amax_bf16(x.to(DEV)).item() == 1000.0
+
+
+@pytest.mark.parametrize("n,fmt,margin", [(16, "e4m3", 0), (4, "e5m2", 2), (1, "e4m3", 0), (100, "e4m3", 1)])
+def test_ring_push_kernel_matches_the_formula_on_host_tensors(n, fmt, margin):
+    """The one-launch record-then-refresh against the same pushes made with host
+    tensors (fp8.py:87-89,147-173: true divisions, floor 1e-12), bit for bit."""
+    from astrai_amd.extension.fp8 import DelayedScaling, FP8TensorMeta
+    recipe = DelayedScaling(history_len=n, margin=margin)
+    dev_meta, cpu_meta = FP8TensorMeta(torch.device(DEV), recipe), FP8TensorMeta(torch.device("cpu"), recipe)
+    g = torch.Generator().manual_seed(n)
+    for step in range(2 * n + 3):
+        amax = (torch.rand(1, generator=g) * 10 ** float(torch.randint(-3, 4, (1,), generator=g))).float()
+        if step == 3:
+            amax = torch.zeros(1)  # the floor
+        dev_meta.update_x(amax.to(DEV), fmt)
+        cpu_meta.update_x(amax, fmt)
+        assert dev_meta.x_idx == cpu_meta.x_idx
+        assert torch.equal(dev_meta.x_hist.cpu(), cpu_meta.x_hist), f"step {step}"
+        assert torch.equal(dev_meta.x_scale.cpu(), cpu_meta.x_scale), f"step {step}"
+
+
+@pytest.mark.parametrize("recipe_name", ["dynamic", "delayed"])
+def test_weight_code_cache_changes_no_output(recipe_name):
+    """fp8_cache_weights keeps a weight's codes while its version counter stands
+    still. The same call sequence (repeated forwards, an in-place weight update,
+    more forwards) with and without it gives equal outputs and equal ring state."""
+    from astrai_amd.extension import fp8 as P
+
+    def run(cache):
+        st = P.fp8_state()
+        st.reset()
+        torch.manual_seed(33)
+        x = torch.randn(48, 96).to(torch.bfloat16).to(DEV)
+        w = torch.randn(40, 96).to(torch.bfloat16).to(DEV)
+        b = torch.randn(40).to(torch.bfloat16).to(DEV)
+        recipe = P.DynamicScaling() if recipe_name == "dynamic" else P.DelayedScaling(history_len=4)
+        outs = []
+        with P.fp8_autocast(True, recipe=recipe, fp8_format="e4m3"):
+            P.fp8_cache_weights(cache)
+            for step in range(14):
+                if step == 5:
+                    w.mul_(3.0)          # bumps the version: codes must be remade
+                if step == 9:
+                    w[0, 0] = 50.0       # a new peak: the ring must see it
+                outs.append(F.linear(x * (1 + step % 3), w, b if step % 2 else None))
+            meta = st.get_weight_meta(w)
+            state = (meta.w_hist.clone(), meta.w_scale.clone(), meta.x_hist.clone(), meta.x_scale.clone())
+        st.reset()
+        return outs, state
+
+    plain, plain_state = run(False)
+    cached, cached_state = run(True)
+    for i, (a, c) in enumerate(zip(plain, cached)):
+        assert torch.equal(a, c), f"step {i}"
+    if recipe_name == "delayed":
+        for a, c in zip(plain_state, cached_state):
+            assert torch.equal(a, c)
+
+
 def test_int8_autocast_linear_matches_oracle_and_caches_weights():
     from astrai_amd.extension import w8a8
     x, w, b = O.make_inputs(23, 10, 200, 512, bias=True)

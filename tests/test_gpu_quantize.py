@@ -79,6 +79,34 @@ def test_fp8_quantize_noncontiguous_input(C):
     assert got.shape == (96, 64) and torch.equal(_codes(got), _codes(want))
 
 
+@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("shape", [(1, 1), (1, 33), (33, 1), (17, 9), (128, 64), (130, 72), (16, 8),
+                                   (48, 20), (129, 65), (256, 7), (19, 128), (1000, 520), (0, 8),
+                                   (2048, 4096)])
+def test_fp8_quantize_transposed_codes(C, shape, fmt):
+    """One pass gives the codes of x and of x.t().contiguous() (the copies
+    csrc/kernels/fp8/mm.cu:298-311 quantizes) and the amax, bit-exact, for
+    aligned, ragged and single-row/column matrices."""
+    print(f"case shape={shape} fmt={fmt}", flush=True)
+    g = torch.Generator().manual_seed(7 + shape[0] * 31 + shape[1])
+    x = (torch.randn(*shape, generator=g) * 3).to(torch.bfloat16)
+    s = torch.tensor([0.037 if fmt == 0 else 0.0011])
+    x8, x8t, amax = C.quantize_transpose_bf16(x.to(DEV), s.to(DEV), fmt, want_rowmajor=True,
+                                              want_amax=True)
+    assert x8.shape == shape and x8t.shape == (shape[1], shape[0])
+    if x.numel() == 0:
+        assert amax.item() == 0.0
+        return
+    want, _ = O.fp8_quantize_saturating(x, s, fmt)
+    assert x8.dtype == want.dtype and x8t.dtype == want.dtype
+    assert torch.equal(_codes(x8), _codes(want))
+    assert torch.equal(_codes(x8t), _codes(want).t().contiguous())
+    assert amax.item() == x.abs().max().item()
+    none8, only_t, zero = C.quantize_transpose_bf16(x.to(DEV), s.to(DEV), fmt)
+    assert none8 is None and zero.item() == 0.0
+    assert torch.equal(_codes(only_t), _codes(x8t))
+
+
 @pytest.mark.parametrize("rows,k", [(1, 8), (3, 24), (16, 2048), (5, 33), (2, 9000), (7, 16384), (64, 4096), (0, 32)])
 def test_int8_rows_bit_exact(C, rows, k):
     print(f"case rows={rows} k={k}", flush=True)
