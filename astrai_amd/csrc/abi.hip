@@ -234,6 +234,30 @@ int astrai_w8a8_attn_decode_bf16(const void* q, const void* k_cache, const void*
     return check_launch("attn_decode_bf16");
 }
 
+int astrai_w8a8_attn_prefill_bf16(const void* q, const void* k_cache, const void* v_cache,
+                                  const int64_t* positions, void* out, int64_t batch, int64_t seq,
+                                  int64_t n_heads, int64_t n_kv_heads, int64_t head_dim,
+                                  int64_t max_len, float scale, void* stream) {
+    if (!q || !k_cache || !v_cache || !positions || !out)
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_prefill_bf16: null pointer");
+    if (batch < 0 || seq < 0 || n_heads <= 0 || n_kv_heads <= 0 || max_len <= 0 ||
+        n_heads % n_kv_heads || seq > (1 << 24) || batch > (1 << 20))
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_prefill_bf16: bad dims");
+    if (!w8a8::attn_prefill_supported((int)n_heads, (int)n_kv_heads, (int)head_dim))
+        return fail(ASTRAI_W8A8_UNSUPPORTED,
+                    "attn_prefill_bf16: needs head_dim 128 and n_heads / n_kv_heads in {2, 4, 8}");
+    if (max_len >= ((int64_t)1 << 30))
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "attn_prefill_bf16: max_len must stay under 2^30");
+    if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out))
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_prefill_bf16: pointers must be 16-byte aligned");
+    if (batch == 0 || seq == 0) return ASTRAI_W8A8_OK;
+    w8a8::AttnPrefillArgs a{q, k_cache, v_cache, positions, out, (int)batch, (int)seq, (int)n_heads,
+                            (int)n_kv_heads, (int)head_dim, max_len, scale};
+    if (!w8a8::launch_attn_prefill(a, static_cast<hipStream_t>(stream)))
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "attn_prefill_bf16: shape not supported");
+    return check_launch("attn_prefill_bf16");
+}
+
 int astrai_w8a8_quantize_bf16_fp8_block128_act(const void* x, void* x8, float* sa, int64_t m,
                                                int64_t k, void* stream) {
     if (!x || !x8 || !sa) return fail(ASTRAI_W8A8_BAD_ARG, "quantize_block128_act: null pointer");

@@ -85,6 +85,21 @@ struct AttnDecodeArgs {
 int64_t attn_decode_workspace_floats(int batch, int n_kv_heads, int nsplit, int nq);
 bool launch_attn_decode(const AttnDecodeArgs& a, hipStream_t stream);
 
+// attn_prefill.hip: causal grouped-query attention of a block of new tokens against
+// the dense bf16 KV cache; head_dim 128, n_heads / n_kv_heads in {2, 4, 8}
+struct AttnPrefillArgs {
+    const void* q;             // bf16 [batch, n_heads, seq, 128]
+    const void* k_cache;       // bf16 [batch, n_kv_heads, max_len, 128]
+    const void* v_cache;       // same
+    const int64_t* positions;  // int64 [seq]: position of each new token (keys <= it are attended)
+    void* out;                 // bf16 [batch, seq, n_heads * 128]
+    int batch, seq, n_heads, n_kv_heads, head_dim;
+    int64_t max_len;
+    float scale;
+};
+bool attn_prefill_supported(int n_heads, int n_kv_heads, int head_dim);
+bool launch_attn_prefill(const AttnPrefillArgs& a, hipStream_t stream);
+
 // gemm_int8.hip / gemm_fp8.hip / gemm_fp8_block.hip: tiled MFMA kernels.
 // Require k % 16 == 0 and m*k, n*k < 2^31 bytes; return false if the shape is
 // not accepted (the caller then uses the generic kernel).

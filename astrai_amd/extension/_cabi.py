@@ -43,6 +43,8 @@ PROTOTYPES = {
     "astrai_w8a8_rope_cache_write_bf16": (
         [_P, _I64, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _P], _INT),
     "astrai_w8a8_attn_decode_workspace_floats": ([_I64, _I64, _I64, _I64], _I64),
+    "astrai_w8a8_attn_prefill_bf16": (
+        [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, ctypes.c_float, _P], _INT),
     "astrai_w8a8_attn_decode_bf16": (
         [_P, _P, _P, _P, _P, _I64, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, ctypes.c_float, _P],
         _INT),
@@ -558,6 +560,41 @@ def attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, p
             ws.data_ptr(), ws.numel(), _ptr(out), _ptr(oq), _ptr(os_), b, s, h, hkv, d, max_len, nsplit,
             float(scale), _stream(q)), lib)
     return (oq, os_) if quantized else out
+
+
+def attn_prefill_supported(n_heads: int, n_kv_heads: int, head_dim: int) -> bool:
+    return head_dim == 128 and n_heads % n_kv_heads == 0 and n_heads // n_kv_heads in (2, 4, 8)
+
+
+def attn_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                 positions: torch.Tensor, scale: Optional[float] = None) -> torch.Tensor:
+    """Causal attention of ``q [batch, n_heads, seq, 128]`` (bf16) against the dense caches
+    ``[batch, n_kv_heads, max_len, 128]``; token ``s`` attends keys ``0..positions[s]``.
+    Returns ``[batch, seq, n_heads * 128]`` bf16 (token-major, what ``o_proj`` reads)."""
+    lib = _require()
+    _gpu(q, "attn_prefill")
+    if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
+        raise RuntimeError("q and the caches must be bf16")
+    if q.dim() != 4 or k_cache.dim() != 4 or k_cache.shape != v_cache.shape:
+        raise RuntimeError("q must be [B, H, S, D] and the caches [B, H_kv, max_len, D]")
+    b, h, s, d = q.shape
+    hkv, max_len = k_cache.size(1), k_cache.size(2)
+    if k_cache.size(0) != b or k_cache.size(3) != d:
+        raise RuntimeError("cache batch / head_dim do not match q")
+    if not (q.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise RuntimeError("q and the caches must be contiguous")
+    if positions.dtype != torch.int64 or positions.numel() != s or positions.device != q.device:
+        raise RuntimeError("positions must be int64 [seq] on q's device")
+    if h % hkv:
+        raise RuntimeError("n_heads must be a multiple of n_kv_heads")
+    if scale is None:
+        scale = d ** -0.5
+    with torch.cuda.device(q.device):
+        out = torch.empty((b, s, h * d), device=q.device, dtype=torch.bfloat16)
+        _check(lib.astrai_w8a8_attn_prefill_bf16(
+            q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), positions.contiguous().data_ptr(),
+            out.data_ptr(), b, s, h, hkv, d, max_len, float(scale), _stream(q)), lib)
+    return out
 
 
 _INT8_ENTRY = {

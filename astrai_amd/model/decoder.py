@@ -189,7 +189,8 @@ class GQA(nn.Module):
         cache: rotation, permutes and the cache write are one kernel. Returns the attention
         output already quantized per token, ``(int8 [B*S, dim], fp32 [B*S, 1])``: for a few new
         tokens straight out of the split-context attention kernel (mask from ``positions``,
-        token-major), otherwise SDPA followed by the quantizer."""
+        token-major), for longer blocks the causal block kernel followed by the quantizer
+        (SDPA only for head layouts neither kernel takes)."""
         from astrai_amd.extension import _cabi
         from astrai_amd.extension.ops import int8 as I
         b, s, _ = qkv.shape
@@ -199,6 +200,10 @@ class GQA(nn.Module):
         if _cabi.attn_decode_supported(self.n_heads, self.n_kv_heads, s, self.head_dim):
             return _cabi.attn_decode(q, kv_cache.k[self.layer_id], kv_cache.v[self.layer_id], positions,
                                      quantized=True)
+        if _cabi.attn_prefill_supported(self.n_heads, self.n_kv_heads, self.head_dim):
+            # causal block kernel: no mask tensor, no head expansion, token-major output
+            return I.quantize_int8_per_token(
+                _cabi.attn_prefill(q, kv_cache.k[self.layer_id], kv_cache.v[self.layer_id], positions))
         out = self._attend_cache(q, kv_cache, key_mask)
         return I.quantize_int8_per_token(out.permute(0, 2, 1, 3).reshape(b, s, self.dim))
 

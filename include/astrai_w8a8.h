@@ -188,6 +188,27 @@ int astrai_w8a8_attn_decode_bf16(const void* q_bf16, const void* k_cache_bf16, c
                                  int64_t nsplit, float scale, void* stream);
 
 /*
+ * Causal grouped-query attention of a block of `seq` new tokens per sequence against
+ * the dense KV cache (prefill, whole or chunked). Replaces the same reference code as
+ * attn_decode_bf16 for long query blocks: head expansion
+ * (astrai/extension/backend/attention.py:244-253), the mask tensor and SDPA
+ * (:443-498), and the permute back to token-major of
+ * astrai/model/components/attention.py:19-85. Key blocks that no query of a block may
+ * see are skipped; the mask is computed from positions.
+ *   q, k_cache, v_cache, positions  as for attn_decode_bf16 (keys at positions <= the
+ *              largest positions[s] must have been written)
+ *   out        bf16 [batch, seq, n_heads * 128]
+ * bf16 MFMAs for q.k^T and p.v (p rounded to bf16, as SDPA's flash kernels do), fp32
+ * softmax statistics and accumulation, one rounding of the output to bf16.
+ * head_dim == 128, n_heads / n_kv_heads in {2, 4, 8}. Allocates nothing, no workspace.
+ */
+int astrai_w8a8_attn_prefill_bf16(const void* q_bf16, const void* k_cache_bf16,
+                                  const void* v_cache_bf16, const int64_t* positions,
+                                  void* out_bf16, int64_t batch, int64_t seq, int64_t n_heads,
+                                  int64_t n_kv_heads, int64_t head_dim, int64_t max_len,
+                                  float scale, void* stream);
+
+/*
  * bf16 -> e4m3fn with one scale per 1x128 K-group (activations) or per 128x128
  * block (weights). No counterpart in the reference. K must be a multiple of 128.
  *   act:    sa[m,kb]  = max(max |x[m,128kb..128kb+127]|, 1e-12) / 448,   sa is [M, K/128]
