@@ -246,8 +246,10 @@ int astrai_w8a8_attn_prefill_bf16(const void* q, const void* k_cache, const void
     if (!w8a8::attn_prefill_supported((int)n_heads, (int)n_kv_heads, (int)head_dim))
         return fail(ASTRAI_W8A8_UNSUPPORTED,
                     "attn_prefill_bf16: needs head_dim 128 and n_heads / n_kv_heads in {2, 4, 8}");
-    if (max_len >= ((int64_t)1 << 30))
-        return fail(ASTRAI_W8A8_UNSUPPORTED, "attn_prefill_bf16: max_len must stay under 2^30");
+    if (max_len * 256 >= ((int64_t)1 << 32))
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "attn_prefill_bf16: one head of the cache must stay under 4 GiB");
+    if (!(scale > 0.0f))
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_prefill_bf16: scale must be positive");
     if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out))
         return fail(ASTRAI_W8A8_BAD_ARG, "attn_prefill_bf16: pointers must be 16-byte aligned");
     if (batch == 0 || seq == 0) return ASTRAI_W8A8_OK;

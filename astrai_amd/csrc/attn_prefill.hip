@@ -20,9 +20,11 @@
 //     stored transposed with its key slots permuted to that order, 136-byte rows
 //     (conflict-free for the transposing 4-byte writes and the 16-byte operand reads);
 //   keys sit in LDS as 256-byte rows of 16-byte chunks XOR-swizzled by row.
-// The next block's keys and values are fetched from the cache into registers while
-// the current block is multiplied.
+// Two LDS buffers: while a block is multiplied, the next one arrives (keys by
+// direct-to-LDS loads, values through registers) and the values of the one after are
+// requested; one barrier per block. Blocks that every query of the wave sees whole skip the masking code.
 #include <climits>
+#include <type_traits>
 
 #include "common.cuh"
 #include "launchers.h"
@@ -41,11 +43,18 @@ constexpr int kKRow = 256;                 // bytes per key row in LDS
 constexpr int kVtRow = 136;                // bytes per value-dim row of V^T in LDS
 constexpr int kKBytes = kKB * kKRow;       // 16 KiB
 constexpr int kVtBytes = kD * kVtRow;      // 17 KiB
+constexpr int kBufBytes = kKBytes + kVtBytes;
 constexpr float kNegBig = -1e30f;          // finite stand-in for -inf: no inf - inf
 
 // slot of key w (0..31 within a 32-key tile) in a V^T row: the S^T accumulator of
 // lane half h holds keys 8g' + 4h + j at register 4g' + j; a 16-key MFMA step t takes
 // registers 8t..8t+7, i.e. keys 16t + 8g + 4h + j (g = 0,1) as its k-index 8h + 4g + j.
+__device__ __forceinline__ void lds_dma16(__amdgpu_buffer_rsrc_t r, uint8_t* lds_wave_base,
+                                          uint32_t voff, uint32_t soff) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+        r, (__attribute__((address_space(3))) void*)lds_wave_base, 16, voff, soff, 0, 0);
+}
+
 __device__ __forceinline__ int vt_slot(int w) {
     return (w & 16) | ((w & 4) << 1) | ((w & 8) >> 1) | (w & 3);
 }
@@ -53,11 +62,9 @@ __device__ __forceinline__ int vt_slot(int w) {
 template <int NREP>
 __global__ __launch_bounds__(64 * NREP, 2) void attn_prefill_kernel(AttnPrefillArgs a) {
     constexpr int THREADS = 64 * NREP;
-    constexpr int K_ITEMS = kKB * 16 / THREADS;        // 16-byte key chunks per thread
+    constexpr int K_DMA = kKB / 4 / NREP;              // 1 KiB key loads per wave and block
     constexpr int V_ITEMS = (kKB / 2) * 16 / THREADS;  // (key pair, 8-dim chunk) items per thread
-    __shared__ __attribute__((aligned(16))) uint8_t lds[kKBytes + kVtBytes];
-    uint8_t* const ks_lds = lds;
-    uint8_t* const vt_lds = lds + kKBytes;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kBufBytes];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -93,16 +100,26 @@ __global__ __launch_bounds__(64 * NREP, 2) void attn_prefill_kernel(AttnPrefillA
     const uint16_t* kc = static_cast<const uint16_t*>(a.k_cache) + cache_off;
     const uint16_t* vc = static_cast<const uint16_t*>(a.v_cache) + cache_off;
 
-    u32x4 kreg[K_ITEMS], vreg[V_ITEMS][2];
-    auto fetch = [&](int kb) {
-        const u32x4 zero = {0u, 0u, 0u, 0u};
+    // keys: straight from the cache into LDS, 1 KiB (four rows) per instruction; lane l
+    // lands at row l/16, chunk position l%16 and therefore asks for chunk (l%16) ^ (row%16).
+    // The descriptor ends after key kmax: later rows arrive as zeros.
+    const __amdgpu_buffer_rsrc_t rk = make_rsrc(kc, (uint32_t)(kmax + 1) * (uint32_t)kKRow);
+    uint32_t k_voff[K_DMA];
 #pragma unroll
-        for (int i = 0; i < K_ITEMS; ++i) {
-            const int item = tid + i * THREADS;
-            const int key = kb * kKB + (item >> 4);
-            kreg[i] = key <= kmax
-                ? *reinterpret_cast<const u32x4*>(kc + (size_t)key * kD + (item & 15) * 8) : zero;
-        }
+    for (int j = 0; j < K_DMA; ++j) {
+        const int row = (wave * K_DMA + j) * 4 + (lane >> 4);
+        k_voff[j] = (uint32_t)row * kKRow + (uint32_t)(((lane & 15) ^ (row & 15)) << 4);
+    }
+    auto dma_k = [&](int kb, int buf) {
+#pragma unroll
+        for (int j = 0; j < K_DMA; ++j)
+            lds_dma16(rk, lds + buf * kBufBytes + (wave * K_DMA + j) * 4 * kKRow,
+                      k_voff[j] + (uint32_t)kb * (kKB * kKRow), 0);
+    };
+    // values: through registers, because they are stored transposed
+    u32x4 vreg[V_ITEMS][2];
+    auto fetch_v = [&](int kb) {
+        const u32x4 zero = {0u, 0u, 0u, 0u};
 #pragma unroll
         for (int i = 0; i < V_ITEMS; ++i) {
             const int item = tid + i * THREADS;
@@ -114,13 +131,8 @@ __global__ __launch_bounds__(64 * NREP, 2) void attn_prefill_kernel(AttnPrefillA
             vreg[i][1] = key + 1 <= kmax ? *reinterpret_cast<const u32x4*>(src + kD) : zero;
         }
     };
-    auto stage = [&]() {
-#pragma unroll
-        for (int i = 0; i < K_ITEMS; ++i) {
-            const int item = tid + i * THREADS;
-            const int row = item >> 4, chunk = item & 15;
-            *reinterpret_cast<u32x4*>(ks_lds + row * kKRow + ((chunk ^ (row & 15)) << 4)) = kreg[i];
-        }
+    auto stage_v = [&](int buf) {
+        uint8_t* const vt_lds = lds + buf * kBufBytes + kKBytes;
 #pragma unroll
         for (int i = 0; i < V_ITEMS; ++i) {
             const int item = tid + i * THREADS;
@@ -131,9 +143,11 @@ __global__ __launch_bounds__(64 * NREP, 2) void attn_prefill_kernel(AttnPrefillA
             const uint32_t hi[4] = {vreg[i][1].x, vreg[i][1].y, vreg[i][1].z, vreg[i][1].w};
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
-                // dims 2p and 2p+1 of the chunk: (key w, key w+1) side by side
-                *reinterpret_cast<uint32_t*>(dst + (2 * p) * kVtRow) = (lo[p] & 0xffffu) | (hi[p] << 16);
-                *reinterpret_cast<uint32_t*>(dst + (2 * p + 1) * kVtRow) = (lo[p] >> 16) | (hi[p] & 0xffff0000u);
+                // dims 2p and 2p+1 of the chunk: (key w, key w+1) side by side, one byte permute each
+                *reinterpret_cast<uint32_t*>(dst + (2 * p) * kVtRow) =
+                    __builtin_amdgcn_perm(hi[p], lo[p], 0x05040100u);
+                *reinterpret_cast<uint32_t*>(dst + (2 * p + 1) * kVtRow) =
+                    __builtin_amdgcn_perm(hi[p], lo[p], 0x07060302u);
             }
         }
     };
@@ -143,70 +157,72 @@ __global__ __launch_bounds__(64 * NREP, 2) void attn_prefill_kernel(AttnPrefillA
     for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
         for (int e = 0; e < 16; ++e) o[dt][e] = 0.0f;
+    // m_run is the reference maximum the probabilities are taken against, in log2 units.
+    // It follows the true running maximum lazily: only when some query of the wave has
+    // outgrown it by more than kSlack does the wave pay for rescaling its 64 accumulators;
+    // until then probabilities may reach 2^kSlack, which fp32 sums and bf16 operands hold.
+    constexpr float kSlack = 8.0f;
     float m_run = kNegBig, l_run = 0.0f;
-    const float c = a.scale * 1.44269504088896340736f;  // scores in log2 units
+    const float c = a.scale * 1.44269504088896340736f;  // scores to log2 units
 
-    fetch(0);
-    for (int kb = 0; kb < nkb; ++kb) {
-        __syncthreads();  // every wave is done reading the previous block
-        stage();
-        __syncthreads();
-        if (kb + 1 < nkb) fetch(kb + 1);
-
+    // one 64-key block out of LDS buffer `buf`; MASK: some key of it lies past some query
+    auto block = [&](auto mask_tag, int kb, const uint8_t* kbuf, const uint8_t* vbuf) {
+        constexpr bool MASK = decltype(mask_tag)::value;
         // ---- S^T = K.Q^T for two 32-key tiles
         f32x16 s[2];
-#pragma unroll
-        for (int ti = 0; ti < 2; ++ti)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) s[ti][e] = 0.0f;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks)
 #pragma unroll
             for (int ti = 0; ti < 2; ++ti) {
                 const int row = ti * 32 + qi;
                 const u32x4 kf = *reinterpret_cast<const u32x4*>(
-                    ks_lds + row * kKRow + (((2 * ks + h) ^ (row & 15)) << 4));
-                s[ti] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                    __builtin_bit_cast(bf16x8, kf), __builtin_bit_cast(bf16x8, qf[ks]), s[ti], 0, 0, 0);
+                    kbuf + row * kKRow + (((2 * ks + h) ^ (row & 15)) << 4));
+                if (ks == 0) {
+                    const f32x16 zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f,
+                                         0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+                    s[ti] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(bf16x8, kf), __builtin_bit_cast(bf16x8, qf[ks]), zero, 0, 0, 0);
+                } else {
+                    s[ti] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(bf16x8, kf), __builtin_bit_cast(bf16x8, qf[ks]), s[ti], 0, 0, 0);
+                }
             }
 
-        // ---- online softmax for this lane's query
-        const bool need_mask = kb * kKB + kKB - 1 > pmin;  // uniform over the wave
+        // ---- online softmax for this lane's query (raw scores; c > 0 keeps their order)
         float m_loc = kNegBig;
 #pragma unroll
         for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                float v = s[ti][e] * c;
-                if (need_mask) {
+                if (MASK) {
                     const int key = kb * kKB + ti * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
-                    v = key <= pq ? v : kNegBig;
+                    s[ti][e] = key <= pq ? s[ti][e] : kNegBig;
                 }
-                s[ti][e] = v;
-                m_loc = fmaxf(m_loc, v);
+                m_loc = fmaxf(m_loc, s[ti][e]);
             }
-        m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 32, kWave));
-        const float m_new = fmaxf(m_run, m_loc);
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        m_run = m_new;
+        m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 32, kWave)) * c;
+        if (__any(m_loc > m_run + kSlack)) {
+            const float m_new = fmaxf(m_run, m_loc);
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            m_run = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) o[dt][e] *= alpha;
+        }
         float l_add = 0.0f;
         uint32_t pk[2][8];
 #pragma unroll
         for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
             for (int e = 0; e < 16; e += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(s[ti][e] - m_new);
-                const float p1 = __builtin_amdgcn_exp2f(s[ti][e + 1] - m_new);
+                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[ti][e], c, -m_run));
+                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[ti][e + 1], c, -m_run));
                 l_add += p0 + p1;
                 pk[ti][e >> 1] = pack_bf16x2(p0, p1);
             }
-        l_run = l_run * alpha + l_add;
-        if (__any(alpha != 1.0f)) {
-#pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) o[dt][e] *= alpha;
-        }
+        l_run += l_add;
 
         // ---- O^T += V^T.P^T, four 16-key steps x four 32-dim tiles
 #pragma unroll
@@ -215,7 +231,7 @@ __global__ __launch_bounds__(64 * NREP, 2) void attn_prefill_kernel(AttnPrefillA
             const u32x4 pf = {pk[ti][4 * t], pk[ti][4 * t + 1], pk[ti][4 * t + 2], pk[ti][4 * t + 3]};
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt) {
-                const uint8_t* src = vt_lds + (dt * 32 + qi) * kVtRow + ti * 64 + t * 32 + h * 16;
+                const uint8_t* src = vbuf + (dt * 32 + qi) * kVtRow + ti * 64 + t * 32 + h * 16;
                 const u32x2 v0 = *reinterpret_cast<const u32x2*>(src);
                 const u32x2 v1 = *reinterpret_cast<const u32x2*>(src + 8);
                 const u32x4 vf = {v0.x, v0.y, v1.x, v1.y};
@@ -223,6 +239,32 @@ __global__ __launch_bounds__(64 * NREP, 2) void attn_prefill_kernel(AttnPrefillA
                     __builtin_bit_cast(bf16x8, vf), __builtin_bit_cast(bf16x8, pf), o[dt], 0, 0, 0);
             }
         }
+    };
+
+    // Two LDS buffers: while block kb is multiplied out of one, block kb+1 goes into the
+    // other (keys by DMA, values from the registers filled an iteration earlier) and the
+    // values of block kb+2 are requested; one barrier per block.
+    const int nfull = min(nkb, (__builtin_amdgcn_readfirstlane(pmin) + 1) / kKB);  // blocks every query sees whole
+    dma_k(0, 0);
+    fetch_v(0);
+    stage_v(0);
+    if (nkb > 1) fetch_v(1);
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): the DMA has landed
+    __syncthreads();
+    for (int kb = 0; kb < nkb; ++kb) {
+        const int cur = kb & 1;
+        if (kb + 1 < nkb) {
+            dma_k(kb + 1, cur ^ 1);
+            stage_v(cur ^ 1);
+        }
+        if (kb + 2 < nkb) fetch_v(kb + 2);
+        const uint8_t* kbuf = lds + cur * kBufBytes;
+        if (kb < nfull)
+            block(std::false_type{}, kb, kbuf, kbuf + kKBytes);
+        else
+            block(std::true_type{}, kb, kbuf, kbuf + kKBytes);
+        __builtin_amdgcn_s_waitcnt(0x0070);
+        __syncthreads();
     }
 
     // ---- normalise and write [batch, seq, heads*128]
