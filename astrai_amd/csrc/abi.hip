@@ -234,6 +234,39 @@ int astrai_w8a8_attn_decode_bf16(const void* q, const void* k_cache, const void*
     return check_launch("attn_decode_bf16");
 }
 
+int astrai_w8a8_attn_paged_decode_bf16(const void* q, const void* k_pool, const void* v_pool,
+                                       const int32_t* req_to_token, const int32_t* req_pool_indices,
+                                       const int32_t* kv_indptr, float* workspace,
+                                       int64_t workspace_floats, void* out, int64_t batch,
+                                       int64_t n_heads, int64_t n_kv_heads, int64_t head_dim,
+                                       int64_t num_slots, int64_t num_requests,
+                                       int64_t max_context_len, int64_t nsplit, float scale,
+                                       void* stream) {
+    if (!q || !k_pool || !v_pool || !req_to_token || !req_pool_indices || !kv_indptr || !workspace || !out)
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_decode_bf16: null pointer");
+    if (batch < 0 || n_heads <= 0 || n_kv_heads <= 0 || num_slots <= 0 || num_requests <= 0 ||
+        max_context_len <= 0 || nsplit <= 0 || nsplit > 64 || batch > 65535 || n_heads % n_kv_heads ||
+        num_slots > INT32_MAX || max_context_len > INT32_MAX)
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_decode_bf16: bad dims");
+    if (head_dim != 128 || n_heads / n_kv_heads > 8 || n_heads > 64)
+        return fail(ASTRAI_W8A8_UNSUPPORTED,
+                    "attn_paged_decode_bf16: needs head_dim 128, n_heads / n_kv_heads <= 8, n_heads <= 64");
+    if (!aligned16(q) || !aligned16(k_pool) || !aligned16(v_pool) || !aligned16(out))
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_decode_bf16: pointers must be 16-byte aligned");
+    if (batch == 0) return ASTRAI_W8A8_OK;
+    const int64_t need = w8a8::attn_decode_workspace_floats((int)batch, (int)n_kv_heads, (int)nsplit,
+                                                            (int)(n_heads / n_kv_heads));
+    if (workspace_floats < need)
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_decode_bf16: workspace too small (%lld floats needed)",
+                    (long long)need);
+    w8a8::AttnDecodeArgs a{q, k_pool, v_pool, nullptr, workspace, out, nullptr, nullptr, (int)batch, 1,
+                           (int)n_heads, (int)n_kv_heads, (int)head_dim, max_context_len, (int)nsplit, scale,
+                           req_to_token, req_pool_indices, kv_indptr, max_context_len, num_slots, num_requests};
+    if (!w8a8::launch_attn_decode(a, static_cast<hipStream_t>(stream)))
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "attn_paged_decode_bf16: shape not supported");
+    return check_launch("attn_paged_decode_bf16");
+}
+
 int astrai_w8a8_attn_prefill_bf16(const void* q, const void* k_cache, const void* v_cache,
                                   const int64_t* positions, void* out, int64_t batch, int64_t seq,
                                   int64_t n_heads, int64_t n_kv_heads, int64_t head_dim,

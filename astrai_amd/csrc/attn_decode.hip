@@ -41,7 +41,15 @@ __device__ __forceinline__ float lane_read(float v, int src_lane) {
 // workspace per (batch, kv head, split): NQ rows of [kD values | max | sum]
 constexpr int kWsRow = kD + 2;
 
-template <int NQ>
+__device__ __forceinline__ int lane_read_i(int v, int src_lane) {
+    return __builtin_amdgcn_ds_bpermute(src_lane << 2, v);
+}
+
+// PAGED: the caches are token-granular pools [slots, n_kv_heads, 128] and key j of
+// sequence b lives in slot req_to_token[req_pool_indices[b]][j]
+// (csrc/kernels/attention/layout_policies.cuh:174-232); every sequence has its own
+// length kv_indptr[b+1] - kv_indptr[b] and one query token, the newest.
+template <int NQ, bool PAGED>
 __global__ __launch_bounds__(256) void attn_decode_partial_kernel(AttnDecodeArgs a) {
     __shared__ float sh_acc[4][NQ][kD];
     __shared__ float sh_ml[4][NQ][2];
@@ -58,10 +66,20 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(AttnDecodeArgs
     // this lane's query row (for the score columns): rep, token, position
     const bool q_live = c16 < nq;
     const int q_rep = q_live ? c16 / a.seq : 0, q_s = q_live ? c16 % a.seq : 0;
-    const int64_t q_pos = q_live ? a.positions[q_s] : -1;
-    int64_t kmax = -1;
-    for (int s = 0; s < a.seq; ++s) kmax = max(kmax, (int64_t)a.positions[s]);
-    kmax = min(kmax, (int64_t)a.max_len - 1);
+    int64_t q_pos, kmax = -1;
+    [[maybe_unused]] const int* table = nullptr;
+    if constexpr (PAGED) {
+        const int64_t len = (int64_t)a.kv_indptr[b + 1] - a.kv_indptr[b];
+        const int64_t req = a.req_pool_indices[b];
+        const bool req_ok = req >= 0 && req < a.num_requests;  // a bad row reads as an empty sequence
+        kmax = req_ok ? min(len, a.rtt_stride) - 1 : -1;
+        q_pos = q_live ? kmax : -1;
+        table = a.req_to_token + (req_ok ? req : 0) * a.rtt_stride;
+    } else {
+        q_pos = q_live ? a.positions[q_s] : -1;
+        for (int s = 0; s < a.seq; ++s) kmax = max(kmax, (int64_t)a.positions[s]);
+        kmax = min(kmax, (int64_t)a.max_len - 1);
+    }
     const int tiles_total = (int)((kmax + 16) >> 4);  // keys 0..kmax
     const int tps = (tiles_total + a.nsplit - 1) / a.nsplit;
     const int t0 = split * tps, t1 = min(t0 + tps, tiles_total);
@@ -75,8 +93,8 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(AttnDecodeArgs
         for (int st = 0; st < 4; ++st)
             qf[st] = q_live ? *reinterpret_cast<const u32x4*>(qrow + 32 * st + 8 * g) : u32x4{0, 0, 0, 0};
     }
-    const int64_t head_off = ((int64_t)b * a.n_kv_heads + hk) * a.max_len * kD;
-    const uint32_t head_bytes = (uint32_t)a.max_len * kD * 2u;
+    const int64_t head_off = PAGED ? 0 : ((int64_t)b * a.n_kv_heads + hk) * a.max_len * kD;
+    const uint32_t head_bytes = PAGED ? 0u : (uint32_t)a.max_len * kD * 2u;
     const __amdgpu_buffer_rsrc_t rk = make_rsrc(static_cast<const uint16_t*>(a.k_cache) + head_off, head_bytes);
     const __amdgpu_buffer_rsrc_t rv = make_rsrc(static_cast<const uint16_t*>(a.v_cache) + head_off, head_bytes);
 
@@ -87,18 +105,46 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(AttnDecodeArgs
 #pragma unroll
         for (int d = 0; d < 8; ++d) acc[q][d] = 0.0f;
 
+    // paged: slot of key 16t + c16, looked up one tile ahead of its use (-1: not attended)
+    auto key_slot = [&](int t) -> int {
+        const int key = (t << 4) + c16;
+        const int slot = (t < t1 && key <= kmax) ? table[key] : -1;
+        return slot < a.num_slots ? slot : -1;
+    };
+    [[maybe_unused]] int slot_next = -1;
+    if constexpr (PAGED) slot_next = key_slot(t0 + wave);
+    const int64_t pool_row = (int64_t)a.n_kv_heads * kD;  // elements from one slot to the next
+
     for (int t = t0 + wave; t < t1; t += 4) {
         const int kb = t << 4;
-        // keys as MFMA rows: lane -> key kb + c16, dims 32*step + 8g
-        u32x4 kf[4];
+        u32x4 kf[4], vf[4];
+        [[maybe_unused]] int vslot[4] = {0, 0, 0, 0};
+        if constexpr (PAGED) {
+            const int slot = slot_next;
+            slot_next = key_slot(t + 4);
+            const u32x4 zero = {0u, 0u, 0u, 0u};
+            const uint16_t* kr = static_cast<const uint16_t*>(a.k_cache) +
+                                 (int64_t)max(slot, 0) * pool_row + hk * kD + 8 * g;
 #pragma unroll
-        for (int st = 0; st < 4; ++st)
-            kf[st] = buf_load16(rk, (uint32_t)(kb + c16) * (kD * 2) + (32 * st + 8 * g) * 2, 0);
-        // values: lane -> key kb + 4g + i, dims 8*c16
-        u32x4 vf[4];
+            for (int st = 0; st < 4; ++st)
+                kf[st] = slot >= 0 ? *reinterpret_cast<const u32x4*>(kr + 32 * st) : zero;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            vf[i] = buf_load16(rv, (uint32_t)(kb + 4 * g + i) * (kD * 2) + c16 * 16, 0);
+            for (int i = 0; i < 4; ++i) {
+                vslot[i] = lane_read_i(slot, 4 * g + i);  // lanes 0..15 hold keys kb..kb+15
+                const uint16_t* vr = static_cast<const uint16_t*>(a.v_cache) +
+                                     (int64_t)max(vslot[i], 0) * pool_row + hk * kD + c16 * 8;
+                vf[i] = vslot[i] >= 0 ? *reinterpret_cast<const u32x4*>(vr) : zero;
+            }
+        } else {
+            // keys as MFMA rows: lane -> key kb + c16, dims 32*step + 8g
+#pragma unroll
+            for (int st = 0; st < 4; ++st)
+                kf[st] = buf_load16(rk, (uint32_t)(kb + c16) * (kD * 2) + (32 * st + 8 * g) * 2, 0);
+            // values: lane -> key kb + 4g + i, dims 8*c16
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                vf[i] = buf_load16(rv, (uint32_t)(kb + 4 * g + i) * (kD * 2) + c16 * 16, 0);
+        }
 
         f32x4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -109,7 +155,8 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(AttnDecodeArgs
         float tm = kNegBig;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const bool ok = q_live && (int64_t)(kb + 4 * g + i) <= q_pos;
+            bool ok = q_live && (int64_t)(kb + 4 * g + i) <= q_pos;
+            if constexpr (PAGED) ok = ok && vslot[i] >= 0;  // negative slot: padding, not attended
             sc[i] = ok ? sc[i] * a.scale : kNegBig;
             tm = fmaxf(tm, sc[i]);
         }
@@ -284,11 +331,19 @@ bool launch_attn_decode(const AttnDecodeArgs& a, hipStream_t stream) {
     if (a.n_heads * kD > kMergeCache * 256 * 8) return false;  // the merge kernel keeps a token's row in registers
     const unsigned grid1 = (unsigned)(a.batch * a.n_kv_heads * a.nsplit);
     const unsigned grid2 = (unsigned)(a.batch * a.seq);
+    const bool paged = a.req_to_token != nullptr;
+    if (paged && (a.seq != 1 || !a.req_pool_indices || !a.kv_indptr || a.rtt_stride <= 0)) return false;
     if (nq <= 4) {
-        attn_decode_partial_kernel<4><<<dim3(grid1), dim3(256), 0, stream>>>(a);
+        if (paged)
+            attn_decode_partial_kernel<4, true><<<dim3(grid1), dim3(256), 0, stream>>>(a);
+        else
+            attn_decode_partial_kernel<4, false><<<dim3(grid1), dim3(256), 0, stream>>>(a);
         attn_decode_merge_kernel<4><<<dim3(grid2), dim3(256), 0, stream>>>(a);
     } else {
-        attn_decode_partial_kernel<8><<<dim3(grid1), dim3(256), 0, stream>>>(a);
+        if (paged)
+            attn_decode_partial_kernel<8, true><<<dim3(grid1), dim3(256), 0, stream>>>(a);
+        else
+            attn_decode_partial_kernel<8, false><<<dim3(grid1), dim3(256), 0, stream>>>(a);
         attn_decode_merge_kernel<8><<<dim3(grid2), dim3(256), 0, stream>>>(a);
     }
     return true;

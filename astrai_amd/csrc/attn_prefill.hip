@@ -60,7 +60,7 @@ __device__ __forceinline__ int vt_slot(int w) {
 }
 
 template <int NREP>
-__global__ __launch_bounds__(64 * NREP, 2) void attn_prefill_kernel(AttnPrefillArgs a) {
+__global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_kernel(AttnPrefillArgs a) {
     constexpr int THREADS = 64 * NREP;
     constexpr int K_DMA = kKB / 4 / NREP;              // 1 KiB key loads per wave and block
     constexpr int V_ITEMS = (kKB / 2) * 16 / THREADS;  // (key pair, 8-dim chunk) items per thread

@@ -81,6 +81,13 @@ struct AttnDecodeArgs {
     int64_t max_len;
     int nsplit;
     float scale;
+    // paged mode (req_to_token != null): seq == 1, the caches are pools [slots, n_kv_heads, 128],
+    // positions is unused and every sequence has its own length
+    const int* req_to_token;      // int32 [requests, rtt_stride]: slot of (request, position)
+    const int* req_pool_indices;  // int32 [batch]: row of req_to_token of each sequence
+    const int* kv_indptr;         // int32 [batch + 1]: prefix sums of the sequence lengths
+    int64_t rtt_stride;
+    int64_t num_slots, num_requests;  // table entries / rows outside these are treated as absent
 };
 int64_t attn_decode_workspace_floats(int batch, int n_kv_heads, int nsplit, int nq);
 bool launch_attn_decode(const AttnDecodeArgs& a, hipStream_t stream);

@@ -43,6 +43,9 @@ PROTOTYPES = {
     "astrai_w8a8_rope_cache_write_bf16": (
         [_P, _I64, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _P], _INT),
     "astrai_w8a8_attn_decode_workspace_floats": ([_I64, _I64, _I64, _I64], _I64),
+    "astrai_w8a8_attn_paged_decode_bf16": (
+        [_P, _P, _P, _P, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
+         ctypes.c_float, _P], _INT),
     "astrai_w8a8_attn_prefill_bf16": (
         [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, ctypes.c_float, _P], _INT),
     "astrai_w8a8_attn_decode_bf16": (
@@ -560,6 +563,78 @@ def attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, p
             ws.data_ptr(), ws.numel(), _ptr(out), _ptr(oq), _ptr(os_), b, s, h, hkv, d, max_len, nsplit,
             float(scale), _stream(q)), lib)
     return (oq, os_) if quantized else out
+
+
+def attn_paged_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                      req_to_token: torch.Tensor, req_pool_indices: torch.Tensor,
+                      kv_indptr: torch.Tensor, new_k: Optional[torch.Tensor] = None,
+                      new_v: Optional[torch.Tensor] = None, mask: Optional[torch.Tensor] = None,
+                      causal_offset: int = -1, scale: float = 0.0, o_part_buf=None, ml_part_buf=None,
+                      out_buf: Optional[torch.Tensor] = None, nsplit: int = 0) -> torch.Tensor:
+    """Paged decode attention with the argument list of the reference's pybind entry
+    (csrc/kernels/attention/paged_decode.cu:69-86): ``q [batch, H, 128]``, flat pools
+    ``[slots, H_kv, 128]``, ``req_to_token`` int32 ``[requests, max_context_len]``,
+    ``req_pool_indices`` int32 ``[batch]``, ``kv_indptr`` int32 ``[batch+1]``; returns
+    ``[batch, H, 128]`` bf16. ``new_k`` / ``new_v`` (``[batch, H_kv, 128]``) are first
+    written to the slot of each sequence's newest position, as the reference's kernel
+    persists them (layout_policies.cuh:226-252). ``causal_offset`` does not change a
+    one-token query (layout_policies.cuh:194-197); the split buffers are not needed
+    (the workspace is allocated here); ``mask`` is not supported."""
+    lib = _require()
+    _gpu(q, "attn_paged_decode")
+    if mask is not None:
+        raise RuntimeError("attn_paged_decode: a key mask is not supported")
+    if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
+        raise RuntimeError("q, k_cache and v_cache must be bf16")
+    if q.dim() != 3 or k_cache.dim() != 3 or k_cache.shape != v_cache.shape:
+        raise RuntimeError("q must be [batch, q_head, head_dim] and the pools [size, kv_head, head_dim]")
+    for t, name in ((req_to_token, "req_to_token"), (req_pool_indices, "req_pool_indices"),
+                    (kv_indptr, "kv_indptr")):
+        if t.dtype != torch.int32 or t.device != q.device:
+            raise RuntimeError(f"{name} must be int32 on q's device")
+    b, h, d = q.shape
+    slots, hkv = k_cache.size(0), k_cache.size(1)
+    if k_cache.size(2) != d:
+        raise RuntimeError("k_cache head_dim mismatch")
+    if h % hkv:
+        raise RuntimeError("q_head must be divisible by kv_head")
+    if req_to_token.dim() != 2 or req_pool_indices.numel() != b or kv_indptr.numel() != b + 1:
+        raise RuntimeError("req_to_token must be 2D, req_pool_indices [batch], kv_indptr [batch+1]")
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise RuntimeError("the pools must be contiguous")
+    if (new_k is None) != (new_v is None):
+        raise RuntimeError("new_k and new_v must be provided together")
+    q_c = q.contiguous()
+    rtt, rpi, ind = req_to_token.contiguous(), req_pool_indices.contiguous(), kv_indptr.contiguous()
+    if scale is None or scale <= 0.0:
+        scale = d ** -0.5
+    if nsplit <= 0:
+        nsplit = max(1, min(16, 1024 // max(1, b * hkv)))
+    with torch.cuda.device(q.device):
+        if new_k is not None:
+            if new_k.shape != (b, hkv, d) or new_v.shape != (b, hkv, d):
+                raise RuntimeError("new K/V shape mismatch")
+            last = (ind[1:] - ind[:-1] - 1).long()
+            dst = rtt[rpi.long(), last.clamp_min(0)].long()
+            live = (last >= 0) & (dst >= 0)
+            dst = torch.where(live, dst, torch.zeros_like(dst))
+            # a sequence of length 0 has no newest position: it rewrites slot 0 with itself
+            k_cache.index_put_((dst,), torch.where(live[:, None, None], new_k, k_cache[dst]))
+            v_cache.index_put_((dst,), torch.where(live[:, None, None], new_v, v_cache[dst]))
+        if out_buf is not None:
+            if not (out_buf.is_cuda and out_buf.is_contiguous() and out_buf.dtype == q.dtype
+                    and out_buf.dim() == 3 and out_buf.size(0) >= b and out_buf.shape[1:] == q.shape[1:]):
+                raise RuntimeError("out_buf must be a contiguous [>=batch, q_head, head_dim] tensor of q's dtype")
+            out = out_buf[:b]
+        else:
+            out = torch.empty((b, h, d), device=q.device, dtype=torch.bfloat16)
+        need = lib.astrai_w8a8_attn_decode_workspace_floats(b, hkv, nsplit, h // hkv)
+        ws = torch.empty(max(need, 1), device=q.device, dtype=torch.float32)
+        _check(lib.astrai_w8a8_attn_paged_decode_bf16(
+            q_c.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), rtt.data_ptr(), rpi.data_ptr(),
+            ind.data_ptr(), ws.data_ptr(), ws.numel(), out.data_ptr(), b, h, hkv, d, slots,
+            rtt.size(0), rtt.size(1), nsplit, float(scale), _stream(q)), lib)
+    return out
 
 
 def attn_prefill_supported(n_heads: int, n_kv_heads: int, head_dim: int) -> bool:

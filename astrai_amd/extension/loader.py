@@ -52,7 +52,13 @@ def _fp8_block_mm_module() -> SimpleNamespace:
     )
 
 
+def _attn_paged_decode_module() -> SimpleNamespace:
+    # the callable of csrc/kernels/attention/paged_decode.cu:69-86, same argument list
+    return SimpleNamespace(attn_paged_decode=_cabi.attn_paged_decode)
+
+
 _FACTORIES = {
+    "attn_paged_decode": _attn_paged_decode_module,
     "fp8_mm": _fp8_mm_module,
     "int8_mm": _int8_mm_module,
     "fp8_block_mm": _fp8_block_mm_module,

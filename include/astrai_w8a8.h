@@ -188,6 +188,32 @@ int astrai_w8a8_attn_decode_bf16(const void* q_bf16, const void* k_cache_bf16, c
                                  int64_t nsplit, float scale, void* stream);
 
 /*
+ * The same decode attention over a token-granular paged cache. Replaces
+ * attn_paged_decode (csrc/kernels/attention/paged_decode.cu:4-67, addressing policy
+ * PagedKV in csrc/kernels/attention/layout_policies.cuh:174-232; Python wrapper
+ * astrai/extension/ops/attention.py:93-147) without its fused append of new_k / new_v
+ * and without the optional key mask.
+ *   q          bf16 [batch, n_heads, 128]: the newest token of every sequence
+ *   k_pool, v_pool  bf16 [num_slots, n_kv_heads, 128]
+ *   req_to_token    int32 [num_requests, max_context_len]: pool slot of (request, position);
+ *              negative entries (and entries >= num_slots) are not attended
+ *   req_pool_indices  int32 [batch]: row of req_to_token of each sequence
+ *   kv_indptr  int32 [batch + 1]: prefix sums of the sequence lengths; sequence b attends
+ *              positions 0 .. kv_indptr[b+1] - kv_indptr[b] - 1
+ *   workspace  as for attn_decode_bf16 with n_query_rows = n_heads / n_kv_heads
+ *   out        bf16 [batch, n_heads, 128]; a sequence of length 0 yields zeros
+ * head_dim == 128, n_heads / n_kv_heads <= 8, n_heads <= 64.
+ */
+int astrai_w8a8_attn_paged_decode_bf16(const void* q_bf16, const void* k_pool_bf16,
+                                       const void* v_pool_bf16, const int32_t* req_to_token,
+                                       const int32_t* req_pool_indices, const int32_t* kv_indptr,
+                                       float* workspace, int64_t workspace_floats, void* out_bf16,
+                                       int64_t batch, int64_t n_heads, int64_t n_kv_heads,
+                                       int64_t head_dim, int64_t num_slots, int64_t num_requests,
+                                       int64_t max_context_len, int64_t nsplit, float scale,
+                                       void* stream);
+
+/*
  * Causal grouped-query attention of a block of `seq` new tokens per sequence against
  * the dense KV cache (prefill, whole or chunked). Replaces the same reference code as
  * attn_decode_bf16 for long query blocks: head expansion

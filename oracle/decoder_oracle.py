@@ -75,6 +75,31 @@ def attn_cached(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
     return out.permute(0, 2, 1, 3).reshape(b, s, h * d).to(q.dtype)
 
 
+def attn_paged_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                      req_to_token: torch.Tensor, req_pool_indices: torch.Tensor,
+                      kv_indptr: torch.Tensor) -> torch.Tensor:
+    """Decode attention over a token-granular paged cache: ``q [B, H, D]``, pools
+    ``[slots, H_kv, D]``; key ``j`` of sequence ``b`` is pool row
+    ``req_to_token[req_pool_indices[b], j]`` for ``j < kv_indptr[b+1] - kv_indptr[b]``,
+    negative rows are skipped (csrc/kernels/attention/layout_policies.cuh:174-232;
+    astrai/extension/ops/attention.py:93-147). ``softmax(q k^T / sqrt(D)) v`` in float32 per
+    sequence, a sequence without keys gives zeros. Returns ``[B, H, D]`` in the input dtype."""
+    b, h, d = q.shape
+    n_rep = h // k_pool.size(1)
+    out = torch.zeros(b, h, d, dtype=torch.float32)
+    for i in range(b):
+        n = int(kv_indptr[i + 1]) - int(kv_indptr[i])
+        rows = req_to_token[int(req_pool_indices[i]), :n].long()
+        rows = rows[rows >= 0]
+        if rows.numel() == 0:
+            continue
+        k = k_pool[rows].float().repeat_interleave(n_rep, dim=1)      # [n, H, D]
+        v = v_pool[rows].float().repeat_interleave(n_rep, dim=1)
+        scores = torch.einsum("hd,nhd->hn", q[i].float(), k) / (d ** 0.5)
+        out[i] = torch.einsum("hn,nhd->hd", torch.softmax(scores, dim=-1), v)
+    return out.to(q.dtype)
+
+
 def repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:
     # x: [B, S, H_kv, D] -> [B, S, H_kv*n_rep, D]
     if n_rep == 1:

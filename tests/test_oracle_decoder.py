@@ -126,3 +126,46 @@ def test_rope_cache_write_is_the_tensor_op_chain():
     torch.testing.assert_close(kc[0, 0, 4], torch.stack([-kx[1], kx[0], -kx[3], kx[2]]))
     torch.testing.assert_close(vc[0, 0, 1], qkv[0, 0, (h + hkv) * d:])
     assert (kc[0, 0, [0, 2, 3]] == -1).all() and (vc[0, 0, [0, 2, 3]] == -1).all()
+
+
+def test_paged_decode_oracle_equals_dense_attention_on_a_scattered_cache():
+    """Scatter a dense cache into a pool through a random slot table: the paged oracle must
+    reproduce the dense one (attn_cached) for every sequence length, including the unused
+    tail of each request row and rows of other requests in between."""
+    g = torch.Generator().manual_seed(12)
+    b, h, hkv, d, max_ctx = 3, 8, 2, 16, 20
+    lens = [20, 7, 1]
+    pool = 97
+    q = torch.randn(b, h, d, generator=g).to(torch.bfloat16)
+    dense_k = torch.randn(b, hkv, max_ctx, d, generator=g).to(torch.bfloat16)
+    dense_v = torch.randn(b, hkv, max_ctx, d, generator=g).to(torch.bfloat16)
+    perm = torch.randperm(pool, generator=g)
+    rows = torch.tensor([4, 0, 2])                       # request rows in a table of 5
+    table = torch.full((5, max_ctx), -1, dtype=torch.int32)
+    k_pool = torch.randn(pool, hkv, d, generator=g).to(torch.bfloat16)   # other tenants' data
+    v_pool = torch.randn(pool, hkv, d, generator=g).to(torch.bfloat16)
+    nxt = 0
+    for i in range(b):
+        for j in range(lens[i]):
+            slot = int(perm[nxt]); nxt += 1
+            table[rows[i], j] = slot
+            k_pool[slot] = dense_k[i, :, j]
+            v_pool[slot] = dense_v[i, :, j]
+    indptr = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    got = D.attn_paged_decode(q, k_pool, v_pool, table, rows.int(), indptr)
+    for i in range(b):
+        want = D.attn_cached(q[i:i + 1].unsqueeze(2), dense_k[i:i + 1], dense_v[i:i + 1],
+                             torch.tensor([lens[i] - 1]))
+        assert torch.equal(got[i].reshape(-1), want.reshape(-1)), i
+
+
+def test_paged_decode_oracle_single_key_and_empty_sequence():
+    """one visible key: the output is that key's value row; no key: zeros"""
+    q = torch.randn(2, 4, 8).to(torch.bfloat16)
+    k_pool = torch.randn(6, 2, 8).to(torch.bfloat16)
+    v_pool = torch.randn(6, 2, 8).to(torch.bfloat16)
+    table = torch.tensor([[5, -1, -1], [3, 1, 2]], dtype=torch.int32)
+    out = D.attn_paged_decode(q, k_pool, v_pool, table, torch.tensor([0, 1], dtype=torch.int32),
+                              torch.tensor([0, 1, 1], dtype=torch.int32))
+    assert torch.equal(out[0], v_pool[5].repeat_interleave(2, dim=0))
+    assert torch.equal(out[1], torch.zeros(4, 8, dtype=torch.bfloat16))
