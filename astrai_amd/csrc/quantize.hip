@@ -70,6 +70,23 @@ __device__ __forceinline__ float block_max(float v, float* slots) {
 }
 
 // ---- per-tensor fp8 -------------------------------------------------------
+// Kernels that report a tensor-wide amax end in an atomic per workgroup on one
+// address, and those are served one after the other (~10 ns each: thousands of
+// workgroups finishing together queue for tens of microseconds). So one workgroup
+// in kEarlyEvery publishes the maximum of its first group of vectors early -- a few
+// dozen atomics that have drained long before the tensor has streamed -- and at the
+// end a workgroup touches the slot only if its share has outgrown what the slot
+// holds by then, which a few dozen out of a thousand do on unsorted data.
+constexpr int kAmaxBlocks = 1024;  // grid cap: the workgroups stride over the tensor
+constexpr int kUnroll = 4;         // independent 16-byte loads in flight per thread
+constexpr int kEarlyEvery = 16;
+
+__device__ __forceinline__ void publish_early(float* amax, float local, float* slots) {
+    const float m = block_max(local, slots);
+    if (threadIdx.x == 0 && m > 0.0f)
+        atomicMax(reinterpret_cast<unsigned int*>(amax), __float_as_uint(m));
+}
+
 template <int Fmt>
 __global__ __launch_bounds__(kThreads) void quantize_fp8_kernel(
     const uint16_t* __restrict__ x, uint8_t* __restrict__ x8, const float* __restrict__ scale,
@@ -79,7 +96,26 @@ __global__ __launch_bounds__(kThreads) void quantize_fp8_kernel(
     float local = 0.0f;
     const int64_t nvec = total >> 3;
     const int64_t stride = (int64_t)gridDim.x * kThreads;
-    for (int64_t v = (int64_t)blockIdx.x * kThreads + threadIdx.x; v < nvec; v += stride) {
+    int64_t v = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    auto group = [&](int64_t v0) {
+        u32x4 raw[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) raw[u] = *reinterpret_cast<const u32x4*>(x + (v0 + u * stride) * 8);
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            float f[8];
+            unpack8(raw[u], f);
+            local = fmaxf(local, amax8(f));
+            *reinterpret_cast<u32x2*>(x8 + (v0 + u * stride) * 8) = quant8_fp8<Fmt>(f, step);
+        }
+    };
+    if (v + (kUnroll - 1) * stride < nvec) {
+        group(v);
+        v += kUnroll * stride;
+    }
+    if (amax && gridDim.x >= 64 && blockIdx.x % kEarlyEvery == 0) publish_early(amax, local, slots);
+    for (; v + (kUnroll - 1) * stride < nvec; v += kUnroll * stride) group(v);
+    for (; v < nvec; v += stride) {
         float f[8];
         unpack8(*reinterpret_cast<const u32x4*>(x + v * 8), f);
         local = fmaxf(local, amax8(f));
@@ -109,7 +145,25 @@ __global__ __launch_bounds__(kThreads) void amax_bf16_kernel(
     float local = 0.0f;
     const int64_t nvec = total >> 3;
     const int64_t stride = (int64_t)gridDim.x * kThreads;
-    for (int64_t v = (int64_t)blockIdx.x * kThreads + threadIdx.x; v < nvec; v += stride) {
+    int64_t v = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    auto group = [&](int64_t v0) {
+        u32x4 raw[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) raw[u] = *reinterpret_cast<const u32x4*>(x + (v0 + u * stride) * 8);
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            float f[8];
+            unpack8(raw[u], f);
+            local = fmaxf(local, amax8(f));
+        }
+    };
+    if (v + (kUnroll - 1) * stride < nvec) {
+        group(v);
+        v += kUnroll * stride;
+    }
+    if (gridDim.x >= 64 && blockIdx.x % kEarlyEvery == 0) publish_early(amax, local, slots);
+    for (; v + (kUnroll - 1) * stride < nvec; v += kUnroll * stride) group(v);
+    for (; v < nvec; v += stride) {
         float f[8];
         unpack8(*reinterpret_cast<const u32x4*>(x + v * 8), f);
         local = fmaxf(local, amax8(f));
@@ -157,72 +211,83 @@ __global__ __launch_bounds__(kThreads) void quantize_transpose_fp8_kernel(
     const float* __restrict__ scale, float* __restrict__ amax, int64_t rows, int64_t cols) {
     __shared__ __attribute__((aligned(16))) uint8_t tile[kTrCols * kTrPitch];
     __shared__ float slots[kThreads / kWave];
-    const int64_t r0 = (int64_t)blockIdx.y * kTrRows, c0 = (int64_t)blockIdx.x * kTrCols;
     const int cc = threadIdx.x & 15, r4 = threadIdx.x >> 4;
     const float step = *scale;
     const bool vec = (cols & 7) == 0;
-    const int64_t c = c0 + cc * 8;
+    const bool runs = (rows & 15) == 0;  // 16-byte pieces stay aligned and inside the matrix
+    const int64_t tiles_x = (cols + kTrCols - 1) / kTrCols;
+    const int64_t ntiles = tiles_x * ((rows + kTrRows - 1) / kTrRows);
     float local = 0.0f;
+    for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        const int64_t r0 = (t / tiles_x) * kTrRows, c0 = (t % tiles_x) * kTrCols;
+        const int64_t c = c0 + cc * 8;
 #pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
-        u32x2 q[4];
+        for (int pass = 0; pass < 2; ++pass) {
+            u32x2 q[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int64_t r = r0 + pass * 64 + r4 * 4 + i;
-            float f[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-            const bool whole = vec && r < rows && c < cols;
-            if (whole) {
-                unpack8(*reinterpret_cast<const u32x4*>(x + r * cols + c), f);
-            } else if (r < rows) {
-#pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    if (c + j < cols) f[j] = bf16_to_f32(x[r * cols + c + j]);
-            }
-            local = fmaxf(local, amax8(f));
-            q[i] = quant8_fp8<Fmt>(f, step);
-            if (x8) {
+            for (int i = 0; i < 4; ++i) {
+                const int64_t r = r0 + pass * 64 + r4 * 4 + i;
+                float f[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+                const bool whole = vec && r < rows && c < cols;
                 if (whole) {
-                    *reinterpret_cast<u32x2*>(x8 + r * cols + c) = q[i];
+                    unpack8(*reinterpret_cast<const u32x4*>(x + r * cols + c), f);
                 } else if (r < rows) {
 #pragma unroll
                     for (int j = 0; j < 8; ++j)
-                        if (c + j < cols)
-                            x8[r * cols + c + j] =
-                                (uint8_t)(((j < 4 ? q[i].x : q[i].y) >> ((j & 3) * 8)) & 0xffu);
+                        if (c + j < cols) f[j] = bf16_to_f32(x[r * cols + c + j]);
+                }
+                local = fmaxf(local, amax8(f));
+                q[i] = quant8_fp8<Fmt>(f, step);
+                if (x8) {
+                    if (whole) {
+                        *reinterpret_cast<u32x2*>(x8 + r * cols + c) = q[i];
+                    } else if (r < rows) {
+#pragma unroll
+                        for (int j = 0; j < 8; ++j)
+                            if (c + j < cols)
+                                x8[r * cols + c + j] =
+                                    (uint8_t)(((j < 4 ? q[i].x : q[i].y) >> ((j & 3) * 8)) & 0xffu);
+                    }
                 }
             }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                uint32_t d = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    d |= (((j < 4 ? q[i].x : q[i].y) >> ((j & 3) * 8)) & 0xffu) << (8 * i);
+                *reinterpret_cast<uint32_t*>(tile + (cc * 8 + j) * kTrPitch + pass * 64 + r4 * 4) = d;
+            }
         }
+        __syncthreads();
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            uint32_t d = 0;
+        for (int h = 0; h < 4; ++h) {
+            const int cl = (threadIdx.x >> 3) + 32 * h;
+            const int64_t ct = c0 + cl, rt = r0 + (threadIdx.x & 7) * 16;
+            if (ct >= cols || rt >= rows) continue;
+            const uint8_t* src = tile + cl * kTrPitch + (threadIdx.x & 7) * 16;
+            u32x4 v;
+            v.x = *reinterpret_cast<const uint32_t*>(src);
+            v.y = *reinterpret_cast<const uint32_t*>(src + 4);
+            v.z = *reinterpret_cast<const uint32_t*>(src + 8);
+            v.w = *reinterpret_cast<const uint32_t*>(src + 12);
+            if (runs) {
+                *reinterpret_cast<u32x4*>(x8t + ct * rows + rt) = v;
+            } else {
+                const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                d |= (((j < 4 ? q[i].x : q[i].y) >> ((j & 3) * 8)) & 0xffu) << (8 * i);
-            *reinterpret_cast<uint32_t*>(tile + (cc * 8 + j) * kTrPitch + pass * 64 + r4 * 4) = d;
+                for (int b = 0; b < 16; ++b)
+                    if (rt + b < rows)
+                        x8t[ct * rows + rt + b] = (uint8_t)((w[b >> 2] >> ((b & 3) * 8)) & 0xffu);
+            }
         }
-    }
-    __syncthreads();
-    const bool runs = (rows & 15) == 0;  // 16-byte pieces stay aligned and inside the matrix
-#pragma unroll
-    for (int h = 0; h < 4; ++h) {
-        const int cl = (threadIdx.x >> 3) + 32 * h;
-        const int64_t ct = c0 + cl, rt = r0 + (threadIdx.x & 7) * 16;
-        if (ct >= cols || rt >= rows) continue;
-        const uint8_t* src = tile + cl * kTrPitch + (threadIdx.x & 7) * 16;
-        u32x4 v;
-        v.x = *reinterpret_cast<const uint32_t*>(src);
-        v.y = *reinterpret_cast<const uint32_t*>(src + 4);
-        v.z = *reinterpret_cast<const uint32_t*>(src + 8);
-        v.w = *reinterpret_cast<const uint32_t*>(src + 12);
-        if (runs) {
-            *reinterpret_cast<u32x4*>(x8t + ct * rows + rt) = v;
-        } else {
-            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-            for (int b = 0; b < 16; ++b)
-                if (rt + b < rows)
-                    x8t[ct * rows + rt + b] = (uint8_t)((w[b >> 2] >> ((b & 3) * 8)) & 0xffu);
-        }
+        // the first tile's maximum goes out early when more tiles follow (block_max also
+        // separates this tile's LDS reads from the next tile's writes)
+        if (amax && t == blockIdx.x && t + gridDim.x < ntiles && gridDim.x >= 64 &&
+            blockIdx.x % kEarlyEvery == 0)
+            publish_early(amax, local, slots);
+        else
+            __syncthreads();
     }
     if (amax) {
         const float m = block_max(local, slots);
@@ -467,9 +532,9 @@ void launch_quantize_fp8(const void* x, void* x8, const float* scale, float* ama
                          int64_t total, int fmt, hipStream_t stream) {
     if (total <= 0) return;
     const int64_t nvec = (total + 7) / 8;
-    int64_t blocks = (nvec + kThreads - 1) / kThreads;
-    // enough workgroups to fill 256 CUs several times over, grid-stride beyond that
-    if (blocks > 256 * 16) blocks = 256 * 16;
+    // two groups of kUnroll vectors per thread where the tensor is large enough
+    int64_t blocks = (nvec + 2 * kUnroll * kThreads - 1) / (2 * kUnroll * kThreads);
+    if (blocks > kAmaxBlocks) blocks = kAmaxBlocks;
     auto xs = static_cast<const uint16_t*>(x);
     auto xo = static_cast<uint8_t*>(x8);
     if (fmt)
@@ -488,8 +553,8 @@ void launch_amax_ring_push(float* hist, int n, int idx, const float* amax, float
 
 void launch_amax_bf16(const void* x, float* amax, int64_t total, hipStream_t stream) {
     if (total <= 0) return;
-    int64_t blocks = ((total + 7) / 8 + kThreads - 1) / kThreads;
-    if (blocks > 256 * 8) blocks = 256 * 8;
+    int64_t blocks = ((total + 7) / 8 + 2 * kUnroll * kThreads - 1) / (2 * kUnroll * kThreads);
+    if (blocks > kAmaxBlocks) blocks = kAmaxBlocks;
     amax_bf16_kernel<<<dim3((unsigned)blocks), dim3(kThreads), 0, stream>>>(
         static_cast<const uint16_t*>(x), amax, total);
 }
@@ -498,7 +563,9 @@ void launch_quantize_transpose_fp8(const void* x, void* x8, void* x8t, const flo
                                    float* amax, int64_t rows, int64_t cols, int fmt,
                                    hipStream_t stream) {
     if (rows <= 0 || cols <= 0) return;
-    const dim3 grid((unsigned)((cols + kTrCols - 1) / kTrCols), (unsigned)((rows + kTrRows - 1) / kTrRows));
+    // two or more tiles per workgroup once there are enough tiles to fill the chip
+    const int64_t ntiles = ((cols + kTrCols - 1) / kTrCols) * ((rows + kTrRows - 1) / kTrRows);
+    const dim3 grid((unsigned)(ntiles <= 256 ? ntiles : (ntiles < 1024 ? (ntiles + 1) / 2 : 512)));
     auto* xi = static_cast<const uint16_t*>(x);
     auto* o = static_cast<uint8_t*>(x8);
     auto* ot = static_cast<uint8_t*>(x8t);

@@ -164,6 +164,9 @@ def main():
     ap.add_argument("--decoder-trace", choices=["modular", "fused"], default=None,
                     help="tracing mode: build the config-4 decoder (Linear-by-Linear int8 path, or the fused "
                          "one), one prefill + 19 eager decode steps, nothing else")
+    ap.add_argument("--trace-kernels", action="store_true",
+                    help="tracing mode: a few launches of every auxiliary kernel (quantizers, policy-path "
+                         "kernels, attention) at the sizes DESIGN.md quotes, nothing else")
     ap.add_argument("--pmc", action="store_true",
                     help="counter-collection mode: a few launches of the headline kernel and of a "
                          "plain 256 MiB device copy (the calibration kernel), nothing else")
@@ -206,6 +209,40 @@ def main():
             greedy_generate(model, ids, 20, use_graph=False)
         torch.cuda.synchronize()
         print(json.dumps({"decoder_trace": args.decoder_trace, "prefill_tokens": 32 * 512, "decode_steps": 19}))
+        return
+
+    if args.trace_kernels:
+        from astrai_amd.extension import get_module
+
+        fp8m = get_module("fp8_mm")
+        x = torch.randn(4096, 4096, device=dev).to(torch.bfloat16)
+        s1 = torch.full((1,), 4.0 / 448.0, device=dev)
+        hist, scale = torch.ones(16, device=dev), torch.ones(1, device=dev)
+        b_, h_, hkv_, s_, n_ = 32, 16, 4, 512, 640
+        q = torch.randn(b_, h_, s_, 128, device=dev).to(torch.bfloat16)
+        kc = torch.randn(b_, hkv_, n_, 128, device=dev).to(torch.bfloat16)
+        vc = torch.randn(b_, hkv_, n_, 128, device=dev).to(torch.bfloat16)
+        pos = torch.arange(s_, device=dev)
+        q1 = q[:, :, -1:].contiguous()
+        last = torch.tensor([n_ - 1], device=dev)
+        k_pool = kc.permute(0, 2, 1, 3).reshape(b_ * n_, hkv_, 128).contiguous()
+        v_pool = vc.permute(0, 2, 1, 3).reshape(b_ * n_, hkv_, 128).contiguous()
+        table = torch.randperm(b_ * n_, device=dev).int().reshape(b_, n_).contiguous()
+        rows = torch.arange(b_, dtype=torch.int32, device=dev)
+        indptr = (torch.arange(b_ + 1, device=dev) * n_).int()
+        for _ in range(5):
+            x8, amax = fp8m.quantize_bf16(x, s1, 0)                    # quantize_fp8_kernel
+            fp8m.quantize_transpose_bf16(x, s1, 0, True, True)         # quantize_transpose_fp8_kernel
+            fp8m.amax_bf16(x)                                          # amax_bf16_kernel
+            fp8m.amax_ring_push(hist, 3, amax, scale, 448.0, 1.0)      # amax_ring_push_kernel
+            _cabi.quantize_int8_rows(x)                                # quantize_int8_rows_kernel
+            _cabi.attn_prefill(q, kc, vc, pos)                         # attn_prefill_kernel
+            _cabi.attn_decode(q1, kc, vc, last)                        # attn_decode_partial/merge (dense)
+            _cabi.attn_paged_decode(q1.reshape(b_, h_, 128), k_pool, v_pool, table, rows, indptr)
+        torch.cuda.synchronize()
+        print(json.dumps({"trace_kernels": "5 launches each; sizes: 4096x4096 bf16 for the quantizers, "
+                                           "32 x 16/4 heads x 512 new tokens x 128 for prefill attention, "
+                                           "32 sequences x 640 keys for decode attention"}))
         return
 
     # ---------------- headline: config 1, fp8 per-tensor 4096^3 ----------------
