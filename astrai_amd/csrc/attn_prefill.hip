@@ -10,19 +10,28 @@
 // output projection reads.
 //
 // One workgroup per (batch, KV head, 32 query tokens); wave r takes query head
-// hk*n_rep + r. Per 64-key block:
+// hk*n_rep + r. Keys are handled in 32-key tiles:
 //   S^T = K.Q^T on v_mfma_f32_32x32x16_bf16 with keys as rows and queries as columns,
-//     so a lane owns ONE query (column lane%32) and 2x16 of its 64 scores: row maxima
+//     so a lane owns ONE query (column lane%32) and 16 of a tile's 32 scores: row maxima
 //     and sums are per-lane reductions plus one exchange with lane^32;
 //   O^T += V^T.P^T with the same instruction: P^T is the S^T accumulator itself,
 //     rounded to bf16 in place (its register order fixes which 8 keys a lane half
-//     contributes per 16-key step), and V^T comes from LDS, where the value tile is
-//     stored transposed with its key slots permuted to that order, 136-byte rows
-//     (conflict-free for the transposing 4-byte writes and the 16-byte operand reads);
-//   keys sit in LDS as 256-byte rows of 16-byte chunks XOR-swizzled by row.
-// Two LDS buffers: while a block is multiplied, the next one arrives (keys by
-// direct-to-LDS loads, values through registers) and the values of the one after are
-// requested; one barrier per block. Blocks that every query of the wave sees whole skip the masking code.
+//     contributes per 16-key step), and the V^T operand is read out of the row-major
+//     value tile with ds_read_b64_tr_b16, the LDS read that hands each lane of a
+//     16-lane group four values down a column (four keys of one dim);
+//   keys and values sit in LDS as 256-byte rows of 16-byte chunks XOR-swizzled by row
+//     (keys by row%16 for the 32-row operand reads, values by 4*(row%4) for the
+//     transposing reads, which touch four consecutive rows at a time).
+// A wave's instruction stream is a software pipeline over tiles, written out and
+// pinned with sched_barrier: the eight score MFMAs of tile T+1 are interleaved with
+// the exponentials of tile T, and the eight P.V MFMAs of tile T with the masking and
+// row maximum of tile T+1, so the matrix pipe and the vector ALU work at the same
+// time inside one wave (a wave issues in order: a softmax phase between two MFMA
+// phases leaves each unit idle while the other runs). Keys and values arrive by
+// direct-to-LDS loads, keys into a ring of four tiles, values into two 64-key buffers,
+// both one 64-key block ahead; one workgroup barrier per block; no staging registers. Tiles that every
+// query of the wave sees whole skip the masking code; the accumulators are rescaled
+// only when a row maximum has outgrown the reference maximum by 2^8.
 #include <climits>
 #include <type_traits>
 
@@ -40,31 +49,24 @@ constexpr int kD = 128;    // head_dim
 constexpr int kQB = 32;    // query tokens per workgroup
 constexpr int kKB = 64;    // keys per block
 constexpr int kKRow = 256;                 // bytes per key row in LDS
-constexpr int kVtRow = 136;                // bytes per value-dim row of V^T in LDS
-constexpr int kKBytes = kKB * kKRow;       // 16 KiB
-constexpr int kVtBytes = kD * kVtRow;      // 17 KiB
-constexpr int kBufBytes = kKBytes + kVtBytes;
+constexpr int kKTileBytes = 32 * kKRow;    // 8 KiB: one 32-key tile
+constexpr int kKRingBytes = 4 * kKTileBytes;
+constexpr int kVBytes = kKB * kKRow;        // 16 KiB: 64 value rows
 constexpr float kNegBig = -1e30f;          // finite stand-in for -inf: no inf - inf
 
-// slot of key w (0..31 within a 32-key tile) in a V^T row: the S^T accumulator of
-// lane half h holds keys 8g' + 4h + j at register 4g' + j; a 16-key MFMA step t takes
-// registers 8t..8t+7, i.e. keys 16t + 8g + 4h + j (g = 0,1) as its k-index 8h + 4g + j.
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+
 __device__ __forceinline__ void lds_dma16(__amdgpu_buffer_rsrc_t r, uint8_t* lds_wave_base,
                                           uint32_t voff, uint32_t soff) {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(
         r, (__attribute__((address_space(3))) void*)lds_wave_base, 16, voff, soff, 0, 0);
 }
 
-__device__ __forceinline__ int vt_slot(int w) {
-    return (w & 16) | ((w & 4) << 1) | ((w & 8) >> 1) | (w & 3);
-}
-
 template <int NREP>
 __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_kernel(AttnPrefillArgs a) {
     constexpr int THREADS = 64 * NREP;
     constexpr int K_DMA = kKB / 4 / NREP;              // 1 KiB key loads per wave and block
-    constexpr int V_ITEMS = (kKB / 2) * 16 / THREADS;  // (key pair, 8-dim chunk) items per thread
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kBufBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kKRingBytes + 2 * kVBytes];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -76,19 +78,11 @@ __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_ker
     const int b = bk / a.n_kv_heads, hk = bk % a.n_kv_heads;
     const int head = hk * NREP + wave;
 
-    // this lane's query token and what it may see
+    // this lane's query token. Its position is requested first and looked at last: the
+    // query rows and the first key tiles do not depend on it.
     const int s_row = qb * kQB + qi;
     const bool row_live = s_row < a.seq;
     int pq = row_live ? (int)a.positions[s_row] : -1;
-    int kmax = pq, pmin = row_live ? pq : INT_MAX;
-#pragma unroll
-    for (int off = 16; off; off >>= 1) {
-        kmax = max(kmax, __shfl_xor(kmax, off, kWave));
-        pmin = min(pmin, __shfl_xor(pmin, off, kWave));
-    }
-    kmax = min(kmax, (int)a.max_len - 1);
-    if (!row_live) pq = kmax;  // rows past the end see everything and are never stored
-    const int nkb = kmax / kKB + 1;
 
     const uint16_t* qrow = static_cast<const uint16_t*>(a.q) +
         (((size_t)b * a.n_heads + head) * a.seq + min(s_row, a.seq - 1)) * kD;
@@ -102,54 +96,56 @@ __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_ker
 
     // keys: straight from the cache into LDS, 1 KiB (four rows) per instruction; lane l
     // lands at row l/16, chunk position l%16 and therefore asks for chunk (l%16) ^ (row%16).
-    // The descriptor ends after key kmax: later rows arrive as zeros.
-    const __amdgpu_buffer_rsrc_t rk = make_rsrc(kc, (uint32_t)(kmax + 1) * (uint32_t)kKRow);
+    // The descriptor covers the whole cache row range: whatever a row past the newest
+    // position holds, its scores are replaced (not scaled) by the mask.
+    const __amdgpu_buffer_rsrc_t rk = make_rsrc(kc, (uint32_t)a.max_len * (uint32_t)kKRow);
     uint32_t k_voff[K_DMA];
 #pragma unroll
     for (int j = 0; j < K_DMA; ++j) {
         const int row = (wave * K_DMA + j) * 4 + (lane >> 4);
         k_voff[j] = (uint32_t)row * kKRow + (uint32_t)(((lane & 15) ^ (row & 15)) << 4);
     }
-    auto dma_k = [&](int kb, int buf) {
+    // tiles t0 and t0+1 (64 keys) into their ring slots
+    auto dma_k = [&](int t0) {
+#pragma unroll
+        for (int j = 0; j < K_DMA; ++j) {
+            const int inst = wave * K_DMA + j;  // 16 instructions of 4 rows; 8 per tile
+            lds_dma16(rk, lds + ((t0 + (inst >> 3)) & 3) * kKTileBytes + (inst & 7) * 4 * kKRow,
+                      k_voff[j] + (uint32_t)t0 * kKTileBytes, 0);
+        }
+    };
+    dma_k(0);
+    dma_k(1);
+
+    // what the block's queries may see
+    int kmax = pq, pmin = row_live ? pq : INT_MAX;
+#pragma unroll
+    for (int off = 16; off; off >>= 1) {
+        kmax = max(kmax, __shfl_xor(kmax, off, kWave));
+        pmin = min(pmin, __shfl_xor(pmin, off, kWave));
+    }
+    // every lane holds the same extremes by now: keep them in scalar registers (loop bounds,
+    // the value descriptor's size)
+    kmax = min(__builtin_amdgcn_readfirstlane(kmax), (int)a.max_len - 1);
+    pmin = __builtin_amdgcn_readfirstlane(pmin);
+    if (!row_live) pq = kmax;  // rows past the end see everything and are never stored
+    const int nkb = kmax / kKB + 1;
+
+    // values: the same way into a 64-row buffer; chunk position (l%16) holds chunk
+    // (l%16) ^ 4*(row%4). Rows past kmax arrive as zeros, so a stale cache row can never
+    // meet a zero probability as 0 * NaN.
+    const __amdgpu_buffer_rsrc_t rv = make_rsrc(vc, (uint32_t)(kmax + 1) * (uint32_t)kKRow);
+    uint32_t v_voff[K_DMA];
+#pragma unroll
+    for (int j = 0; j < K_DMA; ++j) {
+        const int row = (wave * K_DMA + j) * 4 + (lane >> 4);
+        v_voff[j] = (uint32_t)row * kKRow + (uint32_t)(((lane & 15) ^ (4 * (row & 3))) << 4);
+    }
+    auto dma_v = [&](int kb) {
 #pragma unroll
         for (int j = 0; j < K_DMA; ++j)
-            lds_dma16(rk, lds + buf * kBufBytes + (wave * K_DMA + j) * 4 * kKRow,
-                      k_voff[j] + (uint32_t)kb * (kKB * kKRow), 0);
-    };
-    // values: through registers, because they are stored transposed
-    u32x4 vreg[V_ITEMS][2];
-    auto fetch_v = [&](int kb) {
-        const u32x4 zero = {0u, 0u, 0u, 0u};
-#pragma unroll
-        for (int i = 0; i < V_ITEMS; ++i) {
-            const int item = tid + i * THREADS;
-            const int chunk = ((item >> 7) << 2) | (item & 3);
-            const int key = kb * kKB + 2 * ((item >> 2) & 31);
-            const uint16_t* src = vc + (size_t)key * kD + chunk * 8;
-            // keys past kmax may never have been written: they must not reach P.V as 0 * garbage
-            vreg[i][0] = key <= kmax ? *reinterpret_cast<const u32x4*>(src) : zero;
-            vreg[i][1] = key + 1 <= kmax ? *reinterpret_cast<const u32x4*>(src + kD) : zero;
-        }
-    };
-    auto stage_v = [&](int buf) {
-        uint8_t* const vt_lds = lds + buf * kBufBytes + kKBytes;
-#pragma unroll
-        for (int i = 0; i < V_ITEMS; ++i) {
-            const int item = tid + i * THREADS;
-            const int chunk = ((item >> 7) << 2) | (item & 3);
-            const int w = 2 * ((item >> 2) & 31);  // even key of the pair within the block
-            uint8_t* dst = vt_lds + (chunk * 8) * kVtRow + ((w & 32) + vt_slot(w & 31)) * 2;
-            const uint32_t lo[4] = {vreg[i][0].x, vreg[i][0].y, vreg[i][0].z, vreg[i][0].w};
-            const uint32_t hi[4] = {vreg[i][1].x, vreg[i][1].y, vreg[i][1].z, vreg[i][1].w};
-#pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                // dims 2p and 2p+1 of the chunk: (key w, key w+1) side by side, one byte permute each
-                *reinterpret_cast<uint32_t*>(dst + (2 * p) * kVtRow) =
-                    __builtin_amdgcn_perm(hi[p], lo[p], 0x05040100u);
-                *reinterpret_cast<uint32_t*>(dst + (2 * p + 1) * kVtRow) =
-                    __builtin_amdgcn_perm(hi[p], lo[p], 0x07060302u);
-            }
-        }
+            lds_dma16(rv, lds + kKRingBytes + (kb & 1) * kVBytes + (wave * K_DMA + j) * 4 * kKRow,
+                      v_voff[j] + (uint32_t)kb * kVBytes, 0);
     };
 
     f32x16 o[4];
@@ -164,45 +160,56 @@ __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_ker
     constexpr float kSlack = 8.0f;
     float m_run = kNegBig, l_run = 0.0f;
     const float c = a.scale * 1.44269504088896340736f;  // scores to log2 units
-
-    // one 64-key block out of LDS buffer `buf`; MASK: some key of it lies past some query
-    auto block = [&](auto mask_tag, int kb, const uint8_t* kbuf, const uint8_t* vbuf) {
+    const f32x16 zero16 = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f,
+                           0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    // byte offset of this lane's k-step 0 key chunk inside a tile, and of its V^T row
+    const int k_lane = qi * kKRow;
+    // V^T operand of 32 dims x 16 keys: two transposing reads. In each 16-lane group, lane
+    // 4j+q points at row j, dims 4q..4q+3 of a 4-row x 16-dim patch and receives dim (its
+    // index in the group) of rows 0..3. Lane half h takes rows 4h..4h+3 and 8+4h..8+4h+3 of
+    // the 16-key step: the keys its P^T registers hold (register 4g+j = key 8g + 4h + j).
+    // (bits 6-7 of the offset are dt ^ j: the dim tile is XORed into the offset as well)
+    const int v_lane0 = [&] {
+        const int sl = lane & 15, j = sl >> 2, q = sl & 3, g1 = (lane >> 4) & 1;
+        return (4 * h + j) * kKRow + ((((2 * g1 + (q >> 1)) ^ (4 * j)) << 4) | ((q & 1) << 3));
+    }();
+    // key operand of k-step ks: chunk (2ks + h) ^ (row % 16) of this lane's row. The tile
+    // offset and the row offset are multiples of 256, so the k-step can be XORed into the
+    // whole byte offset: one address register per tile instead of eight.
+    const int k_lane0 = k_lane + ((h ^ (qi & 15)) << 4);
+    auto k_frag = [&](int tile_off, int ks) -> u32x4 {
+        return *reinterpret_cast<const u32x4*>(lds + ((tile_off + k_lane0) ^ (ks << 5)));
+    };
+    auto v_frag = [&](int vt_off, int t, int dt) -> u32x4 {
+        typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
+        const uint8_t* src = lds + ((vt_off + v_lane0) ^ (dt << 6)) + t * 16 * kKRow;
+        const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src));
+        const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(src + 8 * kKRow));
+        const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+        return u32x4{l2.x, l2.y, h2.x, h2.y};
+    };
+    // masking and this lane's share of the row maximum of tile T (raw scores; c > 0 keeps order)
+    auto mask_max4 = [&](auto mask_tag, int T, f32x16& s, int g, float m) -> float {
         constexpr bool MASK = decltype(mask_tag)::value;
-        // ---- S^T = K.Q^T for two 32-key tiles
-        f32x16 s[2];
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks)
-#pragma unroll
-            for (int ti = 0; ti < 2; ++ti) {
-                const int row = ti * 32 + qi;
-                const u32x4 kf = *reinterpret_cast<const u32x4*>(
-                    kbuf + row * kKRow + (((2 * ks + h) ^ (row & 15)) << 4));
-                if (ks == 0) {
-                    const f32x16 zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f,
-                                         0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-                    s[ti] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                        __builtin_bit_cast(bf16x8, kf), __builtin_bit_cast(bf16x8, qf[ks]), zero, 0, 0, 0);
-                } else {
-                    s[ti] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                        __builtin_bit_cast(bf16x8, kf), __builtin_bit_cast(bf16x8, qf[ks]), s[ti], 0, 0, 0);
-                }
+        for (int j = 0; j < 4; ++j) {
+            const int e = 4 * g + j;
+            if (MASK) {
+                const int key = T * 32 + g * 8 + h * 4 + j;
+                s[e] = key <= pq ? s[e] : kNegBig;
             }
+            m = fmaxf(m, s[e]);
+        }
+        return m;
+    };
 
-        // ---- online softmax for this lane's query (raw scores; c > 0 keeps their order)
-        float m_loc = kNegBig;
-#pragma unroll
-        for (int ti = 0; ti < 2; ++ti)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                if (MASK) {
-                    const int key = kb * kKB + ti * 32 + (e >> 2) * 8 + h * 4 + (e & 3);
-                    s[ti][e] = key <= pq ? s[ti][e] : kNegBig;
-                }
-                m_loc = fmaxf(m_loc, s[ti][e]);
-            }
-        m_loc = fmaxf(m_loc, __shfl_xor(m_loc, 32, kWave)) * c;
-        if (__any(m_loc > m_run + kSlack)) {
-            const float m_new = fmaxf(m_run, m_loc);
+    // One tile step. In: s_in = raw (masked) scores of tile T, m_in = its row maximum (both lane
+    // halves). Out: P.V of tile T added to o; s_out = scores of tile T+1, m_out = their maximum.
+    auto step = [&](auto mask_tag, int T, f32x16& s_in, float m_in, f32x16& s_out, float& m_out,
+                    int vt /* LDS offset of the 32 value rows of tile T */) {
+        const float m_sc = m_in * c;
+        if (__any(m_sc > m_run + kSlack)) {
+            const float m_new = fmaxf(m_run, m_sc);
             const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
             m_run = m_new;
             l_run *= alpha;
@@ -211,68 +218,87 @@ __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_ker
 #pragma unroll
                 for (int e = 0; e < 16; ++e) o[dt][e] *= alpha;
         }
+        const int kt = ((T + 1) & 3) * kKTileBytes;
+        uint32_t pk[8];
         float l_add = 0.0f;
-        uint32_t pk[2][8];
+        u32x4 kf[8], vf[8];
+        kf[0] = k_frag(kt, 0);
+        kf[1] = k_frag(kt, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- eight score MFMAs of tile T+1, each followed by two exponentials of tile T
 #pragma unroll
-        for (int ti = 0; ti < 2; ++ti)
-#pragma unroll
-            for (int e = 0; e < 16; e += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[ti][e], c, -m_run));
-                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[ti][e + 1], c, -m_run));
-                l_add += p0 + p1;
-                pk[ti][e >> 1] = pack_bf16x2(p0, p1);
-            }
-        l_run += l_add;
-
-        // ---- O^T += V^T.P^T, four 16-key steps x four 32-dim tiles
-#pragma unroll
-        for (int st = 0; st < 4; ++st) {
-            const int ti = st >> 1, t = st & 1;
-            const u32x4 pf = {pk[ti][4 * t], pk[ti][4 * t + 1], pk[ti][4 * t + 2], pk[ti][4 * t + 3]};
-#pragma unroll
-            for (int dt = 0; dt < 4; ++dt) {
-                const uint8_t* src = vbuf + (dt * 32 + qi) * kVtRow + ti * 64 + t * 32 + h * 16;
-                const u32x2 v0 = *reinterpret_cast<const u32x2*>(src);
-                const u32x2 v1 = *reinterpret_cast<const u32x2*>(src + 8);
-                const u32x4 vf = {v0.x, v0.y, v1.x, v1.y};
-                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                    __builtin_bit_cast(bf16x8, vf), __builtin_bit_cast(bf16x8, pf), o[dt], 0, 0, 0);
-            }
+        for (int ks = 0; ks < 8; ++ks) {
+            if (ks + 2 < 8) kf[ks + 2] = k_frag(kt, ks + 2);
+            if (ks >= 6) vf[ks - 6] = v_frag(vt, 0, ks - 6);
+            s_out = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                __builtin_bit_cast(bf16x8, kf[ks]), __builtin_bit_cast(bf16x8, qf[ks]),
+                ks == 0 ? zero16 : s_out, 0, 0, 0);
+            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_in[2 * ks], c, -m_run));
+            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_in[2 * ks + 1], c, -m_run));
+            l_add += p0 + p1;
+            pk[ks] = pack_bf16x2(p0, p1);
+            __builtin_amdgcn_sched_barrier(0);
         }
+        l_run += l_add;
+        // ---- eight P.V MFMAs of tile T, the later ones followed by the maximum of tile T+1
+        float m = kNegBig;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int t = i >> 2, dt = i & 3;
+            if (i + 2 < 8) vf[i + 2] = v_frag(vt, (i + 2) >> 2, (i + 2) & 3);
+            const u32x4 pf = {pk[4 * t], pk[4 * t + 1], pk[4 * t + 2], pk[4 * t + 3]};
+            o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                __builtin_bit_cast(bf16x8, vf[i]), __builtin_bit_cast(bf16x8, pf), o[dt], 0, 0, 0);
+            if (i >= 4) m = mask_max4(mask_tag, T + 1, s_out, i - 4, m);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        m_out = fmaxf(m, __shfl_xor(m, 32, kWave));
     };
 
-    // Two LDS buffers: while block kb is multiplied out of one, block kb+1 goes into the
-    // other (keys by DMA, values from the registers filled an iteration earlier) and the
-    // values of block kb+2 are requested; one barrier per block.
-    const int nfull = min(nkb, (__builtin_amdgcn_readfirstlane(pmin) + 1) / kKB);  // blocks every query sees whole
-    dma_k(0, 0);
-    fetch_v(0);
-    stage_v(0);
-    if (nkb > 1) fetch_v(1);
-    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): the DMA has landed
+    // ---- prologue: tiles 0..2 and the first value block; scores of tile 0
+    const int tfull = (__builtin_amdgcn_readfirstlane(pmin) + 1) / 32;  // tiles every query sees whole
+    const int nfast = max(tfull - 1, 0) / 2;  // blocks whose steps only produce unmasked tiles
+    dma_v(0);
+    // tile 0 needs the queries and the key tiles, not the values: wait for everything but
+    // this wave's K_DMA value loads (the newest), which get the scores of tile 0 to land
+    __builtin_amdgcn_s_waitcnt(0x0f70 | K_DMA);  // vmcnt(K_DMA)
     __syncthreads();
+    f32x16 sa, sb;
+    float ma, mb;
+    {
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks)
+            sa = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                __builtin_bit_cast(bf16x8, k_frag(0, ks)), __builtin_bit_cast(bf16x8, qf[ks]),
+                ks == 0 ? zero16 : sa, 0, 0, 0);
+        float m = kNegBig;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) m = mask_max4(std::true_type{}, 0, sa, g, m);
+        ma = fmaxf(m, __shfl_xor(m, 32, kWave));
+    }
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    __syncthreads();  // values landed; tile 0's ring slot is overwritten by the first block's loads
     for (int kb = 0; kb < nkb; ++kb) {
         const int cur = kb & 1;
-        if (kb + 1 < nkb) {
-            dma_k(kb + 1, cur ^ 1);
-            stage_v(cur ^ 1);
+        dma_k(2 * kb + 3);  // tiles 2kb+3, 2kb+4: their slots held tiles 2kb-1 and 2kb
+        if (kb + 1 < nkb) dma_v(kb + 1);
+        const int vt = kKRingBytes + cur * kVBytes;
+        if (kb < nfast) {
+            step(std::false_type{}, 2 * kb, sa, ma, sb, mb, vt);
+            step(std::false_type{}, 2 * kb + 1, sb, mb, sa, ma, vt + 32 * kKRow);
+        } else {
+            step(std::true_type{}, 2 * kb, sa, ma, sb, mb, vt);
+            step(std::true_type{}, 2 * kb + 1, sb, mb, sa, ma, vt + 32 * kKRow);
         }
-        if (kb + 2 < nkb) fetch_v(kb + 2);
-        const uint8_t* kbuf = lds + cur * kBufBytes;
-        if (kb < nfull)
-            block(std::false_type{}, kb, kbuf, kbuf + kKBytes);
-        else
-            block(std::true_type{}, kb, kbuf, kbuf + kKBytes);
         __builtin_amdgcn_s_waitcnt(0x0070);
         __syncthreads();
     }
-
-    // ---- normalise and write [batch, seq, heads*128]
+    // ---- normalise and write [batch, seq, heads*128]: through this wave's quarter of the
+    // (now idle) key ring, so that the 32 x 128 tile leaves as whole 256-byte rows
     l_run += __shfl_xor(l_run, 32, kWave);
     const float inv = 1.0f / l_run;
-    if (row_live) {
-        uint16_t* orow = static_cast<uint16_t*>(a.out) +
-            (((size_t)b * a.seq + s_row) * a.n_heads + head) * kD;
+    {
+        uint8_t* const mine = lds + wave * kKTileBytes;
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
@@ -280,8 +306,19 @@ __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_ker
                 u32x2 w;
                 w.x = pack_bf16x2(o[dt][4 * g] * inv, o[dt][4 * g + 1] * inv);
                 w.y = pack_bf16x2(o[dt][4 * g + 2] * inv, o[dt][4 * g + 3] * inv);
-                *reinterpret_cast<u32x2*>(orow + dt * 32 + g * 8 + h * 4) = w;
+                // row qi, dims 32dt + 8g + 4h ..+3: chunk 4dt+g (XOR-swizzled by row), half h
+                *reinterpret_cast<u32x2*>(mine + qi * kKRow + (((4 * dt + g) ^ (qi & 15)) << 4) + h * 8) = w;
             }
+        uint16_t* const obase = static_cast<uint16_t*>(a.out) +
+            (((size_t)b * a.seq + qb * kQB) * a.n_heads + head) * kD;
+        const int r4 = lane >> 4, c16 = lane & 15;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int row = i * 4 + r4;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(mine + row * kKRow + ((c16 ^ (row & 15)) << 4));
+            if (qb * kQB + row < a.seq)
+                *reinterpret_cast<u32x4*>(obase + (size_t)row * a.n_heads * kD + c16 * 8) = v;
+        }
     }
 }
 
