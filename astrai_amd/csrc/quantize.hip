@@ -47,12 +47,31 @@ __device__ __forceinline__ uint32_t quant1_int8(float f, float step) {
     return (uint32_t)(int)q & 0xffu;
 }
 
+// Eight codes, exactly rint(f / step) clamped to +-127, without eight IEEE divisions:
+// t = f * (1 / step) is within two ulps of the quotient and |t| stays below 2^8 where a
+// code can still change, so rint(t) can differ from rint(f / step) only when t lies within
+// 2^-14 of a half-integer. Lanes that see such a value (about one vector in a thousand)
+// redo their eight with the division.
 __device__ __forceinline__ u32x2 quant8_int8(const float (&f)[8], float step) {
+    const float inv = 1.0f / step;
+    float r[8];
+    bool risky = false;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float t = f[j] * inv;
+        r[j] = rintf(t);
+        risky |= fabsf(t - r[j]) > 0.5f - 0x1p-14f;
+    }
+    if (risky) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) r[j] = rintf(f[j] / step);
+    }
+    uint32_t c[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) c[j] = (uint32_t)(int)__builtin_amdgcn_fmed3f(r[j], -127.0f, 127.0f) & 0xffu;
     u32x2 o;
-    o.x = quant1_int8(f[0], step) | (quant1_int8(f[1], step) << 8) |
-          (quant1_int8(f[2], step) << 16) | (quant1_int8(f[3], step) << 24);
-    o.y = quant1_int8(f[4], step) | (quant1_int8(f[5], step) << 8) |
-          (quant1_int8(f[6], step) << 16) | (quant1_int8(f[7], step) << 24);
+    o.x = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+    o.y = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
     return o;
 }
 
@@ -435,6 +454,13 @@ __global__ __launch_bounds__(kThreads) void add_rmsnorm_quantize_int8_rows_kerne
     }
 }
 
+// silu(g) = g / (1 + exp(-g)) on the hardware's exp2 and reciprocal (each within one ulp
+// in fp32, far inside the bf16 rounding that follows): the library expf and an IEEE division
+// made this bandwidth kernel compute-bound.
+__device__ __forceinline__ float silu_f32(float g) {
+    return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.44269504088896340736f));
+}
+
 // h = bf16(up * bf16(silu(gate))), silu(g) = g / (1 + exp(-g)) in fp32: the bf16
 // arithmetic of ``up(x) * F.silu(gate(x))`` (model/components/mlp.py:41); then the
 // per-row int8 quantizer on h. gate and up rows are `ld` elements apart (they may
@@ -456,7 +482,7 @@ __global__ __launch_bounds__(kThreads) void silu_mul_quantize_int8_rows_kernel(
             unpack8(*reinterpret_cast<const u32x4*>(up + row * ld + i * 8), v[c]);
 #pragma unroll
             for (int j = 0; j < 8; ++j)
-                v[c][j] = round_bf16(v[c][j] * round_bf16(g[j] / (1.0f + expf(-g[j]))));
+                v[c][j] = round_bf16(v[c][j] * round_bf16(silu_f32(g[j])));
             local = fmaxf(local, amax8(v[c]));
             if (h_out) *reinterpret_cast<u32x4*>(h_out + row * width + i * 8) = pack8(v[c]);
         }
