@@ -547,7 +547,7 @@ def attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, p
     if scale is None:
         scale = d ** -0.5
     if nsplit <= 0:
-        nsplit = max(1, min(16, 1024 // max(1, b * hkv)))
+        nsplit = max(1, min(16, 384 // max(1, b * hkv)))  # a few hundred workgroups: more splits cost more in the merge than they hide
     nq = (h // hkv) * s
     with torch.cuda.device(q.device):
         need = lib.astrai_w8a8_attn_decode_workspace_floats(b, hkv, nsplit, nq)
@@ -609,7 +609,7 @@ def attn_paged_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     if scale is None or scale <= 0.0:
         scale = d ** -0.5
     if nsplit <= 0:
-        nsplit = max(1, min(16, 1024 // max(1, b * hkv)))
+        nsplit = max(1, min(16, 384 // max(1, b * hkv)))  # a few hundred workgroups: more splits cost more in the merge than they hide
     with torch.cuda.device(q.device):
         if new_k is not None:
             if new_k.shape != (b, hkv, d) or new_v.shape != (b, hkv, d):
