@@ -134,9 +134,12 @@ __device__ __forceinline__ void lds_dma16(__amdgpu_buffer_rsrc_t r, uint8_t* lds
 // Phase-timestamp hooks for the kernel's own profiling harness; compiled out
 // of the library.
 #ifdef W8A8_PP_TIMING
+#ifndef PP_BLOCK
+#define PP_BLOCK 0  // the workgroup whose waves record their stamps
+#endif
 __device__ unsigned long long* g_pp_dbg;
 #define PP_STAMP_INIT()                                                                   \
-    const bool pp_rec = (blockIdx.x == 0) && ((threadIdx.x & 63) == 0);                   \
+    const bool pp_rec = (blockIdx.x == PP_BLOCK) && ((threadIdx.x & 63) == 0);                   \
     unsigned long long* pp_my = g_pp_dbg + (threadIdx.x >> 6) * 256;                      \
     int pp_ti = 0;
 #define PP_STAMP()                                              \
