@@ -166,14 +166,14 @@ def main():
                          "one), one prefill + 19 eager decode steps, nothing else")
     ap.add_argument("--trace-kernels", action="store_true",
                     help="tracing mode: a few launches of every auxiliary kernel (quantizers, policy-path "
-                         "kernels, attention) at the sizes DESIGN.md quotes, nothing else")
+                         "kernels, attention) at 4096 x 4096 / config-4 sizes, nothing else")
     ap.add_argument("--pmc", action="store_true",
                     help="counter-collection mode: a few launches of the headline kernel and of a "
                          "plain 256 MiB device copy (the calibration kernel), nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU's share of the path: run with --gpus 1 "
-                 "(no multi-GPU leg exists; the sharding is described in DESIGN.md)")
+                 "(no multi-GPU leg exists: the path shards by output columns or by K, one collective at most)")
 
     import torch
 

@@ -61,7 +61,7 @@ def test_cast_rne_ties_subnormals_overflow(golden, name):
             assert gt == c and gc == c, (hex(b), _f32(b), gt, gc, c)
 
 
-def test_boundaries_called_out_by_the_survey():
+def test_rounding_and_overflow_boundaries():
     # e4m3fn: 17->16, 19->20, 21->20, 23->24 (ties to even), 2^-10 -> 0, 464 -> 448, 465 -> NaN
     x = torch.tensor([17.0, 19.0, 21.0, 23.0, 2.0**-10, 464.0, 465.0])
     y = x.to(torch.float8_e4m3fn).float()
