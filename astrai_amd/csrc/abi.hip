@@ -293,6 +293,44 @@ int astrai_w8a8_attn_prefill_bf16(const void* q, const void* k_cache, const void
     return check_launch("attn_prefill_bf16");
 }
 
+int astrai_w8a8_attn_paged_prefill_bf16(const void* q, const void* k_pool, const void* v_pool,
+                                        const int32_t* req_to_token, const int32_t* req_pool_indices,
+                                        const int32_t* kv_indptr, const int32_t* qo_indptr,
+                                        const int32_t* q_tile_to_batch, const int32_t* q_tile_to_index,
+                                        void* out, int64_t num_q_tiles, int64_t n_heads,
+                                        int64_t n_kv_heads, int64_t head_dim, int64_t num_slots,
+                                        int64_t num_requests, int64_t max_context_len, int causal,
+                                        float scale, void* stream) {
+    if (!q || !k_pool || !v_pool || !req_to_token || !req_pool_indices || !kv_indptr || !qo_indptr ||
+        !q_tile_to_batch || !q_tile_to_index || !out)
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_prefill_bf16: null pointer");
+    if (num_q_tiles < 0 || n_heads <= 0 || n_kv_heads <= 0 || num_slots <= 0 || num_requests <= 0 ||
+        max_context_len <= 0 || n_heads % n_kv_heads || num_q_tiles > (1 << 24) ||
+        max_context_len > INT32_MAX)
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_prefill_bf16: bad dims");
+    if (!w8a8::attn_prefill_supported((int)n_heads, (int)n_kv_heads, (int)head_dim))
+        return fail(ASTRAI_W8A8_UNSUPPORTED,
+                    "attn_paged_prefill_bf16: needs head_dim 128 and n_heads / n_kv_heads in {2, 4, 8}");
+    if (num_slots * n_kv_heads * 256 >= ((int64_t)1 << 32))
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "attn_paged_prefill_bf16: a pool must stay under 4 GiB");
+    if (!(scale > 0.0f)) return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_prefill_bf16: scale must be positive");
+    if (!aligned16(q) || !aligned16(k_pool) || !aligned16(v_pool) || !aligned16(out))
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_prefill_bf16: pointers must be 16-byte aligned");
+    if (num_q_tiles == 0) return ASTRAI_W8A8_OK;
+    w8a8::AttnPrefillArgs a{};
+    a.q = q; a.k_cache = k_pool; a.v_cache = v_pool; a.out = out;
+    a.n_heads = (int)n_heads; a.n_kv_heads = (int)n_kv_heads; a.head_dim = (int)head_dim;
+    a.scale = scale;
+    a.req_to_token = req_to_token; a.req_pool_indices = req_pool_indices;
+    a.kv_indptr = kv_indptr; a.qo_indptr = qo_indptr;
+    a.q_tile_to_batch = q_tile_to_batch; a.q_tile_to_index = q_tile_to_index;
+    a.num_q_tiles = (int)num_q_tiles; a.causal = causal ? 1 : 0;
+    a.rtt_stride = max_context_len; a.num_slots = num_slots; a.num_requests = num_requests;
+    if (!w8a8::launch_attn_prefill(a, static_cast<hipStream_t>(stream)))
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "attn_paged_prefill_bf16: shape not supported");
+    return check_launch("attn_paged_prefill_bf16");
+}
+
 int astrai_w8a8_quantize_bf16_fp8_block128_act(const void* x, void* x8, float* sa, int64_t m,
                                                int64_t k, void* stream) {
     if (!x || !x8 || !sa) return fail(ASTRAI_W8A8_BAD_ARG, "quantize_block128_act: null pointer");

@@ -62,7 +62,15 @@ __device__ __forceinline__ void lds_dma16(__amdgpu_buffer_rsrc_t r, uint8_t* lds
         r, (__attribute__((address_space(3))) void*)lds_wave_base, 16, voff, soff, 0, 0);
 }
 
-template <int NREP>
+// PAGED: the queries are packed [total_q, heads, 128] with per-request row ranges
+// (qo_indptr), the caches are token-granular pools [slots, kv_heads, 128] reached through
+// req_to_token, and a 64-row query tile t of the caller's schedule belongs to request
+// q_tile_to_batch[t], rows 64 * q_tile_to_index[t] .. of it (csrc/kernels/attention/
+// paged_prefill.cu:4-34, layout_policies.cuh:67-93,174-232; the schedule is built in
+// astrai/inference/cache/pool.py:219-234). Two workgroups share a tile. Query row i of a
+// request of q_len rows and kv_len keys sees keys 0 .. kv_len - q_len + i (all of them
+// without the causal flag), so nothing has to be fetched to know the key range.
+template <int NREP, bool PAGED>
 __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_kernel(AttnPrefillArgs a) {
     constexpr int THREADS = 64 * NREP;
     constexpr int K_DMA = kKB / 4 / NREP;              // 1 KiB key loads per wave and block
@@ -71,81 +79,156 @@ __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_ker
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int qi = lane & 31, h = lane >> 5;
-    const int nqb = (a.seq + kQB - 1) / kQB;
-    const int groups = a.batch * a.n_kv_heads;
-    const int qb = nqb - 1 - (int)(blockIdx.x / groups);  // longest key ranges first
-    const int bk = (int)(blockIdx.x % groups);
-    const int b = bk / a.n_kv_heads, hk = bk % a.n_kv_heads;
+
+    int hk, rows_total, row0;   // KV head; query rows of the sequence; first row of this block
+    int64_t tok0;               // index of row 0 of the sequence in the token-major output
+    const uint16_t* qbase;      // row 0 of the sequence, this wave's head
+    int64_t q_row_stride;       // elements between consecutive query rows
+    int pq, kmax, pmin;         // this lane's newest visible key; the block's extremes
+    [[maybe_unused]] const int* table = nullptr;
+    [[maybe_unused]] int kv_len = 0, b_dense = 0;
+    if constexpr (PAGED) {
+        const int idx = (int)blockIdx.x;
+        hk = idx % a.n_kv_heads;
+        const int sub = (idx / a.n_kv_heads) & 1, tile = idx / (2 * a.n_kv_heads);
+        const int req_i = a.q_tile_to_batch[tile];
+        const int q_start = a.qo_indptr[req_i];
+        rows_total = a.qo_indptr[req_i + 1] - q_start;
+        row0 = a.q_tile_to_index[tile] * 64 + sub * kQB;
+        if (row0 >= rows_total) return;  // the tile's second half lies past the request
+        const int64_t req = a.req_pool_indices[req_i];
+        const bool req_ok = req >= 0 && req < a.num_requests;  // a bad row reads as an empty sequence
+        kv_len = req_ok ? (int)min((int64_t)(a.kv_indptr[req_i + 1] - a.kv_indptr[req_i]), a.rtt_stride) : 0;
+        table = a.req_to_token + (req_ok ? req : 0) * a.rtt_stride;
+        tok0 = q_start;
+        q_row_stride = (int64_t)a.n_heads * kD;
+        qbase = static_cast<const uint16_t*>(a.q) + ((int64_t)q_start * a.n_heads + hk * NREP + wave) * kD;
+        const int last = min(row0 + kQB, rows_total) - 1;
+        const int shift = a.causal ? kv_len - rows_total : INT_MIN;
+        pq = a.causal ? min(shift + row0 + qi, kv_len - 1) : kv_len - 1;
+        kmax = a.causal ? min(shift + last, kv_len - 1) : kv_len - 1;
+        pmin = a.causal ? min(shift + row0, kv_len - 1) : kv_len - 1;
+    } else {
+        const int nqb = (a.seq + kQB - 1) / kQB;
+        const int groups = a.batch * a.n_kv_heads;
+        const int qb = nqb - 1 - (int)(blockIdx.x / groups);  // longest key ranges first
+        const int bk = (int)(blockIdx.x % groups);
+        const int b = bk / a.n_kv_heads;
+        b_dense = b;
+        hk = bk % a.n_kv_heads;
+        rows_total = a.seq;
+        row0 = qb * kQB;
+        tok0 = (int64_t)b * a.seq;
+        q_row_stride = kD;
+        qbase = static_cast<const uint16_t*>(a.q) + ((int64_t)b * a.n_heads + hk * NREP + wave) * a.seq * kD;
+        // The position is requested first and looked at last: the query rows and the first
+        // key tiles do not depend on it.
+        pq = row0 + qi < a.seq ? (int)a.positions[row0 + qi] : -1;
+        kmax = pmin = 0;
+    }
     const int head = hk * NREP + wave;
+    const int s_row = row0 + qi;
+    const bool row_live = s_row < rows_total;
 
-    // this lane's query token. Its position is requested first and looked at last: the
-    // query rows and the first key tiles do not depend on it.
-    const int s_row = qb * kQB + qi;
-    const bool row_live = s_row < a.seq;
-    int pq = row_live ? (int)a.positions[s_row] : -1;
-
-    const uint16_t* qrow = static_cast<const uint16_t*>(a.q) +
-        (((size_t)b * a.n_heads + head) * a.seq + min(s_row, a.seq - 1)) * kD;
+    const uint16_t* qrow = qbase + (int64_t)min(s_row, rows_total - 1) * q_row_stride;
     u32x4 qf[8];
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) qf[ks] = *reinterpret_cast<const u32x4*>(qrow + ks * 16 + h * 8);
 
-    const size_t cache_off = ((size_t)b * a.n_kv_heads + hk) * (size_t)a.max_len * kD;
-    const uint16_t* kc = static_cast<const uint16_t*>(a.k_cache) + cache_off;
-    const uint16_t* vc = static_cast<const uint16_t*>(a.v_cache) + cache_off;
-
     // keys: straight from the cache into LDS, 1 KiB (four rows) per instruction; lane l
     // lands at row l/16, chunk position l%16 and therefore asks for chunk (l%16) ^ (row%16).
-    // The descriptor covers the whole cache row range: whatever a row past the newest
-    // position holds, its scores are replaced (not scaled) by the mask.
-    const __amdgpu_buffer_rsrc_t rk = make_rsrc(kc, (uint32_t)a.max_len * (uint32_t)kKRow);
-    uint32_t k_voff[K_DMA];
+    // Dense cache: the descriptor covers the whole row range of this (batch, KV head):
+    // whatever a row past the newest position holds, its scores are replaced (not scaled)
+    // by the mask. Paged: the descriptor covers the pool and each lane looks up the slot of
+    // its row; rows past the sequence ask for an offset outside it and arrive as zeros.
+    const int64_t pool_row = (int64_t)a.n_kv_heads * kKRow;  // bytes from one slot to the next
+    const size_t cache_off = PAGED ? (size_t)hk * kD
+                                   : ((size_t)b_dense * a.n_kv_heads + hk) * (size_t)a.max_len * kD;
+    const uint16_t* kc = static_cast<const uint16_t*>(a.k_cache) + cache_off;
+    const uint16_t* vc = static_cast<const uint16_t*>(a.v_cache) + cache_off;
+    const uint32_t pool_bytes = PAGED ? (uint32_t)(a.num_slots * pool_row - hk * kKRow) : 0u;
+    const __amdgpu_buffer_rsrc_t rk = make_rsrc(kc, PAGED ? pool_bytes : (uint32_t)a.max_len * (uint32_t)kKRow);
+    // Paged: one load per wave fetches the slots of all rows its next loads cover (lane l <
+    // RPW: this wave's l-th key row; the next RPW lanes: its value rows); the loads take each
+    // row's slot from the lane that holds it. Looked up one block ahead, so that the table
+    // access is not a second memory round trip in front of every load.
+    constexpr int RPW = 4 * K_DMA;  // rows of a 64-row block that this wave loads
+    auto lookup = [&](int t0, int kbv) -> int {
+        const int l = lane & (2 * RPW - 1);  // (lanes past 2 RPW repeat the pattern, unused)
+        const int key = l < RPW ? t0 * 32 + wave * RPW + l : kbv * kKB + wave * RPW + (l - RPW);
+        int slot = (key <= kmax) ? table[key] : -1;
+        return slot < a.num_slots ? slot : -1;
+    };
+    auto paged_off = [&](int slots, int src_lane, int swz) -> uint32_t {
+        const int slot = __builtin_amdgcn_ds_bpermute(src_lane << 2, slots);
+        return slot >= 0 ? (uint32_t)(slot * pool_row) + (uint32_t)(((lane & 15) ^ swz) << 4) : kOutOfRange;
+    };
+    [[maybe_unused]] uint32_t k_voff[K_DMA];
+    if constexpr (!PAGED) {
 #pragma unroll
-    for (int j = 0; j < K_DMA; ++j) {
-        const int row = (wave * K_DMA + j) * 4 + (lane >> 4);
-        k_voff[j] = (uint32_t)row * kKRow + (uint32_t)(((lane & 15) ^ (row & 15)) << 4);
+        for (int j = 0; j < K_DMA; ++j) {
+            const int row = (wave * K_DMA + j) * 4 + (lane >> 4);
+            k_voff[j] = (uint32_t)row * kKRow + (uint32_t)(((lane & 15) ^ (row & 15)) << 4);
+        }
     }
     // tiles t0 and t0+1 (64 keys) into their ring slots
-    auto dma_k = [&](int t0) {
+    auto dma_k = [&](int t0, [[maybe_unused]] int slots) {
 #pragma unroll
         for (int j = 0; j < K_DMA; ++j) {
             const int inst = wave * K_DMA + j;  // 16 instructions of 4 rows; 8 per tile
-            lds_dma16(rk, lds + ((t0 + (inst >> 3)) & 3) * kKTileBytes + (inst & 7) * 4 * kKRow,
-                      k_voff[j] + (uint32_t)t0 * kKTileBytes, 0);
+            const int row = inst * 4 + (lane >> 4);
+            const uint32_t off = PAGED ? paged_off(slots, j * 4 + (lane >> 4), row & 15)
+                                       : k_voff[j] + (uint32_t)t0 * kKTileBytes;
+            lds_dma16(rk, lds + ((t0 + (inst >> 3)) & 3) * kKTileBytes + (inst & 7) * 4 * kKRow, off, 0);
         }
     };
-    dma_k(0);
-    dma_k(1);
-
-    // what the block's queries may see
-    int kmax = pq, pmin = row_live ? pq : INT_MAX;
-#pragma unroll
-    for (int off = 16; off; off >>= 1) {
-        kmax = max(kmax, __shfl_xor(kmax, off, kWave));
-        pmin = min(pmin, __shfl_xor(pmin, off, kWave));
+    [[maybe_unused]] int slots = 0;
+    if constexpr (PAGED) {
+        dma_k(0, lookup(0, 0));
+        slots = lookup(1, 0);  // tiles 1, 2 and value block 0
+    } else {
+        dma_k(0, 0);
     }
-    // every lane holds the same extremes by now: keep them in scalar registers (loop bounds,
-    // the value descriptor's size)
-    kmax = min(__builtin_amdgcn_readfirstlane(kmax), (int)a.max_len - 1);
-    pmin = __builtin_amdgcn_readfirstlane(pmin);
+    dma_k(1, slots);
+
+    if constexpr (!PAGED) {
+        // what the block's queries may see
+        kmax = pq;
+        pmin = row_live ? pq : INT_MAX;
+#pragma unroll
+        for (int off = 16; off; off >>= 1) {
+            kmax = max(kmax, __shfl_xor(kmax, off, kWave));
+            pmin = min(pmin, __shfl_xor(pmin, off, kWave));
+        }
+        // every lane holds the same extremes by now: keep them in scalar registers (loop
+        // bounds, the value descriptor's size)
+        kmax = min(__builtin_amdgcn_readfirstlane(kmax), (int)a.max_len - 1);
+        pmin = __builtin_amdgcn_readfirstlane(pmin);
+    }
+    const bool sees_a_key = pq >= 0;
     if (!row_live) pq = kmax;  // rows past the end see everything and are never stored
-    const int nkb = kmax / kKB + 1;
+    const int nkb = kmax / kKB + 1;  // (kmax = -1, an empty sequence: one block of masked keys)
 
     // values: the same way into a 64-row buffer; chunk position (l%16) holds chunk
     // (l%16) ^ 4*(row%4). Rows past kmax arrive as zeros, so a stale cache row can never
     // meet a zero probability as 0 * NaN.
-    const __amdgpu_buffer_rsrc_t rv = make_rsrc(vc, (uint32_t)(kmax + 1) * (uint32_t)kKRow);
-    uint32_t v_voff[K_DMA];
+    const __amdgpu_buffer_rsrc_t rv = make_rsrc(vc, PAGED ? pool_bytes : (uint32_t)(kmax + 1) * (uint32_t)kKRow);
+    [[maybe_unused]] uint32_t v_voff[K_DMA];
+    if constexpr (!PAGED) {
 #pragma unroll
-    for (int j = 0; j < K_DMA; ++j) {
-        const int row = (wave * K_DMA + j) * 4 + (lane >> 4);
-        v_voff[j] = (uint32_t)row * kKRow + (uint32_t)(((lane & 15) ^ (4 * (row & 3))) << 4);
+        for (int j = 0; j < K_DMA; ++j) {
+            const int row = (wave * K_DMA + j) * 4 + (lane >> 4);
+            v_voff[j] = (uint32_t)row * kKRow + (uint32_t)(((lane & 15) ^ (4 * (row & 3))) << 4);
+        }
     }
-    auto dma_v = [&](int kb) {
+    auto dma_v = [&](int kb, [[maybe_unused]] int slots) {
 #pragma unroll
-        for (int j = 0; j < K_DMA; ++j)
-            lds_dma16(rv, lds + kKRingBytes + (kb & 1) * kVBytes + (wave * K_DMA + j) * 4 * kKRow,
-                      v_voff[j] + (uint32_t)kb * kVBytes, 0);
+        for (int j = 0; j < K_DMA; ++j) {
+            const int row = (wave * K_DMA + j) * 4 + (lane >> 4);
+            const uint32_t off = PAGED ? paged_off(slots, RPW + j * 4 + (lane >> 4), 4 * (row & 3))
+                                       : v_voff[j] + (uint32_t)kb * kVBytes;
+            lds_dma16(rv, lds + kKRingBytes + (kb & 1) * kVBytes + (wave * K_DMA + j) * 4 * kKRow, off, 0);
+        }
     };
 
     f32x16 o[4];
@@ -258,7 +341,8 @@ __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_ker
     // ---- prologue: tiles 0..2 and the first value block; scores of tile 0
     const int tfull = (__builtin_amdgcn_readfirstlane(pmin) + 1) / 32;  // tiles every query sees whole
     const int nfast = max(tfull - 1, 0) / 2;  // blocks whose steps only produce unmasked tiles
-    dma_v(0);
+    dma_v(0, slots);
+    if constexpr (PAGED) slots = lookup(3, 1);  // what the first block's loads will ask for
     // tile 0 needs the queries and the key tiles, not the values: wait for everything but
     // this wave's K_DMA value loads (the newest), which get the scores of tile 0 to land
     __builtin_amdgcn_s_waitcnt(0x0f70 | K_DMA);  // vmcnt(K_DMA)
@@ -280,8 +364,9 @@ __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_ker
     __syncthreads();  // values landed; tile 0's ring slot is overwritten by the first block's loads
     for (int kb = 0; kb < nkb; ++kb) {
         const int cur = kb & 1;
-        dma_k(2 * kb + 3);  // tiles 2kb+3, 2kb+4: their slots held tiles 2kb-1 and 2kb
-        if (kb + 1 < nkb) dma_v(kb + 1);
+        dma_k(2 * kb + 3, slots);  // tiles 2kb+3, 2kb+4: their ring slots held tiles 2kb-1 and 2kb
+        if (kb + 1 < nkb) dma_v(kb + 1, slots);
+        if constexpr (PAGED) slots = lookup(2 * kb + 5, kb + 2);  // for the next block's loads
         const int vt = kKRingBytes + cur * kVBytes;
         if (kb < nfast) {
             step(std::false_type{}, 2 * kb, sa, ma, sb, mb, vt);
@@ -296,7 +381,8 @@ __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_ker
     // ---- normalise and write [batch, seq, heads*128]: through this wave's quarter of the
     // (now idle) key ring, so that the 32 x 128 tile leaves as whole 256-byte rows
     l_run += __shfl_xor(l_run, 32, kWave);
-    const float inv = 1.0f / l_run;
+    // a row that sees no key at all (empty sequence, or more queries than keys) yields zeros
+    const float inv = (l_run > 0.0f && sees_a_key) ? 1.0f / l_run : 0.0f;
     {
         uint8_t* const mine = lds + wave * kKTileBytes;
 #pragma unroll
@@ -309,14 +395,13 @@ __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_ker
                 // row qi, dims 32dt + 8g + 4h ..+3: chunk 4dt+g (XOR-swizzled by row), half h
                 *reinterpret_cast<u32x2*>(mine + qi * kKRow + (((4 * dt + g) ^ (qi & 15)) << 4) + h * 8) = w;
             }
-        uint16_t* const obase = static_cast<uint16_t*>(a.out) +
-            (((size_t)b * a.seq + qb * kQB) * a.n_heads + head) * kD;
+        uint16_t* const obase = static_cast<uint16_t*>(a.out) + ((tok0 + row0) * a.n_heads + head) * kD;
         const int r4 = lane >> 4, c16 = lane & 15;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int row = i * 4 + r4;
             const u32x4 v = *reinterpret_cast<const u32x4*>(mine + row * kKRow + ((c16 ^ (row & 15)) << 4));
-            if (qb * kQB + row < a.seq)
+            if (row0 + row < rows_total)
                 *reinterpret_cast<u32x4*>(obase + (size_t)row * a.n_heads * kD + c16 * 8) = v;
         }
     }
@@ -332,17 +417,35 @@ bool attn_prefill_supported(int n_heads, int n_kv_heads, int head_dim) {
 
 bool launch_attn_prefill(const AttnPrefillArgs& a, hipStream_t stream) {
     if (!attn_prefill_supported(a.n_heads, a.n_kv_heads, a.head_dim)) return false;
-    if (a.batch <= 0 || a.seq <= 0 || a.max_len <= 0) return false;
+    const bool paged = a.req_to_token != nullptr;
     const int n_rep = a.n_heads / a.n_kv_heads;
-    const int64_t wgs = (int64_t)((a.seq + kQB - 1) / kQB) * a.batch * a.n_kv_heads;
+    int64_t wgs;
+    if (paged) {
+        if (!a.req_pool_indices || !a.kv_indptr || !a.qo_indptr || !a.q_tile_to_batch || !a.q_tile_to_index ||
+            a.num_q_tiles <= 0 || a.rtt_stride <= 0 || a.num_slots <= 0 || a.num_requests <= 0)
+            return false;
+        if (a.num_slots * (int64_t)a.n_kv_heads * kKRow >= ((int64_t)1 << 32)) return false;  // 32-bit pool offsets
+        wgs = (int64_t)a.num_q_tiles * 2 * a.n_kv_heads;
+    } else {
+        if (a.batch <= 0 || a.seq <= 0 || a.max_len <= 0) return false;
+        wgs = (int64_t)((a.seq + kQB - 1) / kQB) * a.batch * a.n_kv_heads;
+    }
     if (wgs > INT_MAX) return false;
     const dim3 grid((unsigned)wgs);
+#define W8A8_LAUNCH_PREFILL(R)                                                          \
+    do {                                                                                \
+        if (paged)                                                                      \
+            attn_prefill_kernel<R, true><<<grid, dim3(64 * R), 0, stream>>>(a);         \
+        else                                                                            \
+            attn_prefill_kernel<R, false><<<grid, dim3(64 * R), 0, stream>>>(a);        \
+    } while (0)
     if (n_rep == 2)
-        attn_prefill_kernel<2><<<grid, dim3(128), 0, stream>>>(a);
+        W8A8_LAUNCH_PREFILL(2);
     else if (n_rep == 4)
-        attn_prefill_kernel<4><<<grid, dim3(256), 0, stream>>>(a);
+        W8A8_LAUNCH_PREFILL(4);
     else
-        attn_prefill_kernel<8><<<grid, dim3(512), 0, stream>>>(a);
+        W8A8_LAUNCH_PREFILL(8);
+#undef W8A8_LAUNCH_PREFILL
     return true;
 }
 

@@ -103,6 +103,17 @@ struct AttnPrefillArgs {
     int batch, seq, n_heads, n_kv_heads, head_dim;
     int64_t max_len;
     float scale;
+    // paged mode (req_to_token != null): q and out are packed [total_q, n_heads, 128], the
+    // caches are pools [slots, n_kv_heads, 128]; positions, batch, seq and max_len are unused
+    const int* req_to_token;      // int32 [requests, rtt_stride]: slot of (request, position)
+    const int* req_pool_indices;  // int32 [batch]: row of req_to_token of each sequence
+    const int* kv_indptr;         // int32 [batch + 1]: prefix sums of the key counts
+    const int* qo_indptr;         // int32 [batch + 1]: prefix sums of the query row counts
+    const int* q_tile_to_batch;   // int32 [num_q_tiles]: sequence of each 64-row query tile
+    const int* q_tile_to_index;   // int32 [num_q_tiles]: index of the tile within its sequence
+    int num_q_tiles;
+    int causal;                   // row i of a sequence sees keys 0 .. kv_len - q_len + i; else all keys
+    int64_t rtt_stride, num_slots, num_requests;
 };
 bool attn_prefill_supported(int n_heads, int n_kv_heads, int head_dim);
 bool launch_attn_prefill(const AttnPrefillArgs& a, hipStream_t stream);

@@ -46,6 +46,9 @@ PROTOTYPES = {
     "astrai_w8a8_attn_paged_decode_bf16": (
         [_P, _P, _P, _P, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
          ctypes.c_float, _P], _INT),
+    "astrai_w8a8_attn_paged_prefill_bf16": (
+        [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _INT,
+         ctypes.c_float, _P], _INT),
     "astrai_w8a8_attn_prefill_bf16": (
         [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, ctypes.c_float, _P], _INT),
     "astrai_w8a8_attn_decode_bf16": (
@@ -635,6 +638,75 @@ def attn_paged_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
             ind.data_ptr(), ws.data_ptr(), ws.numel(), out.data_ptr(), b, h, hkv, d, slots,
             rtt.size(0), rtt.size(1), nsplit, float(scale), _stream(q)), lib)
     return out
+
+
+Q_TILE_ROWS = 64  # rows per tile of the schedule the reference builds (astrai/inference/workspace.py:13)
+
+
+def attn_paged_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                       req_to_token: torch.Tensor, req_pool_indices: torch.Tensor,
+                       kv_indptr: torch.Tensor, qo_indptr: torch.Tensor,
+                       q_tile_to_batch: torch.Tensor, q_tile_to_index: torch.Tensor,
+                       mask: Optional[torch.Tensor] = None, causal_offset: int = -1,
+                       scale: float = 0.0) -> torch.Tensor:
+    """Ragged paged prefill with the argument list of the reference's pybind entry
+    (csrc/kernels/attention/paged_prefill.cu:36-52): packed ``q [total_q, H, 128]``, flat
+    pools, ``req_to_token`` / ``req_pool_indices`` / ``kv_indptr`` / ``qo_indptr`` int32, and
+    the schedule of 64-row query tiles. ``causal_offset >= 0`` asks for the causal mask (the
+    wrapper passes 0 for ``is_causal``, astrai/extension/ops/attention.py:188); ``mask`` is
+    not supported. Returns ``[total_q, H, 128]`` bf16."""
+    lib = _require()
+    _gpu(q, "attn_paged_prefill")
+    if mask is not None:
+        raise RuntimeError("attn_paged_prefill: a key mask is not supported")
+    if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
+        raise RuntimeError("q, k_cache and v_cache must be bf16")
+    if q.dim() != 3 or k_cache.dim() != 3 or k_cache.shape != v_cache.shape:
+        raise RuntimeError("q must be [total_q, q_head, head_dim] and the pools [size, kv_head, head_dim]")
+    ints = ((req_to_token, "req_to_token"), (req_pool_indices, "req_pool_indices"), (kv_indptr, "kv_indptr"),
+            (qo_indptr, "qo_indptr"), (q_tile_to_batch, "q_tile_to_batch"), (q_tile_to_index, "q_tile_to_index"))
+    for t, name in ints:
+        if t.dtype != torch.int32 or t.device != q.device:
+            raise RuntimeError(f"{name} must be int32 on q's device")
+    total_q, h, d = q.shape
+    slots, hkv = k_cache.size(0), k_cache.size(1)
+    b = req_pool_indices.numel()
+    if k_cache.size(2) != d:
+        raise RuntimeError("k_cache head_dim mismatch")
+    if h % hkv:
+        raise RuntimeError("q_head must be divisible by kv_head")
+    if req_to_token.dim() != 2 or kv_indptr.numel() != b + 1 or qo_indptr.numel() != b + 1:
+        raise RuntimeError("req_to_token must be 2D, kv_indptr and qo_indptr [batch+1]")
+    if q_tile_to_batch.dim() != 1 or q_tile_to_batch.shape != q_tile_to_index.shape:
+        raise RuntimeError("q_tile_to_batch and q_tile_to_index must be 1D of equal length")
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise RuntimeError("the pools must be contiguous")
+    q_c = q.contiguous()
+    tensors = [t.contiguous() for t, _ in ints]
+    if scale is None or scale <= 0.0:
+        scale = d ** -0.5
+    with torch.cuda.device(q.device):
+        # (rows that no tile of the schedule covers are left unwritten, as by the reference)
+        out = torch.empty((total_q, h, d), device=q.device, dtype=torch.bfloat16)
+        _check(lib.astrai_w8a8_attn_paged_prefill_bf16(
+            q_c.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), *[t.data_ptr() for t in tensors],
+            out.data_ptr(), q_tile_to_batch.numel(), h, hkv, d, slots, req_to_token.size(0),
+            req_to_token.size(1), 1 if causal_offset >= 0 else 0, float(scale), _stream(q)), lib)
+    return out
+
+
+def paged_prefill_schedule(q_lens, device):
+    """``(qo_indptr, q_tile_to_batch, q_tile_to_index)`` for per-sequence query row counts,
+    built as astrai/inference/cache/pool.py:219-234 builds them (64-row tiles)."""
+    qo = [0]
+    tb, ti = [], []
+    for i, n in enumerate(q_lens):
+        qo.append(qo[-1] + int(n))
+        nt = (int(n) + Q_TILE_ROWS - 1) // Q_TILE_ROWS
+        tb += [i] * nt
+        ti += list(range(nt))
+    mk = lambda v: torch.tensor(v, dtype=torch.int32, device=device)
+    return mk(qo), mk(tb), mk(ti)
 
 
 def attn_prefill_supported(n_heads: int, n_kv_heads: int, head_dim: int) -> bool:

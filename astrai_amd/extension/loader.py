@@ -57,8 +57,14 @@ def _attn_paged_decode_module() -> SimpleNamespace:
     return SimpleNamespace(attn_paged_decode=_cabi.attn_paged_decode)
 
 
+def _attn_paged_prefill_module() -> SimpleNamespace:
+    # the callable of csrc/kernels/attention/paged_prefill.cu:36-52, same argument list
+    return SimpleNamespace(attn_paged_prefill=_cabi.attn_paged_prefill)
+
+
 _FACTORIES = {
     "attn_paged_decode": _attn_paged_decode_module,
+    "attn_paged_prefill": _attn_paged_prefill_module,
     "fp8_mm": _fp8_mm_module,
     "int8_mm": _int8_mm_module,
     "fp8_block_mm": _fp8_block_mm_module,

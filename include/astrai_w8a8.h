@@ -235,6 +235,34 @@ int astrai_w8a8_attn_prefill_bf16(const void* q_bf16, const void* k_cache_bf16,
                                   float scale, void* stream);
 
 /*
+ * The same causal block attention over ragged sequences in a token-granular paged cache.
+ * Replaces attn_paged_prefill (csrc/kernels/attention/paged_prefill.cu:4-52, addressing
+ * policies PackedQSchedule / PagedKV in csrc/kernels/attention/layout_policies.cuh:67-93,
+ * 174-232; Python wrapper astrai/extension/ops/attention.py:150-207) without the optional
+ * key mask.
+ *   q, out     bf16 [total_q, n_heads, 128]: the query rows of all sequences, packed
+ *   k_pool, v_pool, req_to_token, req_pool_indices, kv_indptr  as for attn_paged_decode_bf16
+ *   qo_indptr  int32 [batch + 1]: prefix sums of the sequences' query row counts
+ *   q_tile_to_batch, q_tile_to_index  int32 [num_q_tiles]: the caller's schedule of 64-row
+ *              query tiles (astrai/inference/cache/pool.py:219-234): sequence of tile t, and
+ *              its index within that sequence
+ *   causal     non-zero: row i of a sequence with q_len rows and kv_len keys attends keys
+ *              0 .. kv_len - q_len + i (layout_policies.cuh:190-193); zero: all kv_len keys.
+ *              A row that may see no key yields zeros.
+ * Same arithmetic as attn_prefill_bf16. head_dim == 128, n_heads / n_kv_heads in {2, 4, 8},
+ * num_slots * n_kv_heads * 256 < 2^32. Allocates nothing, no workspace.
+ */
+int astrai_w8a8_attn_paged_prefill_bf16(const void* q_bf16, const void* k_pool_bf16,
+                                        const void* v_pool_bf16, const int32_t* req_to_token,
+                                        const int32_t* req_pool_indices, const int32_t* kv_indptr,
+                                        const int32_t* qo_indptr, const int32_t* q_tile_to_batch,
+                                        const int32_t* q_tile_to_index, void* out_bf16,
+                                        int64_t num_q_tiles, int64_t n_heads, int64_t n_kv_heads,
+                                        int64_t head_dim, int64_t num_slots, int64_t num_requests,
+                                        int64_t max_context_len, int causal, float scale,
+                                        void* stream);
+
+/*
  * bf16 -> e4m3fn with one scale per 1x128 K-group (activations) or per 128x128
  * block (weights). No counterpart in the reference. K must be a multiple of 128.
  *   act:    sa[m,kb]  = max(max |x[m,128kb..128kb+127]|, 1e-12) / 448,   sa is [M, K/128]

@@ -100,6 +100,38 @@ def attn_paged_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tenso
     return out.to(q.dtype)
 
 
+def attn_paged_prefill(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                       req_to_token: torch.Tensor, req_pool_indices: torch.Tensor,
+                       kv_indptr: torch.Tensor, qo_indptr: torch.Tensor,
+                       causal: bool = True) -> torch.Tensor:
+    """Ragged prefill over the paged cache: packed ``q [total_q, H, D]``; sequence ``b`` owns
+    rows ``qo_indptr[b] .. qo_indptr[b+1]`` and keys ``req_to_token[req_pool_indices[b], :kv_len]``;
+    with ``causal`` row ``i`` of it sees keys ``0 .. kv_len - q_len + i``
+    (csrc/kernels/attention/layout_policies.cuh:67-93,174-232). float32 softmax attention per
+    sequence; a row that sees no key gives zeros. Returns ``[total_q, H, D]`` in the input dtype."""
+    total_q, h, d = q.shape
+    n_rep = h // k_pool.size(1)
+    out = torch.zeros(total_q, h, d, dtype=torch.float32)
+    for b in range(req_pool_indices.numel()):
+        q0, q1 = int(qo_indptr[b]), int(qo_indptr[b + 1])
+        n = int(kv_indptr[b + 1]) - int(kv_indptr[b])
+        if q1 == q0 or n == 0:
+            continue
+        rows = req_to_token[int(req_pool_indices[b]), :n].long()
+        k = k_pool[rows.clamp_min(0)].float().repeat_interleave(n_rep, dim=1)   # [n, H, D]
+        v = v_pool[rows.clamp_min(0)].float().repeat_interleave(n_rep, dim=1)
+        scores = torch.einsum("qhd,nhd->hqn", q[q0:q1].float(), k) / (d ** 0.5)
+        visible = (rows >= 0)[None, :].expand(q1 - q0, n).clone()
+        if causal:
+            newest = (n - (q1 - q0)) + torch.arange(q1 - q0)
+            visible &= torch.arange(n)[None, :] <= newest[:, None]
+        scores = scores.masked_fill(~visible[None], float("-inf"))
+        p = torch.softmax(scores, dim=-1)
+        p = torch.where(visible.any(-1)[None, :, None], p, torch.zeros_like(p))
+        out[q0:q1] = torch.einsum("hqn,nhd->qhd", p, v)
+    return out.to(q.dtype)
+
+
 def repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:
     # x: [B, S, H_kv, D] -> [B, S, H_kv*n_rep, D]
     if n_rep == 1:

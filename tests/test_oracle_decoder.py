@@ -169,3 +169,39 @@ def test_paged_decode_oracle_single_key_and_empty_sequence():
                               torch.tensor([0, 1, 1], dtype=torch.int32))
     assert torch.equal(out[0], v_pool[5].repeat_interleave(2, dim=0))
     assert torch.equal(out[1], torch.zeros(4, 8, dtype=torch.bfloat16))
+
+
+def test_paged_prefill_oracle_equals_dense_attention_per_sequence():
+    """Ragged sequences scattered into a pool: for each one the paged-prefill oracle must equal
+    the dense oracle (attn_cached) fed with that sequence alone and positions
+    kv_len - q_len + i -- chunked prefill (cached context first) and whole-prompt prefill."""
+    g = torch.Generator().manual_seed(31)
+    h, hkv, d, max_ctx, pool = 4, 2, 16, 24, 80
+    kv_lens, q_lens = [24, 9, 5], [7, 9, 1]
+    dense_k = torch.randn(3, hkv, max_ctx, d, generator=g).to(torch.bfloat16)
+    dense_v = torch.randn(3, hkv, max_ctx, d, generator=g).to(torch.bfloat16)
+    perm = torch.randperm(pool, generator=g)
+    rows = torch.tensor([2, 0, 3], dtype=torch.int32)
+    table = torch.full((4, max_ctx), -1, dtype=torch.int32)
+    k_pool = torch.randn(pool, hkv, d, generator=g).to(torch.bfloat16)
+    v_pool = torch.randn(pool, hkv, d, generator=g).to(torch.bfloat16)
+    nxt = 0
+    for i in range(3):
+        for j in range(kv_lens[i]):
+            slot = int(perm[nxt]); nxt += 1
+            table[rows[i], j] = slot
+            k_pool[slot], v_pool[slot] = dense_k[i, :, j], dense_v[i, :, j]
+    qo = torch.tensor([0, 7, 16, 17], dtype=torch.int32)
+    kvp = torch.tensor([0, 24, 33, 38], dtype=torch.int32)
+    q = torch.randn(17, h, d, generator=g).to(torch.bfloat16)
+    got = D.attn_paged_prefill(q, k_pool, v_pool, table, rows, kvp, qo, causal=True)
+    for i in range(3):
+        qi = q[qo[i]:qo[i + 1]].permute(1, 0, 2).unsqueeze(0)                  # [1, H, q_len, D]
+        pos = kv_lens[i] - q_lens[i] + torch.arange(q_lens[i])
+        want = D.attn_cached(qi, dense_k[i:i + 1], dense_v[i:i + 1], pos)      # [1, q_len, H*D]
+        assert torch.equal(got[qo[i]:qo[i + 1]].reshape(q_lens[i], -1), want[0]), i
+    # without the causal flag every row sees all kv_len keys
+    full = D.attn_paged_prefill(q, k_pool, v_pool, table, rows, kvp, qo, causal=False)
+    qi = q[0:7].permute(1, 0, 2).unsqueeze(0)
+    want = D.attn_cached(qi, dense_k[0:1], dense_v[0:1], torch.full((7,), 23))
+    assert torch.equal(full[0:7].reshape(7, -1), want[0])
