@@ -18,6 +18,7 @@ stays on the device as tiny tensor ops; nothing here reads a value back to the
 host, so the path stays stream-ordered and graph-capturable.
 """
 
+import weakref
 from contextlib import contextmanager
 from dataclasses import dataclass
 from enum import Enum
@@ -143,9 +144,10 @@ class FP8TensorMeta:
         self._x = _AmaxRing(device, n)
         self._g = _AmaxRing(device, n)
         # host-side bookkeeping of FP8State.cache_weights
+        self.w_ref = None     # weakref to the tensor object whose pushes are being counted
         self.w_version = -1   # weight._version at the last push into the weight ring
         self.w_repeats = 0    # consecutive pushes made from that same version
-        self.w_cached = None  # (version, w8, amax_w) quantized with the settled step
+        self.w_cached = None  # (weakref to the weight, version, w8, amax_w): codes made with the settled step
 
     w_hist, w_idx = _ring_property("_w", "hist"), _ring_property("_w", "idx")
     w_scale, w_init = _ring_property("_w", "scale"), _ring_property("_w", "seeded")
@@ -165,19 +167,24 @@ class FP8TensorMeta:
 
     def init_w(self, w: torch.Tensor, fmt: str) -> None:
         self._w.seed(w, self.recipe, fmt)
+        self.w_ref = weakref.ref(w)
         self.w_version, self.w_repeats = w._version, self.recipe.history_len
+
+    def _same_weight(self, w: torch.Tensor) -> bool:
+        # same tensor object (an address can be reused by another tensor), same contents
+        return self.w_ref is not None and self.w_ref() is w and self.w_version == w._version
 
     def w_settled(self, w: torch.Tensor) -> bool:
         """True when every slot of the weight ring holds the amax of ``w`` as it is
         now, so that one more push would change neither the ring nor the step."""
-        return self.w_version == w._version and self.w_repeats >= self.recipe.history_len
+        return self._same_weight(w) and self.w_repeats >= self.recipe.history_len
 
     def note_w_push(self, w: torch.Tensor) -> None:
         self.w_cached = None  # the step may have moved with this push
-        if self.w_version == w._version:
+        if self._same_weight(w):
             self.w_repeats += 1
         else:
-            self.w_version, self.w_repeats = w._version, 1
+            self.w_ref, self.w_version, self.w_repeats = weakref.ref(w), w._version, 1
 
     def init_x(self, x: torch.Tensor, fmt: str) -> None:
         self._x.seed(x, self.recipe, fmt)
@@ -217,11 +224,13 @@ class FP8State:
         """``(sw, w8)`` of dynamic scaling, reused while ``w`` is unmodified."""
         key = (w.data_ptr(), w.shape, fmt, self.recipe.margin)
         hit = self._dyn_w.get(key)
-        if hit is not None and hit[0] == w._version:
-            return hit[1], hit[2]
+        # the entry must belong to this very tensor object: an address can be handed to a new
+        # tensor whose version counter happens to match
+        if hit is not None and hit[0]() is w and hit[1] == w._version:
+            return hit[2], hit[3]
         sw = _dynamic_scale(w, self.recipe, fmt)
         w8, _ = quantize_bf16(w, sw, fmt)
-        self._dyn_w[key] = (w._version, sw, w8)
+        self._dyn_w[key] = (weakref.ref(w), w._version, sw, w8)
         return sw, w8
 
     def reset(self) -> None:
@@ -307,13 +316,14 @@ def fp8_linear_forward(x: torch.Tensor, w: torch.Tensor, bias=None):
         # The weight ring already holds this weight's amax in every slot: pushing it
         # again would leave ring and step as they are, so codes made with that step
         # stay valid until the weight is written to.
-        if meta.w_cached is None or meta.w_cached[0] != w._version:
+        hit = meta.w_cached
+        if hit is None or hit[0]() is not w or hit[1] != w._version:
             w8, amax_w = quantize_bf16(w, meta.w_scale, "e4m3")
-            meta.w_cached = (w._version, w8, amax_w)
+            meta.w_cached = (weakref.ref(w), w._version, w8, amax_w)
         x2 = x.reshape(-1, w.size(1))
         x8, amax_x = quantize_bf16(x2, meta.x_scale, "e4m3")
         has_bias = bias is not None and bias.numel() > 0
-        out = mm_fp8_bias(x8, meta.w_cached[1], meta.x_scale, meta.w_scale,
+        out = mm_fp8_bias(x8, meta.w_cached[2], meta.x_scale, meta.w_scale,
                           bias if has_bias else None).reshape(*x.shape[:-1], w.size(0))
         meta.update_x(amax_x, fmt)
         return out
