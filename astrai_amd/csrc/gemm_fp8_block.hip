@@ -11,7 +11,7 @@ namespace w8a8 {
 bool launch_gemm_fp8_block128_tiled(const GemmArgs& g, hipStream_t stream) {
     if (!tiled_shape_ok(g) || (g.k & 127) != 0) return false;
     if (pingpong_shape_ok(g) && (g.n & 7) == 0 && g.out_kind == OUT_BF16) {
-        launch_pingpong<Op32F8<0>, SCALE_BLOCK128>(g, stream);
+        launch_pingpong<Op32F8<0>, SCALE_BLOCK128, PingPongCfgBlock>(g, stream);
         return true;
     }
     // the 256x256 configuration of the generic tiled kernel runs out of registers

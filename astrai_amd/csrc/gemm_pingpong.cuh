@@ -81,21 +81,31 @@ struct Op32F8 {
     }
 };
 
-struct PingPongCfg {
+// MI_ 32-row activation sub-tiles by NI_ 32-row weight sub-tiles per wave; the
+// eight wave tiles cover the 256 x 256 output tile
+template <int MI_, int NI_>
+struct PingPongShape {
     static constexpr int BM = 256, BN = 256, BK = 128;
     static constexpr int THREADS = 512;
-    static constexpr int MI = 4;  // 32-row activation sub-tiles per wave (128 m)
-    static constexpr int NI = 2;  // 32-row weight sub-tiles per wave (64 n)
+    static constexpr int MI = MI_, NI = NI_;
+    static constexpr int WAVE_M = 32 * MI, WAVE_N = 32 * NI;  // rows of m, n per wave
+    static constexpr int WAVES_M = BM / WAVE_M;               // waves along m
+    static_assert(MI * NI == 8 && WAVES_M * (BN / WAVE_N) == 8, "eight waves, eight sub-tiles each");
     static constexpr int OPERAND_STAGE_BYTES = 256 * BK;   // one operand's slab: 32 KiB
     static constexpr int X_STAGES = 3, W_STAGES = 2;
     static constexpr int W_BASE = X_STAGES * OPERAND_STAGE_BYTES;  // weights after activations
     static constexpr int STAGES_BYTES = (X_STAGES + W_STAGES) * OPERAND_STAGE_BYTES;  // 160 KiB
-    static constexpr int EPI_ROW_BYTES = 144;            // 64 bf16 + 16 bytes of padding
-    static constexpr int EPI_WAVE_BYTES = 128 * EPI_ROW_BYTES;
-    // all 160 KiB of the CU's LDS; the epilogue re-uses the space, 8 x 18 KiB
+    static constexpr int EPI_ROW_BYTES = 2 * WAVE_N + 16;  // a row of bf16 + 16 bytes of padding
+    static constexpr int EPI_WAVE_BYTES = WAVE_M * EPI_ROW_BYTES;
+    // all 160 KiB of the CU's LDS; the epilogue re-uses the space
     static constexpr int LDS_BYTES = STAGES_BYTES;
     static_assert(8 * EPI_WAVE_BYTES <= LDS_BYTES, "epilogue staging must fit");
 };
+using PingPongCfg = PingPongShape<4, 2>;     // 128 (m) x 64 (n) wave tiles
+// Block scales: a lane keeps one scale, one ratio and one load in flight per
+// activation sub-tile, so the wave tile is 64 (m) x 128 (n): two sub-tiles of m
+// instead of four, and the 128 columns are exactly one weight block.
+using PingPongCfgBlock = PingPongShape<2, 4>;
 
 // s_waitcnt vmcnt(N) alone: all but the N most recently issued vector-memory
 // loads of this wave have landed (gfx9 encoding: vmcnt in bits 3:0 and 15:14,
@@ -154,10 +164,9 @@ __device__ unsigned long long* g_pp_dbg;
 #define PP_STAMP()
 #endif
 
-template <class Op, int ScaleKind>
-__global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(GemmArgs g) {
+template <class Op, int ScaleKind, class Cfg = PingPongCfg>
+__global__ __launch_bounds__(Cfg::THREADS) void gemm_pingpong_kernel(GemmArgs g) {
     PP_STAMP_INIT();
-    using Cfg = PingPongCfg;
     using Acc = typename Op::Acc;
     constexpr int MI = Cfg::MI, NI = Cfg::NI;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
@@ -166,8 +175,8 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int group = wave >> 2;       // 0: memory phase on even steps, 1: on odd steps
-    const int wave_m = wave & 1;       // 2 x 128 rows of m
-    const int wave_n = (wave >> 1);    // 4 x 64 rows of n
+    const int wave_m = wave % Cfg::WAVES_M;  // which WAVE_M rows of m
+    const int wave_n = wave / Cfg::WAVES_M;  // which WAVE_N rows of n
     const int lrow = lane & 31;
     const int lgrp = lane >> 5;
 
@@ -209,7 +218,14 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
         // per-instruction offsets are re-added here (one v_add each) instead of
         // living in eight registers across the whole loop as hoisted invariants
         uint32_t off_e = ld_off_even, off_o = ld_off_odd;
-        asm volatile("" : "+v"(off_e), "+v"(off_o));
+        if constexpr (ScaleKind == SCALE_BLOCK128) {
+            // one register fewer: rows start at multiples of 128 bytes, so the odd
+            // instructions' chunk c0 ^ 1 is the even offset with bit 4 flipped
+            asm volatile("" : "+v"(off_e));
+            off_o = off_e ^ 16u;
+        } else {
+            asm volatile("" : "+v"(off_e), "+v"(off_o));
+        }
 #pragma unroll
         for (int i = 0; i < 8; ++i)
             lds_dma16(rld, dst + i * 1024, ((i & 1) ? off_o : off_e) + (uint32_t)i * row8, k0);
@@ -226,8 +242,11 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
     const uint32_t pf_off = (uint32_t)(ld_row0 + lane) * (uint32_t)K;
     const i32x4 rld_raw = raw_rsrc(ld_ptr, ld_bytes);
     uint32_t pf_reg = 0;
+    // (not with block scales: measured slower there with the touches than without)
+    constexpr bool kBlk = ScaleKind == SCALE_BLOCK128;
+    constexpr int kTouch = kBlk ? 0 : 1;  // touches per phase
     auto prefetch = [&](int kstep) {
-        if constexpr (ScaleKind == SCALE_BLOCK128) return;  // registers are needed elsewhere
+        if constexpr (kTouch == 0) return;
         const uint32_t k0 = (uint32_t)kstep << 7;
         asm volatile("buffer_load_dword %0, %1, %2, %3 offen"
                      : "+v"(pf_reg) : "v"(pf_off), "s"(rld_raw), "s"(k0) : "memory");
@@ -241,8 +260,8 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
 #pragma unroll
         for (int j = 0; j < 4; ++j) frag_off[j] = lrow * 128 + (((4 * lgrp + j) ^ sw) << 4);
     }
-    const int x_base = (wave_m * 128) * 128;                   // activation rows of this wave
-    const int w_base = Cfg::W_BASE + (wave_n * 64) * 128;      // weight rows of this wave
+    const int x_base = (wave_m * Cfg::WAVE_M) * 128;                // activation rows of this wave
+    const int w_base = Cfg::W_BASE + (wave_n * Cfg::WAVE_N) * 128;  // weight rows of this wave
 
     Acc acc[NI][MI];
 #pragma unroll
@@ -257,6 +276,14 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
     auto read_frags = [&](int xstage, int wstage) {
         const uint8_t* xb = lds + x_base + xstage * Cfg::OPERAND_STAGE_BYTES;
         const uint8_t* wb = lds + w_base + wstage * Cfg::OPERAND_STAGE_BYTES;
+        if constexpr (ScaleKind == SCALE_BLOCK128) {
+            // registers are scarce in this variant: chunk j's position is chunk 0's
+            // with j xor-ed into its two low chunk bits, re-derived at every use
+            int f0 = frag_off[0];
+            asm volatile("" : "+v"(f0));
+#pragma unroll
+            for (int j = 1; j < 4; ++j) frag_off[j] = f0 ^ (j << 4);
+        }
 #pragma unroll
         for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
@@ -280,52 +307,92 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
                     acc[ni][mi] = Op::mma_step(st, wf[ni], xf[mi], acc[ni][mi]);
     };
 
-    // ---- 128-block scales (SCALE_BLOCK128 only). The promotion
+    // ---- 128-block scales (SCALE_BLOCK128 only; wave tile of two activation
+    // sub-tiles by one 128-column weight block). The promotion
     //   out += P_kb * sa[m,kb] * sb[n/128,kb]
     // is run in place on the accumulator: it is kept divided by the current
     // block's scale s_kb = sa*sb, i.e. before slab kb's MFMAs the accumulator is
     // multiplied by s_{kb-1}/s_kb and after the last slab by s_last. That needs no
-    // second register tile for P_kb. Scales below 1e-20 are taken as 1e-20. The
-    // multiplies run in the wave's operand-read phase: placed inside the MFMA
-    // stream (in front of each accumulator's first MFMA of the slab) they were
-    // measured 25% slower still.
-    // A lane owns one m per 32-row sub-tile (4 values) and one weight block.
-    [[maybe_unused]] float blk_s[MI] = {1.0f, 1.0f, 1.0f, 1.0f};   // scale the accumulators are divided by
-    [[maybe_unused]] float blk_next[MI] = {1.0f, 1.0f, 1.0f, 1.0f}; // scale of the slab computed next
+    // second register tile for P_kb. Scales below 1e-20 are taken as 1e-20.
+    // A lane owns one m per 32-row sub-tile and the wave one weight block.
+    //
+    // The multiplies run inside the MFMA stream: eight independent ones fit in the
+    // shadow of one 32x32x64 MFMA. While the eight MFMAs of sub-tile 0 issue,
+    // sub-tile 1 (not yet touched in this slab) is brought to this slab's scale;
+    // while those of sub-tile 1 issue, sub-tile 0 (finished for this slab) is
+    // brought to the next slab's. The scales are therefore requested two slabs
+    // ahead, after the phase's slab loads (a wait in front of a slab load would
+    // delay it), and turned into factors at the start of the next operand-read
+    // phase, when every load older than them has landed long ago: a scale load
+    // issued in the phase that needs it leaves ~1000 cycles of latency exposed.
+    static_assert(!kBlk || (MI == 2 && NI == 4 && Op::STEPS == 2),
+                  "block scales need the 64 (m) x 128 (n) wave tile and two K steps per slab");
+    [[maybe_unused]] float blk_s[2] = {1.0f, 1.0f};  // latest scale consumed, per sub-tile
+    [[maybe_unused]] float blk_r0 = 1.0f;       // sub-tile 0: this slab's scale -> the next slab's
+    [[maybe_unused]] float blk_r1 = 1.0f;       // sub-tile 1: the previous slab's scale -> this slab's
+    [[maybe_unused]] float blk_r1_next = 1.0f;  // the same for the next slab
     [[maybe_unused]] const int kblocks = ksteps;
-    // activation scales through a buffer resource: one 32-bit row offset per lane,
-    // rows past M read as zero (and are clamped like any tiny scale)
+    // lane l asks for the activation scale of row l of the wave's 64 (rows past M
+    // read as zero and are clamped like any tiny scale); the halves of the wave
+    // exchange them at use
     [[maybe_unused]] const __amdgpu_buffer_rsrc_t rsa =
-        make_rsrc(g.sa, (ScaleKind == SCALE_BLOCK128) ? (uint32_t)g.m * (uint32_t)kblocks * 4u : 0u);
+        make_rsrc(g.sa, kBlk ? (uint32_t)g.m * (uint32_t)kblocks * 4u : 0u);
     [[maybe_unused]] const uint32_t sa_off =
-        (uint32_t)(m0 + wave_m * 128 + lrow) * (uint32_t)kblocks * 4u;
+        (uint32_t)(m0 + wave_m * Cfg::WAVE_M + lane) * (uint32_t)kblocks * 4u;
+    [[maybe_unused]] const float* const sb_row =
+        kBlk ? g.sb + (size_t)((n0 + wave_n * Cfg::WAVE_N) >> 7) * kblocks : nullptr;
+    [[maybe_unused]] float blk_sa_ld = 1.0f, blk_sb_ld = 1.0f;  // scales in flight
     [[maybe_unused]] auto load_block_scales = [&](int kb) {
-        if constexpr (ScaleKind == SCALE_BLOCK128) {
-            const int nb = (n0 + wave_n * 64) >> 7;
-            const float sbv = g.sb[(size_t)nb * kblocks + kb];
-#pragma unroll
-            for (int mi = 0; mi < MI; ++mi) {
-                const float sav = __builtin_bit_cast(
-                    float, __builtin_amdgcn_raw_buffer_load_b32(
-                               rsa, sa_off + (uint32_t)(mi * 32) * (uint32_t)kblocks * 4u,
-                               (uint32_t)kb * 4u, 0));
-                blk_next[mi] = fmaxf(sav * sbv, 1e-20f);
-            }
+        if constexpr (kBlk) {
+            kb = min(kb, kblocks - 1);  // past the end: a harmless re-read
+            blk_sb_ld = sb_row[kb];
+            blk_sa_ld = __builtin_bit_cast(
+                float, __builtin_amdgcn_raw_buffer_load_b32(rsa, sa_off, (uint32_t)kb * 4u, 0));
         }
     };
-    // multiply the accumulators by s_prev / s_cur and make s_cur the current scale
-    [[maybe_unused]] auto rescale = [&](bool first) {
-        if constexpr (ScaleKind == SCALE_BLOCK128) {
+    // the scales in flight, per sub-tile
+    [[maybe_unused]] auto landed_scales = [&](float (&next)[2]) {
+        // v_permlane32_swap of a register with itself: first result = the low
+        // half's values in both halves (rows 0..31), second = the high half's
+        const auto both = __builtin_amdgcn_permlane32_swap(
+            __float_as_uint(blk_sa_ld), __float_as_uint(blk_sa_ld), false, false);
+        next[0] = fmaxf(__uint_as_float(both[0]) * blk_sb_ld, 1e-20f);
+        next[1] = fmaxf(__uint_as_float(both[1]) * blk_sb_ld, 1e-20f);
+    };
+    // at the start of slab k's operand-read phase: slab k+1's scales become factors
+    [[maybe_unused]] auto next_factors = [&](int k) {
+        if constexpr (kBlk) {
+            float next[2];
+            landed_scales(next);
+            const bool last = k + 1 >= ksteps;  // no slab follows: stay at this scale
+            blk_r1 = blk_r1_next;
+            // hardware reciprocal (1 ulp) against a 1e-2 output tolerance
+            blk_r0 = last ? 1.0f : blk_s[0] * __builtin_amdgcn_rcpf(next[0]);
+            blk_r1_next = last ? 1.0f : blk_s[1] * __builtin_amdgcn_rcpf(next[1]);
+            blk_s[0] = last ? blk_s[0] : next[0];
+            blk_s[1] = last ? blk_s[1] : next[1];
+        }
+    };
+    // one slab's MFMAs with the rescaling multiplies between them
+    [[maybe_unused]] auto compute_block = [&]() {
+        if constexpr (kBlk) {
 #pragma unroll
-            for (int mi = 0; mi < MI; ++mi) {
-                // hardware reciprocal (1 ulp) against a 1e-2 output tolerance; the IEEE
-                // division sequence also cost the registers that made this variant spill
-                const float r = first ? 1.0f : blk_s[mi] * __builtin_amdgcn_rcpf(blk_next[mi]);
-                blk_s[mi] = blk_next[mi];
-                if (!first) {
+            for (int mi = 0; mi < 2; ++mi) {
+                const float r = mi ? blk_r0 : blk_r1;
 #pragma unroll
-                    for (int ni = 0; ni < NI; ++ni) acc[ni][mi] *= r;
-                }
+                for (int st = 0; st < 2; ++st)
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni) {
+                        acc[ni][mi] = Op::mma_step(st, wf[ni], xf[mi], acc[ni][mi]);
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            const int f = (st * NI + ni) * 8 + j;
+                            float t = acc[f >> 4][mi ^ 1][f & 15] * r;
+                            asm volatile("" : "+v"(t));  // here, not sunk towards its use
+                            acc[f >> 4][mi ^ 1][f & 15] = t;
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
             }
         }
     };
@@ -334,7 +401,12 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
     PP_STAMP();
     issue_loads(0, 0);
     if (ksteps > 1) issue_loads(1, 1);
+    load_block_scales(0);
     __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0) lgkmcnt(0) expcnt(0)
+    if constexpr (kBlk) {
+        landed_scales(blk_s);  // the accumulators start out at slab 0's scale
+        load_block_scales(1);
+    }
     __syncthreads();
     PP_STAMP();
 
@@ -354,10 +426,10 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
     if (group == 0) {
         int xs = 0;  // k % 3
         for (int k = 0; k < ksteps; ++k) {
-            load_block_scales(k);  // lands while the operand reads are in flight
             read_frags(xs, k & 1);
-            rescale(k == 0);       // accumulators now relative to slab k's scale
+            next_factors(k);
             if (k >= 1 && k + 1 < ksteps) issue_loads(k + 1, (k + 1) & 1);
+            load_block_scales(k + 2);
             // always one touch, so that "all but the last one" below means the slab
             // loads; past the end it re-touches the last slab (an L2 hit)
             prefetch(min(k + kPrefetch, ksteps - 1));
@@ -367,11 +439,12 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
             // has MFMAs of the previous slab to issue it goes first (the hardware
             // otherwise favours this, older, wave and starves the other one)
             __builtin_amdgcn_s_setprio(1);
-            compute();
+            if constexpr (kBlk) compute_block();
+            else compute();
             __builtin_amdgcn_s_setprio(0);
             PP_STAMP();
             // the slab loads; the prefetch touch (if any) may stay in flight
-            wait_vmcnt<(ScaleKind == SCALE_BLOCK128) ? 0 : 1>();
+            wait_vmcnt<kTouch>();
             PP_STAMP();
             phase_barrier();  // B_{k+1}
             PP_STAMP();
@@ -380,38 +453,54 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
         }
         phase_barrier();  // matches group 1's final barrier
     } else {
-        int xs = 0;  // k % 3
-        for (int k = 0; k < ksteps; ++k) {
-            __builtin_amdgcn_s_setprio(2);
-            if (k > 0) compute();  // slab k-1
-            __builtin_amdgcn_s_setprio(0);
-            PP_STAMP();
-            load_block_scales(k);
+        // memory phase of slab k and the barrier that ends it
+        auto memory_phase = [&](int k, int xs) {
             read_frags(xs, k & 1);
-            rescale(k == 0);      // slab k-1's MFMAs are issued; next come slab k's
+            next_factors(k);
             const int xs2 = (xs == 0) ? 2 : xs - 1;  // (k + 2) % 3
             const bool more = k + 2 < ksteps;
             if (more) issue_loads(k + 2, xs2);
+            load_block_scales(k + 2);
             prefetch(min(k + 2 + kPrefetch, ksteps - 1));
             wait_lgkmcnt0();
             PP_STAMP();
             // slab k+1 (issued one slab ago) must have landed; this slab's eight
             // loads and the two latest touches may stay in flight
-            // (block scales: this phase's scale loads precede its slab loads and no
-            // touches exist, so the eight slab loads are the only younger ones)
-            if (more) wait_vmcnt<(ScaleKind == SCALE_BLOCK128) ? 8 : 10>();
-            else wait_vmcnt<(ScaleKind == SCALE_BLOCK128) ? 0 : 1>();
+            // (block scales: and this phase's two scale loads)
+            if (more) wait_vmcnt<8 + 2 * kTouch + (kBlk ? 2 : 0)>();
+            else wait_vmcnt<kTouch>();
             PP_STAMP();
             phase_barrier();  // B_{k+1}
             PP_STAMP();
             PP_STAMP();
+        };
+        int xs = 0;  // k % 3
+        if constexpr (kBlk) {
+            // slab 0 has no predecessor to compute: kept out of the loop, whose MFMAs
+            // are then unconditional (under "if (k > 0)" the compiler moved the second
+            // half's multiplies out of the MFMA stream, behind the join)
+            PP_STAMP();
+            memory_phase(0, 0);
+            xs = 1;
+        }
+        for (int k = kBlk ? 1 : 0; k < ksteps; ++k) {
+            __builtin_amdgcn_s_setprio(2);
+            if constexpr (kBlk) {
+                compute_block();  // slab k-1
+            } else {
+                if (k > 0) compute();  // slab k-1
+            }
+            __builtin_amdgcn_s_setprio(0);
+            PP_STAMP();
+            memory_phase(k, xs);
             xs = (xs == 2) ? 0 : xs + 1;
         }
-        compute();  // last slab
+        if constexpr (kBlk) compute_block();  // last slab
+        else compute();
         phase_barrier();
     }
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): no prefetch touch outlives the loop
-    if constexpr (ScaleKind != SCALE_BLOCK128) asm volatile("" :: "v"(pf_reg));
+    asm volatile("" :: "v"(pf_reg));
 
     // ---------------- epilogue ----------------
     PP_STAMP();
@@ -425,7 +514,7 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
         // 0 is here, on registers only).
         uint8_t* const mine = lds + wave * Cfg::EPI_WAVE_BYTES;
         const uint16_t* bias = static_cast<const uint16_t*>(g.bias);
-        const int nw = n0 + wave_n * 64;
+        const int nw = n0 + wave_n * Cfg::WAVE_N;
 #pragma unroll
         for (int ni = 0; ni < NI; ++ni) {
 #pragma unroll
@@ -446,7 +535,7 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
 #pragma unroll
                 for (int mi = 0; mi < MI; ++mi) {
                     const int ml = mi * 32 + lrow;
-                    const int m = m0 + wave_m * 128 + ml;
+                    const int m = m0 + wave_m * Cfg::WAVE_M + ml;
                     float sx = 1.0f;
                     if constexpr (ScaleKind == SCALE_ROWCOL) sx = (m < g.m) ? g.sa[m] : 0.0f;
                     float v[4];
@@ -467,12 +556,14 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
         }
         // same wave reads back: LDS operations of one wave complete in order
         uint16_t* out = static_cast<uint16_t*>(g.out);
-        const int rr = lane >> 3, cc = lane & 7;
+        constexpr int kRowLanes = Cfg::WAVE_N / 8;   // lanes per row, 16 bytes each
+        constexpr int kRowsPer = 64 / kRowLanes;     // rows per store instruction
+        const int rr = lane / kRowLanes, cc = lane % kRowLanes;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int ml = i * 8 + rr;
+        for (int i = 0; i < Cfg::WAVE_M / kRowsPer; ++i) {
+            const int ml = i * kRowsPer + rr;
             const u32x4 v = *reinterpret_cast<const u32x4*>(mine + ml * Cfg::EPI_ROW_BYTES + cc * 16);
-            const int m = m0 + wave_m * 128 + ml;
+            const int m = m0 + wave_m * Cfg::WAVE_M + ml;
             const int n = nw + cc * 8;
             // non-temporal: the output streams to memory during the epilogue instead of
             // sitting dirty in L2 until the end-of-kernel write-back
@@ -482,12 +573,12 @@ __global__ __launch_bounds__(PingPongCfg::THREADS) void gemm_pingpong_kernel(Gem
     } else {
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi) {
-            const int m = m0 + wave_m * 128 + mi * 32 + lrow;
+            const int m = m0 + wave_m * Cfg::WAVE_M + mi * 32 + lrow;
 #pragma unroll
             for (int ni = 0; ni < NI; ++ni) {
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    const int n = n0 + wave_n * 64 + ni * 32 + q * 8 + lgrp * 4;
+                    const int n = n0 + wave_n * Cfg::WAVE_N + ni * 32 + q * 8 + lgrp * 4;
                     typename Op16::Acc v = {acc[ni][mi][4 * q], acc[ni][mi][4 * q + 1],
                                             acc[ni][mi][4 * q + 2], acc[ni][mi][4 * q + 3]};
                     store_subtile<Op16, ScaleKind>(g, es, v, m, n);
@@ -505,11 +596,10 @@ inline bool pingpong_shape_ok(const GemmArgs& g) {
     return tiles >= 192 && g.k >= 256;
 }
 
-template <class Op, int ScaleKind>
+template <class Op, int ScaleKind, class Cfg = PingPongCfg>
 inline void launch_pingpong(const GemmArgs& g, hipStream_t stream) {
-    using Cfg = PingPongCfg;
     const int tiles = ((g.m + Cfg::BM - 1) / Cfg::BM) * ((g.n + Cfg::BN - 1) / Cfg::BN);
-    auto kern = gemm_pingpong_kernel<Op, ScaleKind>;
+    auto kern = gemm_pingpong_kernel<Op, ScaleKind, Cfg>;
     static bool attr_set = false;
     if (!attr_set) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),

@@ -282,6 +282,24 @@ def test_config3_shape_sampled_rows():
     assert_bf16_close(out[rows], O.fp8_gemm_blockscaled(rx8, rw8, rsa, rsb), what="config3 rows")
 
 
+@pytest.mark.parametrize("m,n,k", [(3841, 3336, 256),    # two slabs: the shortest K the large kernel takes
+                                   (4000, 3592, 384),    # three slabs
+                                   (3600, 4096, 1152)])
+def test_block128_large_kernel_wide_scale_range(m, n, k):
+    """The 256x256-tile block-scaled kernel (>= 192 tiles, N % 8 == 0) on ragged M and
+    N, with block scales spread over twelve octaves so that every slab's rescaling
+    factor matters, checked on the whole output."""
+    from astrai_amd.extension.ops import fp8_block as blk
+    print(f"case m={m} n={n} k={k}", flush=True)
+    g = torch.Generator().manual_seed(m + n + k)
+    a8 = (torch.randn(m, k, generator=g) * 2.0).to(torch.float8_e4m3fn)
+    b8 = (torch.randn(n, k, generator=g) * 2.0).to(torch.float8_e4m3fn)
+    sa = torch.exp2(torch.rand(m, k // 128, generator=g) * 12.0 - 6.0)
+    sb = torch.exp2(torch.rand((n + 127) // 128, k // 128, generator=g) * 12.0 - 6.0)
+    out = blk.mm_fp8_blockscaled(a8.to(DEV), b8.to(DEV), sa.to(DEV), sb.to(DEV))
+    assert_bf16_close(out, O.fp8_gemm_blockscaled(a8, b8, sa, sb), what="block128 large")
+
+
 # ---- large ragged shapes: the 256x256-tile kernels with partial edge tiles ----
 
 @pytest.mark.parametrize("m,n,k,bias", [(3900, 4104, 1152, True),    # N % 8 == 0: four-wave kernel
