@@ -72,7 +72,6 @@ __device__ __forceinline__ void lds_dma16(__amdgpu_buffer_rsrc_t r, uint8_t* lds
 // without the causal flag), so nothing has to be fetched to know the key range.
 template <int NREP, bool PAGED>
 __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_kernel(AttnPrefillArgs a) {
-    constexpr int THREADS = 64 * NREP;
     constexpr int K_DMA = kKB / 4 / NREP;              // 1 KiB key loads per wave and block
     __shared__ __attribute__((aligned(16))) uint8_t lds[kKRingBytes + 2 * kVBytes];
 

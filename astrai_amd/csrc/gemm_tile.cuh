@@ -307,12 +307,8 @@ template <class Op, class Cfg, int ScaleKind>
 inline void launch_tiled(const GemmArgs& g, hipStream_t stream) {
     const int tiles = ((g.m + Cfg::BM - 1) / Cfg::BM) * ((g.n + Cfg::BN - 1) / Cfg::BN);
     auto kern = gemm_tiled_kernel<Op, Cfg, ScaleKind>;
-    static bool attr_set = false;  // benign race: the attribute is idempotent
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
-        attr_set = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};
+    allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::LDS_BYTES, lds_allowed);
     kern<<<dim3((unsigned)tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(g);
 }
 

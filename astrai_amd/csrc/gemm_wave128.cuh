@@ -359,12 +359,8 @@ inline void launch_wave128(const GemmArgs& g, hipStream_t stream) {
     using Cfg = Wave128Cfg;
     const int tiles = ((g.m + Cfg::BM - 1) / Cfg::BM) * ((g.n + Cfg::BN - 1) / Cfg::BN);
     auto kern = gemm_wave128_kernel<Op, ScaleKind>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
-        attr_set = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};
+    allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::LDS_BYTES, lds_allowed);
     kern<<<dim3((unsigned)tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(g);
 }
 

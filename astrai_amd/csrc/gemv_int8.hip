@@ -385,12 +385,8 @@ void launch_skinny(const GemmArgs& g, hipStream_t stream) {
     static_assert(MB <= 8, "the reduction re-uses the staging space: NW * RG * MB KiB must fit");
     static_assert(lds_bytes <= 160 * 1024, "staging space of all waves must fit in LDS");
     auto kern = skinny_int8_kernel<RG, MB, NW>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-        attr_set = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};
+    allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_allowed);
     const int blocks = (g.n + RG * 16 - 1) / (RG * 16);
     kern<<<dim3((unsigned)blocks), dim3(NW * 64), lds_bytes, stream>>>(g);
 }

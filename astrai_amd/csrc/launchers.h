@@ -6,7 +6,22 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace w8a8 {
+
+// Opt a kernel into more than 64 KiB of dynamic LDS. The attribute belongs to the
+// (kernel, device) pair and a process may drive several devices from several
+// threads, so `done` (one per kernel, static at the call site) keeps one bit per
+// device; setting the attribute twice is harmless.
+inline void allow_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done) {
+    int dev = 0;
+    const bool known = hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64;
+    const uint64_t bit = known ? (uint64_t)1 << dev : 0;
+    if (known && (done.load(std::memory_order_acquire) & bit)) return;
+    (void)hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (known) done.fetch_or(bit, std::memory_order_release);
+}
 
 enum OutKind : int { OUT_BF16 = 0, OUT_E4M3 = 1, OUT_ACC = 2 };
 enum ScaleKind : int { SCALE_TENSOR = 0, SCALE_ROWCOL = 1, SCALE_BLOCK128 = 2 };
