@@ -153,6 +153,35 @@ def _bench_decoder(dev):
     return res
 
 
+def _measured_ceilings():
+    """What a kernel on this very GPU can approach, measured now: a register-resident
+    loop of nothing but MFMAs on random operand bits (the power manager clocks it
+    well below the datasheet rate) and a plain streaming read of a decode-size matrix.
+    The micro-benchmark is a program of its own (astrai_amd/csrc/ubench), started as a
+    child BEFORE this process touches the GPU, and not at all under a profiler (whose
+    preloaded library has the GPU initialised already). Returns {} when it is not
+    built or did not run."""
+    exe = os.path.join(ROOT, "astrai_amd", "csrc", "ubench", "ceilings")
+    if not os.access(exe, os.X_OK):
+        return {}
+    if "rocprof" in os.environ.get("LD_PRELOAD", "") or any(k.startswith("ROCPROF") for k in os.environ):
+        return {}
+    import re
+    import subprocess
+    try:
+        out = subprocess.run([exe], capture_output=True, text=True, timeout=120, check=True).stdout
+    except (OSError, subprocess.SubprocessError):
+        return {}
+    res = {}
+    for key, pat in (("mfma_fp8_random_TFLOPs", r"mfma fp8 32x32x64\s+operands random:\s*([0-9.]+) Tops/s"),
+                     ("mfma_i8_random_TOPs", r"mfma i8 32x32x32\s+operands random:\s*([0-9.]+) Tops/s"),
+                     ("hbm_stream_45MB_GBs", r"hbm read, 45.1 MB per launch[^:]*:\s*[0-9.]+ us per launch, ([0-9.]+) GB/s")):
+        m = re.search(pat, out)
+        if m:
+            res[key] = float(m.group(1))
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -174,6 +203,9 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU's share of the path: run with --gpus 1 "
                  "(no multi-GPU leg exists: the path shards by output columns or by K, one collective at most)")
+
+    tracing = bool(args.decoder_trace or args.trace_kernels or args.pmc)
+    ceilings = {} if tracing else _measured_ceilings()
 
     import torch
 
@@ -312,6 +344,12 @@ def main():
                 "WRITE_SIZE, calibrated on a plain copy; summary in profiles/gemm_fp8_wave128_4096cubed.txt)",
                 "kernel": "gemm_wave128_kernel<Op32F8<e4m3>,per-tensor> (256x256x128, 4 waves)",
                 "avg_launch_us": round(kern_ms * 1e3, 2)}
+    if "mfma_fp8_random_TFLOPs" in ceilings:
+        # the same kernel against what this GPU's MFMA pipe sustains on random operand bits
+        roofline["measured_ceiling"] = {
+            "value": ceilings["mfma_fp8_random_TFLOPs"], "unit": "TFLOP/s",
+            "frac": round(achieved / ceilings["mfma_fp8_random_TFLOPs"], 4),
+            "what": "register-resident v_mfma_f32_32x32x64_f8f6f4 loop, random operand bits, measured in this run"}
 
     # ---------------- CPU baseline: the oracle on this host ----------------
     cpu_baseline = None
@@ -446,6 +484,8 @@ def main():
             ms1 = _graph_time_ms(lambda i: launch(0), 40, 10)
             gemv[f"M{m}"] = {"us": round(ms * 1e3, 2), "GB/s": round(gbs, 0),
                              "frac_hbm_peak": round(gbs / PEAK_HBM_GBS, 4),
+                             **({"frac_measured_stream": round(gbs / ceilings["hbm_stream_45MB_GBs"], 4)}
+                                if "hbm_stream_45MB_GBs" in ceilings else {}),
                              "single_buffer_cache_resident_us": round(ms1 * 1e3, 2)}
         extra["int8_gemv_11008x4096_hbm_ring"] = gemv
         del ring
@@ -489,6 +529,7 @@ def main():
                                "fp32 accumulate, bf16 out, seed 1"},
         "roofline": roofline, "cpu_baseline": cpu_baseline, "extra": extra,
         "host": {"cpu_count": os.cpu_count(), "torch": torch.__version__},
+        "measured_ceilings": ceilings,
     }
     print(json.dumps(line))
 
