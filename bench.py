@@ -196,6 +196,9 @@ def main():
     ap.add_argument("--trace-kernels", action="store_true",
                     help="tracing mode: a few launches of every auxiliary kernel (quantizers, policy-path "
                          "kernels, attention) at 4096 x 4096 / config-4 sizes, nothing else")
+    ap.add_argument("--trace-gemms", action="store_true",
+                    help="tracing mode: a few launches of the large GEMM kernels besides the headline one "
+                         "(int8 4096^3, block-scaled config 3, fp8 with e4m3 output), nothing else")
     ap.add_argument("--pmc", action="store_true",
                     help="counter-collection mode: a few launches of the headline kernel and of a "
                          "plain 256 MiB device copy (the calibration kernel), nothing else")
@@ -204,7 +207,7 @@ def main():
         sys.exit("bench.py measures one GPU's share of the path: run with --gpus 1 "
                  "(no multi-GPU leg exists: the path shards by output columns or by K, one collective at most)")
 
-    tracing = bool(args.decoder_trace or args.trace_kernels or args.pmc)
+    tracing = bool(args.decoder_trace or args.trace_kernels or args.trace_gemms or args.pmc)
     ceilings = {} if tracing else _measured_ceilings()
 
     import torch
@@ -275,6 +278,34 @@ def main():
         print(json.dumps({"trace_kernels": "5 launches each; sizes: 4096x4096 bf16 for the quantizers, "
                                            "32 x 16/4 heads x 512 new tokens x 128 for prefill attention, "
                                            "32 sequences x 640 keys for decode attention"}))
+        return
+
+    if args.trace_gemms:
+        from oracle import w8a8_oracle as O
+
+        xq = torch.randint(-127, 128, (4096, 4096), dtype=torch.int8, device=dev)
+        wq = torch.randint(-127, 128, (4096, 4096), dtype=torch.int8, device=dev)
+        sx, sw = torch.rand(4096, device=dev) + 0.5, torch.rand(4096, device=dev) + 0.5
+        y = torch.empty(4096, 4096, device=dev, dtype=torch.bfloat16)
+        # config 3 data (seed 3, 1% x20 outliers in the weight), quantized on the device
+        x3, w3, _ = O.make_inputs(3, 8192, 2048, 7168, outlier_p=0.01)
+        a3, sa3 = _cabi.quantize_fp8_block128_act(x3.to(dev))
+        b3, sb3 = _cabi.quantize_fp8_block128_weight(w3.to(dev))
+        y3 = torch.empty(8192, 2048, device=dev, dtype=torch.bfloat16)
+        a8 = (torch.randn(4096, 4096, device=dev) * 0.5).to(torch.float8_e4m3fn)
+        b8 = (torch.randn(4096, 4096, device=dev) * 0.5).to(torch.float8_e4m3fn)
+        one = torch.ones(1, device=dev)
+        y8 = torch.empty(4096, 4096, device=dev, dtype=torch.float8_e4m3fn)
+        for _ in range(20):
+            check(lib.astrai_w8a8_gemm_int8_ptpc(xq.data_ptr(), wq.data_ptr(), sx.data_ptr(), sw.data_ptr(), None,
+                                                 y.data_ptr(), 4096, 4096, 4096, 0, stream))
+            check(lib.astrai_w8a8_gemm_fp8_block128(a3.data_ptr(), b3.data_ptr(), sa3.data_ptr(), sb3.data_ptr(),
+                                                    None, y3.data_ptr(), 8192, 2048, 7168, stream))
+            check(lib.astrai_w8a8_gemm_fp8_pt(a8.data_ptr(), b8.data_ptr(), one.data_ptr(), one.data_ptr(),
+                                              one.data_ptr(), None, y8.data_ptr(), 4096, 4096, 4096, 0, 1, stream))
+        torch.cuda.synchronize()
+        print(json.dumps({"trace_gemms": "20 launches each: int8 4096^3 per-token x per-channel (bf16 out), fp8 "
+                                         "128-block 8192x2048x7168 on config-3 data, fp8 4096^3 with e4m3 output"}))
         return
 
     # ---------------- headline: config 1, fp8 per-tensor 4096^3 ----------------
