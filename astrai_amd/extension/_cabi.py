@@ -205,8 +205,10 @@ def mm_fp8(a: torch.Tensor, b: torch.Tensor, sa: torch.Tensor, sb: torch.Tensor,
         out = torch.empty((m, n), device=a.device,
                           dtype=torch.float8_e4m3fn if out_dtype else torch.bfloat16)
         if m and n:
-            if k == 0:
+            if k == 0:  # an empty sum: zeros (plus the bias)
                 out.zero_()
+                if bias is not None:
+                    out.copy_(bias.expand(m, n))
             else:
                 _check(lib.astrai_w8a8_gemm_fp8_pt(
                     a_c.data_ptr(), b_c.data_ptr(), sa.data_ptr(), sb.data_ptr(),
