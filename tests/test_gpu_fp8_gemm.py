@@ -229,6 +229,23 @@ def test_config1_sampled_rows_at_full_size(ops):
     assert_bf16_close(out[rows], want, what="config1 rows")
 
 
+def test_random_shape_sweep_fp8(ops):
+    """Forty seeded random shapes, both formats, through the default dispatch."""
+    g = torch.Generator().manual_seed(777)
+    for i in range(40):
+        m = int(torch.randint(1, 400, (1,), generator=g))
+        n = int(torch.randint(1, 600, (1,), generator=g))
+        k = int(torch.randint(1, 1500, (1,), generator=g))
+        fmt = torch.float8_e5m2 if i % 4 == 3 else torch.float8_e4m3fn
+        print(f"case {i}: m={m} n={n} k={k} {fmt}", flush=True)
+        a8 = (torch.randn(m, k, generator=g) * 1.5).to(fmt)
+        b8 = (torch.randn(n, k, generator=g) * 1.5).to(fmt)
+        sa = torch.rand(1, generator=g) + 0.25
+        sb = torch.rand(1, generator=g) + 0.25
+        out = ops.mm_fp8(a8.to(DEV), b8.to(DEV), sa.to(DEV), sb.to(DEV))
+        assert_bf16_close(out, O.fp8_gemm(a8, b8, sa, sb), what=f"sweep {m}x{n}x{k}")
+
+
 # ---- 128-block scaled ----
 
 @pytest.mark.parametrize("m,n,k", [(3, 130, 256), (64, 128, 128), (130, 200, 384), (257, 513, 1024)])

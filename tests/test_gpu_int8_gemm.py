@@ -36,6 +36,31 @@ def test_int32_accumulator_bit_exact(C, m, n, k):
     assert got.dtype == torch.int32 and torch.equal(got, O.int8_acc(a, b))
 
 
+def test_random_shape_sweep_default_dispatch_bit_exact(C):
+    """Sixty seeded random shapes through the default entry point, whichever kernel
+    it picks (single-token, skinny, tiled, generic): accumulators bit-exact, and the
+    scaled bf16 output bit-equal to the oracle's elementwise epilogue."""
+    g = torch.Generator().manual_seed(20240)
+    for i in range(60):
+        m = int(torch.randint(1, 301, (1,), generator=g))
+        n = int(torch.randint(1, 701, (1,), generator=g))
+        k = int(torch.randint(1, 1201, (1,), generator=g))
+        if i % 3 == 0:
+            k = (k + 255) // 256 * 256   # the skinny kernels need K % 256 == 0
+        if i % 4 == 0:
+            m = 1 + i % 40
+        print(f"case {i}: m={m} n={n} k={k}", flush=True)
+        a, b = _rand_i8(g, m, k), _rand_i8(g, n, k)
+        want = O.int8_acc(a, b)
+        got = C.mm_int8(a.to(DEV), b.to(DEV), None, None, None, 2).cpu()
+        assert torch.equal(got, want), (m, n, k)
+        sa = torch.rand(m, generator=g) * 0.02 + 0.001
+        sb = torch.rand(n, generator=g) * 0.02 + 0.001
+        out = C.mm_int8(a.to(DEV), b.to(DEV), sa.to(DEV), sb.to(DEV), None, 0).cpu()
+        ref = (want.float() * sa[:, None] * sb[None, :]).to(torch.bfloat16)
+        assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), (m, n, k)
+
+
 def test_golden_integer_cases_including_worst_case_magnitude(C, golden):
     for c in golden("int8_small.json")["gemm"]:
         a = torch.tensor(c["a"], dtype=torch.int8)
