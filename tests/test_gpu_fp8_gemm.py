@@ -229,6 +229,29 @@ def test_config1_sampled_rows_at_full_size(ops):
     assert_bf16_close(out[rows], want, what="config1 rows")
 
 
+def test_empty_operands(ops):
+    """No rows, no columns, no elements: shapes and dtypes as for any other input,
+    no launch, no error (the reference allocates the same empty outputs, mm.cu:111-124,154-160)."""
+    from astrai_amd.extension import _cabi
+    s = torch.ones(1, device=DEV)
+    x8, amax = ops.quantize_bf16(torch.empty(0, 64, device=DEV, dtype=torch.bfloat16), s)
+    assert x8.shape == (0, 64) and x8.dtype == torch.float8_e4m3fn and amax.shape == (1,) and float(amax) == 0.0
+    a8 = torch.zeros(0, 64, device=DEV).to(torch.float8_e4m3fn)
+    b8 = torch.zeros(24, 64, device=DEV).to(torch.float8_e4m3fn)
+    out = ops.mm_fp8(a8, b8, s, s)
+    assert out.shape == (0, 24) and out.dtype == torch.bfloat16
+    out = ops.mm_fp8(b8, a8, s, s)
+    assert out.shape == (24, 0)
+    y, ax, aw = _cabi.linear_forward_fp8(torch.empty(2, 0, 64, device=DEV, dtype=torch.bfloat16),
+                                         torch.randn(24, 64, device=DEV).to(torch.bfloat16), None, s, s)
+    assert y.shape == (2, 0, 24) and float(ax) == 0.0 and float(aw) > 0.0
+    xq, sx = _cabi.quantize_int8_rows(torch.empty(0, 128, device=DEV, dtype=torch.bfloat16))
+    assert xq.shape == (0, 128) and sx.numel() == 0
+    acc = _cabi.mm_int8(torch.empty(0, 128, device=DEV, dtype=torch.int8),
+                        torch.zeros(16, 128, device=DEV, dtype=torch.int8), None, None, None, 2)
+    assert acc.shape == (0, 16) and acc.dtype == torch.int32
+
+
 def test_random_shape_sweep_fp8(ops):
     """Forty seeded random shapes, both formats, through the default dispatch."""
     g = torch.Generator().manual_seed(777)
