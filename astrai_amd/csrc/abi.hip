@@ -436,6 +436,37 @@ int astrai_w8a8_gemv_int8_ptpc(const void* a, const void* b, const float* sa, co
     return check_launch("gemv_int8_ptpc");
 }
 
+int astrai_w8a8_gemm_int8_ptpc_rope_cache(const void* a, const void* b, const float* sa,
+                                          const float* sb, const float* freqs,
+                                          const int64_t* positions, void* q_out, void* k_cache,
+                                          void* v_cache, int64_t batch, int64_t seq,
+                                          int64_t n_heads, int64_t n_kv_heads, int64_t head_dim,
+                                          int64_t max_len, int64_t k, void* stream) {
+    const char* what = "gemm_int8_ptpc_rope_cache";
+    if (!a || !b || !sa || !sb || !freqs || !positions || !q_out || !k_cache || !v_cache)
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: null pointer", what);
+    if (batch < 0 || seq < 0 || n_heads <= 0 || n_kv_heads <= 0 || head_dim <= 0 || max_len <= 0 ||
+        k <= 0 || n_heads > 65535 || n_kv_heads > 65535 || head_dim > 65536 || k > kMaxDim ||
+        batch > kMaxDim || seq > kMaxDim)
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: bad dims", what);
+    if (!aligned16(a) || !aligned16(b) || !aligned16(freqs) || !aligned16(q_out) || !aligned16(k_cache) ||
+        !aligned16(v_cache))
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: pointers must be 16-byte aligned", what);
+    const int64_t m = batch * seq, n = (n_heads + 2 * n_kv_heads) * head_dim;
+    if (m == 0) return ASTRAI_W8A8_OK;
+    if (m > 64 || k % 256 || head_dim % 4 || n * k >= ((int64_t)1 << 31))
+        return fail(ASTRAI_W8A8_UNSUPPORTED,
+                    "%s: needs batch * seq <= 64, K a multiple of 256, head_dim a multiple of 4 and a "
+                    "weight matrix under 2 GiB (got m=%lld k=%lld head_dim=%lld)",
+                    what, (long long)m, (long long)k, (long long)head_dim);
+    const w8a8::GemmArgs g = pack(a, b, sa, sb, nullptr, nullptr, nullptr, m, n, k, w8a8::OUT_BF16);
+    const w8a8::RopeCacheArgs rc{nullptr, 0, freqs, positions, q_out, k_cache, v_cache,
+                                 (int)batch, (int)seq, (int)n_heads, (int)n_kv_heads, (int)head_dim, max_len};
+    if (!w8a8::launch_gemm_int8_rope_cache(g, rc, static_cast<hipStream_t>(stream)))
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "%s: shape not supported", what);
+    return check_launch(what);
+}
+
 int astrai_w8a8_gemm_int8_ptpc_tiled(const void* a, const void* b, const float* sa,
                                      const float* sb, const void* bias, void* out, int64_t m,
                                      int64_t n, int64_t k, int out_dtype, void* stream) {

@@ -236,8 +236,15 @@ void launch_dot(const GemmArgs& g, hipStream_t stream) {
 //     cut out of LDS again for the next four groups.
 //   * int32 partials of the four waves are summed through LDS (exact), then the
 //     dequant epilogue.
-template <int RG, int MB, int NW>
-__global__ __launch_bounds__(NW * 64) void skinny_int8_kernel(GemmArgs g) {
+//
+// ROPE: the rows are the fused q|k|v projection of a decoder layer and the epilogue
+// goes on where the separate rotary / cache-write kernel would start: the bf16-rounded
+// value pairs of q and k are rotated (fp32 products and sums rounded one by one, one
+// rounding to bf16 -- the arithmetic of rope_cache.hip on the same rounded inputs),
+// q goes to [batch, heads, seq, head_dim], k and v into the cache at the tokens'
+// positions. A lane's four consecutive columns are two rotation pairs of one head.
+template <int RG, int MB, int NW, bool ROPE>
+__global__ __launch_bounds__(NW * 64) void skinny_int8_kernel(GemmArgs g, RopeCacheArgs rc) {
     constexpr int R = RG * 16;
     constexpr int XB = MB < 4 ? MB : 4;
     constexpr int PASSES = (MB + XB - 1) / XB;
@@ -275,6 +282,27 @@ __global__ __launch_bounds__(NW * 64) void skinny_int8_kernel(GemmArgs g) {
             const bool in = live && en + j < g.n;
             e_sw[ti][j] = in ? g.sb[en + j] : 0.0f;
             e_b[ti][j] = (in && g.bias) ? bf16_to_f32(static_cast<const uint16_t*>(g.bias)[en + j]) : 0.0f;
+        }
+    }
+    // ROPE: (cos, sin) of the lane's two pairs and the token's cache slot, per task
+    [[maybe_unused]] f32x4 e_cs[TASKS];
+    [[maybe_unused]] int64_t e_pos[TASKS];
+    if constexpr (ROPE) {
+#pragma unroll
+        for (int ti = 0; ti < TASKS; ++ti) {
+            const int t = wave + ti * NW;
+            const int m = (t % MB) * 16 + lrow;
+            const int en = n0 + (t / MB) * 16 + lgrp * 4;
+            e_cs[ti] = f32x4{1.0f, 0.0f, 1.0f, 0.0f};
+            e_pos[ti] = -1;
+            if (t < RG * MB && m < g.m && en < g.n) {
+                const int sq = m % rc.seq;
+                const int d = en % rc.head_dim;
+                e_pos[ti] = rc.positions[sq];
+                if (en < (rc.n_heads + rc.n_kv_heads) * rc.head_dim)
+                    e_cs[ti] = *reinterpret_cast<const f32x4*>(
+                        rc.freqs + ((int64_t)sq * (rc.head_dim >> 1) + (d >> 1)) * 2);
+            }
         }
     }
 
@@ -365,6 +393,42 @@ __global__ __launch_bounds__(NW * 64) void skinny_int8_kernel(GemmArgs g) {
             const float f = (float)sum[j] * e_sx[ti] * e_sw[ti][j];
             v[j] = f + e_b[ti][j];
         }
+        if constexpr (ROPE) {
+            // what the plain epilogue would have stored, as the rotary kernel would read it
+            u32x2 pk;
+            pk.x = pack_bf16x2(v[0], v[1]);
+            pk.y = pack_bf16x2(v[2], v[3]);
+            const int hh = en / rc.head_dim, d = en - hh * rc.head_dim;
+            const int bt = m / rc.seq, sq = m - bt * rc.seq;
+            if (hh < rc.n_heads + rc.n_kv_heads) {
+                const float x[4] = {__uint_as_float(pk.x << 16), __uint_as_float(pk.x & 0xffff0000u),
+                                    __uint_as_float(pk.y << 16), __uint_as_float(pk.y & 0xffff0000u)};
+                float y[4];
+#pragma unroll
+                for (int p = 0; p < 2; ++p) {
+#pragma clang fp contract(off)
+                    const float c = e_cs[ti][2 * p], sn = e_cs[ti][2 * p + 1];
+                    const float xe = x[2 * p], xo = x[2 * p + 1];
+                    const float a0 = xe * c, a1 = xo * sn, b0 = xe * sn, b1 = xo * c;
+                    y[2 * p] = a0 - a1;
+                    y[2 * p + 1] = b0 + b1;
+                }
+                pk.x = pack_bf16x2(y[0], y[1]);
+                pk.y = pack_bf16x2(y[2], y[3]);
+            }
+            if (hh < rc.n_heads) {
+                uint16_t* dst = static_cast<uint16_t*>(rc.q_out) +
+                                (((int64_t)bt * rc.n_heads + hh) * rc.seq + sq) * rc.head_dim + d;
+                *reinterpret_cast<u32x2*>(dst) = pk;
+            } else if (e_pos[ti] >= 0 && e_pos[ti] < rc.max_len) {  // a slot outside the cache: nothing
+                const bool is_k = hh < rc.n_heads + rc.n_kv_heads;
+                const int hk = hh - rc.n_heads - (is_k ? 0 : rc.n_kv_heads);
+                uint16_t* dst = static_cast<uint16_t*>(is_k ? rc.k_cache : rc.v_cache) +
+                                (((int64_t)bt * rc.n_kv_heads + hk) * rc.max_len + e_pos[ti]) * rc.head_dim + d;
+                *reinterpret_cast<u32x2*>(dst) = pk;
+            }
+            continue;
+        }
         uint16_t* out = static_cast<uint16_t*>(g.out);
         if ((g.n & 3) == 0) {
             u32x2 pk;
@@ -379,16 +443,27 @@ __global__ __launch_bounds__(NW * 64) void skinny_int8_kernel(GemmArgs g) {
     }
 }
 
-template <int RG, int MB, int NW>
-void launch_skinny(const GemmArgs& g, hipStream_t stream) {
+template <int RG, int MB, int NW, bool ROPE = false>
+void launch_skinny(const GemmArgs& g, hipStream_t stream, const RopeCacheArgs& rc = RopeCacheArgs{}) {
     constexpr int lds_bytes = NW * RG * 16 * 512;
     static_assert(MB <= 8, "the reduction re-uses the staging space: NW * RG * MB KiB must fit");
     static_assert(lds_bytes <= 160 * 1024, "staging space of all waves must fit in LDS");
-    auto kern = skinny_int8_kernel<RG, MB, NW>;
+    auto kern = skinny_int8_kernel<RG, MB, NW, ROPE>;
     static std::atomic<uint64_t> lds_allowed{0};
     allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_allowed);
     const int blocks = (g.n + RG * 16 - 1) / (RG * 16);
-    kern<<<dim3((unsigned)blocks), dim3(NW * 64), lds_bytes, stream>>>(g);
+    kern<<<dim3((unsigned)blocks), dim3(NW * 64), lds_bytes, stream>>>(g, rc);
+}
+
+// the q|k|v projection with rotary and cache write in the epilogue: up to 64 tokens
+template <int RG, int NW>
+void launch_skinny_rope_mb(const GemmArgs& g, const RopeCacheArgs& rc, hipStream_t stream) {
+    switch ((g.m + 15) / 16) {
+        case 1: launch_skinny<RG, 1, NW, true>(g, stream, rc); break;
+        case 2: launch_skinny<RG, 2, NW, true>(g, stream, rc); break;
+        case 3: launch_skinny<RG, 3, NW, true>(g, stream, rc); break;
+        default: launch_skinny<RG, 4, NW, true>(g, stream, rc); break;
+    }
 }
 
 template <int RG, int NW>
@@ -425,6 +500,21 @@ void launch_lds(const GemmArgs& g, hipStream_t stream) {
 }
 
 }  // namespace
+
+bool launch_gemm_int8_rope_cache(const GemmArgs& g, const RopeCacheArgs& rc, hipStream_t stream) {
+    if (g.m <= 0 || g.m > 64 || g.n <= 0 || g.k <= 0 || (g.k & 255) != 0 || (g.n & 3) != 0) return false;
+    if (g.out_kind != OUT_BF16 || g.bias != nullptr || (rc.head_dim & 3) != 0) return false;
+    if (g.m != rc.batch * rc.seq || g.n != (rc.n_heads + 2 * rc.n_kv_heads) * rc.head_dim) return false;
+    if ((int64_t)g.n * g.k >= ((int64_t)1 << 31)) return false;
+    // the same workgroup shapes as the plain skinny launch
+    const int nsteps = (g.k + 511) >> 9;
+    if ((g.n + 47) / 48 >= 192) launch_skinny_rope_mb<3, 4>(g, rc, stream);
+    else if ((g.n + 31) / 32 >= 192) launch_skinny_rope_mb<2, 4>(g, rc, stream);
+    else if (nsteps <= 4 || (g.n + 15) / 16 >= 512) launch_skinny_rope_mb<1, 4>(g, rc, stream);
+    else if (nsteps <= 8) launch_skinny_rope_mb<1, 8>(g, rc, stream);
+    else launch_skinny_rope_mb<1, 16>(g, rc, stream);
+    return true;
+}
 
 bool launch_gemv_int8(const GemmArgs& g, hipStream_t stream) {
     if (g.m <= 0 || g.m > 128 || g.n <= 0 || g.k <= 0 || (g.k & 255) != 0) return false;

@@ -146,5 +146,8 @@ void launch_gemm_generic(const GemmArgs& g, int op /*0=i8,1=e4m3,2=e5m2*/, int s
 
 // gemv_int8.hip: skinny int8 kernel, m <= 64, k % 256 == 0.
 bool launch_gemv_int8(const GemmArgs& g, hipStream_t stream);
+// the fused q|k|v projection of up to 64 tokens with rotary embedding and KV-cache write
+// in the epilogue (g.out unused; rc.qkv / rc.ld unused); false when the shape does not fit
+bool launch_gemm_int8_rope_cache(const GemmArgs& g, const RopeCacheArgs& rc, hipStream_t stream);
 
 }  // namespace w8a8

@@ -61,6 +61,8 @@ PROTOTYPES = {
     "astrai_w8a8_gemm_int8_ptpc": ([_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _INT, _P], _INT),
     "astrai_w8a8_gemv_int8_ptpc": ([_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _INT, _P], _INT),
     "astrai_w8a8_gemm_int8_ptpc_tiled": ([_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _INT, _P], _INT),
+    "astrai_w8a8_gemm_int8_ptpc_rope_cache": (
+        [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _P], _INT),
 }
 
 _lib: Optional[ctypes.CDLL] = None
@@ -795,6 +797,54 @@ def mm_int8(a: torch.Tensor, b: torch.Tensor, sa: Optional[torch.Tensor],
                 _check(fn(a_c.data_ptr(), b_c.data_ptr(), _ptr(sa), _ptr(sb), _ptr(bias),
                           out.data_ptr(), m, n, k, out_dtype, _stream(a)), lib)
     return out
+
+
+def mm_int8_rope_cache_supported(tokens: int, k: int, head_dim: int) -> bool:
+    """Shapes the fused q|k|v projection + rotary + cache-write kernel takes."""
+    return 0 < tokens <= 64 and k % 256 == 0 and head_dim % 4 == 0
+
+
+def mm_int8_rope_cache(a: torch.Tensor, wqkv: torch.Tensor, sa: torch.Tensor, sb: torch.Tensor,
+                       freqs: torch.Tensor, positions: torch.Tensor, k_cache: torch.Tensor,
+                       v_cache: torch.Tensor, batch: int, seq: int, n_heads: int, n_kv_heads: int,
+                       head_dim: int) -> torch.Tensor:
+    """``mm_int8(a, wqkv, sa, sb)`` followed by :func:`rope_cache_write` on its output, as one
+    kernel and bit for bit the same: ``a`` int8 ``[batch*seq, K]`` (at most 64 rows), ``wqkv``
+    int8 ``[(n_heads + 2 n_kv_heads) * head_dim, K]``. Writes k and v into the caches at
+    ``positions`` and returns the rotated q as ``[batch, n_heads, seq, head_dim]``."""
+    lib = _require()
+    _gpu(a, "mm_int8_rope_cache")
+    if a.dtype != torch.int8 or wqkv.dtype != torch.int8 or a.dim() != 2 or wqkv.dim() != 2:
+        raise RuntimeError("a and wqkv must be 2D int8")
+    m, k = a.shape
+    n = (n_heads + 2 * n_kv_heads) * head_dim
+    if m != batch * seq or wqkv.size(0) != n or wqkv.size(1) != k:
+        raise RuntimeError("a must be [batch*seq, K] and wqkv [(n_heads + 2 n_kv_heads) * head_dim, K]")
+    if not mm_int8_rope_cache_supported(m, k, head_dim):
+        raise RuntimeError("mm_int8_rope_cache: needs at most 64 tokens, K % 256 == 0, head_dim % 4 == 0")
+    sa = _check_vec(sa, a, m, "sa")
+    sb = _check_vec(sb, a, n, "sb")
+    if k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
+        raise RuntimeError("the caches must be bf16")
+    if freqs.dtype != torch.float32 or tuple(freqs.shape[-3:]) != (seq, head_dim // 2, 2):
+        raise RuntimeError("freqs must be fp32 [seq, head_dim/2, 2]")
+    if positions.dtype != torch.int64 or positions.numel() != seq:
+        raise RuntimeError("positions must be int64 [seq]")
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous()) or k_cache.shape != v_cache.shape:
+        raise RuntimeError("caches must be contiguous and of one shape")
+    if k_cache.dim() != 4 or k_cache.size(0) != batch or k_cache.size(1) != n_kv_heads or k_cache.size(3) != head_dim:
+        raise RuntimeError("caches must be [batch, n_kv_heads, max_len, head_dim]")
+    for t in (wqkv, freqs, positions, k_cache, v_cache):
+        if t.device != a.device:
+            raise RuntimeError("all tensors must be on a's device")
+    a_c, w_c = a.contiguous(), wqkv.contiguous()
+    with torch.cuda.device(a.device):
+        q_out = torch.empty((batch, n_heads, seq, head_dim), device=a.device, dtype=torch.bfloat16)
+        _check(lib.astrai_w8a8_gemm_int8_ptpc_rope_cache(
+            a_c.data_ptr(), w_c.data_ptr(), sa.data_ptr(), sb.data_ptr(), freqs.contiguous().data_ptr(),
+            positions.contiguous().data_ptr(), q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+            batch, seq, n_heads, n_kv_heads, head_dim, k_cache.size(2), k, _stream(a)), lib)
+    return q_out
 
 
 def quantize_fp8_block128_act(x: torch.Tensor):

@@ -192,11 +192,17 @@ class GQA(nn.Module):
         token-major), for longer blocks the causal block kernel followed by the quantizer
         (SDPA only for head layouts neither kernel takes)."""
         from astrai_amd.extension import _cabi
-        from astrai_amd.extension.ops import int8 as I
-        b, s, _ = qkv.shape
         q = _cabi.rope_cache_write(qkv, rotary_emb[0], positions, kv_cache.k[self.layer_id],
                                    kv_cache.v[self.layer_id], self.n_heads, self.n_kv_heads,
                                    self.head_dim)
+        return self.attend_rotated(q, kv_cache, positions, key_mask)
+
+    def attend_rotated(self, q: Tensor, kv_cache: DenseKVCache, positions: Tensor, key_mask: Tensor):
+        """The attention of :meth:`core_fused_qkv` for an already rotated ``q [B, H, S, D]``
+        whose keys and values are in the cache."""
+        from astrai_amd.extension import _cabi
+        from astrai_amd.extension.ops import int8 as I
+        b, _, s, _ = q.shape
         if _cabi.attn_decode_supported(self.n_heads, self.n_kv_heads, s, self.head_dim):
             return _cabi.attn_decode(q, kv_cache.k[self.layer_id], kv_cache.v[self.layer_id], positions,
                                      quantized=True)
@@ -243,6 +249,7 @@ class DecoderBlock(nn.Module):
         """``x`` plus the not yet added residual branch ``pending`` (``None`` for the first
         block) is the block input; returns ``(h, mlp_out)`` whose sum is the block output -- the
         add is left to the next norm kernel, which also has to read both."""
+        from astrai_amd.extension import _cabi
         from astrai_amd.extension.ops import int8 as I
         f, att = self.fused_int8, self.attention
         b, s, d = x.shape
@@ -250,14 +257,21 @@ class DecoderBlock(nn.Module):
                                                res=pending)
         if xsum is not None:
             x = xsum
-        qkv = I.mm_int8(xq, f.wqkv, sx, f.sqkv).reshape(b, s, -1)
-        if kv_cache is not None:
-            aq, sa = att.core_fused_qkv(qkv, rotary_emb, kv_cache, positions, key_mask)
-        else:
+        if kv_cache is None:
+            qkv = I.mm_int8(xq, f.wqkv, sx, f.sqkv).reshape(b, s, -1)
             nq, nkv = att.n_heads * att.head_dim, att.n_kv_heads * att.head_dim
             aq, sa = I.quantize_int8_per_token(
                 att.core(qkv[..., :nq], qkv[..., nq:nq + nkv], qkv[..., nq + nkv:], rotary_emb, None,
                          positions, key_mask))
+        elif _cabi.mm_int8_rope_cache_supported(b * s, d, att.head_dim):
+            # a few new tokens: the projection's epilogue rotates q and k and writes the cache
+            q = _cabi.mm_int8_rope_cache(xq, f.wqkv, sx, f.sqkv, rotary_emb[0], positions,
+                                         kv_cache.k[att.layer_id], kv_cache.v[att.layer_id],
+                                         b, s, att.n_heads, att.n_kv_heads, att.head_dim)
+            aq, sa = att.attend_rotated(q, kv_cache, positions, key_mask)
+        else:
+            qkv = I.mm_int8(xq, f.wqkv, sx, f.sqkv).reshape(b, s, -1)
+            aq, sa = att.core_fused_qkv(qkv, rotary_emb, kv_cache, positions, key_mask)
         o = I.mm_int8(aq, f.wo, sa, f.so).reshape(b, s, d)
         # h = attention + x, then its norm, quantized: one kernel
         hq, sh, h = I.rmsnorm_quantize_int8(o, self.post_attention_norm.weight,

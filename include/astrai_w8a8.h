@@ -323,6 +323,27 @@ int astrai_w8a8_gemv_int8_ptpc(const void* a, const void* b, const float* sa,
                                void* stream);
 
 /*
+ * The fused q|k|v projection of a decoder layer for a few new tokens
+ * (batch * seq <= 64), with what follows it in the reference done in the GEMM's
+ * epilogue: the rotary embedding of q and k (astrai/extension/backend/rotary.py:25-33),
+ * the permutes and the KV-cache write (astrai/model/components/attention.py:19-85).
+ * Equal, bit for bit, to astrai_w8a8_gemm_int8_ptpc (bf16 out, no bias) followed by
+ * astrai_w8a8_rope_cache_write_bf16 on its output:
+ *   a int8 [batch*seq, K] with sa fp32 [batch*seq]; b int8 [(n_heads + 2 n_kv_heads) * head_dim, K]
+ *   (rows: q heads | k heads | v heads) with sb fp32 per row; freqs, positions, q_out,
+ *   k_cache, v_cache as for astrai_w8a8_rope_cache_write_bf16.
+ * Needs K % 256 == 0 and head_dim % 4 == 0; ASTRAI_W8A8_UNSUPPORTED otherwise (run the two
+ * calls instead).
+ */
+int astrai_w8a8_gemm_int8_ptpc_rope_cache(const void* a, const void* b, const float* sa,
+                                          const float* sb, const float* freqs,
+                                          const int64_t* positions, void* q_out_bf16,
+                                          void* k_cache_bf16, void* v_cache_bf16, int64_t batch,
+                                          int64_t seq, int64_t n_heads, int64_t n_kv_heads,
+                                          int64_t head_dim, int64_t max_len, int64_t k,
+                                          void* stream);
+
+/*
  * The tiled MFMA int8 kernel on its own (no skinny dispatch), for tests and
  * benchmarks that must name the kernel they measure.
  */

@@ -61,3 +61,59 @@ def test_rope_cache_write_rejects_bad_arguments():
     with pytest.raises(RuntimeError, match="features"):
         _cabi.rope_cache_write(qkv, torch.zeros(1, 8, 2, device=DEV), torch.zeros(1, dtype=torch.long, device=DEV),
                                kc, kc.clone(), 2, 1, 16)
+
+
+@pytest.mark.parametrize("b,s,h,hkv,d,max_len,k", [
+    (32, 1, 16, 4, 128, 640, 2048),    # config-4 decode step
+    (1, 1, 16, 4, 128, 64, 2048),      # one sequence
+    (3, 7, 4, 2, 64, 32, 512),         # a short block of new tokens, 21 rows
+    (4, 16, 2, 1, 16, 40, 256),        # 64 rows: the largest the fused kernel takes
+    (5, 1, 8, 8, 32, 16, 1024),        # no grouping, 16-row workgroups of eight waves
+    (2, 3, 96, 8, 128, 16, 256),       # a wide projection: 48-row workgroups
+])
+def test_projection_with_rotary_epilogue_equals_the_two_kernels(b, s, h, hkv, d, max_len, k):
+    """The fused q|k|v projection + rotary + cache write against the int8 GEMM followed by
+    the rotary / cache-write kernel: q and both caches bit for bit, untouched slots untouched."""
+    from astrai_amd.extension import _cabi
+    print(f"case b={b} s={s} h={h} hkv={hkv} d={d} max_len={max_len} k={k}", flush=True)
+    g = torch.Generator().manual_seed(b * 1000 + s * 10 + d + k)
+    n = (h + 2 * hkv) * d
+    a = torch.randint(-127, 128, (b * s, k), generator=g, dtype=torch.int8).to(DEV)
+    w = torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int8).to(DEV)
+    sa = (torch.rand(b * s, generator=g) * 0.01 + 0.001).to(DEV)
+    sb = (torch.rand(n, generator=g) * 0.01 + 0.001).to(DEV)
+    table = D.rotary_table(d, max_len, 10000.0)
+    positions = torch.randperm(max_len, generator=g)[:s].sort().values
+    freqs = table.index_select(0, positions).to(DEV)
+    pos = positions.to(DEV)
+    kc = torch.randn(b, hkv, max_len, d, generator=g).to(torch.bfloat16)
+    vc = torch.randn(b, hkv, max_len, d, generator=g).to(torch.bfloat16)
+    k1, v1, k2, v2 = kc.to(DEV), vc.to(DEV), kc.to(DEV), vc.to(DEV)
+    qkv = _cabi.mm_int8(a, w, sa, sb).reshape(b, s, n)
+    q_want = _cabi.rope_cache_write(qkv, freqs, pos, k1, v1, h, hkv, d)
+    assert _cabi.mm_int8_rope_cache_supported(b * s, k, d)
+    q_got = _cabi.mm_int8_rope_cache(a, w, sa, sb, freqs, pos, k2, v2, b, s, h, hkv, d)
+    for name, got, want in (("q", q_got, q_want), ("k_cache", k2, k1), ("v_cache", v2, v1)):
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), name
+
+
+def test_projection_with_rotary_epilogue_limits():
+    from astrai_amd.extension import _cabi
+    assert not _cabi.mm_int8_rope_cache_supported(65, 2048, 128)
+    assert not _cabi.mm_int8_rope_cache_supported(8, 2048 + 128, 128)
+    a = torch.zeros(65, 256, dtype=torch.int8, device=DEV)
+    w = torch.zeros(4 * 16, 256, dtype=torch.int8, device=DEV)
+    kc = torch.zeros(65, 1, 4, 16, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError, match="at most 64"):
+        _cabi.mm_int8_rope_cache(a, w, torch.ones(65, device=DEV), torch.ones(64, device=DEV),
+                                 torch.zeros(1, 8, 2, device=DEV), torch.zeros(1, dtype=torch.long, device=DEV),
+                                 kc, kc.clone(), 65, 1, 2, 1, 16)
+    # a slot outside the cache writes nothing, q is still produced
+    a = torch.ones(2, 256, dtype=torch.int8, device=DEV)
+    kc = torch.zeros(2, 1, 4, 16, dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros_like(kc)
+    q = _cabi.mm_int8_rope_cache(a, torch.ones(64, 256, dtype=torch.int8, device=DEV), torch.ones(2, device=DEV),
+                                 torch.ones(64, device=DEV), D.rotary_table(16, 8, 10000.0)[:1].to(DEV),
+                                 torch.tensor([4], device=DEV), kc, vc, 2, 1, 2, 1, 16)
+    torch.cuda.synchronize()
+    assert q.abs().sum().item() > 0 and kc.abs().sum().item() == 0 and vc.abs().sum().item() == 0
