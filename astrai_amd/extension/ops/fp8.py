@@ -1,176 +1,173 @@
-"""FP8 kernel interface adapter: same names, signatures, defaults and scale
-semantics as the reference's ``astrai/extension/ops/fp8.py``.
+"""fp8 primitives of the MI355X backend, behind the call surface AstrAI's policy
+layer uses (reference: ``astrai/extension/ops/fp8.py``).
 
-- ``quantize_bf16(x, scale, fmt) -> (x8, amax)``          (ops/fp8.py:125-132)
-- ``mm_fp8(a8, b8, sa, sb, out_dtype, out_scale) -> out``   (ops/fp8.py:135-154)
-- ``linear_forward_fp8(x, w, bias, sx, sw) -> (out, amax_x, amax_w)``  (:157-166)
-- ``linear_backward_fp8(g, x, w, masks, sg, sw, sx, fmt)``  (:169-184)
+What the reference exposes and where (all in its ``ops/fp8.py``):
 
-Scales are quantization *steps* (``x8 = x / scale``); every primitive computes
-its own inverse; ``amax`` values are returned, never passed in. The custom ops
-``custom::fp8_quantize`` / ``custom::fp8_gemm`` keep the reference's schemas
-(ops/fp8.py:55-58,85-93) so ``torch.compile`` traces them the same way.
+===========================  ============================================  =========
+callable                     returns                                       lines
+===========================  ============================================  =========
+``quantize_bf16``            ``(codes, amax)``                             125-132
+``mm_fp8``                   ``a8 @ b8.T * sa * sb`` (bf16 or e4m3)        135-154
+``linear_forward_fp8``       ``(out, amax_x, amax_w)``                     157-166
+``linear_backward_fp8``      ``(grad_x, grad_w, grad_bias, amax_grad)``    169-184
+``custom::fp8_quantize``     dispatcher op behind ``quantize_bf16``        55-58
+``custom::fp8_gemm``         dispatcher op behind ``mm_fp8``               85-93
+===========================  ============================================  =========
 
-The reference also registers pure-PyTorch ``cpu`` kernels (ops/fp8.py:78-82,
-116-122). Those are its CPU oracle; this backend ships no CPU arithmetic at
-all, so the ops raise for CPU tensors instead of computing.
+Conventions kept from there: a scale is the quantization step (codes are
+``x / scale``, results are multiplied by it), nobody passes reciprocals, an
+amax is handed back as a fresh one-element fp32 tensor. Format names are
+``"e4m3"`` / ``"e5m2"``, output names ``"bf16"`` / ``"e4m3"``; their position in
+the tuples below is the integer the kernels take.
+
+One deliberate difference: the reference registers ``cpu`` kernels in plain
+PyTorch (its lines 78-82 and 116-122). They are its CPU oracle. This backend
+computes nothing on the CPU, so both dispatcher ops fail for CPU tensors.
 """
 
-from typing import Optional
+from __future__ import annotations
+
+from typing import Optional, Sequence, Tuple
 
 import torch
+from torch import Tensor
 from torch.library import custom_op
 
-from astrai_amd.extension.loader import get_module, is_available
+from astrai_amd.extension import loader
 
-# fmt string -> kernel int (0 = E4M3, 1 = E5M2)
-_FMT_TO_INT = {"e4m3": 0, "e5m2": 1}
-
-_MOD: Optional[object] = None
-
-
-def _mod() -> object:
-    global _MOD
-    if _MOD is None:
-        if not is_available("fp8_mm"):
-            raise RuntimeError(
-                "HIP kernel 'fp8_mm' is not available. Build with `make -C astrai_amd/csrc`."
-            )
-        _MOD = get_module("fp8_mm")
-    return _MOD
+_FORMATS: Tuple[str, ...] = ("e4m3", "e5m2")
+_OUTPUTS: Tuple[str, ...] = ("bf16", "e4m3")
+_CODE_DTYPES = (torch.float8_e4m3fn, torch.float8_e5m2)
 
 
-def _no_cpu(op: str):
-    raise RuntimeError(
-        f"{op}: this backend has no CPU implementation; pass tensors on the MI355X device"
-    )
+class _Kernels:
+    """The registry entry ``fp8_mm``, looked up on first use."""
+
+    _entry = None
+
+    @classmethod
+    def get(cls):
+        if cls._entry is None:
+            entry = loader.get_module("fp8_mm") if loader.is_available("fp8_mm") else None
+            if entry is None:
+                raise RuntimeError(
+                    "the 'fp8_mm' kernels are missing: libastrai_w8a8.so did not load "
+                    "(build it with `make -C astrai_amd/csrc`)")
+            cls._entry = entry
+        return cls._entry
 
 
-def _fmt_int(fmt: str) -> int:
-    try:
-        return _FMT_TO_INT[fmt]
-    except KeyError:
-        raise ValueError(f"unsupported fp8 format {fmt!r} (expected 'e4m3' or 'e5m2')")
+def _position(name: str, names: Sequence[str], what: str) -> int:
+    if name not in names:
+        raise ValueError(f"{what} must be one of {', '.join(map(repr, names))}; got {name!r}")
+    return names.index(name)
 
 
-@custom_op("custom::fp8_quantize", mutates_args=())
-def fp8_quantize(
-    x: torch.Tensor, scale: torch.Tensor, fmt: int
-) -> tuple[torch.Tensor, torch.Tensor]:
-    """BF16 -> FP8 quantize with fused amax; returns ``(x8, amax)``."""
-    _no_cpu("custom::fp8_quantize")
+def _all_bf16(what: str, *tensors: Tensor) -> None:
+    bad = [str(t.dtype) for t in tensors if t.dtype != torch.bfloat16]
+    if bad:
+        raise TypeError(f"{what} takes bf16 tensors only (found {', '.join(bad)})")
 
 
-@fp8_quantize.register_fake
-def _fp8_quantize_fake(x, scale, fmt):
-    dtype = torch.float8_e5m2 if fmt else torch.float8_e4m3fn
-    return (
-        torch.empty(x.shape, device=x.device, dtype=dtype),
-        torch.empty(1, device=x.device, dtype=torch.float32),
-    )
+def _device_only(op: str):
+    raise RuntimeError(f"{op} has no CPU kernel in this backend: move the tensors to the GPU")
 
 
-@fp8_quantize.register_kernel("cuda")
-def _fp8_quantize_cuda(x, scale, fmt):
-    if x.dtype != torch.bfloat16:
-        raise TypeError(f"fp8 quantize requires bf16 input, got {x.dtype}")
-    return _mod().quantize_bf16(x, scale, int(fmt))
+# ---------------------------------------------------------------------------
+# dispatcher ops. Schemas are spelled out (they are the reference's, so traced
+# graphs look the same); each op gets a shape function and a device kernel.
+# ---------------------------------------------------------------------------
+
+def _quantize_entry(x, scale, fmt):
+    _device_only("custom::fp8_quantize")
 
 
-@custom_op("custom::fp8_gemm", mutates_args=())
-def fp8_gemm(
-    a: torch.Tensor,
-    b: torch.Tensor,
-    sa: torch.Tensor,
-    sb: torch.Tensor,
-    out_dtype: int = 0,
-    out_scale: Optional[torch.Tensor] = None,
-) -> torch.Tensor:
-    """FP8 GEMM: ``a @ b^T * (sa * sb)`` with FP32 accumulation.
-
-    ``out_dtype``: 0 = BF16 (default), 1 = FP8 E4M3 (requires ``out_scale``).
-    """
-    _no_cpu("custom::fp8_gemm")
+def _quantize_shapes(x, scale, fmt):
+    codes = x.new_empty(x.shape, dtype=_CODE_DTYPES[1 if fmt else 0])
+    return codes, x.new_empty(1, dtype=torch.float32)
 
 
-@fp8_gemm.register_fake
-def _fp8_gemm_fake(a, b, sa, sb, out_dtype=0, out_scale=None):
-    dtype = torch.float8_e4m3fn if out_dtype else torch.bfloat16
-    return torch.empty((a.size(0), b.size(0)), device=a.device, dtype=dtype)
+def _quantize_device(x, scale, fmt):
+    _all_bf16("custom::fp8_quantize", x)
+    return _Kernels.get().quantize_bf16(x, scale, int(fmt))
 
 
-@fp8_gemm.register_kernel("cuda")
-def _fp8_gemm_cuda(a, b, sa, sb, out_dtype=0, out_scale=None):
-    if a.dtype != b.dtype or a.dtype not in (torch.float8_e4m3fn, torch.float8_e5m2):
-        raise TypeError(
-            f"fp8 GEMM requires matching fp8 inputs, got {a.dtype}/{b.dtype}"
-        )
-    return _mod().mm_fp8(a, b, sa, sb, int(out_dtype), out_scale)
+def _gemm_entry(a, b, sa, sb, out_dtype=0, out_scale=None):
+    _device_only("custom::fp8_gemm")
 
 
-def quantize_bf16(x: torch.Tensor, scale: torch.Tensor, fmt: str = "e4m3"):
-    """BF16 -> FP8 quantize with fused amax; returns ``(x8, amax)``.
-
-    ``scale`` is the quantization step (device scalar); ``fmt`` selects E4M3 or
-    E5M2. ``amax`` is a fresh 1-element float32 tensor.
-    """
-    return fp8_quantize(x, scale, _fmt_int(fmt))
+def _gemm_shapes(a, b, sa, sb, out_dtype=0, out_scale=None):
+    return a.new_empty((a.shape[0], b.shape[0]),
+                       dtype=torch.float8_e4m3fn if out_dtype else torch.bfloat16)
 
 
-def amax_bf16(x: torch.Tensor) -> torch.Tensor:
-    """``x.abs().amax()`` as a fresh float32 ``[1]`` tensor from one read of a bf16
-    device tensor (what dynamic scaling measures before it quantizes)."""
-    if x.dtype != torch.bfloat16:
-        raise TypeError(f"amax_bf16 requires a bf16 input, got {x.dtype}")
-    return _mod().amax_bf16(x)
+def _gemm_device(a, b, sa, sb, out_dtype=0, out_scale=None):
+    if a.dtype not in _CODE_DTYPES or b.dtype != a.dtype:
+        raise TypeError(f"custom::fp8_gemm takes two fp8 operands of one format (found {a.dtype} and {b.dtype})")
+    return _Kernels.get().mm_fp8(a, b, sa, sb, int(out_dtype), out_scale)
 
 
-def amax_ring_push(hist, idx: int, amax, scale, fmax: float, pow2_margin: float) -> None:
-    """Delayed scaling's record-then-refresh on device rings, in place, one launch."""
-    _mod().amax_ring_push(hist, idx, amax, scale, fmax, pow2_margin)
+fp8_quantize = custom_op("custom::fp8_quantize", _quantize_entry, mutates_args=(),
+                         schema="(Tensor x, Tensor scale, int fmt) -> (Tensor, Tensor)")
+fp8_quantize.register_fake(_quantize_shapes)
+fp8_quantize.register_kernel("cuda")(_quantize_device)
+
+fp8_gemm = custom_op("custom::fp8_gemm", _gemm_entry, mutates_args=(),
+                     schema="(Tensor a, Tensor b, Tensor sa, Tensor sb, int out_dtype=0, "
+                            "Tensor? out_scale=None) -> Tensor")
+fp8_gemm.register_fake(_gemm_shapes)
+fp8_gemm.register_kernel("cuda")(_gemm_device)
 
 
-def mm_fp8_bias(a, b, sa, sb, bias: Optional[torch.Tensor]) -> torch.Tensor:
-    """``mm_fp8`` to bf16 with the bias added before the single rounding, the
-    epilogue of the fused forward (csrc/kernels/fp8/gemm.cuh:405-435)."""
-    return _mod().mm_fp8(a, b, sa, sb, 0, None, bias)
+# ---------------------------------------------------------------------------
+# the four primitives (string-level arguments) and this backend's additions
+# ---------------------------------------------------------------------------
+
+def quantize_bf16(x: Tensor, scale: Tensor, fmt: str = "e4m3"):
+    """Codes of ``x / scale`` in the named fp8 format plus ``max |x|`` of the
+    unscaled input, from one pass over ``x``. ``scale``: fp32 scalar on ``x``'s device."""
+    return fp8_quantize(x, scale, _position(fmt, _FORMATS, "fmt"))
 
 
-def mm_fp8(
-    a: torch.Tensor,
-    b: torch.Tensor,
-    sa: torch.Tensor,
-    sb: torch.Tensor,
-    out_dtype: str = "bf16",
-    out_scale: Optional[torch.Tensor] = None,
-) -> torch.Tensor:
-    """Pre-quantized FP8 GEMM: ``a @ b^T * (sa * sb)``; ``out_dtype`` is
-    ``"bf16"`` (default) or ``"e4m3"`` (requires ``out_scale``)."""
-    if out_dtype not in ("bf16", "e4m3"):
-        raise ValueError(
-            f"unsupported out_dtype {out_dtype!r} (expected 'bf16' or 'e4m3')"
-        )
-    return fp8_gemm(a, b, sa, sb, int(out_dtype == "e4m3"), out_scale)
+def mm_fp8(a: Tensor, b: Tensor, sa: Tensor, sb: Tensor, out_dtype: str = "bf16",
+           out_scale: Optional[Tensor] = None) -> Tensor:
+    """GEMM of fp8 codes ``a [M, K]`` and ``b [N, K]`` with fp32 accumulation, scaled by
+    ``sa * sb``; as bf16, or as e4m3 codes of the result times ``out_scale``."""
+    return fp8_gemm(a, b, sa, sb, _position(out_dtype, _OUTPUTS, "out_dtype"), out_scale)
 
 
-def linear_forward_fp8(x, w, bias, sx, sw):
-    """BF16 linear forward through E4M3; returns ``(out, amax_x, amax_w)``.
-    ``bias`` may be ``None``."""
-    if not (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16):
-        raise TypeError(f"fp8 forward requires bf16 inputs, got {x.dtype}/{w.dtype}")
-    if bias is None:
-        bias = torch.empty(0, device=x.device, dtype=x.dtype)
-    return _mod().linear_forward_fp8(x, w, bias, sx, sw)
+def mm_fp8_bias(a: Tensor, b: Tensor, sa: Tensor, sb: Tensor, bias: Optional[Tensor]) -> Tensor:
+    """``mm_fp8`` to bf16 with a bf16 ``bias [N]`` added in fp32 ahead of the one rounding:
+    the epilogue order of the reference's fused forward (csrc/kernels/fp8/gemm.cuh:405-435)."""
+    return _Kernels.get().mm_fp8(a, b, sa, sb, 0, None, bias)
 
 
-def linear_backward_fp8(g, x, w, masks, sg, sw, sx, fmt: str = "e5m2"):
-    """FP8 linear backward; returns ``(grad_input, grad_weight, grad_bias, amax_g)``."""
-    if not (
-        g.dtype == torch.bfloat16
-        and x.dtype == torch.bfloat16
-        and w.dtype == torch.bfloat16
-    ):
-        raise TypeError(
-            f"fp8 backward requires bf16 inputs, got {g.dtype}/{x.dtype}/{w.dtype}"
-        )
-    return _mod().linear_backward_fp8(g, x, w, list(masks), sg, sw, sx, _fmt_int(fmt))
+def linear_forward_fp8(x: Tensor, w: Tensor, bias: Optional[Tensor], sx: Tensor, sw: Tensor):
+    """``x @ w.T (+ bias)`` through e4m3 codes of both; also hands back the amax of ``x``
+    and of ``w``. No bias: ``None``."""
+    _all_bf16("linear_forward_fp8", x, w)
+    no_bias = x.new_empty(0) if bias is None else bias  # the kernel entry wants a tensor
+    return _Kernels.get().linear_forward_fp8(x, w, no_bias, sx, sw)
+
+
+def linear_backward_fp8(g: Tensor, x: Tensor, w: Tensor, masks, sg: Tensor, sw: Tensor,
+                        sx: Tensor, fmt: str = "e5m2"):
+    """The three gradients of a linear layer from fp8 codes, which of them being chosen by
+    ``masks`` (input, weight, bias), and the amax of ``g``."""
+    _all_bf16("linear_backward_fp8", g, x, w)
+    return _Kernels.get().linear_backward_fp8(g, x, w, [bool(m) for m in masks], sg, sw, sx,
+                                              _position(fmt, _FORMATS, "fmt"))
+
+
+def amax_bf16(x: Tensor) -> Tensor:
+    """``max |x|`` of a bf16 device tensor as a fresh fp32 ``[1]`` tensor, one read of ``x``
+    (what dynamic scaling measures before it can quantize)."""
+    _all_bf16("amax_bf16", x)
+    return _Kernels.get().amax_bf16(x)
+
+
+def amax_ring_push(hist: Tensor, idx: int, amax: Tensor, scale: Tensor, fmax: float,
+                   pow2_margin: float) -> None:
+    """Delayed scaling's bookkeeping for one tensor in one launch, in place: the new amax
+    goes into slot ``idx`` of the ring, the scale becomes ``max(ring) / fmax / pow2_margin``."""
+    _Kernels.get().amax_ring_push(hist, idx, amax, scale, fmax, pow2_margin)

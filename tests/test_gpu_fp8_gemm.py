@@ -202,7 +202,7 @@ def test_mm_fp8_rejects_bad_arguments(ops):
     a8 = torch.zeros(4, 16, dtype=torch.float8_e4m3fn, device=DEV)
     b5 = torch.zeros(4, 16, dtype=torch.float8_e5m2, device=DEV)
     one = torch.ones(1, device=DEV)
-    with pytest.raises(TypeError, match="matching fp8"):
+    with pytest.raises(TypeError, match="one format"):
         ops.mm_fp8(a8, b5, one, one)                       # ops/fp8.py:109-112
     with pytest.raises(RuntimeError, match="out_scale"):
         ops.mm_fp8(a8, a8, one, one, out_dtype="e4m3")     # mm.cu:158
@@ -210,7 +210,7 @@ def test_mm_fp8_rejects_bad_arguments(ops):
         ops.mm_fp8(a8, a8, torch.ones(2, device=DEV), one)  # mm.cu:49-54
     with pytest.raises(RuntimeError, match="inner dim"):
         ops.mm_fp8(a8, a8[:, :8].contiguous(), one, one)
-    with pytest.raises(TypeError, match="bf16 input"):
+    with pytest.raises(TypeError, match="bf16 tensors only"):
         ops.quantize_bf16(torch.zeros(4, device=DEV), one)
 
 

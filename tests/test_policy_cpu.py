@@ -83,25 +83,25 @@ def test_ring_wraps_and_forgets_old_peaks():
 
 def test_ops_have_no_cpu_arithmetic():
     x = torch.randn(4, 8).to(torch.bfloat16)
-    with pytest.raises(RuntimeError, match="no CPU implementation"):
+    with pytest.raises(RuntimeError, match="no CPU"):
         ops_fp8.quantize_bf16(x, torch.tensor([0.5]))
     a8 = torch.zeros(2, 2, dtype=torch.float8_e4m3fn)
-    with pytest.raises(RuntimeError, match="no CPU implementation"):
+    with pytest.raises(RuntimeError, match="no CPU"):
         ops_fp8.mm_fp8(a8, a8, torch.ones(1), torch.ones(1))
-    with pytest.raises(RuntimeError, match="no CPU implementation"):
+    with pytest.raises(RuntimeError, match="no CPU"):
         ops_int8.quantize_int8_per_token(x)
-    with pytest.raises(RuntimeError, match="no CPU implementation"):
+    with pytest.raises(RuntimeError, match="no CPU"):
         ops_blk.mm_fp8_blockscaled(a8, a8, torch.ones(2, 1), torch.ones(1, 1))
 
 
 def test_argument_errors_match_the_reference_types():
     x = torch.randn(2, 2).to(torch.bfloat16)
-    with pytest.raises(ValueError, match="unsupported fp8 format"):
+    with pytest.raises(ValueError, match="fmt must be one of"):
         ops_fp8.quantize_bf16(x, torch.tensor([1.0]), "e3m4")   # ops/fp8.py:44-48
     a8 = torch.zeros(2, 2, dtype=torch.float8_e4m3fn)
-    with pytest.raises(ValueError, match="unsupported out_dtype"):
+    with pytest.raises(ValueError, match="out_dtype must be one of"):
         ops_fp8.mm_fp8(a8, a8, torch.ones(1), torch.ones(1), out_dtype="fp16")  # :150-153
-    with pytest.raises(TypeError, match="bf16 inputs"):
+    with pytest.raises(TypeError, match="bf16 tensors only"):
         ops_fp8.linear_forward_fp8(x.float(), x, None, torch.ones(1), torch.ones(1))  # :162-163
 
 
