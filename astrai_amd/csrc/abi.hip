@@ -380,6 +380,22 @@ int astrai_w8a8_gemm_fp8_pt(const void* a8, const void* b8, const float* sa, con
     return check_launch("gemm_fp8_pt");
 }
 
+int astrai_w8a8_gemm_fp8_ptpc(const void* a8, const void* b8, const float* sa, const float* sb,
+                              const void* bias, void* out, int64_t m, int64_t n, int64_t k,
+                              int fmt, void* stream) {
+    if (int rc = check_gemm("gemm_fp8_ptpc", a8, b8, out, m, n, k)) return rc;
+    if (fmt != ASTRAI_W8A8_E4M3 && fmt != ASTRAI_W8A8_E5M2)
+        return fail(ASTRAI_W8A8_BAD_ARG, "gemm_fp8_ptpc: fmt must be 0 (e4m3) or 1 (e5m2)");
+    if (!sa || !sb) return fail(ASTRAI_W8A8_BAD_ARG, "gemm_fp8_ptpc: null scale pointer");
+    if (m == 0 || n == 0) return ASTRAI_W8A8_OK;
+    if (k == 0) return fail(ASTRAI_W8A8_UNSUPPORTED, "gemm_fp8_ptpc: K must be >= 1");
+    auto s = static_cast<hipStream_t>(stream);
+    const w8a8::GemmArgs g = pack(a8, b8, sa, sb, nullptr, bias, out, m, n, k, w8a8::OUT_BF16);
+    if (!w8a8::launch_gemm_fp8_rowcol_tiled(g, fmt, s))
+        w8a8::launch_gemm_generic(g, fmt ? 2 : 1, w8a8::SCALE_ROWCOL, s);
+    return check_launch("gemm_fp8_ptpc");
+}
+
 int astrai_w8a8_gemm_fp8_block128(const void* a8, const void* b8, const float* sa,
                                   const float* sb, const void* bias, void* out, int64_t m,
                                   int64_t n, int64_t k, void* stream) {

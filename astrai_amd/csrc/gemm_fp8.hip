@@ -1,5 +1,5 @@
-// fp8 (OCP e4m3fn / e5m2) MFMA GEMMs, per-tensor scales, optional bias, bf16 /
-// e4m3 / fp32 output. Large shapes run v_mfma_f32_32x32x64_f8f6f4 on 256x256
+// fp8 (OCP e4m3fn / e5m2) MFMA GEMMs, per-tensor scales (optional bias, bf16 /
+// e4m3 / fp32 output) or one scale per activation row and per weight row (bf16 output). Large shapes run v_mfma_f32_32x32x64_f8f6f4 on 256x256
 // tiles: the four-wave 128x128-register-tile kernel for bf16 output, the
 // eight-wave ping-pong kernel for the other outputs; the generic tiled kernel
 // takes everything else.
@@ -9,20 +9,27 @@
 namespace w8a8 {
 
 namespace {
-template <int Fmt>
+template <int Fmt, int ScaleKind>
 void launch_for(const GemmArgs& g, hipStream_t stream) {
 #ifndef W8A8_NO_WAVE128
-    if (wave128_shape_ok(g)) return launch_wave128<Op32F8<Fmt>, SCALE_TENSOR>(g, stream);
+    if (wave128_shape_ok(g)) return launch_wave128<Op32F8<Fmt>, ScaleKind>(g, stream);
 #endif
-    if (pingpong_shape_ok(g)) return launch_pingpong<Op32F8<Fmt>, SCALE_TENSOR>(g, stream);
-    launch_tiled_auto<OpF8<Fmt>, SCALE_TENSOR>(g, stream);
+    if (pingpong_shape_ok(g)) return launch_pingpong<Op32F8<Fmt>, ScaleKind>(g, stream);
+    launch_tiled_auto<OpF8<Fmt>, ScaleKind>(g, stream);
 }
 }  // namespace
 
 bool launch_gemm_fp8_tiled(const GemmArgs& g, int fmt, hipStream_t stream) {
     if (!tiled_shape_ok(g)) return false;
-    if (fmt) launch_for<1>(g, stream);
-    else launch_for<0>(g, stream);
+    if (fmt) launch_for<1, SCALE_TENSOR>(g, stream);
+    else launch_for<0, SCALE_TENSOR>(g, stream);
+    return true;
+}
+
+bool launch_gemm_fp8_rowcol_tiled(const GemmArgs& g, int fmt, hipStream_t stream) {
+    if (!tiled_shape_ok(g) || g.out_kind != OUT_BF16) return false;
+    if (fmt) launch_for<1, SCALE_ROWCOL>(g, stream);
+    else launch_for<0, SCALE_ROWCOL>(g, stream);
     return true;
 }
 

@@ -78,9 +78,11 @@ void launch_gemm_generic(const GemmArgs& g, int op, int scale_kind, hipStream_t 
         else launch<OpI8, SCALE_TENSOR>(g, stream);
     } else if (op == 1) {
         if (scale_kind == SCALE_BLOCK128) launch<OpF8<0>, SCALE_BLOCK128>(g, stream);
+        else if (scale_kind == SCALE_ROWCOL) launch<OpF8<0>, SCALE_ROWCOL>(g, stream);
         else launch<OpF8<0>, SCALE_TENSOR>(g, stream);
     } else {
-        launch<OpF8<1>, SCALE_TENSOR>(g, stream);
+        if (scale_kind == SCALE_ROWCOL) launch<OpF8<1>, SCALE_ROWCOL>(g, stream);
+        else launch<OpF8<1>, SCALE_TENSOR>(g, stream);
     }
 }
 

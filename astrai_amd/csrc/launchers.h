@@ -138,6 +138,8 @@ bool launch_attn_prefill(const AttnPrefillArgs& a, hipStream_t stream);
 // not accepted (the caller then uses the generic kernel).
 bool launch_gemm_int8_tiled(const GemmArgs& g, hipStream_t stream);
 bool launch_gemm_fp8_tiled(const GemmArgs& g, int fmt, hipStream_t stream);
+// sa per activation row [M], sb per weight row [N], bf16 output
+bool launch_gemm_fp8_rowcol_tiled(const GemmArgs& g, int fmt, hipStream_t stream);
 bool launch_gemm_fp8_block128_tiled(const GemmArgs& g, hipStream_t stream);
 
 // gemm_generic.hip: any shape, guarded byte loads, one wave per 16x16 tile.

@@ -57,6 +57,7 @@ PROTOTYPES = {
     "astrai_w8a8_quantize_bf16_fp8_block128_act": ([_P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_quantize_bf16_fp8_block128_weight": ([_P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_gemm_fp8_pt": ([_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _INT, _INT, _P], _INT),
+    "astrai_w8a8_gemm_fp8_ptpc": ([_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _INT, _P], _INT),
     "astrai_w8a8_gemm_fp8_block128": ([_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _INT),
     "astrai_w8a8_gemm_int8_ptpc": ([_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _INT, _P], _INT),
     "astrai_w8a8_gemv_int8_ptpc": ([_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _INT, _P], _INT),
@@ -172,8 +173,12 @@ def quantize_bf16(x: torch.Tensor, scale: torch.Tensor, fmt: int):
 def mm_fp8(a: torch.Tensor, b: torch.Tensor, sa: torch.Tensor, sb: torch.Tensor,
            out_dtype: int = 0, out_scale: Optional[torch.Tensor] = None,
            bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Pre-quantized fp8 GEMM ``a @ b^T * (sa*sb)``. mm.cu:128-184. ``bias`` (bf16
-    ``[N]``, bf16 output only) is an extension used by the fused linear forward."""
+    """Pre-quantized fp8 GEMM ``a @ b^T * sa * sb``. mm.cu:128-184. ``bias`` (bf16
+    ``[N]``, bf16 output only) is an extension used by the fused linear forward.
+    Scales are fp32 scalars, as the reference's binding demands (mm.cu:49-54) -- or,
+    for bf16 output, the shapes its CPU kernel's broadcast accepts besides
+    (ops/fp8.py:118): ``sa`` one step per activation row (``[M]`` / ``[M, 1]``) and / or
+    ``sb`` one per weight row (``[N]`` / ``[1, N]``)."""
     lib = _require()
     _gpu(a, "mm_fp8")
     _gpu(b, "mm_fp8")
@@ -187,8 +192,13 @@ def mm_fp8(a: torch.Tensor, b: torch.Tensor, sa: torch.Tensor, sb: torch.Tensor,
         raise RuntimeError("a and b must be on the same device")
     if a.size(1) != b.size(1):
         raise RuntimeError("inner dim mismatch")
-    _check_scale(sa, a, "sa")
-    _check_scale(sb, a, "sb")
+    per_row = ((sa.numel() > 1 and tuple(sa.shape) in ((a.size(0),), (a.size(0), 1)))
+               or (sb.numel() > 1 and tuple(sb.shape) in ((b.size(0),), (1, b.size(0)))))
+    per_row = per_row and out_dtype == 0
+    if not per_row or sa.numel() == 1:
+        _check_scale(sa, a, "sa")
+    if not per_row or sb.numel() == 1:
+        _check_scale(sb, a, "sb")
     if out_dtype not in (0, 1):
         raise RuntimeError("out_dtype must be 0 (bf16) or 1 (fp8 e4m3)")
     if out_dtype == 1:
@@ -211,6 +221,12 @@ def mm_fp8(a: torch.Tensor, b: torch.Tensor, sa: torch.Tensor, sb: torch.Tensor,
                 out.zero_()
                 if bias is not None:
                     out.copy_(bias.expand(m, n))
+            elif per_row:
+                sa_v = _check_vec(sa.reshape(-1).expand(m) if sa.numel() == 1 else sa.reshape(-1), a, m, "sa")
+                sb_v = _check_vec(sb.reshape(-1).expand(n) if sb.numel() == 1 else sb.reshape(-1), a, n, "sb")
+                _check(lib.astrai_w8a8_gemm_fp8_ptpc(
+                    a_c.data_ptr(), b_c.data_ptr(), sa_v.data_ptr(), sb_v.data_ptr(), _ptr(bias),
+                    out.data_ptr(), m, n, k, 1 if a.dtype == torch.float8_e5m2 else 0, _stream(a)), lib)
             else:
                 _check(lib.astrai_w8a8_gemm_fp8_pt(
                     a_c.data_ptr(), b_c.data_ptr(), sa.data_ptr(), sb.data_ptr(),

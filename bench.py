@@ -432,6 +432,18 @@ def main():
                                        "TFLOP/s": round(flop / (ms * 1e-3) / 1e12, 1)}
         del ai, bi
 
+        # ---- fp8 with one scale per activation row and per weight row
+        sa_rows = sa_d.expand(M).contiguous()
+        sb_rows = sb_d.expand(N).contiguous()
+
+        def step_rowcol():
+            check(lib.astrai_w8a8_gemm_fp8_ptpc(a8.data_ptr(), b8.data_ptr(), sa_rows.data_ptr(),
+                                                sb_rows.data_ptr(), None, out.data_ptr(), M, N, K, 0, stream))
+
+        ms = _event_time_ms(step_rowcol, 500, 300)
+        extra["fp8_gemm_4096_row_and_column_scales"] = {"us": round(ms * 1e3, 2),
+                                                        "TFLOP/s": round(flop / (ms * 1e-3) / 1e12, 1)}
+
         # ---- fp8 linear backward at 4096^3 (dX and dW GEMMs + the three transposing
         # quantizer passes), through the module the registry hands out
         from astrai_amd.extension import get_module

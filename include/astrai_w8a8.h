@@ -290,6 +290,18 @@ int astrai_w8a8_gemm_fp8_pt(const void* a8, const void* b8, const float* sa,
                             int out_dtype, void* stream);
 
 /*
+ * The per-tensor GEMM above with one scale per activation row and one per weight row:
+ *   out[m,n] = bf16( (sum_k a8[m,k] * b8[n,k]) * sa[m] * sb[n] + bias[n] )
+ * sa fp32 [M], sb fp32 [N]. The reference's CUDA binding takes scalars only
+ * (csrc/kernels/fp8/mm.cu:49-54), but the arithmetic its ops are specified by,
+ * `a.float() @ b.float().t() * sa * sb` (astrai/extension/ops/fp8.py:118), broadcasts
+ * sa [M,1] and sb [N]; this entry is that broadcast on the device. bf16 output only.
+ */
+int astrai_w8a8_gemm_fp8_ptpc(const void* a8, const void* b8, const float* sa,
+                              const float* sb, const void* bias_bf16, void* out_bf16,
+                              int64_t m, int64_t n, int64_t k, int fmt, void* stream);
+
+/*
  * Pre-quantized e4m3fn GEMM with 128-block scales. No counterpart in the
  * reference. K must be a multiple of 128.
  *   out[m,n] = bf16( sum_kb (sum_{k in kb} a8[m,k]*b8[n,k]) * sa[m,kb] * sb[n/128,kb] + bias[n] )

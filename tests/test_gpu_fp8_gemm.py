@@ -229,6 +229,34 @@ def test_config1_sampled_rows_at_full_size(ops):
     assert_bf16_close(out[rows], want, what="config1 rows")
 
 
+@pytest.mark.parametrize("m,n,k,fmt,bias", [
+    (17, 9, 33, 0, False),          # any-shape kernel (K % 16 != 0)
+    (130, 200, 384, 0, True),       # small tiles
+    (257, 513, 1024, 1, False),     # e5m2
+    (1024, 1536, 512, 0, True),     # 128x128 tiles
+    (4096, 4096, 256, 0, False),    # 256x256 tiles, four-wave kernel
+    (3841, 4100, 640, 0, True),     # 256x256 tiles, N % 8 != 0: ping-pong kernel
+])
+def test_mm_fp8_row_and_column_scales(ops, m, n, k, fmt, bias):
+    """One step per activation row and per weight row: the broadcast the reference's CPU
+    kernel evaluates (ops/fp8.py:118) although its CUDA binding takes scalars only."""
+    from astrai_amd.extension import _cabi
+    print(f"case m={m} n={n} k={k} fmt={fmt} bias={bias}", flush=True)
+    g = torch.Generator().manual_seed(m + 3 * n + 7 * k)
+    dt = torch.float8_e5m2 if fmt else torch.float8_e4m3fn
+    a8 = (torch.randn(m, k, generator=g) * 1.5).to(dt)
+    b8 = (torch.randn(n, k, generator=g) * 1.5).to(dt)
+    sa = torch.exp2(torch.rand(m, 1, generator=g) * 6.0 - 3.0)
+    sb = torch.exp2(torch.rand(n, generator=g) * 6.0 - 3.0)
+    bvec = torch.randn(n, generator=g).to(torch.bfloat16) if bias else None
+    out = _cabi.mm_fp8(a8.to(DEV), b8.to(DEV), sa.to(DEV), sb.to(DEV), 0, None,
+                       bvec.to(DEV) if bias else None)
+    assert_bf16_close(out, O.fp8_gemm_bias(a8, b8, sa, sb, bvec), what="row/column scales")
+    # through the dispatcher op, and with only one of the two per row
+    out = ops.mm_fp8(a8.to(DEV), b8.to(DEV), sa[:1, 0].to(DEV), sb.reshape(1, n).to(DEV))
+    assert_bf16_close(out, O.fp8_gemm(a8, b8, sa[:1, 0], sb.reshape(1, n)), what="column scales only")
+
+
 def test_empty_operands(ops):
     """No rows, no columns, no elements: shapes and dtypes as for any other input,
     no launch, no error (the reference allocates the same empty outputs, mm.cu:111-124,154-160)."""
