@@ -105,7 +105,11 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(AttnDecodeArgs
 #pragma unroll
         for (int d = 0; d < 8; ++d) acc[q][d] = 0.0f;
 
-    // paged: slot of key 16t + c16, looked up one tile ahead of its use (-1: not attended)
+    // paged: slot of key 16t + c16, looked up one tile ahead of its use. -1: nothing is
+    // fetched, key and value read as zeros; a position inside the sequence whose table
+    // entry is negative ("empty padding") is still attended, with score 0, as in the
+    // reference, which gates the load on the slot and the mask on the position only
+    // (csrc/kernels/attention/layout_policies.cuh:104-110,212-219; decode_split_kv_mma.cuh:75-82,107-110)
     auto key_slot = [&](int t) -> int {
         const int key = (t << 4) + c16;
         const int slot = (t < t1 && key <= kmax) ? table[key] : -1;
@@ -156,7 +160,6 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(AttnDecodeArgs
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             bool ok = q_live && (int64_t)(kb + 4 * g + i) <= q_pos;
-            if constexpr (PAGED) ok = ok && vslot[i] >= 0;  // negative slot: padding, not attended
             sc[i] = ok ? sc[i] * a.scale : kNegBig;
             tm = fmaxf(tm, sc[i]);
         }

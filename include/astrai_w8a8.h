@@ -196,7 +196,10 @@ int astrai_w8a8_attn_decode_bf16(const void* q_bf16, const void* k_cache_bf16, c
  *   q          bf16 [batch, n_heads, 128]: the newest token of every sequence
  *   k_pool, v_pool  bf16 [num_slots, n_kv_heads, 128]
  *   req_to_token    int32 [num_requests, max_context_len]: pool slot of (request, position);
- *              negative entries (and entries >= num_slots) are not attended
+ *              a negative entry ("empty padding"; likewise one >= num_slots) is not
+ *              fetched: its key and value read as zeros, and the position is attended like
+ *              any other, as in the reference (load gated on the slot, mask on the position:
+ *              layout_policies.cuh:104-110,212-219)
  *   req_pool_indices  int32 [batch]: row of req_to_token of each sequence
  *   kv_indptr  int32 [batch + 1]: prefix sums of the sequence lengths; sequence b attends
  *              positions 0 .. kv_indptr[b+1] - kv_indptr[b] - 1

@@ -80,21 +80,25 @@ def attn_paged_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tenso
                       kv_indptr: torch.Tensor) -> torch.Tensor:
     """Decode attention over a token-granular paged cache: ``q [B, H, D]``, pools
     ``[slots, H_kv, D]``; key ``j`` of sequence ``b`` is pool row
-    ``req_to_token[req_pool_indices[b], j]`` for ``j < kv_indptr[b+1] - kv_indptr[b]``,
-    negative rows are skipped (csrc/kernels/attention/layout_policies.cuh:174-232;
-    astrai/extension/ops/attention.py:93-147). ``softmax(q k^T / sqrt(D)) v`` in float32 per
-    sequence, a sequence without keys gives zeros. Returns ``[B, H, D]`` in the input dtype."""
+    ``req_to_token[req_pool_indices[b], j]`` for ``j < kv_indptr[b+1] - kv_indptr[b]``
+    (csrc/kernels/attention/layout_policies.cuh:174-232; astrai/extension/ops/attention.py:93-147).
+    A negative row ("empty padding") is not fetched -- its key and value are zeros -- but the
+    position stays in the attended range [0, kv_len): the reference gates the load on the slot
+    (layout_policies.cuh:104-110,212-219; decode_split_kv_mma.cuh:75-82) and masks by position
+    only (decode_split_kv_mma.cuh:107-110), so such a position enters the softmax with score 0.
+    ``softmax(q k^T / sqrt(D)) v`` in float32 per sequence, a sequence without keys gives
+    zeros. Returns ``[B, H, D]`` in the input dtype."""
     b, h, d = q.shape
     n_rep = h // k_pool.size(1)
     out = torch.zeros(b, h, d, dtype=torch.float32)
     for i in range(b):
         n = int(kv_indptr[i + 1]) - int(kv_indptr[i])
         rows = req_to_token[int(req_pool_indices[i]), :n].long()
-        rows = rows[rows >= 0]
         if rows.numel() == 0:
             continue
-        k = k_pool[rows].float().repeat_interleave(n_rep, dim=1)      # [n, H, D]
-        v = v_pool[rows].float().repeat_interleave(n_rep, dim=1)
+        live = (rows >= 0)[:, None, None]
+        k = torch.where(live, k_pool[rows.clamp_min(0)].float(), torch.zeros(())).repeat_interleave(n_rep, dim=1)
+        v = torch.where(live, v_pool[rows.clamp_min(0)].float(), torch.zeros(())).repeat_interleave(n_rep, dim=1)
         scores = torch.einsum("hd,nhd->hn", q[i].float(), k) / (d ** 0.5)
         out[i] = torch.einsum("hn,nhd->hd", torch.softmax(scores, dim=-1), v)
     return out.to(q.dtype)
@@ -107,8 +111,11 @@ def attn_paged_prefill(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tens
     """Ragged prefill over the paged cache: packed ``q [total_q, H, D]``; sequence ``b`` owns
     rows ``qo_indptr[b] .. qo_indptr[b+1]`` and keys ``req_to_token[req_pool_indices[b], :kv_len]``;
     with ``causal`` row ``i`` of it sees keys ``0 .. kv_len - q_len + i``
-    (csrc/kernels/attention/layout_policies.cuh:67-93,174-232). float32 softmax attention per
-    sequence; a row that sees no key gives zeros. Returns ``[total_q, H, D]`` in the input dtype."""
+    (csrc/kernels/attention/layout_policies.cuh:67-93,174-232). A negative pool row reads as a
+    zero key and a zero value and is attended like any other position (the load is gated on the
+    slot, the mask on the position: prefill_split_q_mma.cuh:84-89,121-124). float32 softmax
+    attention per sequence; a row that sees no position gives zeros. Returns ``[total_q, H, D]``
+    in the input dtype."""
     total_q, h, d = q.shape
     n_rep = h // k_pool.size(1)
     out = torch.zeros(total_q, h, d, dtype=torch.float32)
@@ -118,10 +125,11 @@ def attn_paged_prefill(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tens
         if q1 == q0 or n == 0:
             continue
         rows = req_to_token[int(req_pool_indices[b]), :n].long()
-        k = k_pool[rows.clamp_min(0)].float().repeat_interleave(n_rep, dim=1)   # [n, H, D]
-        v = v_pool[rows.clamp_min(0)].float().repeat_interleave(n_rep, dim=1)
+        live = (rows >= 0)[:, None, None]
+        k = torch.where(live, k_pool[rows.clamp_min(0)].float(), torch.zeros(())).repeat_interleave(n_rep, dim=1)
+        v = torch.where(live, v_pool[rows.clamp_min(0)].float(), torch.zeros(())).repeat_interleave(n_rep, dim=1)
         scores = torch.einsum("qhd,nhd->hqn", q[q0:q1].float(), k) / (d ** 0.5)
-        visible = (rows >= 0)[None, :].expand(q1 - q0, n).clone()
+        visible = torch.ones(q1 - q0, n, dtype=torch.bool)
         if causal:
             newest = (n - (q1 - q0)) + torch.arange(q1 - q0)
             visible &= torch.arange(n)[None, :] <= newest[:, None]

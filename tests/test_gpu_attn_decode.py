@@ -92,3 +92,21 @@ def test_quantized_output_is_the_quantizer_applied_to_the_bf16_output():
     oq, os_ = _cabi.attn_decode(q, kc, vc, pos, nsplit=4, quantized=True)
     wq, ws = O.int8_quantize_rows(out.cpu().reshape(b * s, h * d))
     assert torch.equal(oq.cpu(), wq) and torch.equal(os_.cpu(), ws)
+
+
+def test_decode_random_sweep():
+    """Thirty seeded random layouts: batch, grouping (n_rep * new tokens <= 8), context
+    length, positions of the new tokens and split count all vary."""
+    g = torch.Generator().manual_seed(2718)
+    for i in range(30):
+        n_rep = (1, 2, 4, 8)[int(torch.randint(0, 4, (1,), generator=g))]
+        s = int(torch.randint(1, 8 // n_rep + 1, (1,), generator=g))
+        hkv = int(torch.randint(1, 5, (1,), generator=g))
+        b = int(torch.randint(1, 6, (1,), generator=g))
+        max_len = int(torch.randint(s, 700, (1,), generator=g))
+        first = int(torch.randint(0, max_len - s + 1, (1,), generator=g))
+        positions = list(range(first, first + s))
+        nsplit = (0, 1, 2, 5, 16)[i % 5]
+        print(f"case {i}: b={b} h={hkv * n_rep}/{hkv} s={s} max_len={max_len} pos={positions} nsplit={nsplit}",
+              flush=True)
+        _case(b, hkv * n_rep, hkv, s, max_len, positions, seed=900 + i, nsplit=nsplit)

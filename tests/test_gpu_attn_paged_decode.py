@@ -26,7 +26,7 @@ def _setup(b, h, hkv, lens, max_ctx, pool, seed, n_req=None, holes=False):
         for j in range(lens[i]):
             table[rows[i], j] = int(perm[nxt]); nxt += 1
         if holes and lens[i] > 3:
-            table[rows[i], 1] = -1        # padding inside a sequence: skipped
+            table[rows[i], 1] = -1        # padding inside a sequence: zero key and value
     # slots that no live position maps to hold poison: they must not be read
     unused = perm[nxt:]
     k_pool[unused] = float("nan")
@@ -63,7 +63,7 @@ def test_paged_decode_small_shapes(b, h, hkv, lens, max_ctx):
         assert_bf16_close(_run(args, nsplit), D.attn_paged_decode(*args), what=f"lens={lens} nsplit={nsplit}")
 
 
-def test_paged_decode_skips_negative_and_out_of_pool_slots():
+def test_paged_decode_negative_and_out_of_pool_slots_read_as_zeros():
     args = list(_setup(2, 8, 2, [40, 9], 64, 80, seed=3, holes=True))
     want = D.attn_paged_decode(*args)
     assert_bf16_close(_run(args, 2), want, what="holes")

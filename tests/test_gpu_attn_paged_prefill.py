@@ -115,3 +115,22 @@ def test_paged_prefill_rejects_what_it_does_not_do():
         _cabi.attn_paged_prefill(*args, qo, tb, ti, mask=torch.ones(1, 1, 3, 3, dtype=torch.bool, device=DEV))
     with pytest.raises(RuntimeError, match="int32"):
         _cabi.attn_paged_prefill(*args, qo.long(), tb, ti)
+
+
+def test_paged_prefill_random_sweep():
+    """Twenty seeded random batches: request counts, grouping, cached prefix lengths and new
+    token counts all vary; every third batch is non-causal, every fourth has padding slots."""
+    g = torch.Generator().manual_seed(4242)
+    for i in range(20):
+        n_rep = (2, 4, 8)[int(torch.randint(0, 3, (1,), generator=g))]
+        hkv = int(torch.randint(1, 4, (1,), generator=g))
+        b = int(torch.randint(1, 5, (1,), generator=g))
+        q_lens = [int(torch.randint(1, 150, (1,), generator=g)) for _ in range(b)]
+        kv_lens = [ql + (int(torch.randint(0, 120, (1,), generator=g)) if j % 2 else 0)
+                   for j, ql in enumerate(q_lens)]
+        causal = i % 3 != 2
+        print(f"case {i}: h={hkv * n_rep}/{hkv} kv={kv_lens} q={q_lens} causal={causal}", flush=True)
+        args = _setup(hkv * n_rep, hkv, kv_lens, q_lens, max(kv_lens) + 3, sum(kv_lens) + 7,
+                      seed=500 + i, holes=(i % 4 == 3))
+        got, want = _run(args, q_lens, causal=causal)
+        _close(got, want, f"sweep {i}")

@@ -60,6 +60,21 @@ def test_prefill_small_shapes(b, h, hkv, s, max_len, start):
     _case(b, h, hkv, s, max_len, start, seed=b + h + s + start)
 
 
+def test_prefill_random_shape_sweep():
+    """Thirty seeded random layouts: batch, grouping, chunk length, cache length and the
+    chunk's start all vary, block boundaries (32 query rows, 64 keys) fall anywhere."""
+    g = torch.Generator().manual_seed(31337)
+    for i in range(30):
+        n_rep = (2, 4, 8)[int(torch.randint(0, 3, (1,), generator=g))]
+        hkv = int(torch.randint(1, 4, (1,), generator=g))
+        b = int(torch.randint(1, 4, (1,), generator=g))
+        s = int(torch.randint(1, 200, (1,), generator=g))
+        start = int(torch.randint(0, 150, (1,), generator=g)) if i % 2 else 0
+        max_len = start + s + int(torch.randint(0, 70, (1,), generator=g))
+        print(f"case {i}: b={b} h={hkv * n_rep} hkv={hkv} s={s} max_len={max_len} start={start}", flush=True)
+        _case(b, hkv * n_rep, hkv, s, max_len, start, seed=1000 + i)
+
+
 def test_prefill_config4_shape():
     _case(2, 16, 4, 512, 640, 0, seed=4)
 

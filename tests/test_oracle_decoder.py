@@ -205,3 +205,39 @@ def test_paged_prefill_oracle_equals_dense_attention_per_sequence():
     qi = q[0:7].permute(1, 0, 2).unsqueeze(0)
     want = D.attn_cached(qi, dense_k[0:1], dense_v[0:1], torch.full((7,), 23))
     assert torch.equal(full[0:7].reshape(7, -1), want[0])
+
+
+def test_paged_oracles_read_a_negative_slot_as_a_zero_key_and_value():
+    """The reference gates the K/V load on the slot and the mask on the position only
+    (csrc/kernels/attention/layout_policies.cuh:104-110,212-219; prefill_split_q_mma.cuh:84-89,
+    121-124; decode_split_kv_mma.cuh:75-82,107-110): a negative table entry inside a sequence
+    must act exactly like a slot whose key and value rows are zero -- still attended, score 0 --
+    and not like a shorter sequence."""
+    g = torch.Generator().manual_seed(21)
+    h, hkv, d, pool = 4, 2, 16, 40
+    k_pool = torch.randn(pool, hkv, d, generator=g).to(torch.bfloat16)
+    v_pool = torch.randn(pool, hkv, d, generator=g).to(torch.bfloat16)
+    k_pool[pool - 1] = 0          # a real slot holding a zero key and a zero value
+    v_pool[pool - 1] = 0
+    lens = [9, 5]
+    rows = torch.tensor([1, 0], dtype=torch.int32)
+    table = torch.full((2, 12), -1, dtype=torch.int32)
+    table[1, :9] = torch.arange(9, dtype=torch.int32)
+    table[0, :5] = torch.arange(20, 25, dtype=torch.int32)
+    holes = table.clone(); holes[1, 3] = -1; holes[0, 0] = -1
+    zeros = table.clone(); zeros[1, 3] = pool - 1; zeros[0, 0] = pool - 1
+    indptr = torch.tensor([0, 9, 14], dtype=torch.int32)
+    q1 = torch.randn(2, h, d, generator=g).to(torch.bfloat16)
+    a = D.attn_paged_decode(q1, k_pool, v_pool, holes, rows, indptr)
+    b = D.attn_paged_decode(q1, k_pool, v_pool, zeros, rows, indptr)
+    assert torch.equal(a, b)
+    short = D.attn_paged_decode(q1, k_pool, v_pool, table, rows, indptr)
+    assert not torch.equal(a, short)
+    qo = torch.tensor([0, 9, 12], dtype=torch.int32)      # whole prompt; a 3-row chunk after 2 cached
+    qp = torch.randn(12, h, d, generator=g).to(torch.bfloat16)
+    for causal in (True, False):
+        a = D.attn_paged_prefill(qp, k_pool, v_pool, holes, rows, indptr, qo, causal=causal)
+        b = D.attn_paged_prefill(qp, k_pool, v_pool, zeros, rows, indptr, qo, causal=causal)
+        assert torch.equal(a, b), causal
+    # row 0 of the second sequence sees positions 0..2, all real except the hole at 0
+    assert a.abs().sum() > 0
