@@ -127,3 +127,18 @@ def test_paged_decode_rejects_what_it_does_not_do():
         _cabi.attn_paged_decode(q, k_pool, v_pool, table.long(), rows, indptr)
     with pytest.raises(RuntimeError, match="together"):
         _cabi.attn_paged_decode(q, k_pool, v_pool, table, rows, indptr, new_k=q[:, :1])
+
+
+def test_paged_decode_random_sweep():
+    """Twenty-five seeded random batches: sequence lengths from empty to several hundred,
+    grouping, split counts, padding slots in every other batch."""
+    g = torch.Generator().manual_seed(1618)
+    for i in range(25):
+        n_rep = (1, 2, 4, 8)[int(torch.randint(0, 4, (1,), generator=g))]
+        hkv = int(torch.randint(1, 5, (1,), generator=g))
+        b = int(torch.randint(1, 7, (1,), generator=g))
+        lens = [int(torch.randint(0, 400, (1,), generator=g)) for _ in range(b)]
+        nsplit = (0, 1, 3, 7, 16)[i % 5]
+        print(f"case {i}: h={hkv * n_rep}/{hkv} lens={lens} nsplit={nsplit}", flush=True)
+        args = _setup(b, hkv * n_rep, hkv, lens, max(lens) + 2, sum(lens) + 9, seed=300 + i, holes=bool(i % 2))
+        assert_bf16_close(_run(args, nsplit), D.attn_paged_decode(*args), what=f"sweep {i}")

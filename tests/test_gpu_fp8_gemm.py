@@ -401,3 +401,50 @@ def test_large_ragged_tiles_with_guard_rows(m, n, k, bias):
     cols = torch.cat([torch.arange(0, 2), torch.arange(n - 9, n)])
     want_c = O.fp8_gemm_bias(a8, b8[cols], sa, sb, bvec[cols] if bias else None)
     assert_bf16_close(out[:m, cols], want_c, what="ragged columns")
+
+
+def test_block128_random_shape_sweep():
+    """Seeded random shapes of the block-scaled GEMM, small tiles to the 256x256-tile kernel,
+    ragged M and N, scales over eight octaves, whole output against the oracle."""
+    from astrai_amd.extension.ops import fp8_block as blk
+    g = torch.Generator().manual_seed(909)
+    r = lambda lo, hi: int(torch.randint(lo, hi, (1,), generator=g))
+    shapes = [(r(1, 600), r(1, 700), 128 * r(1, 9)) for _ in range(12)]
+    shapes += [(r(3500, 4200), 8 * r(430, 520), 128 * r(2, 5)) for _ in range(3)]   # >= 192 tiles of 256^2
+    for (m, n, k) in shapes:
+        print(f"case m={m} n={n} k={k}", flush=True)
+        a8 = (torch.randn(m, k, generator=g) * 2.0).to(torch.float8_e4m3fn)
+        b8 = (torch.randn(n, k, generator=g) * 2.0).to(torch.float8_e4m3fn)
+        sa = torch.exp2(torch.rand(m, k // 128, generator=g) * 8.0 - 4.0)
+        sb = torch.exp2(torch.rand((n + 127) // 128, k // 128, generator=g) * 8.0 - 4.0)
+        out = blk.mm_fp8_blockscaled(a8.to(DEV), b8.to(DEV), sa.to(DEV), sb.to(DEV))
+        assert_bf16_close(out, O.fp8_gemm_blockscaled(a8, b8, sa, sb), what=f"block128 {m}x{n}x{k}")
+
+
+def test_linear_forward_backward_random_shape_sweep(ops):
+    """Twelve seeded random layer shapes through the fused forward and the backward (all three
+    gradients), bias in every other case, against the oracle's codes."""
+    g = torch.Generator().manual_seed(2025)
+    r = lambda lo, hi: int(torch.randint(lo, hi, (1,), generator=g))
+    for i in range(12):
+        m, n, k = r(1, 300), r(1, 300), r(1, 500)
+        print(f"case {i}: m={m} n={n} k={k}", flush=True)
+        x = torch.randn(m, k, generator=g).to(torch.bfloat16)
+        w = torch.randn(n, k, generator=g).to(torch.bfloat16)
+        gr = torch.randn(m, n, generator=g).to(torch.bfloat16)
+        bias = torch.randn(n, generator=g).to(torch.bfloat16) if i % 2 else None
+        sx, sw, sg = _scale(x), _scale(w), _scale(gr)
+        out, ax, aw = ops.linear_forward_fp8(x.to(DEV), w.to(DEV), bias.to(DEV) if i % 2 else None,
+                                             sx.to(DEV), sw.to(DEV))
+        want, wax, waw = O.linear_forward_fp8(x, w, bias, sx, sw)
+        assert_bf16_close(out, want, what=f"forward {m}x{n}x{k}")
+        assert ax.item() == wax.item() and aw.item() == waw.item()
+        gx, gw, gb, amax_g = ops.linear_backward_fp8(
+            gr.to(DEV), x.to(DEV), w.to(DEV), [1, 1, 1], sg.to(DEV), sw.to(DEV), sx.to(DEV), "e4m3")
+        qg = O.fp8_quantize(gr, sg, 0)[0].float()
+        qw = O.fp8_quantize(w, sw, 0)[0].float()
+        qx = O.fp8_quantize(x, sx, 0)[0].float()
+        assert_bf16_close(gx, (qg @ qw * sg * sw).to(torch.bfloat16), what=f"dX {m}x{n}x{k}")
+        assert_bf16_close(gw, (qg.t() @ qx * sg * sx).to(torch.bfloat16), what=f"dW {m}x{n}x{k}")
+        torch.testing.assert_close(gb.cpu(), gr.sum(0).to(torch.bfloat16))
+        assert amax_g.item() == gr.abs().max().item()

@@ -78,3 +78,13 @@ def test_fused_entry_points_reject_unsupported(C):
     big = torch.zeros(1, 8200, device=DEV, dtype=torch.bfloat16)
     with pytest.raises(RuntimeError, match="8192"):
         C.silu_mul_quantize_int8(big, big)
+
+
+def test_fused_producers_random_shape_sweep(C):
+    """Seeded random row counts and widths (multiples of 8 up to 8192) through both producers."""
+    g = torch.Generator().manual_seed(808)
+    r = lambda lo, hi: int(torch.randint(lo, hi, (1,), generator=g))
+    for i in range(12):
+        test_add_rmsnorm_quantize(C, r(1, 70), 8 * r(1, 1025), bool(i % 2))
+    for i in range(12):
+        test_silu_mul_quantize(C, r(1, 70), 8 * r(1, 1025), bool(i % 2))

@@ -151,3 +151,17 @@ def test_block128_weight_quantize(C, n, k):
     r8, rs = O.fp8_quantize_weight_block128(w)
     assert sb.shape == rs.shape and torch.equal(sb.cpu(), rs)
     assert torch.equal(_codes(w8), _codes(r8))
+
+
+def test_quantizer_random_shape_sweep(C):
+    """Seeded random shapes through the three quantizers (the checks of the parametrized tests
+    above): transposed fp8 codes, per-row int8, 128-block fp8."""
+    g = torch.Generator().manual_seed(606)
+    r = lambda lo, hi: int(torch.randint(lo, hi, (1,), generator=g))
+    for i in range(12):
+        test_fp8_quantize_transposed_codes(C, (r(1, 700), r(1, 700)), i % 2)
+    for i in range(12):
+        test_int8_rows_bit_exact(C, r(1, 80), r(1, 12000))
+    for i in range(6):
+        test_block128_act_quantize(C, r(1, 400), 128 * r(1, 12))
+        test_block128_weight_quantize(C, r(1, 600), 128 * r(1, 8))

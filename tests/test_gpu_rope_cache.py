@@ -117,3 +117,13 @@ def test_projection_with_rotary_epilogue_limits():
                                  torch.tensor([4], device=DEV), kc, vc, 2, 1, 2, 1, 16)
     torch.cuda.synchronize()
     assert q.abs().sum().item() > 0 and kc.abs().sum().item() == 0 and vc.abs().sum().item() == 0
+
+
+def test_rope_cache_write_random_sweep():
+    """Twenty seeded random layouts of the standalone rotary / cache-write kernel."""
+    g = torch.Generator().manual_seed(5050)
+    r = lambda lo, hi: int(torch.randint(lo, hi, (1,), generator=g))
+    for i in range(20):
+        hkv = r(1, 5); h = hkv * (1, 2, 4, 8)[r(0, 4)]; d = 8 * r(1, 17)
+        b, s = r(1, 6), r(1, 40)
+        test_rope_cache_write_matches_tensor_ops(b, s, h, hkv, d, s + r(0, 50), bool(i % 3 == 0))
