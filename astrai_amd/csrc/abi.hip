@@ -196,6 +196,24 @@ int astrai_w8a8_rope_cache_write_bf16(const void* qkv, int64_t ld, const float* 
     return check_launch("rope_cache_write_bf16");
 }
 
+int astrai_w8a8_rotary_emb_bf16(const void* x, const float* freqs_cis, void* out, int64_t tokens,
+                                int64_t n_heads, int64_t head_dim, void* stream) {
+    if (!x || !freqs_cis || !out) return fail(ASTRAI_W8A8_BAD_ARG, "rotary_emb_bf16: null pointer");
+    if (tokens < 0 || n_heads <= 0 || head_dim <= 0 || n_heads > 65535 || head_dim > 65536 ||
+        tokens > ((int64_t)1 << 40))
+        return fail(ASTRAI_W8A8_BAD_ARG, "rotary_emb_bf16: bad dims");
+    if (head_dim % 2) return fail(ASTRAI_W8A8_BAD_ARG, "rotary_emb_bf16: head_dim must be even");
+    const uintptr_t need = head_dim % 8 ? 3 : 15;  // pair-wise or 16-byte accesses
+    if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out) |
+         reinterpret_cast<uintptr_t>(freqs_cis)) & need)
+        return fail(ASTRAI_W8A8_BAD_ARG, "rotary_emb_bf16: pointers must be %d-byte aligned", (int)need + 1);
+    if (tokens == 0) return ASTRAI_W8A8_OK;
+    if (!w8a8::launch_rotary_emb(x, freqs_cis, out, tokens, (int)n_heads, (int)head_dim,
+                                 static_cast<hipStream_t>(stream)))
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "rotary_emb_bf16: shape not supported");
+    return check_launch("rotary_emb_bf16");
+}
+
 int64_t astrai_w8a8_attn_decode_workspace_floats(int64_t batch, int64_t n_kv_heads, int64_t nsplit,
                                                  int64_t n_query_rows) {
     if (batch <= 0 || n_kv_heads <= 0 || nsplit <= 0 || n_query_rows <= 0 || n_query_rows > 8) return 0;
@@ -242,6 +260,24 @@ int astrai_w8a8_attn_paged_decode_bf16(const void* q, const void* k_pool, const 
                                        int64_t num_slots, int64_t num_requests,
                                        int64_t max_context_len, int64_t nsplit, float scale,
                                        void* stream) {
+    return astrai_w8a8_attn_paged_decode_masked_bf16(q, k_pool, v_pool, req_to_token, req_pool_indices,
+                                                     kv_indptr, nullptr, 0, 0, workspace, workspace_floats,
+                                                     out, batch, n_heads, n_kv_heads, head_dim, num_slots,
+                                                     num_requests, max_context_len, nsplit, scale, stream);
+}
+
+int astrai_w8a8_attn_paged_decode_masked_bf16(const void* q, const void* k_pool, const void* v_pool,
+                                              const int32_t* req_to_token,
+                                              const int32_t* req_pool_indices, const int32_t* kv_indptr,
+                                              const uint8_t* mask, int64_t mask_row_stride,
+                                              int64_t mask_width, float* workspace,
+                                              int64_t workspace_floats, void* out, int64_t batch,
+                                              int64_t n_heads, int64_t n_kv_heads, int64_t head_dim,
+                                              int64_t num_slots, int64_t num_requests,
+                                              int64_t max_context_len, int64_t nsplit, float scale,
+                                              void* stream) {
+    if (mask && (mask_width <= 0 || mask_width > INT32_MAX || mask_row_stride < 0))
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_decode_bf16: bad mask dims");
     if (!q || !k_pool || !v_pool || !req_to_token || !req_pool_indices || !kv_indptr || !workspace || !out)
         return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_decode_bf16: null pointer");
     if (batch < 0 || n_heads <= 0 || n_kv_heads <= 0 || num_slots <= 0 || num_requests <= 0 ||
@@ -261,7 +297,8 @@ int astrai_w8a8_attn_paged_decode_bf16(const void* q, const void* k_pool, const 
                     (long long)need);
     w8a8::AttnDecodeArgs a{q, k_pool, v_pool, nullptr, workspace, out, nullptr, nullptr, (int)batch, 1,
                            (int)n_heads, (int)n_kv_heads, (int)head_dim, max_context_len, (int)nsplit, scale,
-                           req_to_token, req_pool_indices, kv_indptr, max_context_len, num_slots, num_requests};
+                           req_to_token, req_pool_indices, kv_indptr, max_context_len, num_slots, num_requests,
+                           mask, mask_row_stride, (int)mask_width};
     if (!w8a8::launch_attn_decode(a, static_cast<hipStream_t>(stream)))
         return fail(ASTRAI_W8A8_UNSUPPORTED, "attn_paged_decode_bf16: shape not supported");
     return check_launch("attn_paged_decode_bf16");
@@ -301,6 +338,23 @@ int astrai_w8a8_attn_paged_prefill_bf16(const void* q, const void* k_pool, const
                                         int64_t n_kv_heads, int64_t head_dim, int64_t num_slots,
                                         int64_t num_requests, int64_t max_context_len, int causal,
                                         float scale, void* stream) {
+    return astrai_w8a8_attn_paged_prefill_masked_bf16(
+        q, k_pool, v_pool, req_to_token, req_pool_indices, kv_indptr, qo_indptr, q_tile_to_batch,
+        q_tile_to_index, nullptr, 0, 0, 0, 0, 0, out, num_q_tiles, n_heads, n_kv_heads, head_dim, num_slots,
+        num_requests, max_context_len, causal, scale, stream);
+}
+
+int astrai_w8a8_attn_paged_prefill_masked_bf16(
+    const void* q, const void* k_pool, const void* v_pool, const int32_t* req_to_token,
+    const int32_t* req_pool_indices, const int32_t* kv_indptr, const int32_t* qo_indptr,
+    const int32_t* q_tile_to_batch, const int32_t* q_tile_to_index, const uint8_t* mask,
+    int64_t mask_seq_stride, int64_t mask_head_stride, int64_t mask_row_stride, int64_t mask_rows,
+    int64_t mask_width, void* out, int64_t num_q_tiles, int64_t n_heads, int64_t n_kv_heads,
+    int64_t head_dim, int64_t num_slots, int64_t num_requests, int64_t max_context_len, int causal,
+    float scale, void* stream) {
+    if (mask && (mask_width <= 0 || mask_rows <= 0 || mask_width > INT32_MAX || mask_rows > INT32_MAX ||
+                 mask_seq_stride < 0 || mask_head_stride < 0 || mask_row_stride < 0))
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_prefill_bf16: bad mask dims");
     if (!q || !k_pool || !v_pool || !req_to_token || !req_pool_indices || !kv_indptr || !qo_indptr ||
         !q_tile_to_batch || !q_tile_to_index || !out)
         return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_prefill_bf16: null pointer");
@@ -326,6 +380,8 @@ int astrai_w8a8_attn_paged_prefill_bf16(const void* q, const void* k_pool, const
     a.q_tile_to_batch = q_tile_to_batch; a.q_tile_to_index = q_tile_to_index;
     a.num_q_tiles = (int)num_q_tiles; a.causal = causal ? 1 : 0;
     a.rtt_stride = max_context_len; a.num_slots = num_slots; a.num_requests = num_requests;
+    a.mask = mask; a.mask_b_stride = mask_seq_stride; a.mask_h_stride = mask_head_stride;
+    a.mask_l_stride = mask_row_stride; a.mask_rows = (int)mask_rows; a.mask_width = (int)mask_width;
     if (!w8a8::launch_attn_prefill(a, static_cast<hipStream_t>(stream)))
         return fail(ASTRAI_W8A8_UNSUPPORTED, "attn_paged_prefill_bf16: shape not supported");
     return check_launch("attn_paged_prefill_bf16");

@@ -49,7 +49,9 @@ __device__ __forceinline__ int lane_read_i(int v, int src_lane) {
 // sequence b lives in slot req_to_token[req_pool_indices[b]][j]
 // (csrc/kernels/attention/layout_policies.cuh:174-232); every sequence has its own
 // length kv_indptr[b+1] - kv_indptr[b] and one query token, the newest.
-template <int NQ, bool PAGED>
+// MASK (paged only): a bool tensor [batch, mask_width] picks the positions a sequence may
+// attend on top of its length (csrc/kernels/attention/mma_utils.cuh:196-199)
+template <int NQ, bool PAGED, bool MASK = false>
 __global__ __launch_bounds__(256) void attn_decode_partial_kernel(AttnDecodeArgs a) {
     __shared__ float sh_acc[4][NQ][kD];
     __shared__ float sh_ml[4][NQ][2];
@@ -118,10 +120,20 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(AttnDecodeArgs
     [[maybe_unused]] int slot_next = -1;
     if constexpr (PAGED) slot_next = key_slot(t0 + wave);
     const int64_t pool_row = (int64_t)a.n_kv_heads * kD;  // elements from one slot to the next
+    [[maybe_unused]] const uint8_t* mask_row = nullptr;
+    if constexpr (MASK) mask_row = a.mask + (int64_t)b * a.mask_b_stride;
 
     for (int t = t0 + wave; t < t1; t += 4) {
         const int kb = t << 4;
         u32x4 kf[4], vf[4];
+        [[maybe_unused]] uint8_t keep[4] = {1, 1, 1, 1};
+        if constexpr (MASK) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = kb + 4 * g + i;
+                keep[i] = key < a.mask_width ? mask_row[key] : (uint8_t)0;
+            }
+        }
         [[maybe_unused]] int vslot[4] = {0, 0, 0, 0};
         if constexpr (PAGED) {
             const int slot = slot_next;
@@ -160,6 +172,7 @@ __global__ __launch_bounds__(256) void attn_decode_partial_kernel(AttnDecodeArgs
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             bool ok = q_live && (int64_t)(kb + 4 * g + i) <= q_pos;
+            if constexpr (MASK) ok = ok && keep[i] != 0;
             sc[i] = ok ? sc[i] * a.scale : kNegBig;
             tm = fmaxf(tm, sc[i]);
         }
@@ -336,14 +349,19 @@ bool launch_attn_decode(const AttnDecodeArgs& a, hipStream_t stream) {
     const unsigned grid2 = (unsigned)(a.batch * a.seq);
     const bool paged = a.req_to_token != nullptr;
     if (paged && (a.seq != 1 || !a.req_pool_indices || !a.kv_indptr || a.rtt_stride <= 0)) return false;
+    if (a.mask && (!paged || a.mask_width <= 0)) return false;
     if (nq <= 4) {
-        if (paged)
+        if (paged && a.mask)
+            attn_decode_partial_kernel<4, true, true><<<dim3(grid1), dim3(256), 0, stream>>>(a);
+        else if (paged)
             attn_decode_partial_kernel<4, true><<<dim3(grid1), dim3(256), 0, stream>>>(a);
         else
             attn_decode_partial_kernel<4, false><<<dim3(grid1), dim3(256), 0, stream>>>(a);
         attn_decode_merge_kernel<4><<<dim3(grid2), dim3(256), 0, stream>>>(a);
     } else {
-        if (paged)
+        if (paged && a.mask)
+            attn_decode_partial_kernel<8, true, true><<<dim3(grid1), dim3(256), 0, stream>>>(a);
+        else if (paged)
             attn_decode_partial_kernel<8, true><<<dim3(grid1), dim3(256), 0, stream>>>(a);
         else
             attn_decode_partial_kernel<8, false><<<dim3(grid1), dim3(256), 0, stream>>>(a);

@@ -70,7 +70,10 @@ __device__ __forceinline__ void lds_dma16(__amdgpu_buffer_rsrc_t r, uint8_t* lds
 // astrai/inference/cache/pool.py:219-234). Two workgroups share a tile. Query row i of a
 // request of q_len rows and kv_len keys sees keys 0 .. kv_len - q_len + i (all of them
 // without the causal flag), so nothing has to be fetched to know the key range.
-template <int NREP, bool PAGED>
+// MASK (paged only): a bool tensor says, per sequence, (head,) (query row,) and position,
+// what may be attended on top of the causal range (csrc/kernels/attention/mma_utils.cuh:190-199);
+// every tile then takes the masking path.
+template <int NREP, bool PAGED, bool MASK = false>
 __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_kernel(AttnPrefillArgs a) {
     constexpr int K_DMA = kKB / 4 / NREP;              // 1 KiB key loads per wave and block
     __shared__ __attribute__((aligned(16))) uint8_t lds[kKRingBytes + 2 * kVBytes];
@@ -85,12 +88,13 @@ __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_ker
     int64_t q_row_stride;       // elements between consecutive query rows
     int pq, kmax, pmin;         // this lane's newest visible key; the block's extremes
     [[maybe_unused]] const int* table = nullptr;
-    [[maybe_unused]] int kv_len = 0, b_dense = 0;
+    [[maybe_unused]] int kv_len = 0, b_dense = 0, seq_index = 0;
     if constexpr (PAGED) {
         const int idx = (int)blockIdx.x;
         hk = idx % a.n_kv_heads;
         const int sub = (idx / a.n_kv_heads) & 1, tile = idx / (2 * a.n_kv_heads);
         const int req_i = a.q_tile_to_batch[tile];
+        seq_index = req_i;
         const int q_start = a.qo_indptr[req_i];
         rows_total = a.qo_indptr[req_i + 1] - q_start;
         row0 = a.q_tile_to_index[tile] * 64 + sub * kQB;
@@ -128,6 +132,16 @@ __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_ker
     const int head = hk * NREP + wave;
     const int s_row = row0 + qi;
     const bool row_live = s_row < rows_total;
+    // this lane's row of the mask and how many of its positions the mask covers (none for a
+    // query row the mask has no row for: nothing is read there and nothing attended)
+    [[maybe_unused]] const uint8_t* mask_row = nullptr;
+    [[maybe_unused]] int mask_keys = 0;
+    if constexpr (MASK) {
+        const bool covered = row_live && (a.mask_l_stride == 0 || s_row < a.mask_rows);
+        mask_row = a.mask + (int64_t)seq_index * a.mask_b_stride + (int64_t)head * a.mask_h_stride +
+                   (int64_t)(covered ? s_row : 0) * a.mask_l_stride;
+        mask_keys = covered ? a.mask_width : 0;
+    }
 
     const uint16_t* qrow = qbase + (int64_t)min(s_row, rows_total - 1) * q_row_stride;
     u32x4 qf[8];
@@ -272,13 +286,15 @@ __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_ker
     };
     // masking and this lane's share of the row maximum of tile T (raw scores; c > 0 keeps order)
     auto mask_max4 = [&](auto mask_tag, int T, f32x16& s, int g, float m) -> float {
-        constexpr bool MASK = decltype(mask_tag)::value;
+        constexpr bool PARTIAL = decltype(mask_tag)::value;  // some score of the tile may be hidden
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int e = 4 * g + j;
-            if (MASK) {
+            if (PARTIAL) {
                 const int key = T * 32 + g * 8 + h * 4 + j;
-                s[e] = key <= pq ? s[e] : kNegBig;
+                bool visible = key <= pq;
+                if constexpr (MASK) visible = visible && key < mask_keys && mask_row[key] != 0;
+                s[e] = visible ? s[e] : kNegBig;
             }
             m = fmaxf(m, s[e]);
         }
@@ -339,7 +355,7 @@ __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_ker
 
     // ---- prologue: tiles 0..2 and the first value block; scores of tile 0
     const int tfull = (__builtin_amdgcn_readfirstlane(pmin) + 1) / 32;  // tiles every query sees whole
-    const int nfast = max(tfull - 1, 0) / 2;  // blocks whose steps only produce unmasked tiles
+    const int nfast = MASK ? 0 : max(tfull - 1, 0) / 2;  // blocks whose steps only produce unmasked tiles
     dma_v(0, slots);
     if constexpr (PAGED) slots = lookup(3, 1);  // what the first block's loads will ask for
     // tile 0 needs the queries and the key tiles, not the values: wait for everything but
@@ -381,7 +397,10 @@ __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_ker
     // (now idle) key ring, so that the 32 x 128 tile leaves as whole 256-byte rows
     l_run += __shfl_xor(l_run, 32, kWave);
     // a row that sees no key at all (empty sequence, or more queries than keys) yields zeros
-    const float inv = (l_run > 0.0f && sees_a_key) ? 1.0f / l_run : 0.0f;
+    // (with a mask tensor a row may have met nothing but masked scores: its reference maximum
+    // then still is the stand-in for -inf, times c once it has been through a rescale)
+    const bool met_a_key = !MASK || m_run > 0.5f * kNegBig * fminf(c, 1.0f);
+    const float inv = (l_run > 0.0f && sees_a_key && met_a_key) ? 1.0f / l_run : 0.0f;
     {
         uint8_t* const mine = lds + wave * kKTileBytes;
 #pragma unroll
@@ -417,6 +436,7 @@ bool attn_prefill_supported(int n_heads, int n_kv_heads, int head_dim) {
 bool launch_attn_prefill(const AttnPrefillArgs& a, hipStream_t stream) {
     if (!attn_prefill_supported(a.n_heads, a.n_kv_heads, a.head_dim)) return false;
     const bool paged = a.req_to_token != nullptr;
+    if (a.mask && (!paged || a.mask_width <= 0 || a.mask_rows <= 0)) return false;
     const int n_rep = a.n_heads / a.n_kv_heads;
     int64_t wgs;
     if (paged) {
@@ -433,7 +453,9 @@ bool launch_attn_prefill(const AttnPrefillArgs& a, hipStream_t stream) {
     const dim3 grid((unsigned)wgs);
 #define W8A8_LAUNCH_PREFILL(R)                                                          \
     do {                                                                                \
-        if (paged)                                                                      \
+        if (paged && a.mask)                                                            \
+            attn_prefill_kernel<R, true, true><<<grid, dim3(64 * R), 0, stream>>>(a);   \
+        else if (paged)                                                                 \
             attn_prefill_kernel<R, true><<<grid, dim3(64 * R), 0, stream>>>(a);         \
         else                                                                            \
             attn_prefill_kernel<R, false><<<grid, dim3(64 * R), 0, stream>>>(a);        \

@@ -80,6 +80,10 @@ struct RopeCacheArgs {
     int64_t max_len;
 };
 void launch_rope_cache_write(const RopeCacheArgs& a, hipStream_t stream);
+// x, out bf16 [tokens, heads, head_dim]; freqs fp32 [tokens, head_dim/2, 2] (cos, sin) per token.
+// head_dim must be even; false if it is not.
+bool launch_rotary_emb(const void* x, const float* freqs, void* out, int64_t tokens, int heads,
+                       int head_dim, hipStream_t stream);
 
 // attn_decode.hip: grouped-query attention of a few new tokens against the dense
 // bf16 KV cache, split over the context; head_dim 128, n_rep * seq <= 8
@@ -103,6 +107,12 @@ struct AttnDecodeArgs {
     const int* kv_indptr;         // int32 [batch + 1]: prefix sums of the sequence lengths
     int64_t rtt_stride;
     int64_t num_slots, num_requests;  // table entries / rows outside these are treated as absent
+    // paged mode only, optional: bool [batch, mask_width] with row stride mask_b_stride; position
+    // j of sequence b is attended only where mask[b][j] is non-zero, positions at or past
+    // mask_width are not attended (csrc/kernels/attention/entry_utils.cuh:226-237, mma_utils.cuh:196-199)
+    const uint8_t* mask;
+    int64_t mask_b_stride;
+    int mask_width;
 };
 int64_t attn_decode_workspace_floats(int batch, int n_kv_heads, int nsplit, int nq);
 bool launch_attn_decode(const AttnDecodeArgs& a, hipStream_t stream);
@@ -129,6 +139,14 @@ struct AttnPrefillArgs {
     int num_q_tiles;
     int causal;                   // row i of a sequence sees keys 0 .. kv_len - q_len + i; else all keys
     int64_t rtt_stride, num_slots, num_requests;
+    // paged mode only, optional: bool mask addressed as mask[b * mask_b_stride + head *
+    // mask_h_stride + row * mask_l_stride + key] with b the sequence, row the query row inside
+    // the sequence and key the position (csrc/kernels/attention/entry_utils.cuh:326-346,
+    // mma_utils.cuh:190-199). A stride of 0 broadcasts that axis. Rows at or past mask_rows (when
+    // mask_l_stride != 0) and keys at or past mask_width are not attended.
+    const uint8_t* mask;
+    int64_t mask_b_stride, mask_h_stride, mask_l_stride;
+    int mask_rows, mask_width;
 };
 bool attn_prefill_supported(int n_heads, int n_kv_heads, int head_dim);
 bool launch_attn_prefill(const AttnPrefillArgs& a, hipStream_t stream);

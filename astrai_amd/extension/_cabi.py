@@ -49,6 +49,13 @@ PROTOTYPES = {
     "astrai_w8a8_attn_paged_prefill_bf16": (
         [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _INT,
          ctypes.c_float, _P], _INT),
+    "astrai_w8a8_rotary_emb_bf16": ([_P, _P, _P, _I64, _I64, _I64, _P], _INT),
+    "astrai_w8a8_attn_paged_decode_masked_bf16": (
+        [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
+         _I64, ctypes.c_float, _P], _INT),
+    "astrai_w8a8_attn_paged_prefill_masked_bf16": (
+        [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _P, _I64, _I64, _I64, _I64,
+         _I64, _I64, _I64, _INT, ctypes.c_float, _P], _INT),
     "astrai_w8a8_attn_prefill_bf16": (
         [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, ctypes.c_float, _P], _INT),
     "astrai_w8a8_attn_decode_bf16": (
@@ -499,6 +506,48 @@ def silu_mul_quantize_int8(gate: torch.Tensor, up: torch.Tensor, want_h: bool = 
     return hq, s, None if h is None else h.reshape(gate.shape)
 
 
+def rotary_emb(x: torch.Tensor, freqs_cis: torch.Tensor) -> torch.Tensor:
+    """Rotate adjacent pairs of ``x`` (bf16, packed ``[tokens, heads, head_dim]`` or dense
+    ``[batch, seq, heads, head_dim]``) by ``freqs_cis`` (fp32, the same token axes followed by
+    ``[head_dim/2, 2]`` = cos, sin); a new tensor of ``x``'s shape. Argument checks and
+    messages of the reference's entry (csrc/kernels/rotary/rotary_emb.cu:47-93)."""
+    lib = _require()
+    if not x.is_cuda:
+        raise RuntimeError("x must be on CUDA")
+    if not freqs_cis.is_cuda:
+        raise RuntimeError("freqs_cis must be on CUDA")
+    if x.dtype != torch.bfloat16:
+        raise RuntimeError("x must be bf16")
+    if x.dim() not in (3, 4):
+        raise RuntimeError("x must be [tokens, n_heads, head_dim] or [batch, seq_len, n_heads, head_dim]")
+    if not x.is_contiguous():
+        raise RuntimeError("x must be contiguous")
+    if freqs_cis.dim() != x.dim():
+        raise RuntimeError("freqs_cis rank must match x rank")
+    if not freqs_cis.is_contiguous():
+        raise RuntimeError("freqs_cis must be contiguous")
+    if freqs_cis.dtype != torch.float32:
+        raise RuntimeError("freqs_cis must be f32")
+    if freqs_cis.device != x.device:
+        raise RuntimeError("freqs_cis must be on x's device")
+    tokens = x.size(0) if x.dim() == 3 else x.size(0) * x.size(1)
+    heads, head_dim = x.size(-2), x.size(-1)
+    if head_dim % 2:
+        raise RuntimeError("head_dim must be even")
+    if freqs_cis.numel() != tokens * head_dim:
+        raise RuntimeError("freqs_cis token or rotary dimension mismatch")
+    if freqs_cis.size(-2) != head_dim // 2:
+        raise RuntimeError("freqs_cis dim/2 mismatch")
+    if freqs_cis.size(-1) != 2:
+        raise RuntimeError("freqs_cis last dim must be 2 [cos, sin]")
+    with torch.cuda.device(x.device):
+        out = torch.empty_like(x)
+        if x.numel():
+            _check(lib.astrai_w8a8_rotary_emb_bf16(x.data_ptr(), freqs_cis.data_ptr(), out.data_ptr(),
+                                                   tokens, heads, head_dim, _stream(x)), lib)
+    return out
+
+
 def rope_cache_write(qkv: torch.Tensor, freqs: torch.Tensor, positions: torch.Tensor,
                      k_cache: torch.Tensor, v_cache: torch.Tensor, n_heads: int, n_kv_heads: int,
                      head_dim: int) -> torch.Tensor:
@@ -602,11 +651,19 @@ def attn_paged_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     written to the slot of each sequence's newest position, as the reference's kernel
     persists them (layout_policies.cuh:226-252). ``causal_offset`` does not change a
     one-token query (layout_policies.cuh:194-197); the split buffers are not needed
-    (the workspace is allocated here); ``mask`` is not supported."""
+    (the workspace is allocated here). ``mask``: bool ``[batch, width]``, True = attend
+    that position (entry_utils.cuh:226-237); positions past ``width`` are not attended."""
     lib = _require()
     _gpu(q, "attn_paged_decode")
     if mask is not None:
-        raise RuntimeError("attn_paged_decode: a key mask is not supported")
+        if not mask.is_cuda or mask.dtype != torch.bool:
+            raise RuntimeError("mask must be bool CUDA")
+        if mask.dim() != 2 or mask.size(0) != q.size(0):
+            raise RuntimeError("mask batch mismatch: a decode mask is [batch, kv positions]")
+        if mask.size(1) == 0:
+            raise RuntimeError("mask kv_len mismatch: the mask has no positions")
+        if mask.stride(1) != 1:
+            mask = mask.contiguous()
     if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
         raise RuntimeError("q, k_cache and v_cache must be bf16")
     if q.dim() != 3 or k_cache.dim() != 3 or k_cache.shape != v_cache.shape:
@@ -653,10 +710,11 @@ def attn_paged_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
             out = torch.empty((b, h, d), device=q.device, dtype=torch.bfloat16)
         need = lib.astrai_w8a8_attn_decode_workspace_floats(b, hkv, nsplit, h // hkv)
         ws = torch.empty(max(need, 1), device=q.device, dtype=torch.float32)
-        _check(lib.astrai_w8a8_attn_paged_decode_bf16(
+        m_ptr, m_stride, m_width = (mask.data_ptr(), mask.stride(0), mask.size(1)) if mask is not None else (0, 0, 0)
+        _check(lib.astrai_w8a8_attn_paged_decode_masked_bf16(
             q_c.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), rtt.data_ptr(), rpi.data_ptr(),
-            ind.data_ptr(), ws.data_ptr(), ws.numel(), out.data_ptr(), b, h, hkv, d, slots,
-            rtt.size(0), rtt.size(1), nsplit, float(scale), _stream(q)), lib)
+            ind.data_ptr(), m_ptr, m_stride, m_width, ws.data_ptr(), ws.numel(), out.data_ptr(), b, h, hkv,
+            d, slots, rtt.size(0), rtt.size(1), nsplit, float(scale), _stream(q)), lib)
     return out
 
 
@@ -673,12 +731,33 @@ def attn_paged_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Te
     (csrc/kernels/attention/paged_prefill.cu:36-52): packed ``q [total_q, H, 128]``, flat
     pools, ``req_to_token`` / ``req_pool_indices`` / ``kv_indptr`` / ``qo_indptr`` int32, and
     the schedule of 64-row query tiles. ``causal_offset >= 0`` asks for the causal mask (the
-    wrapper passes 0 for ``is_causal``, astrai/extension/ops/attention.py:188); ``mask`` is
-    not supported. Returns ``[total_q, H, 128]`` bf16."""
+    wrapper passes 0 for ``is_causal``, astrai/extension/ops/attention.py:188). ``mask``:
+    bool, True = attend, ``[batch, kv]`` or ``[batch, 1 | H, rows, kv]`` with ``rows`` counted
+    inside each sequence (entry_utils.cuh:326-346); rows and positions the mask does not hold
+    are not attended. Returns ``[total_q, H, 128]`` bf16."""
     lib = _require()
     _gpu(q, "attn_paged_prefill")
+    m_args = (0, 0, 0, 0, 0, 0)
     if mask is not None:
-        raise RuntimeError("attn_paged_prefill: a key mask is not supported")
+        if not mask.is_cuda or mask.dtype != torch.bool:
+            raise RuntimeError("mask must be bool CUDA")
+        if mask.dim() not in (2, 4):
+            raise RuntimeError("mask must be 2D or 4D")
+        if mask.size(0) != req_pool_indices.numel():
+            raise RuntimeError("mask batch mismatch")
+        if mask.dim() == 4 and mask.size(1) not in (1, q.size(1)):
+            raise RuntimeError("mask head mismatch")
+        if mask.dim() == 4 and mask.size(2) == 0:
+            raise RuntimeError("mask q_len mismatch")
+        if mask.size(-1) == 0:
+            raise RuntimeError("mask kv_len mismatch: the mask has no positions")
+        if mask.stride(-1) != 1:
+            mask = mask.contiguous()
+        if mask.dim() == 2:
+            m_args = (mask.data_ptr(), mask.stride(0), 0, 0, 1, mask.size(1))
+        else:
+            m_args = (mask.data_ptr(), mask.stride(0), 0 if mask.size(1) == 1 else mask.stride(1),
+                      0 if mask.size(2) == 1 else mask.stride(2), mask.size(2), mask.size(3))
     if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
         raise RuntimeError("q, k_cache and v_cache must be bf16")
     if q.dim() != 3 or k_cache.dim() != 3 or k_cache.shape != v_cache.shape:
@@ -708,9 +787,9 @@ def attn_paged_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Te
     with torch.cuda.device(q.device):
         # (rows that no tile of the schedule covers are left unwritten, as by the reference)
         out = torch.empty((total_q, h, d), device=q.device, dtype=torch.bfloat16)
-        _check(lib.astrai_w8a8_attn_paged_prefill_bf16(
+        _check(lib.astrai_w8a8_attn_paged_prefill_masked_bf16(
             q_c.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), *[t.data_ptr() for t in tensors],
-            out.data_ptr(), q_tile_to_batch.numel(), h, hkv, d, slots, req_to_token.size(0),
+            *m_args, out.data_ptr(), q_tile_to_batch.numel(), h, hkv, d, slots, req_to_token.size(0),
             req_to_token.size(1), 1 if causal_offset >= 0 else 0, float(scale), _stream(q)), lib)
     return out
 
@@ -933,3 +1012,156 @@ def mm_fp8_block128(a: torch.Tensor, b: torch.Tensor, sa: torch.Tensor, sb: torc
                 a_c.data_ptr(), b_c.data_ptr(), sa.data_ptr(), sb.data_ptr(), _ptr(bias),
                 out.data_ptr(), m, n, k, _stream(a)), lib)
     return out
+
+
+# ---------------------------------------------------------------------------
+# The reference's dense entries attn_decode / attn_prefill (q, k, v tensors in either
+# layout, csrc/kernels/attention/decode.cu:4-67 and prefill.cu) on top of the kernels above.
+# ---------------------------------------------------------------------------
+
+BHLD, BLHD = 0, 1  # the reference's TensorLayout (csrc/kernels/attention/common.h)
+
+_index_cache: dict = {}
+
+
+def _identity_paging(batch: int, kv_len: int, device):
+    """``(req_to_token, req_pool_indices)`` that address a token-major ``[batch, kv_len, ...]``
+    tensor, viewed as a pool of ``batch * kv_len`` slots, sequence by sequence."""
+    key = ("page", batch, kv_len, str(device))
+    if key not in _index_cache:
+        if len(_index_cache) > 64:
+            _index_cache.clear()
+        table = torch.arange(batch * kv_len, dtype=torch.int32, device=device).reshape(batch, kv_len)
+        _index_cache[key] = (table, torch.arange(batch, dtype=torch.int32, device=device))
+    return _index_cache[key]
+
+
+def _dense_args(q, k, v, layout, what):
+    if not (q.is_cuda and k.is_cuda and v.is_cuda):
+        raise RuntimeError(f"{what}: q, k and v must be CUDA tensors")
+    if q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16:
+        raise RuntimeError(f"{what}: q, k and v must be bf16")
+    if k.shape != v.shape:
+        raise RuntimeError("K and V must have identical shapes")
+    if q.dim() != 4 or k.dim() != 4:
+        raise RuntimeError("Q/K/V must be 4D")
+    if layout not in (BHLD, BLHD):
+        raise RuntimeError(f"{what}: layout must be 0 (BHLD) or 1 (BLHD)")
+    l_ax, h_ax = (2, 1) if layout == BHLD else (1, 2)
+    b, q_len, h, d = q.size(0), q.size(l_ax), q.size(h_ax), q.size(3)
+    kv_len, hkv = k.size(l_ax), k.size(h_ax)
+    if k.size(0) != b:
+        raise RuntimeError("K/V batch must match Q")
+    if h % hkv:
+        raise RuntimeError("q_head must be divisible by kv_head")
+    if k.size(3) != d:
+        raise RuntimeError("K/V head_dim must match Q")
+    return b, q_len, kv_len, h, hkv, d
+
+
+def _dense_mask(mask, b, q_len, kv_len, h):
+    """The reference's 2D / 3D / 4D mask (entry_utils.cuh:56-86) as ``[b, 1 | h, 1 | q_len, kv_len]``."""
+    if mask is None:
+        return None
+    if not mask.is_cuda:
+        raise RuntimeError("mask must be on CUDA")
+    if mask.dtype != torch.bool:
+        raise RuntimeError("mask must be bool")
+    if mask.size(0) != b:
+        raise RuntimeError("mask batch mismatch")
+    if mask.size(-1) != kv_len:
+        raise RuntimeError("mask kv_len mismatch")
+    if mask.dim() == 2:
+        return mask[:, None, None, :]
+    if mask.dim() == 3:
+        if mask.size(1) not in (1, q_len):
+            raise RuntimeError("mask q_len mismatch")
+        return mask[:, None]
+    if mask.dim() == 4:
+        if mask.size(1) not in (1, h):
+            raise RuntimeError("mask head mismatch")
+        if mask.size(2) not in (1, q_len):
+            raise RuntimeError("mask q_len mismatch")
+        return mask
+    raise RuntimeError("mask must be 2D, 3D, or 4D")
+
+
+def _token_major(t, layout):
+    return (t.transpose(1, 2) if layout == BHLD else t).contiguous()
+
+
+def attn_decode_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Optional[torch.Tensor] = None,
+                    causal_offset: int = -1, scale: float = 0.0, layout: int = BHLD,
+                    o_part_buf=None, ml_part_buf=None) -> torch.Tensor:
+    """The reference's ``attn_decode`` entry (csrc/kernels/attention/decode.cu:4-67): one query
+    token per sequence against ``k`` / ``v`` tensors, ``[batch, heads, len, 128]`` (layout 0) or
+    ``[batch, len, heads, 128]`` (layout 1); the result has ``q``'s layout. ``causal_offset >= 0``
+    limits the keys to ``0 .. causal_offset`` (layout_policies.cuh:138-141), ``mask`` (bool, True =
+    attend) is ``[batch, kv_len]``, ``[batch, 1, kv_len]`` or ``[batch, 1, 1, kv_len]``. The split
+    buffers are not needed. Layout 0 without a mask runs the dense-cache kernel in place; the
+    other cases run the paged kernel over the token-major tensors (layout 0 is copied for it)."""
+    b, q_len, kv_len, h, hkv, d = _dense_args(q, k, v, layout, "attn_decode")
+    if q_len != 1:
+        raise RuntimeError("Q seq_len must be 1")
+    m4 = _dense_mask(mask, b, 1, kv_len, h)
+    if m4 is not None and m4.size(1) != 1:
+        raise RuntimeError("attn_decode: a mask per head is not supported")
+    if d != 128 or h // hkv > 8 or h > 64:
+        raise RuntimeError("attn_decode needs head_dim 128, n_heads / n_kv_heads <= 8, n_heads <= 64")
+    attend = kv_len if causal_offset < 0 else min(kv_len, causal_offset + 1)
+    with torch.cuda.device(q.device):
+        if kv_len == 0 or b == 0:
+            return torch.zeros_like(q)
+        if layout == BHLD and m4 is None and k.is_contiguous() and v.is_contiguous():
+            pos = torch.full((1,), attend - 1, dtype=torch.int64, device=q.device)
+            out = attn_decode(q.contiguous(), k, v, pos, scale=scale if scale > 0 else None)
+            return out.reshape(b, h, 1, d)
+        k_tm, v_tm = _token_major(k, layout), _token_major(v, layout)
+        table, rows = _identity_paging(b, kv_len, q.device)
+        indptr = (torch.arange(b + 1, dtype=torch.int32, device=q.device) * attend)
+        out = attn_paged_decode(q.reshape(b, h, d), k_tm.view(b * kv_len, hkv, d), v_tm.view(b * kv_len, hkv, d),
+                                table, rows, indptr, mask=None if m4 is None else m4[:, 0, 0], scale=scale)
+    return out.reshape(q.shape)  # one token: both layouts have the same memory order
+
+
+def attn_prefill_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Optional[torch.Tensor] = None,
+                     causal_offset: int = -1, scale: float = 0.0, layout: int = BHLD) -> torch.Tensor:
+    """The reference's ``attn_prefill`` entry (csrc/kernels/attention/prefill.cu): a block of
+    query rows per sequence against ``k`` / ``v`` tensors in either layout; the result has
+    ``q``'s layout. ``causal_offset >= 0``: row ``i`` sees keys ``0 .. i + causal_offset``
+    (prefill_split_q_mma.cuh:121-124); ``mask`` (bool, True = attend) is ``[batch, kv_len]``,
+    ``[batch, 1 | q_len, kv_len]`` or ``[batch, 1 | heads, 1 | q_len, kv_len]``. Layout 0 without
+    a mask runs the dense-cache kernel in place; the other cases run the ragged paged kernel
+    over the token-major tensors (layout 0 is copied for it); an offset other than
+    ``kv_len - q_len`` is expressed through the mask."""
+    b, q_len, kv_len, h, hkv, d = _dense_args(q, k, v, layout, "attn_prefill")
+    m4 = _dense_mask(mask, b, q_len, kv_len, h)
+    if not attn_prefill_supported(h, hkv, d):
+        raise RuntimeError("attn_prefill needs head_dim 128 and n_heads / n_kv_heads in {2, 4, 8}")
+    with torch.cuda.device(q.device):
+        if kv_len == 0 or b == 0 or q_len == 0:
+            return torch.zeros_like(q)
+        rows_i = torch.arange(q_len, dtype=torch.int64, device=q.device)
+        if layout == BHLD and m4 is None and k.is_contiguous() and v.is_contiguous():
+            pos = torch.full_like(rows_i, kv_len - 1) if causal_offset < 0 else (rows_i + causal_offset).clamp_max(kv_len - 1)
+            out = attn_prefill(q.contiguous(), k, v, pos, scale=scale if scale > 0 else None)
+            return out.view(b, q_len, h, d).transpose(1, 2)
+        causal = causal_offset >= 0 and causal_offset == kv_len - q_len
+        if causal_offset >= 0 and not causal:
+            band = torch.arange(kv_len, device=q.device)[None, :] <= (rows_i + causal_offset)[:, None]
+            band = band[None, None].expand(b, 1, q_len, kv_len)
+            m4 = band if m4 is None else (m4 & band)
+        q_tm = _token_major(q, layout)
+        k_tm, v_tm = _token_major(k, layout), _token_major(v, layout)
+        table, rows = _identity_paging(b, kv_len, q.device)
+        key = ("sched", b, q_len, str(q.device))
+        if key not in _index_cache:
+            _index_cache[key] = paged_prefill_schedule([q_len] * b, q.device)
+        qo, tb, ti = _index_cache[key]
+        kvp = torch.arange(b + 1, dtype=torch.int32, device=q.device) * kv_len
+        out = attn_paged_prefill(q_tm.view(b * q_len, h, d), k_tm.view(b * kv_len, hkv, d),
+                                 v_tm.view(b * kv_len, hkv, d), table, rows, kvp, qo, tb, ti, mask=m4,
+                                 causal_offset=0 if causal else -1, scale=scale)
+    out = out.view(b, q_len, h, d)
+    return out if layout == BLHD else out.transpose(1, 2)
+

@@ -62,7 +62,25 @@ def _attn_paged_prefill_module() -> SimpleNamespace:
     return SimpleNamespace(attn_paged_prefill=_cabi.attn_paged_prefill)
 
 
+def _attn_decode_module() -> SimpleNamespace:
+    # the callable of csrc/kernels/attention/decode.cu:4-67 (q, k, v tensors in either layout)
+    return SimpleNamespace(attn_decode=_cabi.attn_decode_qkv)
+
+
+def _attn_prefill_module() -> SimpleNamespace:
+    # the callable of csrc/kernels/attention/prefill.cu, same argument list
+    return SimpleNamespace(attn_prefill=_cabi.attn_prefill_qkv)
+
+
+def _rotary_emb_module() -> SimpleNamespace:
+    # the callable of csrc/kernels/rotary/rotary_emb.cu:47-93
+    return SimpleNamespace(rotary_emb=_cabi.rotary_emb)
+
+
 _FACTORIES = {
+    "attn_decode": _attn_decode_module,
+    "attn_prefill": _attn_prefill_module,
+    "rotary_emb": _rotary_emb_module,
     "attn_paged_decode": _attn_paged_decode_module,
     "attn_paged_prefill": _attn_paged_prefill_module,
     "fp8_mm": _fp8_mm_module,

@@ -158,6 +158,21 @@ int astrai_w8a8_rope_cache_write_bf16(const void* qkv_bf16, int64_t ld, const fl
                                       int64_t head_dim, int64_t max_len, void* stream);
 
 /*
+ * Rotary embedding alone. Replaces rotary_emb (csrc/kernels/rotary/rotary_emb.cu:6-45 kernel,
+ * :47-93 entry; Python wrapper astrai/extension/ops/rotary.py:24-39).
+ *   x, out     bf16 [tokens, n_heads, head_dim], contiguous (a dense [batch, seq, ...] tensor
+ *              is the same memory with tokens = batch * seq)
+ *   freqs_cis  fp32 [tokens, head_dim/2, 2]: each token's own (cos, sin) rows
+ *   out[t,h,2i] = x[t,h,2i] cos - x[t,h,2i+1] sin;  out[t,h,2i+1] = x[t,h,2i] sin + x[t,h,2i+1] cos
+ *   with every product and sum rounded in fp32 and one rounding to bf16: bit for bit the
+ *   fp32 tensor arithmetic of astrai/extension/backend/rotary.py:25-33 (the reference's own
+ *   kernel leaves the contraction of a*b - c*d to its compiler).
+ * head_dim even; pointers 16-byte aligned when head_dim % 8 == 0, else 4-byte.
+ */
+int astrai_w8a8_rotary_emb_bf16(const void* x_bf16, const float* freqs_cis, void* out_bf16,
+                                int64_t tokens, int64_t n_heads, int64_t head_dim, void* stream);
+
+/*
  * Grouped-query attention of the `seq` newest tokens of every sequence against the
  * dense KV cache (decode step; split over the context and merged). Replaces the
  * cached branch of GQA.forward / the decode attention backend
@@ -191,8 +206,8 @@ int astrai_w8a8_attn_decode_bf16(const void* q_bf16, const void* k_cache_bf16, c
  * The same decode attention over a token-granular paged cache. Replaces
  * attn_paged_decode (csrc/kernels/attention/paged_decode.cu:4-67, addressing policy
  * PagedKV in csrc/kernels/attention/layout_policies.cuh:174-232; Python wrapper
- * astrai/extension/ops/attention.py:93-147) without its fused append of new_k / new_v
- * and without the optional key mask.
+ * astrai/extension/ops/attention.py:93-147) without its fused append of new_k / new_v;
+ * the variant with the optional key mask follows.
  *   q          bf16 [batch, n_heads, 128]: the newest token of every sequence
  *   k_pool, v_pool  bf16 [num_slots, n_kv_heads, 128]
  *   req_to_token    int32 [num_requests, max_context_len]: pool slot of (request, position);
@@ -215,6 +230,27 @@ int astrai_w8a8_attn_paged_decode_bf16(const void* q_bf16, const void* k_pool_bf
                                        int64_t head_dim, int64_t num_slots, int64_t num_requests,
                                        int64_t max_context_len, int64_t nsplit, float scale,
                                        void* stream);
+
+/*
+ * attn_paged_decode_bf16 with the reference's optional key mask (the `mask` argument of
+ * csrc/kernels/attention/paged_decode.cu:13, packed at entry_utils.cuh:226-237 and applied
+ * at mma_utils.cuh:196-199).
+ *   mask       bool (one byte each) [batch, mask_width], rows mask_row_stride bytes apart:
+ *              position j of sequence b is attended only where mask[b][j] != 0. Positions
+ *              at or past mask_width are not attended (the reference reads past the row
+ *              there). A sequence with every position masked yields zeros. NULL: no mask,
+ *              mask_row_stride and mask_width are ignored.
+ */
+int astrai_w8a8_attn_paged_decode_masked_bf16(const void* q_bf16, const void* k_pool_bf16,
+                                              const void* v_pool_bf16, const int32_t* req_to_token,
+                                              const int32_t* req_pool_indices, const int32_t* kv_indptr,
+                                              const uint8_t* mask, int64_t mask_row_stride,
+                                              int64_t mask_width, float* workspace,
+                                              int64_t workspace_floats, void* out_bf16, int64_t batch,
+                                              int64_t n_heads, int64_t n_kv_heads, int64_t head_dim,
+                                              int64_t num_slots, int64_t num_requests,
+                                              int64_t max_context_len, int64_t nsplit, float scale,
+                                              void* stream);
 
 /*
  * Causal grouped-query attention of a block of `seq` new tokens per sequence against
@@ -241,8 +277,8 @@ int astrai_w8a8_attn_prefill_bf16(const void* q_bf16, const void* k_cache_bf16,
  * The same causal block attention over ragged sequences in a token-granular paged cache.
  * Replaces attn_paged_prefill (csrc/kernels/attention/paged_prefill.cu:4-52, addressing
  * policies PackedQSchedule / PagedKV in csrc/kernels/attention/layout_policies.cuh:67-93,
- * 174-232; Python wrapper astrai/extension/ops/attention.py:150-207) without the optional
- * key mask.
+ * 174-232; Python wrapper astrai/extension/ops/attention.py:150-207); the variant with the
+ * optional mask follows.
  *   q, out     bf16 [total_q, n_heads, 128]: the query rows of all sequences, packed
  *   k_pool, v_pool, req_to_token, req_pool_indices, kv_indptr  as for attn_paged_decode_bf16
  *   qo_indptr  int32 [batch + 1]: prefix sums of the sequences' query row counts
@@ -264,6 +300,29 @@ int astrai_w8a8_attn_paged_prefill_bf16(const void* q_bf16, const void* k_pool_b
                                         int64_t head_dim, int64_t num_slots, int64_t num_requests,
                                         int64_t max_context_len, int causal, float scale,
                                         void* stream);
+
+/*
+ * attn_paged_prefill_bf16 with the reference's optional mask (the `mask` argument of
+ * csrc/kernels/attention/paged_prefill.cu:14: 2D [batch, kv] or 4D [batch, 1 | n_heads,
+ * rows, kv], packed into three strides at entry_utils.cuh:326-346 and applied at
+ * mma_utils.cuh:190-199).
+ *   mask       bool (one byte each); query row r (counted inside its sequence) of sequence b
+ *              and head h attends position j, on top of the causal range, only where
+ *              mask[b * mask_seq_stride + h * mask_head_stride + r * mask_row_stride + j] != 0.
+ *              A stride of 0 broadcasts that axis (a 2D mask has head and row stride 0).
+ *   mask_rows  rows the mask holds per sequence (used when mask_row_stride != 0): rows at or
+ *              past it attend nothing and yield zeros
+ *   mask_width positions a row of the mask holds: positions at or past it are not attended
+ *              (the reference reads past the row in both cases). NULL mask: no mask.
+ */
+int astrai_w8a8_attn_paged_prefill_masked_bf16(
+    const void* q_bf16, const void* k_pool_bf16, const void* v_pool_bf16,
+    const int32_t* req_to_token, const int32_t* req_pool_indices, const int32_t* kv_indptr,
+    const int32_t* qo_indptr, const int32_t* q_tile_to_batch, const int32_t* q_tile_to_index,
+    const uint8_t* mask, int64_t mask_seq_stride, int64_t mask_head_stride, int64_t mask_row_stride,
+    int64_t mask_rows, int64_t mask_width, void* out_bf16, int64_t num_q_tiles, int64_t n_heads,
+    int64_t n_kv_heads, int64_t head_dim, int64_t num_slots, int64_t num_requests,
+    int64_t max_context_len, int causal, float scale, void* stream);
 
 /*
  * bf16 -> e4m3fn with one scale per 1x128 K-group (activations) or per 128x128

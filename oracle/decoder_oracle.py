@@ -16,7 +16,7 @@ so that it shares no code with the product's modules. Arithmetic followed:
 
 from __future__ import annotations
 
-from typing import Callable, Dict
+from typing import Callable, Dict, Optional
 
 import torch
 import torch.nn.functional as F
@@ -77,7 +77,7 @@ def attn_cached(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
 
 def attn_paged_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                       req_to_token: torch.Tensor, req_pool_indices: torch.Tensor,
-                      kv_indptr: torch.Tensor) -> torch.Tensor:
+                      kv_indptr: torch.Tensor, mask: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Decode attention over a token-granular paged cache: ``q [B, H, D]``, pools
     ``[slots, H_kv, D]``; key ``j`` of sequence ``b`` is pool row
     ``req_to_token[req_pool_indices[b], j]`` for ``j < kv_indptr[b+1] - kv_indptr[b]``
@@ -86,8 +86,12 @@ def attn_paged_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tenso
     position stays in the attended range [0, kv_len): the reference gates the load on the slot
     (layout_policies.cuh:104-110,212-219; decode_split_kv_mma.cuh:75-82) and masks by position
     only (decode_split_kv_mma.cuh:107-110), so such a position enters the softmax with score 0.
-    ``softmax(q k^T / sqrt(D)) v`` in float32 per sequence, a sequence without keys gives
-    zeros. Returns ``[B, H, D]`` in the input dtype."""
+    ``mask`` (bool ``[B, width]``, indexed by sequence and position, True = attend) hides
+    positions on top of that (csrc/kernels/attention/entry_utils.cuh:226-237,
+    mma_utils.cuh:196-199); the reference reads past a mask narrower than a sequence, here such
+    positions are hidden. ``softmax(q k^T / sqrt(D)) v`` in float32 per sequence; a sequence
+    without a visible key gives zeros (mma_utils.cuh:217-218, the guarded 1/l of the kernels).
+    Returns ``[B, H, D]`` in the input dtype."""
     b, h, d = q.shape
     n_rep = h // k_pool.size(1)
     out = torch.zeros(b, h, d, dtype=torch.float32)
@@ -100,6 +104,13 @@ def attn_paged_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tenso
         k = torch.where(live, k_pool[rows.clamp_min(0)].float(), torch.zeros(())).repeat_interleave(n_rep, dim=1)
         v = torch.where(live, v_pool[rows.clamp_min(0)].float(), torch.zeros(())).repeat_interleave(n_rep, dim=1)
         scores = torch.einsum("hd,nhd->hn", q[i].float(), k) / (d ** 0.5)
+        if mask is not None:
+            seen = torch.zeros(n, dtype=torch.bool)
+            w = min(n, mask.size(1))
+            seen[:w] = mask[i, :w]
+            if not bool(seen.any()):
+                continue
+            scores = scores.masked_fill(~seen[None], float("-inf"))
         out[i] = torch.einsum("hn,nhd->hd", torch.softmax(scores, dim=-1), v)
     return out.to(q.dtype)
 
@@ -107,15 +118,18 @@ def attn_paged_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tenso
 def attn_paged_prefill(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                        req_to_token: torch.Tensor, req_pool_indices: torch.Tensor,
                        kv_indptr: torch.Tensor, qo_indptr: torch.Tensor,
-                       causal: bool = True) -> torch.Tensor:
+                       causal: bool = True, mask: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Ragged prefill over the paged cache: packed ``q [total_q, H, D]``; sequence ``b`` owns
     rows ``qo_indptr[b] .. qo_indptr[b+1]`` and keys ``req_to_token[req_pool_indices[b], :kv_len]``;
     with ``causal`` row ``i`` of it sees keys ``0 .. kv_len - q_len + i``
     (csrc/kernels/attention/layout_policies.cuh:67-93,174-232). A negative pool row reads as a
     zero key and a zero value and is attended like any other position (the load is gated on the
-    slot, the mask on the position: prefill_split_q_mma.cuh:84-89,121-124). float32 softmax
-    attention per sequence; a row that sees no position gives zeros. Returns ``[total_q, H, D]``
-    in the input dtype."""
+    slot, the mask on the position: prefill_split_q_mma.cuh:84-89,121-124). ``mask`` (bool, True
+    = attend): ``[B, kv]``, or ``[B, 1 | H, rows, kv]`` with ``rows`` 1 (every row) or counted
+    inside each sequence, combined with the causal range by "and" (entry_utils.cuh:326-346,
+    mma_utils.cuh:190-199); the reference reads past a mask with fewer rows or positions than
+    a sequence, here those are hidden. float32 softmax attention per sequence; a row that sees
+    no position gives zeros. Returns ``[total_q, H, D]`` in the input dtype."""
     total_q, h, d = q.shape
     n_rep = h // k_pool.size(1)
     out = torch.zeros(total_q, h, d, dtype=torch.float32)
@@ -133,11 +147,56 @@ def attn_paged_prefill(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tens
         if causal:
             newest = (n - (q1 - q0)) + torch.arange(q1 - q0)
             visible &= torch.arange(n)[None, :] <= newest[:, None]
-        scores = scores.masked_fill(~visible[None], float("-inf"))
+        visible = visible[None].expand(h, -1, -1)
+        if mask is not None:
+            m4 = mask[b][None, None, :] if mask.dim() == 2 else mask[b]      # [1 | H, rows, kv]
+            cover = torch.zeros(m4.size(0), q1 - q0, n, dtype=torch.bool)
+            w = min(n, m4.size(-1))
+            if m4.size(1) == 1:
+                cover[:, :, :w] = m4[:, :, :w]
+            else:
+                r = min(q1 - q0, m4.size(1))
+                cover[:, :r, :w] = m4[:, :r, :w]
+            visible = visible & cover
+        scores = scores.masked_fill(~visible, float("-inf"))
         p = torch.softmax(scores, dim=-1)
-        p = torch.where(visible.any(-1)[None, :, None], p, torch.zeros_like(p))
+        p = torch.where(visible.any(-1)[:, :, None], p, torch.zeros_like(p))
         out[q0:q1] = torch.einsum("hqn,nhd->qhd", p, v)
     return out.to(q.dtype)
+
+
+def attn_dense(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Optional[torch.Tensor] = None,
+               causal_offset: int = -1, layout: int = 1) -> torch.Tensor:
+    """The reference's dense kernels attn_decode / attn_prefill as one formula: ``q``, ``k``,
+    ``v`` in layout 1 ``[B, L, H, D]`` or 0 ``[B, H, L, D]``; query head ``h`` reads KV head
+    ``h // n_rep``; with ``causal_offset >= 0`` row ``i`` sees keys ``j <= i + causal_offset``
+    (csrc/kernels/attention/prefill_split_q_mma.cuh:121-124; for the one row of a decode
+    call that is layout_policies.cuh:138-141); ``mask`` (bool, True = attend) is ``[B, kv]``,
+    ``[B, 1 | q, kv]`` or ``[B, 1 | H, 1 | q, kv]`` (entry_utils.cuh:56-86), "and"-ed with the
+    causal range (mma_utils.cuh:196-199). float32 ``softmax(q k^T / sqrt(D)) v``; a row that
+    sees nothing gives zeros. Returns ``q``'s shape and dtype."""
+    if layout == 1:
+        q, k, v = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
+    b, h, lq, d = q.shape
+    n_rep, lk = h // k.size(1), k.size(2)
+    kf = k.float().repeat_interleave(n_rep, dim=1)
+    vf = v.float().repeat_interleave(n_rep, dim=1)
+    scores = q.float() @ kf.transpose(-1, -2) / (d ** 0.5)             # [B, H, lq, lk]
+    visible = torch.ones(b, h, lq, lk, dtype=torch.bool)
+    if causal_offset >= 0:
+        visible &= (torch.arange(lk)[None, :] <= torch.arange(lq)[:, None] + causal_offset)[None, None]
+    if mask is not None:
+        m = mask
+        if m.dim() == 2:
+            m = m[:, None, None, :]
+        elif m.dim() == 3:
+            m = m[:, None]
+        visible = visible & m
+    scores = scores.masked_fill(~visible, float("-inf"))
+    p = torch.softmax(scores, dim=-1)
+    p = torch.where(visible.any(-1, keepdim=True), p, torch.zeros_like(p))
+    out = (p @ vf).to(q.dtype)
+    return out.transpose(1, 2) if layout == 1 else out
 
 
 def repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:

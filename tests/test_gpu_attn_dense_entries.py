@@ -1,0 +1,185 @@
+"""The reference's dense attention entry points (attn_decode / attn_prefill on q, k, v tensors
+in either layout, boolean is_causal, optional masks) and its rotary_emb entry, through the
+registry and the ops wrappers, against the oracle."""
+
+import pytest
+import torch
+
+from oracle import decoder_oracle as D
+from tests.helpers import assert_bf16_close
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _close(got, want, what):
+    """Prefill bound (probabilities and output rounded to bf16): |y - ref| <= 2e-2 |ref| + four
+    bf16 ulps at rms(ref)."""
+    g, w = got.float().cpu(), want.float().cpu()
+    assert g.shape == w.shape, (g.shape, w.shape)
+    assert torch.isfinite(g).all(), f"{what}: non-finite output"
+    rms = w.pow(2).mean().sqrt().item()
+    err = (g - w).abs()
+    bad = err > 2e-2 * w.abs() + 2.0 ** -6 * rms
+    assert not bad.any(), f"{what}: {int(bad.sum())} of {bad.numel()} outside tolerance; worst {err.max().item():.4g}"
+
+
+def _qkv(b, lq, lk, h, hkv, seed, layout=1):
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda l, n: torch.randn(b, l, n, 128, generator=g).to(torch.bfloat16)
+    q, k, v = mk(lq, h), mk(lk, hkv), mk(lk, hkv)
+    if layout == 0:
+        q, k, v = (t.transpose(1, 2).contiguous() for t in (q, k, v))
+    return q, k, v
+
+
+def test_registry_lists_the_reference_kernel_names():
+    from astrai_amd.extension import KERNEL_NAMES, get_module, is_available
+    for name in ("attn_decode", "attn_prefill", "attn_paged_decode", "attn_paged_prefill", "rotary_emb", "fp8_mm"):
+        assert name in KERNEL_NAMES and is_available(name)
+        assert callable(getattr(get_module(name), name))      # csrc/CMakeLists.txt:55-62: module name = entry name
+
+
+@pytest.mark.parametrize("h,hkv", [(16, 4), (8, 8), (16, 2)])
+@pytest.mark.parametrize("is_causal", [False, True])
+def test_ops_attn_decode_blhd(h, hkv, is_causal):
+    from astrai_amd.extension import ops
+    q, k, v = _qkv(3, 1, 77, h, hkv, seed=h + hkv)
+    got = ops.attn_decode(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=is_causal)
+    assert got.shape == q.shape and got.dtype == torch.bfloat16
+    assert_bf16_close(got, D.attn_dense(q, k, v), what=f"decode {h}/{hkv}")   # one row: causal sees every key
+    g = torch.Generator().manual_seed(3)
+    mask = torch.rand(3, 77, generator=g) < 0.6
+    mask[2] = False                                      # a hidden sequence: zeros
+    for m in (mask, mask[:, None, :]):
+        got = ops.attn_decode(q.to(DEV), k.to(DEV), v.to(DEV), mask=m.to(DEV), is_causal=is_causal)
+        assert_bf16_close(got, D.attn_dense(q, k, v, mask=m), what=f"decode mask {tuple(m.shape)}")
+        assert got[2].abs().sum() == 0
+
+
+@pytest.mark.parametrize("layout", [0, 1])
+def test_registry_attn_decode_layouts_and_offsets(layout):
+    """The pybind-level entry: layout code, causal_offset as a key limit (layout_policies.cuh:
+    138-141), strided inputs."""
+    from astrai_amd.extension import get_module
+    fn = get_module("attn_decode").attn_decode
+    q, k, v = _qkv(2, 1, 130, 8, 2, seed=11, layout=layout)
+    dev = [t.to(DEV) for t in (q, k, v)]
+    for off in (-1, 0, 40, 129, 500):
+        got = fn(*dev, causal_offset=off, layout=layout)
+        assert got.shape == q.shape
+        assert_bf16_close(got, D.attn_dense(q, k, v, causal_offset=off, layout=layout), what=f"layout {layout} offset {off}")
+    mask = torch.rand(2, 130, generator=torch.Generator().manual_seed(1)) < 0.5
+    got = fn(*dev, mask=mask.to(DEV), causal_offset=100, layout=layout)
+    assert_bf16_close(got, D.attn_dense(q, k, v, mask=mask, causal_offset=100, layout=layout), what="mask and offset")
+    # a key tensor that is a window of a longer buffer (non-contiguous)
+    g = torch.Generator().manual_seed(5)
+    shape = (2, 200, 2, 128) if layout == 1 else (2, 2, 200, 128)
+    big_k = torch.randn(shape, generator=g).to(torch.bfloat16)
+    big_v = torch.randn(shape, generator=g).to(torch.bfloat16)
+    win = (slice(None), slice(20, 150)) if layout == 1 else (slice(None), slice(None), slice(20, 150))
+    got = fn(dev[0], big_k.to(DEV)[win], big_v.to(DEV)[win], layout=layout)
+    assert_bf16_close(got, D.attn_dense(q, big_k[win], big_v[win], layout=layout), what="window")
+
+
+@pytest.mark.parametrize("h,hkv,lq,lk", [(8, 2, 70, 70), (16, 4, 33, 150), (4, 2, 128, 128), (16, 2, 5, 64)])
+@pytest.mark.parametrize("is_causal", [False, True])
+def test_ops_attn_prefill_blhd(h, hkv, lq, lk, is_causal):
+    from astrai_amd.extension import ops
+    q, k, v = _qkv(2, lq, lk, h, hkv, seed=lq + lk)
+    off = lk - lq if is_causal else -1
+    got = ops.attn_prefill(q.to(DEV), k.to(DEV), v.to(DEV), is_causal=is_causal)
+    assert got.shape == q.shape and got.dtype == torch.bfloat16
+    _close(got, D.attn_dense(q, k, v, causal_offset=off), f"prefill {h}/{hkv} {lq}x{lk} causal={is_causal}")
+    g = torch.Generator().manual_seed(9)
+    m2 = torch.rand(2, lk, generator=g) < 0.7
+    m3 = torch.rand(2, lq, lk, generator=g) < 0.7
+    m3[1, lq // 2] = False                                # a hidden row: zeros
+    for m in (m2, m3):
+        got = ops.attn_prefill(q.to(DEV), k.to(DEV), v.to(DEV), mask=m.to(DEV), is_causal=is_causal)
+        _close(got, D.attn_dense(q, k, v, mask=m, causal_offset=off), f"prefill mask {tuple(m.shape)}")
+    assert got[1, lq // 2].abs().sum() == 0
+
+
+@pytest.mark.parametrize("layout", [0, 1])
+def test_registry_attn_prefill_layouts_offsets_and_4d_masks(layout):
+    from astrai_amd.extension import get_module
+    fn = get_module("attn_prefill").attn_prefill
+    b, lq, lk, h, hkv = 2, 90, 140, 8, 2
+    q, k, v = _qkv(b, lq, lk, h, hkv, seed=21, layout=layout)
+    dev = [t.to(DEV) for t in (q, k, v)]
+    for off in (-1, lk - lq, 0, 10, 1000):               # aligned to the end, to the start, in between, past everything
+        got = fn(*dev, causal_offset=off, layout=layout)
+        assert got.shape == q.shape
+        _close(got, D.attn_dense(q, k, v, causal_offset=off, layout=layout), f"layout {layout} offset {off}")
+    g = torch.Generator().manual_seed(2)
+    for shape in ((b, 1, 1, lk), (b, h, 1, lk), (b, 1, lq, lk), (b, h, lq, lk)):
+        m = torch.rand(shape, generator=g) < 0.6
+        got = fn(*dev, mask=m.to(DEV), causal_offset=lk - lq, layout=layout)
+        _close(got, D.attn_dense(q, k, v, mask=m, causal_offset=lk - lq, layout=layout), f"4D mask {shape}")
+        got = fn(*dev, mask=m.to(DEV), causal_offset=7, layout=layout)
+        _close(got, D.attn_dense(q, k, v, mask=m, causal_offset=7, layout=layout), f"4D mask {shape}, offset 7")
+
+
+def test_dense_entries_reject_what_the_reference_rejects():
+    from astrai_amd.extension import get_module
+    dec, pre = get_module("attn_decode").attn_decode, get_module("attn_prefill").attn_prefill
+    q, k, v = (t.to(DEV) for t in _qkv(2, 1, 16, 8, 2, seed=1))
+    with pytest.raises(RuntimeError, match="seq_len must be 1"):
+        dec(k[:, :2].repeat(1, 1, 4, 1), k, v, layout=1)
+    with pytest.raises(RuntimeError, match="identical shapes"):
+        dec(q, k, v[:, :8], layout=1)
+    with pytest.raises(RuntimeError, match="4D"):
+        dec(q[0], k, v, layout=1)
+    with pytest.raises(RuntimeError, match="bf16"):
+        dec(q.float(), k, v, layout=1)
+    with pytest.raises(RuntimeError, match="divisible"):
+        dec(q[:, :, :3], k, v, layout=1)
+    with pytest.raises(RuntimeError, match="mask kv_len"):
+        dec(q, k, v, mask=torch.ones(2, 15, dtype=torch.bool, device=DEV), layout=1)
+    with pytest.raises(RuntimeError, match="mask batch"):
+        pre(q, k, v, mask=torch.ones(3, 16, dtype=torch.bool, device=DEV), layout=1)
+    with pytest.raises(RuntimeError, match="mask must be bool"):
+        pre(q, k, v, mask=torch.ones(2, 16, device=DEV), layout=1)
+    with pytest.raises(RuntimeError, match="head_dim 128"):
+        pre(q[..., :64], k[..., :64], v[..., :64], layout=1)
+
+
+@pytest.mark.parametrize("shape", [(37, 16, 128), (2, 19, 4, 128), (5, 3, 64), (4, 2, 6), (1, 1, 2), (0, 4, 128)])
+def test_rotary_emb_equals_the_fp32_tensor_arithmetic(shape):
+    """Bit for bit the reference's torch path (astrai/extension/backend/rotary.py:25-33): complex
+    multiply in fp32, one rounding to bf16. Packed and dense inputs, head_dim with and without
+    16-byte rows, empty input."""
+    from astrai_amd.extension import ops
+    g = torch.Generator().manual_seed(sum(shape))
+    x = (torch.randn(shape, generator=g) * 3).to(torch.bfloat16)
+    ang = torch.rand(*shape[:-2], shape[-1] // 2, generator=g) * 6.28318
+    freqs = torch.stack([torch.cos(ang), torch.sin(ang)], dim=-1)
+    got = ops.rotary_emb(x.to(DEV), freqs.to(DEV))
+    assert got.shape == x.shape and got.dtype == torch.bfloat16
+    if x.numel():
+        assert torch.equal(got.cpu(), D.apply_rotary(x, freqs))
+
+
+def test_rotary_emb_large_and_argument_checks():
+    from astrai_amd.extension import get_module, ops
+    fn = get_module("rotary_emb").rotary_emb
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(4, 512, 16, 128, generator=g).to(torch.bfloat16)
+    table = D.rotary_table(128, 600, 10000.0)
+    pos = torch.randint(0, 600, (4, 512), generator=g)
+    freqs = table[pos]                                    # [4, 512, 64, 2]: each token's own row
+    got = fn(x.to(DEV), freqs.to(DEV))
+    assert torch.equal(got.cpu(), D.apply_rotary(x, freqs))
+    # the wrapper copies non-contiguous inputs; the entry refuses them like the reference's
+    xt = x.transpose(0, 1)                                # [512, 4, 16, 128] view
+    ft = freqs.transpose(0, 1)
+    assert torch.equal(ops.rotary_emb(xt.to(DEV), ft.to(DEV)).cpu(), D.apply_rotary(xt, ft))
+    xd, fd = x.to(DEV), freqs.to(DEV)
+    for args, msg in (((xd.transpose(0, 1), fd), "x must be contiguous"),
+                      ((xd, fd.transpose(0, 1)), "freqs_cis must be contiguous"),
+                      ((xd.float(), fd), "x must be bf16"), ((xd, fd.double()), "freqs_cis must be f32"),
+                      ((xd, fd[0]), "rank"), ((xd, fd[:3]), "mismatch"), ((xd[0, 0], fd[0, 0]), "x must be"),
+                      ((xd.cpu(), fd), "CUDA")):
+        with pytest.raises(RuntimeError, match=msg):
+            fn(*args)

@@ -35,10 +35,10 @@ def _setup(b, h, hkv, lens, max_ctx, pool, seed, n_req=None, holes=False):
     return q, k_pool, v_pool, table, rows, indptr
 
 
-def _run(args, nsplit=0, **kw):
+def _run(args, nsplit=0, mask=None, **kw):
     from astrai_amd.extension import _cabi
     dev = [t.to(DEV) for t in args]
-    return _cabi.attn_paged_decode(*dev, nsplit=nsplit, **kw)
+    return _cabi.attn_paged_decode(*dev, nsplit=nsplit, mask=None if mask is None else mask.to(DEV), **kw)
 
 
 @pytest.mark.parametrize("nsplit", [0, 1, 5])
@@ -121,12 +121,35 @@ def test_paged_decode_equals_dense_kernel_on_the_same_cache():
 def test_paged_decode_rejects_what_it_does_not_do():
     from astrai_amd.extension import _cabi
     q, k_pool, v_pool, table, rows, indptr = [t.to(DEV) for t in _setup(1, 4, 1, [3], 8, 8, seed=2)]
-    with pytest.raises(RuntimeError, match="mask"):
-        _cabi.attn_paged_decode(q, k_pool, v_pool, table, rows, indptr, mask=torch.ones(1, 8, dtype=torch.bool, device=DEV))
+    ok = torch.ones(1, 8, dtype=torch.bool, device=DEV)
+    for bad, msg in ((ok.float(), "bool"), (ok.cpu(), "CUDA"), (ok.expand(2, 8), "batch"), (ok[:, :0], "kv_len")):
+        with pytest.raises(RuntimeError, match=msg):
+            _cabi.attn_paged_decode(q, k_pool, v_pool, table, rows, indptr, mask=bad)
     with pytest.raises(RuntimeError, match="int32"):
         _cabi.attn_paged_decode(q, k_pool, v_pool, table.long(), rows, indptr)
     with pytest.raises(RuntimeError, match="together"):
         _cabi.attn_paged_decode(q, k_pool, v_pool, table, rows, indptr, new_k=q[:, :1])
+
+
+@pytest.mark.parametrize("nsplit", [0, 1, 4])
+def test_paged_decode_with_a_key_mask(nsplit):
+    """The reference's optional mask [batch, positions], True = attend, indexed by sequence
+    (not by table row) and position (csrc/kernels/attention/entry_utils.cuh:226-237)."""
+    lens = [300, 1, 17, 64, 0, 33]
+    args = _setup(6, 16, 4, lens, 320, sum(lens) + 20, seed=12, holes=True)
+    g = torch.Generator().manual_seed(5)
+    mask = torch.rand(6, 320, generator=g) < 0.6
+    mask[3, :64] = False                      # a sequence with every position hidden: zeros
+    mask[0, 100:260] = False                  # whole tiles (and whole splits) hidden
+    got = _run(args, nsplit, mask=mask)
+    assert_bf16_close(got, D.attn_paged_decode(*args, mask=mask), what=f"masked nsplit={nsplit}")
+    assert got[3].abs().sum() == 0 and got[4].abs().sum() == 0
+    # a mask narrower than the sequences (strided view): the positions past it are hidden
+    narrow = torch.ones(6, 640, dtype=torch.bool)[:, 5:205]
+    assert narrow.stride(0) == 640
+    assert_bf16_close(_run(args, nsplit, mask=narrow), D.attn_paged_decode(*args, mask=narrow), what="narrow mask")
+    # an all-True mask is the unmasked kernel, bit for bit
+    assert torch.equal(_run(args, nsplit, mask=torch.ones(6, 320, dtype=torch.bool)), _run(args, nsplit))
 
 
 def test_paged_decode_random_sweep():
@@ -142,3 +165,7 @@ def test_paged_decode_random_sweep():
         print(f"case {i}: h={hkv * n_rep}/{hkv} lens={lens} nsplit={nsplit}", flush=True)
         args = _setup(b, hkv * n_rep, hkv, lens, max(lens) + 2, sum(lens) + 9, seed=300 + i, holes=bool(i % 2))
         assert_bf16_close(_run(args, nsplit), D.attn_paged_decode(*args), what=f"sweep {i}")
+        if i % 3 == 0:
+            mask = torch.rand(b, max(lens) + 2, generator=g) < 0.5
+            assert_bf16_close(_run(args, nsplit, mask=mask), D.attn_paged_decode(*args, mask=mask),
+                              what=f"sweep {i} with a mask")

@@ -45,12 +45,13 @@ def _setup(h, hkv, kv_lens, q_lens, max_ctx, pool, seed, holes=False):
     return q, k_pool, v_pool, table, rows, kvp
 
 
-def _run(args, q_lens, causal=True):
+def _run(args, q_lens, causal=True, mask=None):
     from astrai_amd.extension import _cabi
     qo, tb, ti = _cabi.paged_prefill_schedule(q_lens, DEV)
     dev = [t.to(DEV) for t in args]
-    got = _cabi.attn_paged_prefill(*dev, qo, tb, ti, causal_offset=0 if causal else -1)
-    want = D.attn_paged_prefill(*args, qo.cpu(), causal=causal)
+    got = _cabi.attn_paged_prefill(*dev, qo, tb, ti, causal_offset=0 if causal else -1,
+                                   mask=None if mask is None else mask.to(DEV))
+    want = D.attn_paged_prefill(*args, qo.cpu(), causal=causal, mask=mask)
     return got, want
 
 
@@ -111,10 +112,63 @@ def test_paged_prefill_rejects_what_it_does_not_do():
     from astrai_amd.extension import _cabi
     args = [t.to(DEV) for t in _setup(4, 1, [3], [3], 8, 8, seed=2)]
     qo, tb, ti = _cabi.paged_prefill_schedule([3], DEV)
-    with pytest.raises(RuntimeError, match="mask"):
-        _cabi.attn_paged_prefill(*args, qo, tb, ti, mask=torch.ones(1, 1, 3, 3, dtype=torch.bool, device=DEV))
     with pytest.raises(RuntimeError, match="int32"):
         _cabi.attn_paged_prefill(*args, qo.long(), tb, ti)
+    # the reference's mask checks (csrc/kernels/attention/entry_utils.cuh:326-346)
+    ok = torch.ones(1, 1, 3, 3, dtype=torch.bool, device=DEV)
+    for bad, msg in ((ok.float(), "bool"), (ok.cpu(), "CUDA"), (ok[0], "2D or 4D"),
+                     (ok.expand(2, 1, 3, 3), "batch"), (ok.expand(1, 3, 3, 3), "head"),
+                     (ok[:, :, :0], "q_len"), (ok[..., :0], "kv_len")):
+        with pytest.raises(RuntimeError, match=msg):
+            _cabi.attn_paged_prefill(*args, qo, tb, ti, mask=bad)
+
+
+def _random_mask(shape, seed, keep=0.7):
+    g = torch.Generator().manual_seed(seed)
+    return torch.rand(shape, generator=g) < keep
+
+
+@pytest.mark.parametrize("kind", ["2d", "4d_rows", "4d_heads", "4d_one_row"])
+@pytest.mark.parametrize("causal", [True, False])
+def test_paged_prefill_with_a_mask_tensor(kind, causal):
+    """The reference's optional mask: [batch, kv] or [batch, 1 | H, rows, kv], True = attend,
+    rows counted inside each sequence, 'and'-ed with the causal range."""
+    h, hkv = 8, 2
+    kv_lens, q_lens = [150, 70, 40], [150, 30, 40]
+    width = max(kv_lens) + 5
+    args = _setup(h, hkv, kv_lens, q_lens, width, sum(kv_lens) + 11, seed=17, holes=True)
+    shape = {"2d": (3, width), "4d_rows": (3, 1, max(q_lens), width),
+             "4d_heads": (3, h, max(q_lens), width), "4d_one_row": (3, h, 1, width)}[kind]
+    mask = _random_mask(shape, seed=len(kind))
+    if mask.dim() == 4 and mask.size(2) > 1:
+        mask[1, :, 3] = False            # a row that sees nothing: zeros
+        mask[0, :, :, :64] = False       # sequence 0: the whole first key block hidden from every row
+    print(f"case {kind} causal={causal}", flush=True)
+    got, want = _run(args, q_lens, causal=causal, mask=mask)
+    _close(got, want, f"mask {kind} causal={causal}")
+    if mask.dim() == 4 and mask.size(2) > 1:
+        assert got[150 + 3].abs().sum() == 0
+
+
+def test_paged_prefill_mask_smaller_than_the_sequences_and_strided():
+    """Rows and positions that the mask does not hold are not attended; the mask may be a
+    strided view (only its innermost stride has to be 1) or a batch broadcast."""
+    h, hkv = 4, 2
+    kv_lens, q_lens = [100, 90], [60, 90]
+    args = _setup(h, hkv, kv_lens, q_lens, 128, 220, seed=23)
+    big = _random_mask((2, 1, 80, 256), seed=5, keep=0.8)
+    mask = big[:, :, :, 10:90]                 # 80 rows, 80 positions, row stride 256
+    got, want = _run(args, q_lens, causal=True, mask=mask)
+    _close(got, want, "narrow strided mask")
+    assert got[60 + 80:].abs().sum() == 0      # rows 80.. of sequence 1: no row in the mask
+    one = _random_mask((1, 128), seed=6).expand(2, 128)    # batch stride 0
+    got, want = _run(args, q_lens, causal=False, mask=one)
+    _close(got, want, "batch-broadcast mask")
+    # an all-True mask is the unmasked kernel's result
+    full = torch.ones(2, 128, dtype=torch.bool)
+    got, _ = _run(args, q_lens, causal=True, mask=full)
+    plain, _ = _run(args, q_lens, causal=True)
+    _close(got, plain, "all-True mask")
 
 
 def test_paged_prefill_random_sweep():
@@ -134,3 +188,8 @@ def test_paged_prefill_random_sweep():
                       seed=500 + i, holes=(i % 4 == 3))
         got, want = _run(args, q_lens, causal=causal)
         _close(got, want, f"sweep {i}")
+        if i % 2:
+            shape = [(b, max(kv_lens) + 3), (b, 1, max(q_lens), max(kv_lens) + 3),
+                     (b, hkv * n_rep, max(q_lens), max(kv_lens))][(i // 2) % 3]
+            got, want = _run(args, q_lens, causal=causal, mask=_random_mask(shape, seed=900 + i, keep=0.5))
+            _close(got, want, f"sweep {i} with a mask {shape}")

@@ -241,3 +241,106 @@ def test_paged_oracles_read_a_negative_slot_as_a_zero_key_and_value():
         assert torch.equal(a, b), causal
     # row 0 of the second sequence sees positions 0..2, all real except the hole at 0
     assert a.abs().sum() > 0
+
+
+def test_paged_oracles_mask_hides_positions_like_removing_them():
+    """The reference's optional mask (csrc/kernels/attention/entry_utils.cuh:226-237,326-346;
+    mma_utils.cuh:190-199) is indexed by sequence (not by the row of req_to_token), query row
+    inside the sequence and position, True = attend, and is combined with the causal range by
+    "and". Pinned by what softmax attention fixes: hiding a position equals a sequence that
+    never held it; an all-True mask changes nothing; the lower triangle as a mask equals the
+    causal flag; a 2D mask equals its 4D broadcast; hiding everything gives zeros."""
+    g = torch.Generator().manual_seed(33)
+    h, hkv, d, pool = 4, 2, 16, 64
+    k_pool = torch.randn(pool, hkv, d, generator=g).to(torch.bfloat16)
+    v_pool = torch.randn(pool, hkv, d, generator=g).to(torch.bfloat16)
+    lens = [9, 6]
+    rows = torch.tensor([2, 0], dtype=torch.int32)          # sequence 0 lives in table row 2
+    table = torch.full((3, 12), -1, dtype=torch.int32)
+    table[2, :9] = torch.arange(30, 39, dtype=torch.int32)
+    table[0, :6] = torch.arange(10, 16, dtype=torch.int32)
+    indptr = torch.tensor([0, 9, 15], dtype=torch.int32)
+    q1 = torch.randn(2, h, d, generator=g).to(torch.bfloat16)
+    plain = D.attn_paged_decode(q1, k_pool, v_pool, table, rows, indptr)
+    assert torch.equal(D.attn_paged_decode(q1, k_pool, v_pool, table, rows, indptr,
+                                           mask=torch.ones(2, 12, dtype=torch.bool)), plain)
+    # hide positions 2 and 7 of sequence 0 and position 0 of sequence 1
+    mask = torch.ones(2, 12, dtype=torch.bool)
+    mask[0, 2] = mask[0, 7] = mask[1, 0] = False
+    got = D.attn_paged_decode(q1, k_pool, v_pool, table, rows, indptr, mask=mask)
+    cut = torch.full((3, 12), -1, dtype=torch.int32)
+    cut[2, :7] = torch.tensor([30, 31, 33, 34, 35, 36, 38], dtype=torch.int32)
+    cut[0, :5] = torch.arange(11, 16, dtype=torch.int32)
+    want = D.attn_paged_decode(q1, k_pool, v_pool, cut, rows, torch.tensor([0, 7, 12], dtype=torch.int32))
+    assert (got.float() - want.float()).abs().max() < 2e-2 and not torch.equal(got, plain)
+    # a mask narrower than a sequence hides the rest; hiding everything gives zeros
+    narrow = D.attn_paged_decode(q1, k_pool, v_pool, table, rows, indptr, mask=torch.ones(2, 4, dtype=torch.bool))
+    first4 = D.attn_paged_decode(q1, k_pool, v_pool, table, rows, torch.tensor([0, 4, 8], dtype=torch.int32))
+    assert torch.equal(narrow, first4)
+    none = mask.clone(); none[1] = False
+    assert D.attn_paged_decode(q1, k_pool, v_pool, table, rows, indptr, mask=none)[1].abs().sum() == 0
+
+    # prefill: whole prompts (q_len == kv_len)
+    qo = torch.tensor([0, 9, 15], dtype=torch.int32)
+    qp = torch.randn(15, h, d, generator=g).to(torch.bfloat16)
+    causal = D.attn_paged_prefill(qp, k_pool, v_pool, table, rows, indptr, qo, causal=True)
+    tri = torch.tril(torch.ones(9, 12, dtype=torch.bool))[None, None].expand(2, 1, 9, 12)
+    as_mask = D.attn_paged_prefill(qp, k_pool, v_pool, table, rows, indptr, qo, causal=False, mask=tri)
+    assert torch.equal(as_mask, causal)
+    both = D.attn_paged_prefill(qp, k_pool, v_pool, table, rows, indptr, qo, causal=True, mask=tri)
+    assert torch.equal(both, causal)
+    m2 = mask
+    m4 = mask[:, None, None, :]
+    a = D.attn_paged_prefill(qp, k_pool, v_pool, table, rows, indptr, qo, causal=True, mask=m2)
+    b = D.attn_paged_prefill(qp, k_pool, v_pool, table, rows, indptr, qo, causal=True, mask=m4)
+    c = D.attn_paged_prefill(qp, k_pool, v_pool, table, rows, indptr, qo, causal=True,
+                             mask=m4.expand(2, h, 9, 12))
+    assert torch.equal(a, b) and torch.equal(a, c) and not torch.equal(a, causal)
+    # row 0 of sequence 1 sees only position 0, which the mask hides: zeros
+    assert a[9].abs().sum() == 0 and a[10].abs().sum() > 0
+    # a per-head mask: head 1 of sequence 0 loses position 0, the other heads keep it
+    per_head = torch.ones(2, h, 9, 12, dtype=torch.bool)
+    per_head[0, 1, :, 0] = False
+    e = D.attn_paged_prefill(qp, k_pool, v_pool, table, rows, indptr, qo, causal=True, mask=per_head)
+    assert torch.equal(e[:, [0, 2, 3]], causal[:, [0, 2, 3]]) and torch.equal(e[9:], causal[9:])
+    assert e[0, 1].abs().sum() == 0 and not torch.equal(e[1:9, 1], causal[1:9, 1])
+
+
+def test_attn_dense_oracle_against_sdpa_and_the_paged_oracle():
+    """The dense-entry oracle, pinned on the CPU by a library routine (torch's scaled-dot-product
+    attention in float32: causal flag, boolean mask, grouped heads expanded by hand) and by the
+    paged oracle on the same keys addressed through an identity table."""
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(8)
+    b, h, hkv, lq, lk, d = 2, 4, 2, 5, 9, 16
+    q = torch.randn(b, lq, h, d, generator=g)
+    k = torch.randn(b, lk, hkv, d, generator=g)
+    v = torch.randn(b, lk, hkv, d, generator=g)
+    kx, vx = k.repeat_interleave(2, dim=2), v.repeat_interleave(2, dim=2)
+    sd = lambda **kw: F.scaled_dot_product_attention(q.transpose(1, 2), kx.transpose(1, 2), vx.transpose(1, 2), **kw).transpose(1, 2)
+    assert torch.allclose(D.attn_dense(q, k, v), sd(), atol=1e-5)
+    # bottom-right aligned causal range = offset kv_len - q_len
+    band = torch.arange(lk)[None, :] <= torch.arange(lq)[:, None] + (lk - lq)
+    assert torch.allclose(D.attn_dense(q, k, v, causal_offset=lk - lq), sd(attn_mask=band), atol=1e-5)
+    # top-left aligned (offset 0) is SDPA's is_causal
+    assert torch.allclose(D.attn_dense(q, k, v, causal_offset=0), sd(is_causal=True), atol=1e-5)
+    m3 = torch.rand(b, lq, lk, generator=g) < 0.7
+    m3[..., 0] = True
+    assert torch.allclose(D.attn_dense(q, k, v, mask=m3), sd(attn_mask=m3[:, None]), atol=1e-5)
+    m2 = m3[:, 0]
+    assert torch.allclose(D.attn_dense(q, k, v, mask=m2, causal_offset=lk - lq),
+                          sd(attn_mask=m2[:, None, None, :] & band), atol=1e-5)
+    # layout 0 is the same numbers transposed
+    a0 = D.attn_dense(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), mask=m3, layout=0)
+    assert torch.equal(a0.transpose(1, 2), D.attn_dense(q, k, v, mask=m3))
+    # the paged oracle over an identity table
+    table = torch.arange(b * lk, dtype=torch.int32).reshape(b, lk)
+    rows = torch.arange(b, dtype=torch.int32)
+    kvp = (torch.arange(b + 1) * lk).int()
+    qo = (torch.arange(b + 1) * lq).int()
+    paged = D.attn_paged_prefill(q.reshape(b * lq, h, d), k.reshape(b * lk, hkv, d), v.reshape(b * lk, hkv, d),
+                                 table, rows, kvp, qo, causal=True, mask=m3[:, None])
+    assert torch.allclose(paged.reshape(b, lq, h, d), D.attn_dense(q, k, v, mask=m3, causal_offset=lk - lq), atol=1e-6)
+    # a hidden row gives zeros, not NaN
+    none = m3.clone(); none[1, 2] = False
+    assert D.attn_dense(q, k, v, mask=none)[1, 2].abs().sum() == 0
