@@ -293,7 +293,12 @@ __global__ __launch_bounds__(64 * NREP, NREP >= 4 ? 2 : 1) void attn_prefill_ker
             if (PARTIAL) {
                 const int key = T * 32 + g * 8 + h * 4 + j;
                 bool visible = key <= pq;
-                if constexpr (MASK) visible = visible && key < mask_keys && mask_row[key] != 0;
+                if constexpr (MASK) {
+                    // (the byte is fetched whether or not it is needed, from a clamped index:
+                    // four independent loads per group instead of four dependent branches)
+                    const uint8_t keep = mask_row[max(min(key, mask_keys - 1), 0)];
+                    visible = visible && key < mask_keys && keep != 0;
+                }
                 s[e] = visible ? s[e] : kNegBig;
             }
             m = fmaxf(m, s[e]);
