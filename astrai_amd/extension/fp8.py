@@ -220,6 +220,10 @@ class FP8State:
             meta = self._metas[key] = FP8TensorMeta(w.device, self.recipe)
         return meta
 
+    def peek_weight_meta(self, w: torch.Tensor) -> Optional[FP8TensorMeta]:
+        """The scaling state of ``w`` if it has any; never creates one."""
+        return self._metas.get((w.data_ptr(), w.shape, w.dtype))
+
     def dynamic_weight(self, w: torch.Tensor, fmt: str):
         """``(sw, w8)`` of dynamic scaling, reused while ``w`` is unmodified."""
         key = (w.data_ptr(), w.shape, fmt, self.recipe.margin)

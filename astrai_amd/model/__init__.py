@@ -11,7 +11,8 @@ from astrai_amd.model.decoder import (
     unfuse_int8_weights,
 )
 
-from astrai_amd.model.checkpoint import load_int8_checkpoint, save_int8_checkpoint
+from astrai_amd.model.checkpoint import (load_fp8_scaling, load_int8_checkpoint, save_fp8_scaling,
+                                         save_int8_checkpoint)
 
-__all__ = ["load_int8_checkpoint", "save_int8_checkpoint", "AutoRegressiveLM", "AutoRegressiveLMConfig", "DenseKVCache", "greedy_generate",
+__all__ = ["load_fp8_scaling", "save_fp8_scaling", "load_int8_checkpoint", "save_int8_checkpoint", "AutoRegressiveLM", "AutoRegressiveLMConfig", "DenseKVCache", "greedy_generate",
            "fuse_int8_weights", "unfuse_int8_weights"]

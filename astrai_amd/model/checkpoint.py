@@ -105,3 +105,81 @@ def load_int8_checkpoint(save_dir: str, device="cuda", fuse: bool = True) -> Aut
     if fuse:
         fuse_int8_weights(model)  # concatenates what the cache holds: the stored integers
     return model
+
+
+# ---------------------------------------------------------------------------
+# fp8 delayed scaling: the amax histories and steps of every Linear weight, so that a
+# resumed run quantizes its next step with the steps the interrupted run had reached
+# (the reference keeps them in process memory only, keyed by the weight's address:
+# astrai/extension/fp8.py:111-213; its Checkpoint has no slot for them).
+# ---------------------------------------------------------------------------
+
+_FP8_FILE = "fp8_scaling.safetensors"
+_RINGS = ("w", "x", "g")
+
+
+@torch.no_grad()
+def save_fp8_scaling(model: torch.nn.Module, save_dir: str) -> int:
+    """Write ``fp8_scaling.safetensors`` into ``save_dir`` and record the recipe in
+    ``meta.json`` (created, or extended if it exists). Per parameter ``<name>`` that has
+    scaling state: ``<name>.fp8_{w,x,g}_hist`` fp32 ``[history_len]``, ``<name>.fp8_{w,x,g}_scale``
+    fp32 ``[1]``, ``<name>.fp8_cursor`` int64 ``[3]`` (next slot of each ring) and
+    ``<name>.fp8_seeded`` int64 ``[3]``. Returns the number of parameters written."""
+    from astrai_amd.extension.fp8 import fp8_state
+
+    state = fp8_state()
+    path = Path(save_dir)
+    path.mkdir(parents=True, exist_ok=True)
+    tensors: Dict[str, torch.Tensor] = {}
+    count = 0
+    for name, p in model.named_parameters():
+        meta = state.peek_weight_meta(p)
+        if meta is None:
+            continue
+        count += 1
+        for r in _RINGS:
+            tensors[f"{name}.fp8_{r}_hist"] = getattr(meta, f"{r}_hist").detach().float().cpu().contiguous()
+            tensors[f"{name}.fp8_{r}_scale"] = getattr(meta, f"{r}_scale").detach().float().cpu().contiguous()
+        tensors[f"{name}.fp8_cursor"] = torch.tensor([getattr(meta, f"{r}_idx") for r in _RINGS], dtype=torch.int64)
+        tensors[f"{name}.fp8_seeded"] = torch.tensor([int(getattr(meta, f"{r}_init")) for r in _RINGS], dtype=torch.int64)
+    st.save_file(tensors, str(path / _FP8_FILE))
+    meta_path = path / _META_FILE
+    meta = json.loads(meta_path.read_text()) if meta_path.exists() else {}
+    meta["fp8_scaling"] = {"recipe": type(state.recipe).__name__, "history_len": state.recipe.history_len,
+                           "margin": state.recipe.margin, "fp8_format": state.fp8_format.value,
+                           "parameters": count}
+    meta_path.write_text(json.dumps(meta, indent=2))
+    return count
+
+
+@torch.no_grad()
+def load_fp8_scaling(model: torch.nn.Module, save_dir: str) -> int:
+    """Restore what :func:`save_fp8_scaling` wrote into the process's fp8 state, for the
+    parameters of ``model`` (on whatever device they live), under the recipe that is active
+    now. A history of another length is refused: its steps would not be the saved run's.
+    Returns the number of parameters restored."""
+    from astrai_amd.extension.fp8 import fp8_state
+
+    state = fp8_state()
+    path = Path(save_dir)
+    tensors = st.load_file(str(path / _FP8_FILE))  # safetensors: data only, nothing executed
+    count = 0
+    for name, p in model.named_parameters():
+        if f"{name}.fp8_cursor" not in tensors:
+            continue
+        hist_len = tensors[f"{name}.fp8_w_hist"].numel()
+        if hist_len != state.recipe.history_len:
+            raise ValueError(f"{name}: saved amax history has {hist_len} slots, the active recipe "
+                             f"{state.recipe.history_len}")
+        meta = state.get_weight_meta(p)
+        cursor = tensors[f"{name}.fp8_cursor"].tolist()
+        seeded = tensors[f"{name}.fp8_seeded"].tolist()
+        for i, r in enumerate(_RINGS):
+            getattr(meta, f"{r}_hist").copy_(tensors[f"{name}.fp8_{r}_hist"])
+            getattr(meta, f"{r}_scale").copy_(tensors[f"{name}.fp8_{r}_scale"])
+            setattr(meta, f"{r}_idx", int(cursor[i]) % hist_len)
+            setattr(meta, f"{r}_init", bool(seeded[i]))
+        meta.w_cached = None
+        count += 1
+    return count
+

@@ -140,3 +140,65 @@ def test_int8_autocast_restores():
             assert not w8a8.int8_linear_enabled()
         assert w8a8.int8_linear_enabled()
     assert not w8a8.int8_linear_enabled()
+
+
+def test_fp8_scaling_state_survives_a_checkpoint(tmp_path):
+    """Delayed scaling resumed from ``save_fp8_scaling`` continues exactly where the saved run
+    stood: same histories, cursors, steps, and the same steps after further updates as a run
+    that was never interrupted."""
+    import json
+    from astrai_amd.model.checkpoint import load_fp8_scaling, save_fp8_scaling
+
+    def feed(model, amaxes):
+        st = fp8_state()
+        for p, vals in zip(model.parameters(), amaxes):
+            meta = st.get_weight_meta(p)
+            if not meta.w_init:
+                meta.init_w(p, "e4m3")
+            for a in vals:
+                meta.update_x(torch.tensor([a]), "e4m3")
+                meta.update_g(torch.tensor([a * 0.01]), "e5m2")
+                meta.update_w(torch.tensor([a * 0.5]), "e4m3")
+
+    def snapshot(model):
+        st = fp8_state()
+        out = []
+        for p in model.parameters():
+            m = st.peek_weight_meta(p)
+            out.append(None if m is None else
+                       [t.clone() for t in (m.w_hist, m.x_hist, m.g_hist, m.w_scale, m.x_scale, m.g_scale)]
+                       + [m.w_idx, m.x_idx, m.g_idx, m.w_init])
+        return out
+
+    def same(a, b):
+        return all((x is None and y is None) or all(torch.equal(u, v) if torch.is_tensor(u) else u == v
+                                                    for u, v in zip(x, y)) for x, y in zip(a, b))
+
+    torch.manual_seed(0)
+    model = torch.nn.Sequential(torch.nn.Linear(8, 4, bias=False), torch.nn.Linear(4, 2, bias=False))
+    first = [[3.0, 7.0, 2.0, 9.0, 1.0], [0.5, 0.25]]
+    later = [[4.0, 4.0, 30.0], [0.125, 2.0, 1.0, 1.0, 1.0]]
+    st = fp8_state()
+    st.reset()
+    try:
+        with fp8_autocast(update_interval=4, margin=1):
+            feed(model, first)
+            before = snapshot(model)
+            assert save_fp8_scaling(model, str(tmp_path)) == 2
+            feed(model, later)
+            uninterrupted = snapshot(model)
+            # a fresh process: no state; the weights are the same tensors of a re-built model
+            st._metas.clear()
+            assert all(s is None for s in snapshot(model))
+            assert load_fp8_scaling(model, str(tmp_path)) == 2
+            assert same(snapshot(model), before)
+            feed(model, later)
+            assert same(snapshot(model), uninterrupted)
+        info = json.loads((tmp_path / "meta.json").read_text())["fp8_scaling"]
+        assert info == {"recipe": "DelayedScaling", "history_len": 4, "margin": 1, "fp8_format": "hybrid",
+                        "parameters": 2}
+        with fp8_autocast(update_interval=8):
+            with pytest.raises(ValueError, match="slots"):
+                load_fp8_scaling(model, str(tmp_path))
+    finally:
+        st.reset()
