@@ -387,6 +387,64 @@ int astrai_w8a8_attn_paged_prefill_masked_bf16(
     return check_launch("attn_paged_prefill_bf16");
 }
 
+int64_t astrai_w8a8_attn_paged_rows_workspace_floats(int64_t batch_or_tiles, int64_t n_heads,
+                                                     int64_t n_kv_heads, int64_t head_dim,
+                                                     int64_t nsplit, int prefill) {
+    if (batch_or_tiles <= 0 || nsplit <= 0 || nsplit > 64 || n_heads <= 0 || n_kv_heads <= 0 ||
+        n_heads > 65535 || !w8a8::attn_rows_supported((int)n_heads, (int)n_kv_heads, (int)head_dim))
+        return 0;
+    return w8a8::attn_rows_workspace_floats(batch_or_tiles, (int)n_heads, (int)n_kv_heads, (int)head_dim,
+                                            (int)nsplit, prefill != 0);
+}
+
+int astrai_w8a8_attn_paged_rows_bf16(
+    const void* q, const void* k_pool, const void* v_pool, const int32_t* req_to_token,
+    const int32_t* req_pool_indices, const int32_t* kv_indptr, const int32_t* qo_indptr,
+    const int32_t* q_tile_to_batch, const int32_t* q_tile_to_index, const uint8_t* mask,
+    int64_t mask_seq_stride, int64_t mask_head_stride, int64_t mask_row_stride, int64_t mask_rows,
+    int64_t mask_width, float* workspace, int64_t workspace_floats, void* out, int64_t batch_or_tiles,
+    int64_t n_heads, int64_t n_kv_heads, int64_t head_dim, int64_t num_slots, int64_t num_requests,
+    int64_t max_context_len, int causal, int64_t nsplit, float scale, void* stream) {
+    if (!q || !k_pool || !v_pool || !req_to_token || !req_pool_indices || !kv_indptr || !workspace || !out)
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_rows_bf16: null pointer");
+    const bool prefill = qo_indptr != nullptr;
+    if (prefill && (!q_tile_to_batch || !q_tile_to_index))
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_rows_bf16: a prefill call needs the tile schedule");
+    if (batch_or_tiles < 0 || n_heads <= 0 || n_kv_heads <= 0 || n_heads > 65535 || num_slots <= 0 ||
+        num_requests <= 0 || max_context_len <= 0 || nsplit <= 0 || nsplit > 64 || n_heads % n_kv_heads ||
+        num_slots > INT32_MAX || max_context_len > INT32_MAX || batch_or_tiles > (1 << 24))
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_rows_bf16: bad dims");
+    if (!w8a8::attn_rows_supported((int)n_heads, (int)n_kv_heads, (int)head_dim))
+        return fail(ASTRAI_W8A8_UNSUPPORTED,
+                    "attn_paged_rows_bf16: needs head_dim in {32, 64, 128, 256} and n_heads / n_kv_heads <= 8");
+    if (mask && (mask_width <= 0 || mask_rows <= 0 || mask_width > INT32_MAX || mask_rows > INT32_MAX ||
+                 mask_seq_stride < 0 || mask_head_stride < 0 || mask_row_stride < 0))
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_rows_bf16: bad mask dims");
+    if (!(scale > 0.0f)) return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_rows_bf16: scale must be positive");
+    if (!aligned16(q) || !aligned16(k_pool) || !aligned16(v_pool) || !aligned16(out))
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_rows_bf16: pointers must be 16-byte aligned");
+    if (batch_or_tiles == 0) return ASTRAI_W8A8_OK;
+    const int64_t need = w8a8::attn_rows_workspace_floats(batch_or_tiles, (int)n_heads, (int)n_kv_heads,
+                                                          (int)head_dim, (int)nsplit, prefill);
+    if (workspace_floats < need)
+        return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_rows_bf16: workspace too small (%lld floats needed)",
+                    (long long)need);
+    w8a8::AttnRowsArgs a{};
+    a.q = q; a.k_cache = k_pool; a.v_cache = v_pool; a.req_to_token = req_to_token;
+    a.req_pool_indices = req_pool_indices; a.kv_indptr = kv_indptr; a.qo_indptr = qo_indptr;
+    a.q_tile_to_batch = q_tile_to_batch; a.q_tile_to_index = q_tile_to_index;
+    a.ws = workspace; a.out = out; a.num_blocks = batch_or_tiles;
+    a.n_heads = (int)n_heads; a.n_kv_heads = (int)n_kv_heads; a.head_dim = (int)head_dim; a.nsplit = (int)nsplit;
+    a.causal = (prefill && causal) ? 1 : 0;
+    a.scale = scale;
+    a.rtt_stride = max_context_len; a.num_slots = num_slots; a.num_requests = num_requests;
+    a.mask = mask; a.mask_b_stride = mask_seq_stride; a.mask_h_stride = mask_head_stride;
+    a.mask_l_stride = mask_row_stride; a.mask_rows = (int)mask_rows; a.mask_width = (int)mask_width;
+    if (!w8a8::launch_attn_rows(a, static_cast<hipStream_t>(stream)))
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "attn_paged_rows_bf16: shape not supported");
+    return check_launch("attn_paged_rows_bf16");
+}
+
 int astrai_w8a8_quantize_bf16_fp8_block128_act(const void* x, void* x8, float* sa, int64_t m,
                                                int64_t k, void* stream) {
     if (!x || !x8 || !sa) return fail(ASTRAI_W8A8_BAD_ARG, "quantize_block128_act: null pointer");

@@ -151,6 +151,37 @@ struct AttnPrefillArgs {
 bool attn_prefill_supported(int n_heads, int n_kv_heads, int head_dim);
 bool launch_attn_prefill(const AttnPrefillArgs& a, hipStream_t stream);
 
+// attn_rows.hip: paged attention for every head_dim in {32, 64, 128, 256} and every
+// n_heads / n_kv_heads <= 8; decode (qo_indptr == null: sequence b owns packed row b) and
+// ragged prefill (row ranges and the 64-row tile schedule, as for attn_prefill's paged mode)
+struct AttnRowsArgs {
+    const void* q;                // bf16 [total_q, n_heads, head_dim]
+    const void* k_cache;          // bf16 [num_slots, n_kv_heads, head_dim]
+    const void* v_cache;          // same
+    const int* req_to_token;      // int32 [num_requests, rtt_stride]
+    const int* req_pool_indices;  // int32 [batch]
+    const int* kv_indptr;         // int32 [batch + 1]
+    const int* qo_indptr;         // int32 [batch + 1], or null for decode
+    const int* q_tile_to_batch;   // int32 [num_blocks] (prefill)
+    const int* q_tile_to_index;   // int32 [num_blocks] (prefill)
+    float* ws;                    // attn_rows_workspace_floats(...) floats
+    void* out;                    // bf16 [total_q, n_heads, head_dim]
+    int64_t num_blocks;           // decode: batch; prefill: 64-row tiles of the schedule
+    int n_heads, n_kv_heads, head_dim, nsplit;
+    int causal;                   // prefill: row i of a sequence sees keys 0 .. kv_len - q_len + i
+    float scale;
+    int64_t rtt_stride, num_slots, num_requests;
+    // optional bool mask, addressed as for AttnPrefillArgs (decode: row 0 of every sequence)
+    const uint8_t* mask;
+    int64_t mask_b_stride, mask_h_stride, mask_l_stride;
+    int mask_rows, mask_width;
+    int rows_per_block, blocks_per_tile;  // filled in by the launcher
+};
+bool attn_rows_supported(int n_heads, int n_kv_heads, int head_dim);
+int64_t attn_rows_workspace_floats(int64_t batch_or_tiles, int n_heads, int n_kv_heads, int head_dim,
+                                   int nsplit, bool prefill);
+bool launch_attn_rows(AttnRowsArgs a, hipStream_t stream);
+
 // gemm_int8.hip / gemm_fp8.hip / gemm_fp8_block.hip: tiled MFMA kernels.
 // Require k % 16 == 0 and m*k, n*k < 2^31 bytes; return false if the shape is
 // not accepted (the caller then uses the generic kernel).

@@ -50,6 +50,10 @@ PROTOTYPES = {
         [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _INT,
          ctypes.c_float, _P], _INT),
     "astrai_w8a8_rotary_emb_bf16": ([_P, _P, _P, _I64, _I64, _I64, _P], _INT),
+    "astrai_w8a8_attn_paged_rows_workspace_floats": ([_I64, _I64, _I64, _I64, _I64, _INT], _I64),
+    "astrai_w8a8_attn_paged_rows_bf16": (
+        [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _P, _I64, _P, _I64, _I64,
+         _I64, _I64, _I64, _I64, _I64, _INT, _I64, ctypes.c_float, _P], _INT),
     "astrai_w8a8_attn_paged_decode_masked_bf16": (
         [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
          _I64, ctypes.c_float, _P], _INT),
@@ -708,14 +712,37 @@ def attn_paged_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
             out = out_buf[:b]
         else:
             out = torch.empty((b, h, d), device=q.device, dtype=torch.bfloat16)
+        m_ptr, m_stride, m_width = (mask.data_ptr(), mask.stride(0), mask.size(1)) if mask is not None else (0, 0, 0)
+        if d != 128 or h > 64:  # the shapes only the general kernel takes
+            _paged_rows(lib, q_c, k_cache, v_cache, rtt, rpi, ind, None, (m_ptr, m_stride, 0, 0, 1, m_width),
+                        out, b, nsplit, False, scale)
+            return out
         need = lib.astrai_w8a8_attn_decode_workspace_floats(b, hkv, nsplit, h // hkv)
         ws = torch.empty(max(need, 1), device=q.device, dtype=torch.float32)
-        m_ptr, m_stride, m_width = (mask.data_ptr(), mask.stride(0), mask.size(1)) if mask is not None else (0, 0, 0)
         _check(lib.astrai_w8a8_attn_paged_decode_masked_bf16(
             q_c.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), rtt.data_ptr(), rpi.data_ptr(),
             ind.data_ptr(), m_ptr, m_stride, m_width, ws.data_ptr(), ws.numel(), out.data_ptr(), b, h, hkv,
             d, slots, rtt.size(0), rtt.size(1), nsplit, float(scale), _stream(q)), lib)
     return out
+
+
+def _paged_rows(lib, q, k_pool, v_pool, rtt, rpi, kv_indptr, schedule, m_args, out, count, nsplit, causal,
+                scale) -> None:
+    """The general paged kernel (any head_dim in {32, 64, 128, 256}, n_rep <= 8). ``schedule``:
+    ``(qo_indptr, q_tile_to_batch, q_tile_to_index)`` for a prefill call (``count`` = tiles),
+    None for decode (``count`` = batch)."""
+    h, d, hkv = q.size(1), q.size(2), k_pool.size(1)
+    prefill = schedule is not None
+    need = lib.astrai_w8a8_attn_paged_rows_workspace_floats(count, h, hkv, d, nsplit, 1 if prefill else 0)
+    if count and need <= 0:
+        raise RuntimeError(f"paged attention needs head_dim in (32, 64, 128, 256) and n_heads / n_kv_heads <= 8; "
+                           f"got head_dim {d}, {h} / {hkv} heads")
+    ws = torch.empty(max(need, 1), device=q.device, dtype=torch.float32)
+    sched = [t.data_ptr() for t in schedule] if prefill else [0, 0, 0]
+    _check(lib.astrai_w8a8_attn_paged_rows_bf16(
+        q.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), rtt.data_ptr(), rpi.data_ptr(), kv_indptr.data_ptr(),
+        *sched, *m_args, ws.data_ptr(), ws.numel(), out.data_ptr(), count, h, hkv, d, k_pool.size(0), rtt.size(0),
+        rtt.size(1), 1 if causal else 0, nsplit, float(scale), _stream(q)), lib)
 
 
 Q_TILE_ROWS = 64  # rows per tile of the schedule the reference builds (astrai/inference/workspace.py:13)
@@ -787,6 +814,12 @@ def attn_paged_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Te
     with torch.cuda.device(q.device):
         # (rows that no tile of the schedule covers are left unwritten, as by the reference)
         out = torch.empty((total_q, h, d), device=q.device, dtype=torch.bfloat16)
+        if not attn_prefill_supported(h, hkv, d):  # the shapes only the general kernel takes
+            tiles = q_tile_to_batch.numel()
+            blocks = tiles * 8 * hkv                 # at least: 8 row blocks per 64-row tile
+            _paged_rows(lib, q_c, k_cache, v_cache, tensors[0], tensors[1], tensors[2], tensors[3:], m_args,
+                        out, tiles, max(1, min(16, 384 // max(1, blocks))), causal_offset >= 0, scale)
+            return out
         _check(lib.astrai_w8a8_attn_paged_prefill_masked_bf16(
             q_c.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), *[t.data_ptr() for t in tensors],
             *m_args, out.data_ptr(), q_tile_to_batch.numel(), h, hkv, d, slots, req_to_token.size(0),
@@ -1106,13 +1139,13 @@ def attn_decode_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Opt
     m4 = _dense_mask(mask, b, 1, kv_len, h)
     if m4 is not None and m4.size(1) != 1:
         raise RuntimeError("attn_decode: a mask per head is not supported")
-    if d != 128 or h // hkv > 8 or h > 64:
-        raise RuntimeError("attn_decode needs head_dim 128, n_heads / n_kv_heads <= 8, n_heads <= 64")
+    if d not in (32, 64, 128, 256) or h // hkv > 8:
+        raise RuntimeError("attn_decode needs head_dim in (32, 64, 128, 256) and n_heads / n_kv_heads <= 8")
     attend = kv_len if causal_offset < 0 else min(kv_len, causal_offset + 1)
     with torch.cuda.device(q.device):
         if kv_len == 0 or b == 0:
             return torch.zeros_like(q)
-        if layout == BHLD and m4 is None and k.is_contiguous() and v.is_contiguous():
+        if layout == BHLD and m4 is None and k.is_contiguous() and v.is_contiguous() and d == 128 and h <= 64:
             pos = torch.full((1,), attend - 1, dtype=torch.int64, device=q.device)
             out = attn_decode(q.contiguous(), k, v, pos, scale=scale if scale > 0 else None)
             return out.reshape(b, h, 1, d)
@@ -1136,13 +1169,13 @@ def attn_prefill_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Op
     ``kv_len - q_len`` is expressed through the mask."""
     b, q_len, kv_len, h, hkv, d = _dense_args(q, k, v, layout, "attn_prefill")
     m4 = _dense_mask(mask, b, q_len, kv_len, h)
-    if not attn_prefill_supported(h, hkv, d):
-        raise RuntimeError("attn_prefill needs head_dim 128 and n_heads / n_kv_heads in {2, 4, 8}")
+    if d not in (32, 64, 128, 256) or h // hkv > 8:
+        raise RuntimeError("attn_prefill needs head_dim in (32, 64, 128, 256) and n_heads / n_kv_heads <= 8")
     with torch.cuda.device(q.device):
         if kv_len == 0 or b == 0 or q_len == 0:
             return torch.zeros_like(q)
         rows_i = torch.arange(q_len, dtype=torch.int64, device=q.device)
-        if layout == BHLD and m4 is None and k.is_contiguous() and v.is_contiguous():
+        if layout == BHLD and m4 is None and k.is_contiguous() and v.is_contiguous() and attn_prefill_supported(h, hkv, d):
             pos = torch.full_like(rows_i, kv_len - 1) if causal_offset < 0 else (rows_i + causal_offset).clamp_max(kv_len - 1)
             out = attn_prefill(q.contiguous(), k, v, pos, scale=scale if scale > 0 else None)
             return out.view(b, q_len, h, d).transpose(1, 2)

@@ -325,6 +325,34 @@ int astrai_w8a8_attn_paged_prefill_masked_bf16(
     int64_t max_context_len, int causal, float scale, void* stream);
 
 /*
+ * Paged attention for the shapes the tuned kernels above do not take: head_dim 32, 64, 128 or
+ * 256 and any n_heads / n_kv_heads up to 8 -- the reference's paged kernels accept those
+ * head_dims and any grouping (astrai/extension/backend/attention.py:518-527; its tests run
+ * head_dim 64, tests/extension/conftest.py:9-20). One entry for both reference entries:
+ *   qo_indptr == NULL  decode, as attn_paged_decode_masked_bf16: q / out [batch, n_heads,
+ *              head_dim], batch_or_tiles = batch, causal ignored, mask rows / strides as for a
+ *              2D mask (head and row stride 0)
+ *   qo_indptr != NULL  ragged prefill, as attn_paged_prefill_masked_bf16: packed q / out
+ *              [total_q, n_heads, head_dim], the 64-row tile schedule, batch_or_tiles = tiles
+ * Same arithmetic as attn_decode_bf16 (bf16 MFMA scores, fp32 softmax and P.V, one rounding);
+ * correct for every shape, not tuned (prefill re-reads the keys once per block of at most
+ * 8 / (n_heads / n_kv_heads) rows). workspace: attn_paged_rows_workspace_floats(...) floats,
+ * 0 from that function = unsupported shape. nsplit in [1, 64] splits the context.
+ */
+int64_t astrai_w8a8_attn_paged_rows_workspace_floats(int64_t batch_or_tiles, int64_t n_heads,
+                                                     int64_t n_kv_heads, int64_t head_dim,
+                                                     int64_t nsplit, int prefill);
+int astrai_w8a8_attn_paged_rows_bf16(
+    const void* q_bf16, const void* k_pool_bf16, const void* v_pool_bf16,
+    const int32_t* req_to_token, const int32_t* req_pool_indices, const int32_t* kv_indptr,
+    const int32_t* qo_indptr, const int32_t* q_tile_to_batch, const int32_t* q_tile_to_index,
+    const uint8_t* mask, int64_t mask_seq_stride, int64_t mask_head_stride, int64_t mask_row_stride,
+    int64_t mask_rows, int64_t mask_width, float* workspace, int64_t workspace_floats, void* out_bf16,
+    int64_t batch_or_tiles, int64_t n_heads, int64_t n_kv_heads, int64_t head_dim, int64_t num_slots,
+    int64_t num_requests, int64_t max_context_len, int causal, int64_t nsplit, float scale,
+    void* stream);
+
+/*
  * bf16 -> e4m3fn with one scale per 1x128 K-group (activations) or per 128x128
  * block (weights). No counterpart in the reference. K must be a multiple of 128.
  *   act:    sa[m,kb]  = max(max |x[m,128kb..128kb+127]|, 1e-12) / 448,   sa is [M, K/128]

@@ -141,8 +141,8 @@ def test_dense_entries_reject_what_the_reference_rejects():
         pre(q, k, v, mask=torch.ones(3, 16, dtype=torch.bool, device=DEV), layout=1)
     with pytest.raises(RuntimeError, match="mask must be bool"):
         pre(q, k, v, mask=torch.ones(2, 16, device=DEV), layout=1)
-    with pytest.raises(RuntimeError, match="head_dim 128"):
-        pre(q[..., :64], k[..., :64], v[..., :64], layout=1)
+    with pytest.raises(RuntimeError, match="head_dim"):
+        pre(q[..., :48], k[..., :48], v[..., :48], layout=1)
 
 
 @pytest.mark.parametrize("shape", [(37, 16, 128), (2, 19, 4, 128), (5, 3, 64), (4, 2, 6), (1, 1, 2), (0, 4, 128)])
@@ -183,3 +183,111 @@ def test_rotary_emb_large_and_argument_checks():
                       ((xd.cpu(), fd), "CUDA")):
         with pytest.raises(RuntimeError, match=msg):
             fn(*args)
+
+
+# ---- the general paged kernel: head_dim 32 / 64 / 256, any grouping up to 8 ----
+
+def _paged_case(b, h, hkv, d, kv_lens, q_lens, seed, holes=False):
+    g = torch.Generator().manual_seed(seed)
+    total_q, pool = sum(q_lens), sum(kv_lens) + 9
+    q = torch.randn(total_q, h, d, generator=g).to(torch.bfloat16)
+    k_pool = torch.randn(pool, hkv, d, generator=g).to(torch.bfloat16)
+    v_pool = torch.randn(pool, hkv, d, generator=g).to(torch.bfloat16)
+    rows = torch.randperm(b + 2, generator=g)[:b].int()
+    table = torch.full((b + 2, max(kv_lens) + 3), -1, dtype=torch.int32)
+    perm = torch.randperm(pool, generator=g)
+    nxt = 0
+    for i in range(b):
+        table[rows[i], :kv_lens[i]] = perm[nxt:nxt + kv_lens[i]].int()
+        nxt += kv_lens[i]
+        if holes and kv_lens[i] > 4:
+            table[rows[i], 2] = -1
+    k_pool[perm[nxt:]] = float("nan")         # slots no live position maps to must not be read
+    v_pool[perm[nxt:]] = float("nan")
+    kvp = torch.tensor([0] + torch.tensor(kv_lens).cumsum(0).tolist(), dtype=torch.int32)
+    return q, k_pool, v_pool, table, rows, kvp
+
+
+@pytest.mark.parametrize("d", [32, 64, 256])
+@pytest.mark.parametrize("h,hkv", [(2, 1), (4, 4), (6, 2), (8, 1), (16, 4)])
+def test_paged_decode_other_head_dims_and_groupings(d, h, hkv):
+    """head_dim 64 with 2 heads on 1 KV head is the reference's own test model
+    (tests/extension/conftest.py:9-20)."""
+    from astrai_amd.extension import ops
+    lens = [70, 1, 0, 33, 150]
+    args = _paged_case(5, h, hkv, d, lens, [1] * 5, seed=d + h, holes=True)
+    dev = [t.to(DEV) for t in args]
+    want = D.attn_paged_decode(*args)
+    got = ops.attn_paged_decode(*dev, is_causal=True)
+    assert got.shape == (5, h, d)
+    assert_bf16_close(got, want, what=f"decode d={d} {h}/{hkv}")
+    assert got[2].abs().sum() == 0
+    mask = torch.rand(5, max(lens) + 3, generator=torch.Generator().manual_seed(d)) < 0.6
+    got = ops.attn_paged_decode(*dev, mask=mask.to(DEV), is_causal=True)
+    assert_bf16_close(got, D.attn_paged_decode(*args, mask=mask), what=f"decode d={d} {h}/{hkv} mask")
+    from astrai_amd.extension import _cabi
+    for nsplit in (1, 3):
+        got = _cabi.attn_paged_decode(*dev, nsplit=nsplit)
+        assert_bf16_close(got, want, what=f"decode d={d} nsplit={nsplit}")
+
+
+@pytest.mark.parametrize("d,h,hkv", [(64, 2, 1), (64, 4, 4), (32, 8, 1), (256, 4, 2), (128, 4, 4), (128, 6, 2), (64, 16, 2)])
+@pytest.mark.parametrize("causal", [True, False])
+def test_paged_prefill_other_head_dims_and_groupings(d, h, hkv, causal):
+    """The shapes the MFMA prefill kernel does not take (head_dim != 128, or a grouping other
+    than 2 / 4 / 8, multi-head attention included) run the general kernel."""
+    from astrai_amd.extension import _cabi, ops
+    kv_lens, q_lens = [100, 37, 64, 5], [70, 37, 1, 5]
+    args = _paged_case(4, h, hkv, d, kv_lens, q_lens, seed=d + h + hkv, holes=True)
+    dev = [t.to(DEV) for t in args]
+    qo, tb, ti = _cabi.paged_prefill_schedule(q_lens, DEV)
+    got = ops.attn_paged_prefill(*dev, qo, tb, ti, is_causal=causal)
+    assert got.shape == (sum(q_lens), h, d)
+    _close(got, D.attn_paged_prefill(*args, qo.cpu(), causal=causal), f"prefill d={d} {h}/{hkv} causal={causal}")
+    g = torch.Generator().manual_seed(d)
+    for shape in ((4, max(kv_lens) + 3), (4, 1, max(q_lens), max(kv_lens)), (4, h, max(q_lens), max(kv_lens))):
+        mask = torch.rand(shape, generator=g) < 0.6
+        got = ops.attn_paged_prefill(*dev, qo, tb, ti, mask=mask.to(DEV), is_causal=causal)
+        _close(got, D.attn_paged_prefill(*args, qo.cpu(), causal=causal, mask=mask), f"prefill d={d} mask {shape}")
+
+
+def test_general_kernel_agrees_with_the_tuned_kernels_where_both_apply():
+    """head_dim 128, grouping 4: the rows entry through the C ABI against the tuned paged kernels."""
+    import ctypes
+    from astrai_amd.extension import _cabi
+    lib = _cabi.load()
+    kv_lens, q_lens = [300, 64, 129], [300, 1, 60]
+    args = _paged_case(3, 16, 4, 128, kv_lens, q_lens, seed=5)
+    q, kp, vp, table, rows, kvp = [t.to(DEV) for t in args]
+    qo, tb, ti = _cabi.paged_prefill_schedule(q_lens, DEV)
+    tuned = _cabi.attn_paged_prefill(q, kp, vp, table, rows, kvp, qo, tb, ti, causal_offset=0)
+    out = torch.empty_like(tuned)
+    _cabi._paged_rows(lib, q, kp, vp, table, rows, kvp, (qo, tb, ti), (0, 0, 0, 0, 0, 0), out, tb.numel(), 2, True,
+                      128 ** -0.5)
+    _close(out, tuned, "rows kernel vs MFMA prefill kernel")
+    q1 = q[:3].contiguous()
+    tuned = _cabi.attn_paged_decode(q1, kp, vp, table, rows, kvp, nsplit=2)
+    out = torch.empty_like(tuned)
+    _cabi._paged_rows(lib, q1, kp, vp, table, rows, kvp, None, (0, 0, 0, 0, 0, 0), out, 3, 2, False, 128 ** -0.5)
+    assert torch.equal(out, tuned)                 # same arithmetic, same split points
+
+
+@pytest.mark.parametrize("layout", [0, 1])
+def test_dense_entries_head_dim_64_like_the_reference_test_model(layout):
+    from astrai_amd.extension import get_module
+    dec, pre = get_module("attn_decode").attn_decode, get_module("attn_prefill").attn_prefill
+    g = torch.Generator().manual_seed(64)
+    b, lq, lk, h, hkv, d = 2, 16, 40, 2, 1, 64
+    mk = lambda l, n: torch.randn(b, l, n, d, generator=g).to(torch.bfloat16)
+    q, k, v = mk(lq, h), mk(lk, hkv), mk(lk, hkv)
+    if layout == 0:
+        q, k, v = (t.transpose(1, 2).contiguous() for t in (q, k, v))
+    dev = [t.to(DEV) for t in (q, k, v)]
+    for off in (-1, lk - lq, 0):
+        _close(pre(*dev, causal_offset=off, layout=layout), D.attn_dense(q, k, v, causal_offset=off, layout=layout),
+               f"prefill layout {layout} offset {off}")
+    q1 = q[:, :, :1].contiguous() if layout == 0 else q[:, :1].contiguous()
+    got = dec(q1.to(DEV), dev[1], dev[2], causal_offset=lk - 1, layout=layout)
+    assert_bf16_close(got, D.attn_dense(q1, k, v, layout=layout), what=f"decode layout {layout}")
+    with pytest.raises(RuntimeError, match="head_dim"):
+        pre(dev[0][..., :48], dev[1][..., :48], dev[2][..., :48], layout=layout)
