@@ -130,3 +130,35 @@ def test_int8_checkpoint_round_trip(tmp_path):
         got = loaded(ids)["logits"]
     w8a8.int8_state().reset()
     assert torch.equal(got, want)
+
+
+def test_reference_test_model_config_modular_and_fused():
+    """The model the reference's extension tests build (tests/extension/conftest.py:9-20: hidden
+    128, 2 heads on 1 KV head, head_dim 64, FFN 256, 2 layers, vocabulary 1000): K = 128 and 256
+    GEMMs, a 2-head grouping, through both int8 paths, with a cache, against the oracle."""
+    from astrai_amd.extension import w8a8
+    from astrai_amd.model import DenseKVCache, fuse_int8_weights, greedy_generate
+    cfg, model = _model(9, vocab_size=1000, hidden_size=128, num_hidden_layers=2, num_attention_heads=2,
+                        num_key_value_heads=1, intermediate_size=256, max_position_embeddings=64)
+    sd = {k: v.detach().clone() for k, v in model.state_dict().items()}
+    ids = torch.randint(0, cfg.vocab_size, (2, 16), generator=torch.Generator().manual_seed(9))
+    want = D.forward(sd, cfg, ids, D.int8_linear_fn(sd)).float()
+    gm = model.to(DEV)
+    w8a8.int8_state().reset()
+    w8a8.prepare_int8_weights(gm)
+    with torch.no_grad(), w8a8.int8_autocast(True):
+        modular = gm(ids.to(DEV))["logits"].float().cpu()
+        fuse_int8_weights(gm)
+        fused = gm(ids.to(DEV))["logits"].float().cpu()
+        cache = DenseKVCache(cfg, 2, 16, DEV, torch.bfloat16)
+        pre = gm(ids[:, :9].to(DEV), cache, torch.arange(9, device=DEV))["logits"]
+        dec = [gm(ids[:, t:t + 1].to(DEV), cache, torch.tensor([t], device=DEV))["logits"] for t in range(9, 16)]
+        eager = greedy_generate(gm, ids[:, :8].to(DEV), 8, use_graph=False)
+        graph = greedy_generate(gm, ids[:, :8].to(DEV), 8, use_graph=True)
+    w8a8.int8_state().reset()
+    scale = want.abs().max().item()
+    for name, got in (("modular", modular), ("fused", fused), ("cached", torch.cat([pre] + dec, 1).float().cpu())):
+        cos = torch.nn.functional.cosine_similarity(got.flatten(), want.flatten(), dim=0).item()
+        assert cos > 0.999, (name, cos)
+        assert (got - want).abs().max().item() <= 0.05 * scale, name
+    assert torch.equal(eager, graph)
