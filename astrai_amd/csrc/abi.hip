@@ -390,9 +390,9 @@ int astrai_w8a8_attn_paged_prefill_masked_bf16(
 int64_t astrai_w8a8_attn_paged_rows_workspace_floats(int64_t batch_or_tiles, int64_t n_heads,
                                                      int64_t n_kv_heads, int64_t head_dim,
                                                      int64_t nsplit, int prefill) {
-    if (batch_or_tiles <= 0 || nsplit <= 0 || nsplit > 64 || n_heads <= 0 || n_kv_heads <= 0 ||
+    if (batch_or_tiles < 0 || nsplit <= 0 || nsplit > 64 || n_heads <= 0 || n_kv_heads <= 0 ||
         n_heads > 65535 || !w8a8::attn_rows_supported((int)n_heads, (int)n_kv_heads, (int)head_dim))
-        return 0;
+        return -1;
     return w8a8::attn_rows_workspace_floats(batch_or_tiles, (int)n_heads, (int)n_kv_heads, (int)head_dim,
                                             (int)nsplit, prefill != 0);
 }
@@ -405,7 +405,8 @@ int astrai_w8a8_attn_paged_rows_bf16(
     int64_t mask_width, float* workspace, int64_t workspace_floats, void* out, int64_t batch_or_tiles,
     int64_t n_heads, int64_t n_kv_heads, int64_t head_dim, int64_t num_slots, int64_t num_requests,
     int64_t max_context_len, int causal, int64_t nsplit, float scale, void* stream) {
-    if (!q || !k_pool || !v_pool || !req_to_token || !req_pool_indices || !kv_indptr || !workspace || !out)
+    if (!q || !k_pool || !v_pool || !req_to_token || !req_pool_indices || !kv_indptr || !out ||
+        (nsplit > 1 && !workspace))
         return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_rows_bf16: null pointer");
     const bool prefill = qo_indptr != nullptr;
     if (prefill && (!q_tile_to_batch || !q_tile_to_index))
@@ -416,7 +417,7 @@ int astrai_w8a8_attn_paged_rows_bf16(
         return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_rows_bf16: bad dims");
     if (!w8a8::attn_rows_supported((int)n_heads, (int)n_kv_heads, (int)head_dim))
         return fail(ASTRAI_W8A8_UNSUPPORTED,
-                    "attn_paged_rows_bf16: needs head_dim in {32, 64, 128, 256} and n_heads / n_kv_heads <= 8");
+                    "attn_paged_rows_bf16: needs head_dim in {32, 64, 128, 256} and n_heads / n_kv_heads <= 16");
     if (mask && (mask_width <= 0 || mask_rows <= 0 || mask_width > INT32_MAX || mask_rows > INT32_MAX ||
                  mask_seq_stride < 0 || mask_head_stride < 0 || mask_row_stride < 0))
         return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_rows_bf16: bad mask dims");
@@ -426,7 +427,7 @@ int astrai_w8a8_attn_paged_rows_bf16(
     if (batch_or_tiles == 0) return ASTRAI_W8A8_OK;
     const int64_t need = w8a8::attn_rows_workspace_floats(batch_or_tiles, (int)n_heads, (int)n_kv_heads,
                                                           (int)head_dim, (int)nsplit, prefill);
-    if (workspace_floats < need)
+    if (need > 0 && workspace_floats < need)
         return fail(ASTRAI_W8A8_BAD_ARG, "attn_paged_rows_bf16: workspace too small (%lld floats needed)",
                     (long long)need);
     w8a8::AttnRowsArgs a{};

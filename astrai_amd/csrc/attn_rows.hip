@@ -1,19 +1,27 @@
 // Paged grouped-query attention for the shapes the two tuned kernels do not take:
-// head_dim 32, 64, 128 or 256, any n_heads / n_kv_heads up to 8, decode (one query
+// head_dim 32, 64, 128 or 256, any n_heads / n_kv_heads up to 16, decode (one query
 // row per sequence) and ragged prefill (row ranges per sequence) alike. The
 // reference's paged kernels accept head_dim in {32, 64, 128, 256} and any head
 // grouping (astrai/extension/backend/attention.py:518-527,
 // csrc/kernels/attention/dispatchers.cuh); its own tests run head_dim 64
 // (tests/extension/conftest.py:9-20).
 //
-// Same scheme as the decode kernel: the query rows that share a KV head -- n_rep heads
-// times up to 8 / n_rep consecutive rows of a sequence, at most 8 in all -- are the
-// columns of v_mfma_f32_16x16x32_bf16 score tiles whose rows are 16 keys; online
-// softmax in fp32; P.V on the vector ALU; the four waves of a workgroup take key
-// tiles in turn and merge through LDS; the context can be split over workgroups,
-// merged by a second kernel. Every query row carries its own causal limit, so a
-// block of prefill rows is a decode step with several newest tokens. Correct for
-// every shape, not tuned: prefill re-reads the keys once per row block.
+// One wave per (block of query rows, KV head, context split). The query rows that share a
+// KV head -- n_rep heads times up to 16 / n_rep consecutive rows of a sequence, at most
+// 16 in all -- are the columns of 16-key MFMA tiles:
+//   scores  v_mfma_f32_16x16x32_bf16, keys as rows (16 bytes per lane straight from the
+//           pool), so a lane ends up with the scores of one query for keys 4g..4g+3;
+//   softmax online, fp32, per query (its four lanes share through two butterfly steps);
+//   P.V     v_mfma_f32_16x16x16_bf16 per 16 dims with V^T as the row operand -- the 16
+//           value rows of the tile pass through a wave-private LDS patch and come back
+//           transposed (ds_read_tr16_b64) -- and P, already in the column operand's
+//           layout, split into a bf16 head and a bf16 remainder (two MFMAs), so that the
+//           probabilities enter with 16 bits of mantissa.
+// Every query row carries its own causal limit and mask row, so a block of prefill rows is
+// a decode step with several newest tokens. Without a context split the wave normalises
+// and writes bf16 itself; with one it leaves (max, sum, acc) in a workspace for the merge
+// kernel. Correct for every shape, not tuned like the head_dim-128 kernels: prefill
+// re-reads the keys once per row block.
 #include <climits>
 
 #include "common.cuh"
@@ -25,17 +33,16 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
-constexpr int kNQ = 8;             // query rows per workgroup (MFMA columns in use)
+constexpr int kNQ = 16;            // query rows per wave (MFMA columns)
 constexpr float kNegBig = -1e30f;  // finite stand-in for -inf: no inf - inf
 
-__device__ __forceinline__ float lane_read(float v, int src_lane) {
-    return __int_as_float(__builtin_amdgcn_ds_bpermute(src_lane << 2, __float_as_int(v)));
-}
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+
 __device__ __forceinline__ int lane_read_i(int v, int src_lane) {
     return __builtin_amdgcn_ds_bpermute(src_lane << 2, v);
 }
 
-// W 32-bit words (2 W bf16 values) from an address aligned to their size (16 bytes at most)
+// W 32-bit words (2 W bf16 values) from / to an address aligned to their size (16 bytes at most)
 template <int W>
 __device__ __forceinline__ void load_words(const uint16_t* p, uint32_t (&w)[W]) {
     if constexpr (W == 1) {
@@ -51,8 +58,20 @@ __device__ __forceinline__ void load_words(const uint16_t* p, uint32_t (&w)[W]) 
         }
     }
 }
+template <int W>
+__device__ __forceinline__ void store_words(uint8_t* p, const uint32_t (&w)[W]) {
+    if constexpr (W == 1) {
+        *reinterpret_cast<uint32_t*>(p) = w[0];
+    } else if constexpr (W == 2) {
+        *reinterpret_cast<u32x2*>(p) = u32x2{w[0], w[1]};
+    } else {
+#pragma unroll
+        for (int i = 0; i < W / 4; ++i)
+            *reinterpret_cast<u32x4*>(p + 16 * i) = u32x4{w[4 * i], w[4 * i + 1], w[4 * i + 2], w[4 * i + 3]};
+    }
+}
 
-// the row block a workgroup (or a merge workgroup's row) belongs to
+// the row block a wave (or a merge workgroup's row) belongs to
 struct RowBlock {
     int seq;      // sequence (index into req_pool_indices, kv_indptr, qo_indptr, the mask)
     int q_start;  // first packed query row of the sequence
@@ -80,22 +99,25 @@ __device__ __forceinline__ RowBlock row_block(const AttnRowsArgs& a, int block) 
 // workspace per (row block, kv head, split): kNQ rows of [D values | max | sum]
 template <int D, bool MASK>
 __global__ __launch_bounds__(256) void attn_rows_partial_kernel(AttnRowsArgs a) {
-    constexpr int STEPS = D / 32;  // score MFMAs per key tile
-    constexpr int DV = D / 16;     // value dims per lane
+    constexpr int STEPS = D / 32;           // score MFMAs per key tile
+    constexpr int CHUNKS = D / 16;          // 16-dim output chunks
+    constexpr int DV = D / 16;              // value dims a lane fetches per key
     constexpr int WS_ROW = D + 2;
-    __shared__ float sh_acc[4][kNQ][D];
-    __shared__ float sh_ml[4][kNQ][2];
+    constexpr int V_STRIDE = D * 2 + 32;    // bytes per staged value row: the 4 rows of a transposing read hit distinct banks
+    __shared__ __attribute__((aligned(16))) uint8_t v_stage[4][16 * V_STRIDE];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int c16 = lane & 15, g = lane >> 4;
     const int n_rep = a.n_heads / a.n_kv_heads;
     const int rows = a.rows_per_block;
     const int nq = n_rep * rows;  // <= kNQ
-    int wg = blockIdx.x;
-    const int split = wg % a.nsplit;
-    wg /= a.nsplit;
-    const int hk = wg % a.n_kv_heads;
-    const RowBlock rb = row_block(a, wg / a.n_kv_heads);
+    int64_t item = (int64_t)blockIdx.x * 4 + wave;
+    if (item >= a.num_items) return;
+    const int split = (int)(item % a.nsplit);
+    item /= a.nsplit;
+    const int hk = (int)(item % a.n_kv_heads);
+    const int block = (int)(item / a.n_kv_heads);
+    const RowBlock rb = row_block(a, block);
     if (rb.r0 >= rb.q_len) return;  // the schedule's tile reaches past the sequence: nothing reads this block
 
     const int64_t req = a.req_pool_indices[rb.seq];
@@ -138,57 +160,77 @@ __global__ __launch_bounds__(256) void attn_rows_partial_kernel(AttnRowsArgs a) 
     }
 
     float m = kNegBig, l = 0.0f;  // of query c16, equal in its four lanes
-    float acc[kNQ][DV];
+    // o[c][i] = sum over keys of p * v for query c16, dim 16c + 4g + i
+    f32x4 o[CHUNKS];
 #pragma unroll
-    for (int q = 0; q < kNQ; ++q)
-#pragma unroll
-        for (int d = 0; d < DV; ++d) acc[q][d] = 0.0f;
+    for (int c = 0; c < CHUNKS; ++c) o[c] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    // slot of key 16t + c16, looked up one tile ahead of its use. -1 (a negative or
-    // out-of-pool table entry): nothing is fetched, key and value read as zeros, and the
-    // position is attended all the same, as in the reference, which gates the load on the
-    // slot and the mask on the position (csrc/kernels/attention/layout_policies.cuh:104-110,212-219)
+    // slot of key 16t + c16, looked up one tile ahead of its use. -1 (past the newest visible
+    // key, or a negative or out-of-pool table entry): nothing is fetched, key and value read
+    // as zeros; a negative entry inside the sequence is attended all the same, as in the
+    // reference, which gates the load on the slot and the mask on the position
+    // (csrc/kernels/attention/layout_policies.cuh:104-110,212-219)
     auto key_slot = [&](int t) -> int {
         const int key = (t << 4) + c16;
         const int slot = (t < t1 && key <= kmax) ? table[key] : -1;
         return slot < a.num_slots ? slot : -1;
     };
-    int slot_next = key_slot(t0 + wave);
     const int64_t pool_row = (int64_t)a.n_kv_heads * D;  // elements from one slot to the next
+    uint8_t* const stage = v_stage[wave];
+    // where this lane stores the value pieces it fetches (key 4g + i, dims DV c16 ..) and where
+    // its transposing reads point (key 4g + c16 / 4, dims 16c + 4 (c16 % 4) ..: the lane gets
+    // dim 16c + c16 of keys 4g .. 4g+3 back)
+    uint8_t* const st_mine = stage + (4 * g) * V_STRIDE + c16 * DV * 2;
+    const uint8_t* const tr_mine = stage + (4 * g + (c16 >> 2)) * V_STRIDE + (c16 & 3) * 8;
 
-    for (int t = t0 + wave; t < t1; t += 4) {
-        const int kb = t << 4;
-        const int slot = slot_next;
-        slot_next = key_slot(t + 4);
-        u32x4 kf[STEPS];
-        uint32_t vw[4][DV / 2];
-        [[maybe_unused]] uint8_t keep[4] = {1, 1, 1, 1};
+    // operands of one key tile, requested a tile ahead of their use: keys as MFMA rows (lane ->
+    // key 16t + c16, dims 32 step + 8g), values (lane -> keys 16t + 4g + i, dims DV c16 ..), mask bytes
+    u32x4 kf_n[STEPS];
+    uint32_t vw_n[4][DV / 2];
+    [[maybe_unused]] uint8_t keep_n[4] = {1, 1, 1, 1};
+    auto fetch = [&](int t, int slot) {
+        const uint16_t* kr = static_cast<const uint16_t*>(a.k_cache) + (int64_t)max(slot, 0) * pool_row + hk * D + 8 * g;
+#pragma unroll
+        for (int st = 0; st < STEPS; ++st)
+            kf_n[st] = slot >= 0 ? *reinterpret_cast<const u32x4*>(kr + 32 * st) : u32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int vslot = lane_read_i(slot, 4 * g + i);  // lanes 0..15 hold the slots of keys 16t..16t+15
+            const uint16_t* vr = static_cast<const uint16_t*>(a.v_cache) + (int64_t)max(vslot, 0) * pool_row +
+                                 hk * D + c16 * DV;
+            if (vslot >= 0) {
+                load_words<DV / 2>(vr, vw_n[i]);
+            } else {
+#pragma unroll
+                for (int w = 0; w < DV / 2; ++w) vw_n[i][w] = 0u;
+            }
+        }
         if constexpr (MASK) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int key = kb + 4 * g + i;
-                keep[i] = key < mask_keys ? mask_row[key] : (uint8_t)0;
+                const int key = (t << 4) + 4 * g + i;
+                keep_n[i] = key < mask_keys ? mask_row[key] : (uint8_t)0;
             }
         }
-        {
-            const uint16_t* kr = static_cast<const uint16_t*>(a.k_cache) + (int64_t)max(slot, 0) * pool_row +
-                                 hk * D + 8 * g;
+    };
+    fetch(t0, key_slot(t0));
+    int slot_next = key_slot(t0 + 1);
+
+    for (int t = t0; t < t1; ++t) {
+        const int kb = t << 4;
+        u32x4 kf[STEPS];
+        [[maybe_unused]] uint8_t keep[4];
 #pragma unroll
-            for (int st = 0; st < STEPS; ++st)
-                kf[st] = slot >= 0 ? *reinterpret_cast<const u32x4*>(kr + 32 * st) : u32x4{0, 0, 0, 0};
+        for (int st = 0; st < STEPS; ++st) kf[st] = kf_n[st];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int vslot = lane_read_i(slot, 4 * g + i);  // lanes 0..15 hold keys kb..kb+15
-                const uint16_t* vr = static_cast<const uint16_t*>(a.v_cache) + (int64_t)max(vslot, 0) * pool_row +
-                                     hk * D + c16 * DV;
-                if (vslot >= 0) {
-                    load_words<DV / 2>(vr, vw[i]);
-                } else {
+        for (int i = 0; i < 4; ++i) keep[i] = keep_n[i];
+        // values of the tile into the wave's patch (the previous tile's reads are done: same wave, in order)
+        __asm__ volatile("" ::: "memory");
 #pragma unroll
-                    for (int w = 0; w < DV / 2; ++w) vw[i][w] = 0u;
-                }
-            }
-        }
+        for (int i = 0; i < 4; ++i) store_words<DV / 2>(st_mine + i * V_STRIDE, vw_n[i]);
+        __asm__ volatile("" ::: "memory");
+        fetch(t + 1, slot_next);  // (past the last tile every slot is -1: nothing is requested)
+        slot_next = key_slot(t + 2);
 
         f32x4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -219,77 +261,47 @@ __global__ __launch_bounds__(256) void attn_rows_partial_kernel(AttnRowsArgs a) 
         l = l * alpha + ps;
         m = m_new;
 
-        // P.V: this lane needs alpha and p[i] of query q from lane 16g + q
+        // P as the column operand (query c16, keys 4g..4g+3): bf16 head and bf16 remainder
+        const uint32_t h01 = pack_bf16x2(p[0], p[1]), h23 = pack_bf16x2(p[2], p[3]);
+        const uint32_t r01 = pack_bf16x2(p[0] - __uint_as_float(h01 << 16), p[1] - __uint_as_float(h01 & 0xffff0000u));
+        const uint32_t r23 = pack_bf16x2(p[2] - __uint_as_float(h23 << 16), p[3] - __uint_as_float(h23 & 0xffff0000u));
+        const i16x4 p_hi = __builtin_bit_cast(i16x4, u32x2{h01, h23});
+        const i16x4 p_lo = __builtin_bit_cast(i16x4, u32x2{r01, r23});
 #pragma unroll
-        for (int q = 0; q < kNQ; ++q) {
-            const float aq = lane_read(alpha, 16 * g + q);
-#pragma unroll
-            for (int d = 0; d < DV; ++d) acc[q][d] *= aq;
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float v[DV];
-#pragma unroll
-            for (int w = 0; w < DV / 2; ++w) {
-                // a row past the newest visible position was never written: keep it out even at p = 0
-                const uint32_t raw = (kb + 4 * g + i) > kmax ? 0u : vw[i][w];
-                v[2 * w] = __uint_as_float(raw << 16);
-                v[2 * w + 1] = __uint_as_float(raw & 0xffff0000u);
-            }
-#pragma unroll
-            for (int q = 0; q < kNQ; ++q) {
-                const float pq = lane_read(p[i], 16 * g + q);
-#pragma unroll
-                for (int d = 0; d < DV; ++d) acc[q][d] += pq * v[d];
-            }
+        for (int c = 0; c < CHUNKS; ++c) {
+            typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
+            const i16x4 vt = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(tr_mine + c * 32));
+            f32x4 acc = o[c] * alpha;
+            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vt, p_hi, acc, 0, 0, 0);
+            o[c] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vt, p_lo, acc, 0, 0, 0);
         }
     }
 
-    // the four key groups of the wave hold sums over different keys: add them up
+    if (a.nsplit == 1) {
+        // the whole context was this wave's: normalise and write out[row, head, 16c + 4g ..+3]
+        if (!q_live) return;
+        const float inv = l > 0.0f ? 1.0f / l : 0.0f;  // a row with no visible key yields zeros
+        uint16_t* orow = static_cast<uint16_t*>(a.out) + ((int64_t)(rb.q_start + row) * a.n_heads + head) * D + 4 * g;
 #pragma unroll
-    for (int q = 0; q < kNQ; ++q)
-#pragma unroll
-        for (int d = 0; d < DV; ++d) {
-            float v = acc[q][d];
-            v += __shfl_xor(v, 16, kWave);
-            v += __shfl_xor(v, 32, kWave);
-            acc[q][d] = v;
-        }
-    if (g == 0) {
-#pragma unroll
-        for (int q = 0; q < kNQ; ++q)
-#pragma unroll
-            for (int d = 0; d < DV; ++d) sh_acc[wave][q][c16 * DV + d] = acc[q][d];
-        if (c16 < kNQ) {
-            sh_ml[wave][c16][0] = m;
-            sh_ml[wave][c16][1] = l;
-        }
+        for (int c = 0; c < CHUNKS; ++c)
+            *reinterpret_cast<u32x2*>(orow + 16 * c) =
+                u32x2{pack_bf16x2(o[c][0] * inv, o[c][1] * inv), pack_bf16x2(o[c][2] * inv, o[c][3] * inv)};
+        return;
     }
-    __syncthreads();
-    // merge the four waves; thread -> (query, dim)
-    float* ws = a.ws + (int64_t)blockIdx.x * kNQ * WS_ROW;
-    for (int e = threadIdx.x; e < kNQ * D; e += 256) {
-        const int q = e / D, d = e - q * D;
-        float mm = kNegBig;
+    float* ws = a.ws + (((int64_t)block * a.n_kv_heads + hk) * a.nsplit + split) * kNQ * WS_ROW + c16 * WS_ROW;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) mm = fmaxf(mm, sh_ml[w][q][0]);
-        float v = 0.0f, ll = 0.0f;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const float f = __expf(sh_ml[w][q][0] - mm);
-            v += sh_acc[w][q][d] * f;
-            ll += sh_ml[w][q][1] * f;
-        }
-        ws[q * WS_ROW + d] = v;
-        if (d == 0) {
-            ws[q * WS_ROW + D] = mm;
-            ws[q * WS_ROW + D + 1] = ll;
-        }
+    for (int c = 0; c < CHUNKS; ++c) {  // (a workspace row starts on an 8-byte boundary only)
+        *reinterpret_cast<f32x2_hw*>(ws + 16 * c + 4 * g) = f32x2_hw{o[c][0], o[c][1]};
+        *reinterpret_cast<f32x2_hw*>(ws + 16 * c + 4 * g + 2) = f32x2_hw{o[c][2], o[c][3]};
+    }
+    if (g == 0) {
+        ws[D] = m;
+        ws[D + 1] = l;
     }
 }
 
-// One workgroup per query row slot of the schedule (decode: per sequence): merges the
-// splits of every head of the row and writes out[row, head, :] in bf16.
+// With a context split: one workgroup per query row slot of the schedule (decode: per
+// sequence) merges the splits of every head of the row and writes out[row, head, :] in bf16.
 template <int D>
 __global__ __launch_bounds__(256) void attn_rows_merge_kernel(AttnRowsArgs a) {
     constexpr int WS_ROW = D + 2;
@@ -317,12 +329,12 @@ __global__ __launch_bounds__(256) void attn_rows_merge_kernel(AttnRowsArgs a) {
             for (int d = 0; d < 8; ++d) v[d] += r[d0 + d] * f;
         }
         const float inv = ll > 0.0f ? 1.0f / ll : 0.0f;  // a row with no visible key yields zeros
-        u32x4 o;
-        o.x = pack_bf16x2(v[0] * inv, v[1] * inv);
-        o.y = pack_bf16x2(v[2] * inv, v[3] * inv);
-        o.z = pack_bf16x2(v[4] * inv, v[5] * inv);
-        o.w = pack_bf16x2(v[6] * inv, v[7] * inv);
-        *reinterpret_cast<u32x4*>(out + e) = o;
+        u32x4 ov;
+        ov.x = pack_bf16x2(v[0] * inv, v[1] * inv);
+        ov.y = pack_bf16x2(v[2] * inv, v[3] * inv);
+        ov.z = pack_bf16x2(v[4] * inv, v[5] * inv);
+        ov.w = pack_bf16x2(v[6] * inv, v[7] * inv);
+        *reinterpret_cast<u32x4*>(out + e) = ov;
     }
 }
 
@@ -332,7 +344,7 @@ void launch_for_dim(const AttnRowsArgs& a, unsigned grid1, unsigned grid2, hipSt
         attn_rows_partial_kernel<D, true><<<dim3(grid1), dim3(256), 0, stream>>>(a);
     else
         attn_rows_partial_kernel<D, false><<<dim3(grid1), dim3(256), 0, stream>>>(a);
-    attn_rows_merge_kernel<D><<<dim3(grid2), dim3(256), 0, stream>>>(a);
+    if (a.nsplit > 1) attn_rows_merge_kernel<D><<<dim3(grid2), dim3(256), 0, stream>>>(a);
 }
 
 }  // namespace
@@ -359,6 +371,8 @@ int64_t attn_rows_blocks(int64_t batch_or_tiles, int n_heads, int n_kv_heads, bo
 
 int64_t attn_rows_workspace_floats(int64_t batch_or_tiles, int n_heads, int n_kv_heads, int head_dim,
                                    int nsplit, bool prefill) {
+    if (!attn_rows_supported(n_heads, n_kv_heads, head_dim)) return -1;
+    if (nsplit <= 1) return 0;  // each wave owns a whole context and writes the output itself
     return attn_rows_blocks(batch_or_tiles, n_heads, n_kv_heads, prefill) * n_kv_heads * nsplit * kNQ *
            (head_dim + 2);
 }
@@ -366,13 +380,15 @@ int64_t attn_rows_workspace_floats(int64_t batch_or_tiles, int n_heads, int n_kv
 bool launch_attn_rows(AttnRowsArgs a, hipStream_t stream) {
     if (!attn_rows_supported(a.n_heads, a.n_kv_heads, a.head_dim) || a.nsplit <= 0 || a.num_blocks <= 0) return false;
     if (!a.req_to_token || !a.req_pool_indices || !a.kv_indptr || a.rtt_stride <= 0) return false;
+    if (a.nsplit > 1 && !a.ws) return false;
     const bool prefill = a.qo_indptr != nullptr;
     if (prefill && (!a.q_tile_to_batch || !a.q_tile_to_index)) return false;
     if (a.mask && (a.mask_width <= 0 || a.mask_rows <= 0)) return false;
     a.rows_per_block = prefill ? attn_rows_per_block(a.n_heads, a.n_kv_heads) : 1;
     a.blocks_per_tile = prefill ? 64 / a.rows_per_block : 1;
     const int64_t blocks = attn_rows_blocks(a.num_blocks, a.n_heads, a.n_kv_heads, prefill);
-    const int64_t grid1 = blocks * a.n_kv_heads * a.nsplit;
+    a.num_items = blocks * a.n_kv_heads * a.nsplit;  // one wave each, four to a workgroup
+    const int64_t grid1 = (a.num_items + 3) / 4;
     const int64_t grid2 = prefill ? blocks * a.rows_per_block : blocks;
     if (grid1 > INT_MAX || grid2 > INT_MAX) return false;
     switch (a.head_dim) {

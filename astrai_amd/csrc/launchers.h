@@ -176,6 +176,7 @@ struct AttnRowsArgs {
     int64_t mask_b_stride, mask_h_stride, mask_l_stride;
     int mask_rows, mask_width;
     int rows_per_block, blocks_per_tile;  // filled in by the launcher
+    int64_t num_items;                    // (row block, kv head, split) triples, filled in by the launcher
 };
 bool attn_rows_supported(int n_heads, int n_kv_heads, int head_dim);
 int64_t attn_rows_workspace_floats(int64_t batch_or_tiles, int n_heads, int n_kv_heads, int head_dim,

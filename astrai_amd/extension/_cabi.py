@@ -692,6 +692,7 @@ def attn_paged_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     rtt, rpi, ind = req_to_token.contiguous(), req_pool_indices.contiguous(), kv_indptr.contiguous()
     if scale is None or scale <= 0.0:
         scale = d ** -0.5
+    user_nsplit = nsplit > 0
     if nsplit <= 0:
         nsplit = max(1, min(16, 384 // max(1, b * hkv)))  # a few hundred workgroups: more splits cost more in the merge than they hide
     with torch.cuda.device(q.device):
@@ -713,7 +714,9 @@ def attn_paged_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         else:
             out = torch.empty((b, h, d), device=q.device, dtype=torch.bfloat16)
         m_ptr, m_stride, m_width = (mask.data_ptr(), mask.stride(0), mask.size(1)) if mask is not None else (0, 0, 0)
-        if d != 128 or h > 64:  # the shapes only the general kernel takes
+        if d != 128 or h > 64 or h // hkv > 8:  # the shapes only the general kernel takes
+            if not user_nsplit:  # one wave per (sequence, kv head, split): enough of them to fill the chip
+                nsplit = max(1, min(64, 2048 // max(1, b * hkv), rtt.size(1) // 64))
             _paged_rows(lib, q_c, k_cache, v_cache, rtt, rpi, ind, None, (m_ptr, m_stride, 0, 0, 1, m_width),
                         out, b, nsplit, False, scale)
             return out
@@ -734,8 +737,8 @@ def _paged_rows(lib, q, k_pool, v_pool, rtt, rpi, kv_indptr, schedule, m_args, o
     h, d, hkv = q.size(1), q.size(2), k_pool.size(1)
     prefill = schedule is not None
     need = lib.astrai_w8a8_attn_paged_rows_workspace_floats(count, h, hkv, d, nsplit, 1 if prefill else 0)
-    if count and need <= 0:
-        raise RuntimeError(f"paged attention needs head_dim in (32, 64, 128, 256) and n_heads / n_kv_heads <= 8; "
+    if need < 0:
+        raise RuntimeError(f"paged attention needs head_dim in (32, 64, 128, 256) and n_heads / n_kv_heads <= 16; "
                            f"got head_dim {d}, {h} / {hkv} heads")
     ws = torch.empty(max(need, 1), device=q.device, dtype=torch.float32)
     sched = [t.data_ptr() for t in schedule] if prefill else [0, 0, 0]
@@ -816,9 +819,9 @@ def attn_paged_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Te
         out = torch.empty((total_q, h, d), device=q.device, dtype=torch.bfloat16)
         if not attn_prefill_supported(h, hkv, d):  # the shapes only the general kernel takes
             tiles = q_tile_to_batch.numel()
-            blocks = tiles * 8 * hkv                 # at least: 8 row blocks per 64-row tile
+            waves = tiles * 4 * hkv                  # at least: one wave per row block, 4+ blocks per tile
             _paged_rows(lib, q_c, k_cache, v_cache, tensors[0], tensors[1], tensors[2], tensors[3:], m_args,
-                        out, tiles, max(1, min(16, 384 // max(1, blocks))), causal_offset >= 0, scale)
+                        out, tiles, max(1, min(16, 2048 // max(1, waves))), causal_offset >= 0, scale)
             return out
         _check(lib.astrai_w8a8_attn_paged_prefill_masked_bf16(
             q_c.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), *[t.data_ptr() for t in tensors],
@@ -1139,13 +1142,14 @@ def attn_decode_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Opt
     m4 = _dense_mask(mask, b, 1, kv_len, h)
     if m4 is not None and m4.size(1) != 1:
         raise RuntimeError("attn_decode: a mask per head is not supported")
-    if d not in (32, 64, 128, 256) or h // hkv > 8:
-        raise RuntimeError("attn_decode needs head_dim in (32, 64, 128, 256) and n_heads / n_kv_heads <= 8")
+    if d not in (32, 64, 128, 256) or h // hkv > 16:
+        raise RuntimeError("attn_decode needs head_dim in (32, 64, 128, 256) and n_heads / n_kv_heads <= 16")
     attend = kv_len if causal_offset < 0 else min(kv_len, causal_offset + 1)
     with torch.cuda.device(q.device):
         if kv_len == 0 or b == 0:
             return torch.zeros_like(q)
-        if layout == BHLD and m4 is None and k.is_contiguous() and v.is_contiguous() and d == 128 and h <= 64:
+        if layout == BHLD and m4 is None and k.is_contiguous() and v.is_contiguous() and d == 128 and h <= 64 \
+                and h // hkv <= 8:
             pos = torch.full((1,), attend - 1, dtype=torch.int64, device=q.device)
             out = attn_decode(q.contiguous(), k, v, pos, scale=scale if scale > 0 else None)
             return out.reshape(b, h, 1, d)
@@ -1169,8 +1173,8 @@ def attn_prefill_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Op
     ``kv_len - q_len`` is expressed through the mask."""
     b, q_len, kv_len, h, hkv, d = _dense_args(q, k, v, layout, "attn_prefill")
     m4 = _dense_mask(mask, b, q_len, kv_len, h)
-    if d not in (32, 64, 128, 256) or h // hkv > 8:
-        raise RuntimeError("attn_prefill needs head_dim in (32, 64, 128, 256) and n_heads / n_kv_heads <= 8")
+    if d not in (32, 64, 128, 256) or h // hkv > 16:
+        raise RuntimeError("attn_prefill needs head_dim in (32, 64, 128, 256) and n_heads / n_kv_heads <= 16")
     with torch.cuda.device(q.device):
         if kv_len == 0 or b == 0 or q_len == 0:
             return torch.zeros_like(q)

@@ -326,7 +326,7 @@ int astrai_w8a8_attn_paged_prefill_masked_bf16(
 
 /*
  * Paged attention for the shapes the tuned kernels above do not take: head_dim 32, 64, 128 or
- * 256 and any n_heads / n_kv_heads up to 8 -- the reference's paged kernels accept those
+ * 256 and any n_heads / n_kv_heads up to 16 -- the reference's paged kernels accept those
  * head_dims and any grouping (astrai/extension/backend/attention.py:518-527; its tests run
  * head_dim 64, tests/extension/conftest.py:9-20). One entry for both reference entries:
  *   qo_indptr == NULL  decode, as attn_paged_decode_masked_bf16: q / out [batch, n_heads,
@@ -334,10 +334,15 @@ int astrai_w8a8_attn_paged_prefill_masked_bf16(
  *              2D mask (head and row stride 0)
  *   qo_indptr != NULL  ragged prefill, as attn_paged_prefill_masked_bf16: packed q / out
  *              [total_q, n_heads, head_dim], the 64-row tile schedule, batch_or_tiles = tiles
- * Same arithmetic as attn_decode_bf16 (bf16 MFMA scores, fp32 softmax and P.V, one rounding);
- * correct for every shape, not tuned (prefill re-reads the keys once per block of at most
- * 8 / (n_heads / n_kv_heads) rows). workspace: attn_paged_rows_workspace_floats(...) floats,
- * 0 from that function = unsupported shape. nsplit in [1, 64] splits the context.
+ * One wave per (block of up to 16 / (n_heads / n_kv_heads) query rows, KV head, context
+ * split): bf16 MFMAs for the scores and for P.V (P as a bf16 head plus a bf16 remainder), fp32
+ * softmax statistics and accumulation, one rounding of the output. Correct for every shape,
+ * not tuned like the head_dim-128 kernels (prefill re-reads the keys once per row block).
+ *   nsplit     in [1, 64]: 1 = every wave owns a whole context and writes the output itself,
+ *              no workspace (NULL allowed); > 1 = partial results in the workspace and a
+ *              merge kernel
+ *   workspace  attn_paged_rows_workspace_floats(...) floats (0 for nsplit == 1; that function
+ *              returns -1 for a shape this entry does not take)
  */
 int64_t astrai_w8a8_attn_paged_rows_workspace_floats(int64_t batch_or_tiles, int64_t n_heads,
                                                      int64_t n_kv_heads, int64_t head_dim,

@@ -209,7 +209,7 @@ def _paged_case(b, h, hkv, d, kv_lens, q_lens, seed, holes=False):
 
 
 @pytest.mark.parametrize("d", [32, 64, 256])
-@pytest.mark.parametrize("h,hkv", [(2, 1), (4, 4), (6, 2), (8, 1), (16, 4)])
+@pytest.mark.parametrize("h,hkv", [(2, 1), (4, 4), (6, 2), (8, 1), (16, 4), (16, 1), (24, 2)])
 def test_paged_decode_other_head_dims_and_groupings(d, h, hkv):
     """head_dim 64 with 2 heads on 1 KV head is the reference's own test model
     (tests/extension/conftest.py:9-20)."""
@@ -231,7 +231,8 @@ def test_paged_decode_other_head_dims_and_groupings(d, h, hkv):
         assert_bf16_close(got, want, what=f"decode d={d} nsplit={nsplit}")
 
 
-@pytest.mark.parametrize("d,h,hkv", [(64, 2, 1), (64, 4, 4), (32, 8, 1), (256, 4, 2), (128, 4, 4), (128, 6, 2), (64, 16, 2)])
+@pytest.mark.parametrize("d,h,hkv", [(64, 2, 1), (64, 4, 4), (32, 8, 1), (256, 4, 2), (128, 4, 4), (128, 6, 2), (64, 16, 2),
+                                     (128, 16, 1), (64, 10, 2), (256, 3, 3)])
 @pytest.mark.parametrize("causal", [True, False])
 def test_paged_prefill_other_head_dims_and_groupings(d, h, hkv, causal):
     """The shapes the MFMA prefill kernel does not take (head_dim != 128, or a grouping other
@@ -269,7 +270,14 @@ def test_general_kernel_agrees_with_the_tuned_kernels_where_both_apply():
     tuned = _cabi.attn_paged_decode(q1, kp, vp, table, rows, kvp, nsplit=2)
     out = torch.empty_like(tuned)
     _cabi._paged_rows(lib, q1, kp, vp, table, rows, kvp, None, (0, 0, 0, 0, 0, 0), out, 3, 2, False, 128 ** -0.5)
-    assert torch.equal(out, tuned)                 # same arithmetic, same split points
+    assert_bf16_close(out, tuned, what="rows kernel vs tuned decode kernel")
+    out1 = torch.empty_like(tuned)                 # without a split the waves write the output themselves
+    _cabi._paged_rows(lib, q1, kp, vp, table, rows, kvp, None, (0, 0, 0, 0, 0, 0), out1, 3, 1, False, 128 ** -0.5)
+    assert_bf16_close(out1, tuned, what="rows kernel, no split")
+    outp = torch.empty(q.shape, dtype=q.dtype, device=DEV)
+    _cabi._paged_rows(lib, q, kp, vp, table, rows, kvp, (qo, tb, ti), (0, 0, 0, 0, 0, 0), outp, tb.numel(), 1, True,
+                      128 ** -0.5)
+    _close(outp, _cabi.attn_paged_prefill(q, kp, vp, table, rows, kvp, qo, tb, ti, causal_offset=0), "rows prefill, no split")
 
 
 @pytest.mark.parametrize("layout", [0, 1])
