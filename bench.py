@@ -265,6 +265,22 @@ def main():
         table = torch.randperm(b_ * n_, device=dev).int().reshape(b_, n_).contiguous()
         rows = torch.arange(b_, dtype=torch.int32, device=dev)
         indptr = (torch.arange(b_ + 1, device=dev) * n_).int()
+        # the reference-facing attention entries: ragged paged prefill (tuned kernel, with and without a
+        # mask tensor), the same workload at head_dim 64 on the general kernel, rotary embedding
+        qp = q.permute(0, 2, 1, 3).reshape(b_ * s_, h_, 128).contiguous()
+        qo, tb, ti = _cabi.paged_prefill_schedule([s_] * b_, dev)
+        key_mask = torch.ones(b_, n_, dtype=torch.bool, device=dev)
+        q64 = torch.randn(b_ * s_, 2 * h_, 64, device=dev).to(torch.bfloat16)
+        k64 = torch.randn(b_ * n_, 2 * hkv_, 64, device=dev).to(torch.bfloat16)
+        v64 = torch.randn(b_ * n_, 2 * hkv_, 64, device=dev).to(torch.bfloat16)
+        freqs = torch.randn(b_ * s_, 64, 2, device=dev)
+        for _ in range(5):
+            _cabi.attn_paged_prefill(qp, k_pool, v_pool, table, rows, indptr, qo, tb, ti, causal_offset=0)
+            _cabi.attn_paged_prefill(qp, k_pool, v_pool, table, rows, indptr, qo, tb, ti, mask=key_mask,
+                                     causal_offset=0)
+            _cabi.attn_paged_prefill(q64, k64, v64, table, rows, indptr, qo, tb, ti, causal_offset=0)
+            _cabi.attn_paged_decode(q64[:b_].contiguous(), k64, v64, table, rows, indptr)
+            _cabi.rotary_emb(qp, freqs)
         for _ in range(5):
             x8, amax = fp8m.quantize_bf16(x, s1, 0)                    # quantize_fp8_kernel
             fp8m.quantize_transpose_bf16(x, s1, 0, True, True)         # quantize_transpose_fp8_kernel
