@@ -756,7 +756,7 @@ def attn_paged_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Te
                        kv_indptr: torch.Tensor, qo_indptr: torch.Tensor,
                        q_tile_to_batch: torch.Tensor, q_tile_to_index: torch.Tensor,
                        mask: Optional[torch.Tensor] = None, causal_offset: int = -1,
-                       scale: float = 0.0) -> torch.Tensor:
+                       scale: float = 0.0, nsplit: int = 0) -> torch.Tensor:
     """Ragged paged prefill with the argument list of the reference's pybind entry
     (csrc/kernels/attention/paged_prefill.cu:36-52): packed ``q [total_q, H, 128]``, flat
     pools, ``req_to_token`` / ``req_pool_indices`` / ``kv_indptr`` / ``qo_indptr`` int32, and
@@ -764,7 +764,9 @@ def attn_paged_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Te
     wrapper passes 0 for ``is_causal``, astrai/extension/ops/attention.py:188). ``mask``:
     bool, True = attend, ``[batch, kv]`` or ``[batch, 1 | H, rows, kv]`` with ``rows`` counted
     inside each sequence (entry_utils.cuh:326-346); rows and positions the mask does not hold
-    are not attended. Returns ``[total_q, H, 128]`` bf16."""
+    are not attended. Returns ``[total_q, H, head_dim]`` bf16. head_dim 128 with a grouping of
+    2, 4 or 8 runs the MFMA block kernel; other shapes the general kernel, whose context split
+    ``nsplit`` (0: chosen here) only matters for short schedules."""
     lib = _require()
     _gpu(q, "attn_paged_prefill")
     m_args = (0, 0, 0, 0, 0, 0)
@@ -821,7 +823,8 @@ def attn_paged_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Te
             tiles = q_tile_to_batch.numel()
             waves = tiles * 4 * hkv                  # at least: one wave per row block, 4+ blocks per tile
             _paged_rows(lib, q_c, k_cache, v_cache, tensors[0], tensors[1], tensors[2], tensors[3:], m_args,
-                        out, tiles, max(1, min(16, 2048 // max(1, waves))), causal_offset >= 0, scale)
+                        out, tiles, nsplit if nsplit > 0 else max(1, min(16, 2048 // max(1, waves))),
+                        causal_offset >= 0, scale)
             return out
         _check(lib.astrai_w8a8_attn_paged_prefill_masked_bf16(
             q_c.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), *[t.data_ptr() for t in tensors],

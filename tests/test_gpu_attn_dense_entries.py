@@ -244,12 +244,19 @@ def test_paged_prefill_other_head_dims_and_groupings(d, h, hkv, causal):
     qo, tb, ti = _cabi.paged_prefill_schedule(q_lens, DEV)
     got = ops.attn_paged_prefill(*dev, qo, tb, ti, is_causal=causal)
     assert got.shape == (sum(q_lens), h, d)
-    _close(got, D.attn_paged_prefill(*args, qo.cpu(), causal=causal), f"prefill d={d} {h}/{hkv} causal={causal}")
+    want = D.attn_paged_prefill(*args, qo.cpu(), causal=causal)
+    _close(got, want, f"prefill d={d} {h}/{hkv} causal={causal}")
+    off = 0 if causal else -1
+    for nsplit in (1, 3):       # 1: workgroups of four row blocks sharing the key tiles; 3: split context + merge
+        got = _cabi.attn_paged_prefill(*dev, qo, tb, ti, causal_offset=off, nsplit=nsplit)
+        _close(got, want, f"prefill d={d} {h}/{hkv} causal={causal} nsplit={nsplit}")
     g = torch.Generator().manual_seed(d)
     for shape in ((4, max(kv_lens) + 3), (4, 1, max(q_lens), max(kv_lens)), (4, h, max(q_lens), max(kv_lens))):
         mask = torch.rand(shape, generator=g) < 0.6
-        got = ops.attn_paged_prefill(*dev, qo, tb, ti, mask=mask.to(DEV), is_causal=causal)
-        _close(got, D.attn_paged_prefill(*args, qo.cpu(), causal=causal, mask=mask), f"prefill d={d} mask {shape}")
+        want = D.attn_paged_prefill(*args, qo.cpu(), causal=causal, mask=mask)
+        for nsplit in (0, 1):
+            got = _cabi.attn_paged_prefill(*dev, qo, tb, ti, mask=mask.to(DEV), causal_offset=off, nsplit=nsplit)
+            _close(got, want, f"prefill d={d} mask {shape} nsplit={nsplit}")
 
 
 def test_general_kernel_agrees_with_the_tuned_kernels_where_both_apply():
