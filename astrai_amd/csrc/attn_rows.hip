@@ -99,7 +99,8 @@ __device__ __forceinline__ RowBlock row_block(const AttnRowsArgs& a, int block) 
 // One 16-key tile for the 16 query columns of a wave. kf: the keys as MFMA rows (lane -> key
 // c16, dims 32 step + 8g); qf: the queries likewise; keep: mask bytes of this lane's four keys;
 // v_tr: where this lane's transposing reads of the staged value rows point (chunk 0); key0: the
-// position of this lane's first key (tile start + 4g). Updates the running (m, l) of query c16
+// position of this lane's first key (tile start + 4g). Updates the running maximum m of query
+// c16 (equal in its four lanes), this lane's share l of its running sum (finish with query_sum)
 // and its accumulators o[c][i] (dim 16c + 4g + i).
 template <int D, bool MASK>
 __device__ __forceinline__ void tile_step(const u32x4 (&kf)[D / 32], const u32x4 (&qf)[D / 32],
@@ -129,9 +130,7 @@ __device__ __forceinline__ void tile_step(const u32x4 (&kf)[D / 32], const u32x4
         p[i] = (sc[i] > 0.5f * kNegBig) ? __expf(sc[i] - m_new) : 0.0f;
         ps += p[i];
     }
-    ps += __shfl_xor(ps, 16, kWave);
-    ps += __shfl_xor(ps, 32, kWave);
-    l = l * alpha + ps;
+    l = l * alpha + ps;  // this lane's four keys only: the four lanes of a query are added up at the end
     m = m_new;
 
     // P as the column operand (query c16, keys key0 .. key0+3): bf16 head and bf16 remainder
@@ -148,6 +147,11 @@ __device__ __forceinline__ void tile_step(const u32x4 (&kf)[D / 32], const u32x4
         acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vt, p_hi, acc, 0, 0, 0);
         o[c] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vt, p_lo, acc, 0, 0, 0);
     }
+}
+
+__device__ __forceinline__ float query_sum(float l) {
+    l += __shfl_xor(l, 16, kWave);
+    return l + __shfl_xor(l, 32, kWave);
 }
 
 // workspace per (row block, kv head, split): kNQ rows of [D values | max | sum]
@@ -213,7 +217,7 @@ __global__ __launch_bounds__(256) void attn_rows_partial_kernel(AttnRowsArgs a) 
         mask_keys = covered ? a.mask_width : 0;
     }
 
-    float m = kNegBig, l = 0.0f;  // of query c16, equal in its four lanes
+    float m = kNegBig, l = 0.0f;  // running maximum of query c16 (equal in its four lanes); this lane's share of its sum
     // o[c][i] = sum over keys of p * v for query c16, dim 16c + 4g + i
     f32x4 o[CHUNKS];
 #pragma unroll
@@ -289,6 +293,7 @@ __global__ __launch_bounds__(256) void attn_rows_partial_kernel(AttnRowsArgs a) 
         tile_step<D, MASK>(kf, qf, keep, tr_mine, kb + 4 * g, q_live, q_pos, a.scale, m, l, o);
     }
 
+    l = query_sum(l);
     if (a.nsplit == 1) {
         // the whole context was this wave's: normalise and write out[row, head, 16c + 4g ..+3]
         if (!q_live) return;
@@ -430,6 +435,7 @@ __global__ __launch_bounds__(256) void attn_rows_shared_kernel(AttnRowsArgs a) {
             tile_step<D, MASK>(kf, qf, keep, v_stage[buf] + v_get, (t << 4) + 4 * g, q_live, q_pos, a.scale, m, l, o);
         }
     }
+    l = query_sum(l);
     if (!q_live) return;
     const float inv = l > 0.0f ? 1.0f / l : 0.0f;  // a row with no visible key yields zeros
     uint16_t* orow = static_cast<uint16_t*>(a.out) + ((int64_t)(rb.q_start + row) * a.n_heads + head) * D + 4 * g;
