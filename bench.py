@@ -297,14 +297,15 @@ def main():
         return
 
     if args.trace_gemms:
-        from oracle import w8a8_oracle as O
-
         xq = torch.randint(-127, 128, (4096, 4096), dtype=torch.int8, device=dev)
         wq = torch.randint(-127, 128, (4096, 4096), dtype=torch.int8, device=dev)
         sx, sw = torch.rand(4096, device=dev) + 0.5, torch.rand(4096, device=dev) + 0.5
         y = torch.empty(4096, 4096, device=dev, dtype=torch.bfloat16)
         # config 3 data (seed 3, 1% x20 outliers in the weight), quantized on the device
-        x3, w3, _ = O.make_inputs(3, 8192, 2048, 7168, outlier_p=0.01)
+        g3 = torch.Generator().manual_seed(3)   # activation, weight, outlier mask, in this order
+        x3 = torch.randn(8192, 7168, generator=g3).to(torch.bfloat16)
+        w3 = torch.randn(2048, 7168, generator=g3) * 0.02
+        w3 = torch.where(torch.rand(2048, 7168, generator=g3) < 0.01, w3 * 20.0, w3).to(torch.bfloat16)
         a3, sa3 = _cabi.quantize_fp8_block128_act(x3.to(dev))
         b3, sb3 = _cabi.quantize_fp8_block128_weight(w3.to(dev))
         y3 = torch.empty(8192, 2048, device=dev, dtype=torch.bfloat16)
