@@ -109,3 +109,53 @@ def test_paged_decode_appends_new_kv_in_kernel():
     kr[out_cache_loc], vr[out_cache_loc] = new_k, new_v
     want = O.attn_paged_decode(q, kr, vr, req_to_token, torch.arange(2, dtype=torch.int32), kv_indptr)
     assert (out.float().cpu() - want.float()).abs().max().item() < 2e-2
+
+
+@pytest.mark.parametrize("d,h,hkv", [(D, 2, 1), (128, 16, 4)])
+def test_paged_decode_graph_replay_is_exact(d, h, hkv):
+    """Kernel-level counterpart of tests/extension/test_backend_equivalence.py:216-272: the decode
+    call (new K/V stored, output into ``out_buf``) captured once into a HIP graph and replayed
+    while the sequences grow; every replay equals the eager call on the same state, bit for bit.
+    Eager work and synchronisations sit between the replays."""
+    from astrai_amd.extension.ops import attn_paged_decode
+    g = torch.Generator().manual_seed(d + h)
+    b, max_ctx, pool = 3, 48, 200
+    k_buf = torch.randn(pool, hkv, d, generator=g).to(torch.bfloat16).to(DEV)
+    v_buf = torch.randn(pool, hkv, d, generator=g).to(torch.bfloat16).to(DEV)
+    table = torch.randperm(pool, generator=g)[: b * max_ctx].int().reshape(b, max_ctx).to(DEV)
+    rows = torch.arange(b, dtype=torch.int32, device=DEV)
+    lens = torch.tensor([5, 17, 30])
+    q = torch.zeros(b, h, d, dtype=torch.bfloat16, device=DEV)
+    new_k = torch.zeros(b, hkv, d, dtype=torch.bfloat16, device=DEV)
+    new_v = torch.zeros_like(new_k)
+    indptr = torch.zeros(b + 1, dtype=torch.int32, device=DEV)
+    out_buf = torch.zeros(b, h, d, dtype=torch.bfloat16, device=DEV)
+
+    def call(kb, vb, out):
+        return attn_paged_decode(q, kb, vb, table, rows, indptr, new_k=new_k, new_v=new_v, is_causal=True, out_buf=out)
+
+    def step_inputs(step):
+        q.copy_(torch.randn(b, h, d, generator=g).to(torch.bfloat16))
+        new_k.copy_(torch.randn(b, hkv, d, generator=g).to(torch.bfloat16))
+        new_v.copy_(torch.randn(b, hkv, d, generator=g).to(torch.bfloat16))
+        indptr.copy_(torch.tensor([0] + (lens + step).cumsum(0).tolist(), dtype=torch.int32))
+
+    step_inputs(1)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                     # warm-up off the capture, on copies of the pools
+        call(k_buf.clone(), v_buf.clone(), torch.empty_like(out_buf))
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(k_buf, v_buf, out_buf)
+    for step in range(1, 6):
+        step_inputs(step)
+        ke, ve = k_buf.clone(), v_buf.clone()          # eager reference on the state before the replay
+        want = call(ke, ve, torch.empty_like(out_buf)).clone()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_buf, want), step
+        assert torch.equal(k_buf, ke) and torch.equal(v_buf, ve), step
