@@ -654,8 +654,9 @@ def attn_paged_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     ``[batch, H, 128]`` bf16. ``new_k`` / ``new_v`` (``[batch, H_kv, 128]``) are first
     written to the slot of each sequence's newest position, as the reference's kernel
     persists them (layout_policies.cuh:226-252). ``causal_offset`` does not change a
-    one-token query (layout_policies.cuh:194-197); the split buffers are not needed
-    (the workspace is allocated here). ``mask``: bool ``[batch, width]``, True = attend
+    one-token query (layout_policies.cuh:194-197); ``o_part_buf`` (fp32, contiguous) serves as
+    the split workspace when it is large enough, otherwise one is allocated here;
+    ``ml_part_buf`` is not needed. ``mask``: bool ``[batch, width]``, True = attend
     that position (entry_utils.cuh:226-237); positions past ``width`` are not attended."""
     lib = _require()
     _gpu(q, "attn_paged_decode")
@@ -718,10 +719,10 @@ def attn_paged_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
             if not user_nsplit:  # one wave per (sequence, kv head, split): enough of them to fill the chip
                 nsplit = max(1, min(64, 2048 // max(1, b * hkv), rtt.size(1) // 64))
             _paged_rows(lib, q_c, k_cache, v_cache, rtt, rpi, ind, None, (m_ptr, m_stride, 0, 0, 1, m_width),
-                        out, b, nsplit, False, scale)
+                        out, b, nsplit, False, scale, o_part_buf)
             return out
         need = lib.astrai_w8a8_attn_decode_workspace_floats(b, hkv, nsplit, h // hkv)
-        ws = torch.empty(max(need, 1), device=q.device, dtype=torch.float32)
+        ws = _scratch(need, q.device, o_part_buf)
         _check(lib.astrai_w8a8_attn_paged_decode_masked_bf16(
             q_c.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), rtt.data_ptr(), rpi.data_ptr(),
             ind.data_ptr(), m_ptr, m_stride, m_width, ws.data_ptr(), ws.numel(), out.data_ptr(), b, h, hkv,
@@ -729,8 +730,18 @@ def attn_paged_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     return out
 
 
+def _scratch(need: int, device, given: Optional[torch.Tensor]) -> torch.Tensor:
+    """``need`` fp32 elements of scratch: the caller's pre-allocated buffer when it is large
+    enough (the reference's callers hand over their split buffers so that a captured decode step
+    allocates nothing), else a fresh tensor."""
+    if given is not None and given.is_cuda and given.device == device and given.dtype == torch.float32 \
+            and given.is_contiguous() and given.numel() >= need:
+        return given.view(-1)
+    return torch.empty(max(need, 1), device=device, dtype=torch.float32)
+
+
 def _paged_rows(lib, q, k_pool, v_pool, rtt, rpi, kv_indptr, schedule, m_args, out, count, nsplit, causal,
-                scale) -> None:
+                scale, scratch: Optional[torch.Tensor] = None) -> None:
     """The general paged kernel (any head_dim in {32, 64, 128, 256}, n_rep <= 8). ``schedule``:
     ``(qo_indptr, q_tile_to_batch, q_tile_to_index)`` for a prefill call (``count`` = tiles),
     None for decode (``count`` = batch)."""
@@ -740,7 +751,7 @@ def _paged_rows(lib, q, k_pool, v_pool, rtt, rpi, kv_indptr, schedule, m_args, o
     if need < 0:
         raise RuntimeError(f"paged attention needs head_dim in (32, 64, 128, 256) and n_heads / n_kv_heads <= 16; "
                            f"got head_dim {d}, {h} / {hkv} heads")
-    ws = torch.empty(max(need, 1), device=q.device, dtype=torch.float32)
+    ws = _scratch(need, q.device, scratch)
     sched = [t.data_ptr() for t in schedule] if prefill else [0, 0, 0]
     _check(lib.astrai_w8a8_attn_paged_rows_bf16(
         q.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), rtt.data_ptr(), rpi.data_ptr(), kv_indptr.data_ptr(),

@@ -95,6 +95,15 @@ def test_paged_decode_appends_new_kv_like_the_reference_entry():
     got = _cabi.attn_paged_decode(q.to(DEV), kd, vd, table.to(DEV), rows.to(DEV), indptr.to(DEV),
                                   new_k=new_k.to(DEV), new_v=new_v.to(DEV), out_buf=out_buf)
     assert_bf16_close(got, want, what="append")
+    # the caller's split buffer is used as the workspace when it is large enough (and is scribbled on)
+    big = torch.full((1 << 20,), float("nan"), device=DEV)
+    again = _cabi.attn_paged_decode(q.to(DEV), kd, vd, table.to(DEV), rows.to(DEV), indptr.to(DEV), nsplit=4,
+                                    o_part_buf=big, ml_part_buf=torch.empty(8, device=DEV))
+    assert_bf16_close(again, want, what="caller's split buffer")
+    assert torch.isfinite(big[:64]).any()
+    small = _cabi.attn_paged_decode(q.to(DEV), kd, vd, table.to(DEV), rows.to(DEV), indptr.to(DEV), nsplit=4,
+                                    o_part_buf=torch.empty(16, device=DEV))
+    assert torch.equal(small, again)
     assert got.data_ptr() == out_buf.data_ptr() and torch.equal(out_buf[3:].cpu(), torch.zeros(2, 8, 128, dtype=torch.bfloat16))
     live = torch.isfinite(kp.float()).all(-1).all(-1)
     assert torch.equal(kd.cpu()[live], kp[live]) and torch.equal(vd.cpu()[live], vp[live])
