@@ -714,6 +714,8 @@ def attn_paged_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
             out = out_buf[:b]
         else:
             out = torch.empty((b, h, d), device=q.device, dtype=torch.bfloat16)
+        if b == 0:
+            return out  # (an empty tensor has no address to hand over)
         m_ptr, m_stride, m_width = (mask.data_ptr(), mask.stride(0), mask.size(1)) if mask is not None else (0, 0, 0)
         if d != 128 or h > 64 or h // hkv > 8:  # the shapes only the general kernel takes
             if not user_nsplit:  # one wave per (sequence, kv head, split): enough of them to fill the chip
@@ -830,6 +832,8 @@ def attn_paged_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Te
     with torch.cuda.device(q.device):
         # (rows that no tile of the schedule covers are left unwritten, as by the reference)
         out = torch.empty((total_q, h, d), device=q.device, dtype=torch.bfloat16)
+        if total_q == 0 or q_tile_to_batch.numel() == 0:
+            return out  # (an empty tensor has no address to hand over)
         if not attn_prefill_supported(h, hkv, d):  # the shapes only the general kernel takes
             tiles = q_tile_to_batch.numel()
             waves = tiles * 4 * hkv                  # at least: one wave per row block, 4+ blocks per tile

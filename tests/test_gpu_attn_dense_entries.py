@@ -306,3 +306,35 @@ def test_dense_entries_head_dim_64_like_the_reference_test_model(layout):
     assert_bf16_close(got, D.attn_dense(q1, k, v, layout=layout), what=f"decode layout {layout}")
     with pytest.raises(RuntimeError, match="head_dim"):
         pre(dev[0][..., :48], dev[1][..., :48], dev[2][..., :48], layout=layout)
+
+
+@pytest.mark.parametrize("d", [64, 128])
+def test_attention_entries_with_nothing_to_do(d):
+    """Empty batch, empty schedule, sequences without keys or without query rows: shapes come
+    back right, nothing is launched out of bounds, rows without keys are zeros."""
+    from astrai_amd.extension import _cabi, get_module, ops
+    h, hkv = 4, 2
+    kp = torch.randn(16, hkv, d).to(torch.bfloat16).to(DEV)
+    table = torch.arange(16, dtype=torch.int32, device=DEV).reshape(2, 8)
+    none = torch.zeros(0, dtype=torch.int32, device=DEV)
+    zero1 = torch.zeros(1, dtype=torch.int32, device=DEV)
+    q0 = torch.zeros(0, h, d, dtype=torch.bfloat16, device=DEV)
+    assert ops.attn_paged_decode(q0, kp, kp, table, none, zero1).shape == (0, h, d)
+    qo, tb, ti = _cabi.paged_prefill_schedule([], DEV)
+    assert ops.attn_paged_prefill(q0, kp, kp, table, none, zero1, qo, tb, ti, is_causal=True).shape == (0, h, d)
+    # two sequences: the first has rows but no keys, the second keys but no rows
+    q = torch.randn(5, h, d).to(torch.bfloat16).to(DEV)
+    rows = torch.arange(2, dtype=torch.int32, device=DEV)
+    kvp = torch.tensor([0, 0, 6], dtype=torch.int32, device=DEV)
+    qo, tb, ti = _cabi.paged_prefill_schedule([5, 0], DEV)
+    for causal in (True, False):
+        out = ops.attn_paged_prefill(q, kp, kp, table, rows, kvp, qo, tb, ti, is_causal=causal)
+        assert out.shape == (5, h, d) and out.abs().sum() == 0
+    out = ops.attn_paged_decode(q[:2].contiguous(), kp, kp, table, rows, kvp)
+    assert out[0].abs().sum() == 0 and out[1].abs().sum() > 0
+    dec, pre = get_module("attn_decode").attn_decode, get_module("attn_prefill").attn_prefill
+    k0 = torch.zeros(2, 0, hkv, d, dtype=torch.bfloat16, device=DEV)
+    q4 = torch.randn(2, 3, h, d).to(torch.bfloat16).to(DEV)
+    assert pre(q4, k0, k0, layout=1).abs().sum() == 0 and pre(q4, k0, k0, layout=1).shape == q4.shape
+    assert dec(q4[:, :1].contiguous(), k0, k0, layout=1).abs().sum() == 0
+    assert pre(q4[:0], k0[:0], k0[:0], layout=1).shape == (0, 3, h, d)
