@@ -338,3 +338,39 @@ def test_attention_entries_with_nothing_to_do(d):
     assert pre(q4, k0, k0, layout=1).abs().sum() == 0 and pre(q4, k0, k0, layout=1).shape == q4.shape
     assert dec(q4[:, :1].contiguous(), k0, k0, layout=1).abs().sum() == 0
     assert pre(q4[:0], k0[:0], k0[:0], layout=1).shape == (0, 3, h, d)
+
+
+def test_general_kernel_random_sweep():
+    """Thirty seeded random batches through the general kernel: head_dim, grouping (1..16), ragged
+    cached-prefix and new-token counts (some with more rows than keys), causal or not, padding
+    slots, every mask form, every split choice; decode on the same pools."""
+    from astrai_amd.extension import _cabi
+    g = torch.Generator().manual_seed(2718)
+    ri = lambda lo, hi: int(torch.randint(lo, hi, (1,), generator=g))
+    for i in range(30):
+        d = (32, 64, 128, 256)[ri(0, 4)]
+        n_rep = (1, 2, 3, 4, 5, 8, 12, 16)[ri(0, 8)]
+        hkv = ri(1, 4)
+        h = hkv * n_rep
+        b = ri(1, 5)
+        q_lens = [ri(1, 150) for _ in range(b)]
+        kv_lens = [max(1, ql + ri(-20, 100)) for ql in q_lens]
+        causal, nsplit = bool(i % 3), (0, 1, 2, 5)[i % 4]
+        if d == 128 and n_rep in (2, 4, 8):
+            d = 64                                       # (that shape is the tuned kernel's, swept elsewhere)
+        print(f"case {i}: d={d} h={h}/{hkv} kv={kv_lens} q={q_lens} causal={causal} nsplit={nsplit}", flush=True)
+        args = _paged_case(b, h, hkv, d, kv_lens, q_lens, seed=7000 + i, holes=(i % 4 == 1))
+        dev = [t.to(DEV) for t in args]
+        qo, tb, ti = _cabi.paged_prefill_schedule(q_lens, DEV)
+        mask = None
+        if i % 2:
+            w = max(kv_lens) + 3
+            shape = [(b, w), (b, 1, max(q_lens), w), (b, h, max(q_lens), w), (b, h, 1, w)][(i // 2) % 4]
+            mask = torch.rand(shape, generator=g) < 0.6
+        got = _cabi.attn_paged_prefill(*dev, qo, tb, ti, mask=None if mask is None else mask.to(DEV),
+                                       causal_offset=0 if causal else -1, nsplit=nsplit)
+        _close(got, D.attn_paged_prefill(*args, qo.cpu(), causal=causal, mask=mask), f"sweep {i} prefill")
+        m2 = None if mask is None else (torch.rand(b, max(kv_lens) + 3, generator=g) < 0.6)
+        q1 = args[0][:b].contiguous()
+        got = _cabi.attn_paged_decode(q1.to(DEV), *dev[1:], mask=None if m2 is None else m2.to(DEV), nsplit=nsplit)
+        assert_bf16_close(got, D.attn_paged_decode(q1, *args[1:], mask=m2), what=f"sweep {i} decode")
