@@ -1151,15 +1151,13 @@ def attn_decode_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Opt
     token per sequence against ``k`` / ``v`` tensors, ``[batch, heads, len, 128]`` (layout 0) or
     ``[batch, len, heads, 128]`` (layout 1); the result has ``q``'s layout. ``causal_offset >= 0``
     limits the keys to ``0 .. causal_offset`` (layout_policies.cuh:138-141), ``mask`` (bool, True =
-    attend) is ``[batch, kv_len]``, ``[batch, 1, kv_len]`` or ``[batch, 1, 1, kv_len]``. The split
+    attend) is ``[batch, kv_len]``, ``[batch, 1, kv_len]`` or ``[batch, 1 | heads, 1, kv_len]``. The split
     buffers are not needed. Layout 0 without a mask runs the dense-cache kernel in place; the
     other cases run the paged kernel over the token-major tensors (layout 0 is copied for it)."""
     b, q_len, kv_len, h, hkv, d = _dense_args(q, k, v, layout, "attn_decode")
     if q_len != 1:
         raise RuntimeError("Q seq_len must be 1")
     m4 = _dense_mask(mask, b, 1, kv_len, h)
-    if m4 is not None and m4.size(1) != 1:
-        raise RuntimeError("attn_decode: a mask per head is not supported")
     if d not in (32, 64, 128, 256) or h // hkv > 16:
         raise RuntimeError("attn_decode needs head_dim in (32, 64, 128, 256) and n_heads / n_kv_heads <= 16")
     attend = kv_len if causal_offset < 0 else min(kv_len, causal_offset + 1)
@@ -1174,8 +1172,19 @@ def attn_decode_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Opt
         k_tm, v_tm = _token_major(k, layout), _token_major(v, layout)
         table, rows = _identity_paging(b, kv_len, q.device)
         indptr = (torch.arange(b + 1, dtype=torch.int32, device=q.device) * attend)
-        out = attn_paged_decode(q.reshape(b, h, d), k_tm.view(b * kv_len, hkv, d), v_tm.view(b * kv_len, hkv, d),
-                                table, rows, indptr, mask=None if m4 is None else m4[:, 0, 0], scale=scale)
+        q3, k_pool, v_pool = q.reshape(b, h, d), k_tm.view(b * kv_len, hkv, d), v_tm.view(b * kv_len, hkv, d)
+        if m4 is not None and m4.size(1) != 1:
+            # one mask row per head: only the general kernel addresses a mask by head
+            mh = m4[:, :, 0]
+            mh = mh if mh.stride(-1) == 1 else mh.contiguous()
+            out = torch.empty((b, h, d), device=q.device, dtype=torch.bfloat16)
+            nsplit = max(1, min(64, 2048 // max(1, b * hkv), kv_len // 64))
+            _paged_rows(_require(), q3.contiguous(), k_pool, v_pool, table, rows, indptr, None,
+                        (mh.data_ptr(), mh.stride(0), mh.stride(1), 0, 1, mh.size(2)), out, b, nsplit, False,
+                        scale if scale > 0 else d ** -0.5)
+            return out.reshape(q.shape)
+        out = attn_paged_decode(q3, k_pool, v_pool, table, rows, indptr,
+                                mask=None if m4 is None else m4[:, 0, 0], scale=scale)
     return out.reshape(q.shape)  # one token: both layouts have the same memory order
 
 

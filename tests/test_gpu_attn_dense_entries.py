@@ -72,6 +72,9 @@ def test_registry_attn_decode_layouts_and_offsets(layout):
     mask = torch.rand(2, 130, generator=torch.Generator().manual_seed(1)) < 0.5
     got = fn(*dev, mask=mask.to(DEV), causal_offset=100, layout=layout)
     assert_bf16_close(got, D.attn_dense(q, k, v, mask=mask, causal_offset=100, layout=layout), what="mask and offset")
+    per_head = torch.rand(2, 8, 1, 130, generator=torch.Generator().manual_seed(2)) < 0.5
+    got = fn(*dev, mask=per_head.to(DEV), causal_offset=100, layout=layout)
+    assert_bf16_close(got, D.attn_dense(q, k, v, mask=per_head, causal_offset=100, layout=layout), what="mask per head")
     # a key tensor that is a window of a longer buffer (non-contiguous)
     g = torch.Generator().manual_seed(5)
     shape = (2, 200, 2, 128) if layout == 1 else (2, 2, 200, 128)
