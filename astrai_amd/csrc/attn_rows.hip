@@ -3,7 +3,7 @@
 // row per sequence) and ragged prefill (row ranges per sequence) alike. The
 // reference's paged kernels accept head_dim in {32, 64, 128, 256} and any head
 // grouping (astrai/extension/backend/attention.py:518-527,
-// csrc/kernels/attention/dispatchers.cuh); its own tests run head_dim 64
+// csrc/kernels/attention/entry_utils.cuh:13-22); its own tests run head_dim 64
 // (tests/extension/conftest.py:9-20).
 //
 // One wave per (block of query rows, KV head, context split). The query rows that share a
