@@ -20,9 +20,13 @@ amax is handed back as a fresh one-element fp32 tensor. Format names are
 ``"e4m3"`` / ``"e5m2"``, output names ``"bf16"`` / ``"e4m3"``; their position in
 the tuples below is the integer the kernels take.
 
-One deliberate difference: the reference registers ``cpu`` kernels in plain
-PyTorch (its lines 78-82 and 116-122). They are its CPU oracle. This backend
-computes nothing on the CPU, so both dispatcher ops fail for CPU tensors.
+Like the reference, the two dispatcher ops carry three registrations: a shape
+function, the device kernel, and a ``cpu`` kernel in plain PyTorch for CPU
+tensors (its lines 76-82 and 114-122), which the reference's own CPU tests call
+through the op. The device selects the kernel: a GPU tensor never reaches the
+``cpu`` one, and with ``libastrai_w8a8.so`` missing a GPU call raises. The
+primitives this backend adds (``mm_fp8_bias``, ``linear_forward_fp8``, ...) are
+device-only.
 """
 
 from __future__ import annotations
@@ -82,6 +86,12 @@ def _quantize_entry(x, scale, fmt):
     _device_only("custom::fp8_quantize")
 
 
+def _quantize_host(x, scale, fmt):
+    # CPU tensors only (reference ops/fp8.py:76-82): plain cast of x / step, floored amax
+    codes = (x.float() / scale).to(_CODE_DTYPES[1 if fmt else 0])
+    return codes, x.abs().amax().float().reshape(1).clamp_min(1e-12)
+
+
 def _quantize_shapes(x, scale, fmt):
     codes = x.new_empty(x.shape, dtype=_CODE_DTYPES[1 if fmt else 0])
     return codes, x.new_empty(1, dtype=torch.float32)
@@ -94,6 +104,14 @@ def _quantize_device(x, scale, fmt):
 
 def _gemm_entry(a, b, sa, sb, out_dtype=0, out_scale=None):
     _device_only("custom::fp8_gemm")
+
+
+def _gemm_host(a, b, sa, sb, out_dtype=0, out_scale=None):
+    # CPU tensors only (reference ops/fp8.py:114-122); the steps enter by broadcasting
+    acc = a.float() @ b.float().t() * sa * sb
+    if not out_dtype:
+        return acc.to(torch.bfloat16)
+    return (acc if out_scale is None else acc * out_scale).to(torch.float8_e4m3fn)
 
 
 def _gemm_shapes(a, b, sa, sb, out_dtype=0, out_scale=None):
@@ -111,12 +129,14 @@ fp8_quantize = custom_op("custom::fp8_quantize", _quantize_entry, mutates_args=(
                          schema="(Tensor x, Tensor scale, int fmt) -> (Tensor, Tensor)")
 fp8_quantize.register_fake(_quantize_shapes)
 fp8_quantize.register_kernel("cuda")(_quantize_device)
+fp8_quantize.register_kernel("cpu")(_quantize_host)
 
 fp8_gemm = custom_op("custom::fp8_gemm", _gemm_entry, mutates_args=(),
                      schema="(Tensor a, Tensor b, Tensor sa, Tensor sb, int out_dtype=0, "
                             "Tensor? out_scale=None) -> Tensor")
 fp8_gemm.register_fake(_gemm_shapes)
 fp8_gemm.register_kernel("cuda")(_gemm_device)
+fp8_gemm.register_kernel("cpu")(_gemm_host)
 
 
 # ---------------------------------------------------------------------------

@@ -7,9 +7,12 @@ The reference has no int8 policy; this follows the shape of its fp8 one
 autocast-style context manager, an enable switch, and a guard that falls
 through to the stock kernel for anything it does not take. The per-weight cache
 is keyed like the reference's per-weight metas, ``(data_ptr, shape, dtype)``
-(fp8.py:200-208), plus the tensor version so an in-place update re-quantizes.
+(fp8.py:200-208); an entry also holds a weak reference to the tensor object it
+was made for and that tensor's version, so an in-place update re-quantizes and
+a new tensor that lands on a freed weight's address never gets the old codes.
 """
 
+import weakref
 from contextlib import contextmanager
 from typing import Dict, Optional, Tuple
 
@@ -25,24 +28,41 @@ from astrai_amd.extension.ops.int8 import (
 class Int8State:
     def __init__(self):
         self.enabled = False
-        self._weights: Dict[Tuple, Tuple[int, torch.Tensor, torch.Tensor]] = {}
+        # key -> (weakref to the weight, its version, wq, sw)
+        self._weights: Dict[Tuple, Tuple[weakref.ref, int, torch.Tensor, torch.Tensor]] = {}
+
+    @staticmethod
+    def _key(w: torch.Tensor) -> Tuple:
+        return (w.data_ptr(), w.shape, w.dtype)
+
+    def _store(self, w: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor) -> None:
+        dead = [k for k, e in self._weights.items() if e[0]() is None]
+        for k in dead:
+            del self._weights[k]
+        self._weights[self._key(w)] = (weakref.ref(w), w._version, wq, sw)
+
+    def lookup(self, w: torch.Tensor) -> Optional[Tuple[torch.Tensor, torch.Tensor]]:
+        """The cached ``(wq, sw)`` of this very tensor object at its current
+        version, or ``None``."""
+        hit = self._weights.get(self._key(w))
+        if hit is not None and hit[0]() is w and hit[1] == w._version:
+            return hit[2], hit[3]
+        return None
 
     def get_weight(self, w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
         """``(wq int8 [N,K], sw fp32 [N])`` for ``w``, quantizing on first use."""
-        key = (w.data_ptr(), w.shape, w.dtype)
-        hit = self._weights.get(key)
-        if hit is not None and hit[0] == w._version:
-            return hit[1], hit[2]
+        hit = self.lookup(w)
+        if hit is not None:
+            return hit
         wq, sw = quantize_int8_per_channel(w.detach())
-        self._weights[key] = (w._version, wq, sw)
+        self._store(w, wq, sw)
         return wq, sw
 
     def put_weight(self, w: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor) -> None:
         """Install an already quantized form of ``w`` (e.g. from an int8 checkpoint)."""
         if wq.shape != w.shape or wq.dtype != torch.int8 or sw.numel() != w.size(0):
             raise ValueError("wq must be int8 of w's shape and sw one step per output channel")
-        self._weights[(w.data_ptr(), w.shape, w.dtype)] = (
-            w._version, wq.contiguous(), sw.reshape(-1).float().contiguous())
+        self._store(w, wq.contiguous(), sw.reshape(-1).float().contiguous())
 
     def reset(self) -> None:
         self.enabled = False

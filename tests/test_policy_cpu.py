@@ -81,13 +81,36 @@ def test_ring_wraps_and_forgets_old_peaks():
     torch.testing.assert_close(meta.x_scale, torch.tensor([2.0 / 448.0]))
 
 
-def test_ops_have_no_cpu_arithmetic():
+def test_reference_ops_cpu_kernels(golden):
+    """The reference registers cpu kernels on its two dispatcher ops and tests them
+    with these vectors (tests/extension/test_fp8_mma.py:262-293)."""
+    kats = golden("reference_kats.json")
+    torch.manual_seed(0)
+    x = torch.randn(16, 32, dtype=torch.bfloat16)
+    x8, amax = ops_fp8.quantize_bf16(x, torch.tensor([kats["quantize_scale"]]), "e4m3")
+    assert x8.dtype == torch.float8_e4m3fn
+    # dividing by 0.5 is an exact doubling, so the expected codes are the cast of 2x
+    assert torch.equal(x8.view(torch.uint8), (x.float() * 2).to(torch.float8_e4m3fn).view(torch.uint8))
+    torch.testing.assert_close(amax, x.abs().amax().float().reshape(1))
+    x5, _ = ops_fp8.quantize_bf16(x, torch.tensor([1.0]), "e5m2")
+    assert x5.dtype == torch.float8_e5m2
+    k = kats["mm_fp8_cpu"]
+    a8 = torch.tensor(k["a8"]).to(torch.float8_e4m3fn)
+    b8 = torch.tensor(k["b8"]).to(torch.float8_e4m3fn)
+    out = ops_fp8.mm_fp8(a8, b8, torch.tensor([k["sa"]]), torch.tensor([k["sb"]]))
+    assert out.dtype == torch.bfloat16 and out.tolist() == k["out_bf16"]
+    k = kats["mm_fp8_fp8_out_cpu"]
+    out8 = ops_fp8.mm_fp8(a8, b8, torch.tensor([k["sa"]]), torch.tensor([k["sb"]]),
+                          out_dtype="e4m3", out_scale=torch.tensor([k["out_scale"]]))
+    assert out8.dtype == torch.float8_e4m3fn and out8.float().tolist() == k["out_e4m3"]
+    # an all-zero input: the floor keeps the amax positive (ops/fp8.py:81)
+    _, amax0 = ops_fp8.quantize_bf16(torch.zeros(2, 2, dtype=torch.bfloat16), torch.tensor([1.0]))
+    assert float(amax0) == pytest.approx(1e-12)
+
+
+def test_added_ops_have_no_cpu_arithmetic():
     x = torch.randn(4, 8).to(torch.bfloat16)
-    with pytest.raises(RuntimeError, match="no CPU"):
-        ops_fp8.quantize_bf16(x, torch.tensor([0.5]))
     a8 = torch.zeros(2, 2, dtype=torch.float8_e4m3fn)
-    with pytest.raises(RuntimeError, match="no CPU"):
-        ops_fp8.mm_fp8(a8, a8, torch.ones(1), torch.ones(1))
     with pytest.raises(RuntimeError, match="no CPU"):
         ops_int8.quantize_int8_per_token(x)
     with pytest.raises(RuntimeError, match="no CPU"):
@@ -202,3 +225,39 @@ def test_fp8_scaling_state_survives_a_checkpoint(tmp_path):
                 load_fp8_scaling(model, str(tmp_path))
     finally:
         st.reset()
+
+
+def test_int8_weight_cache_is_tied_to_the_tensor_object(monkeypatch):
+    """A cached int8 form belongs to one tensor object at one version: another
+    tensor with the same address, shape and dtype (a freed weight's memory
+    reused) must be quantized afresh, an in-place update too."""
+    calls = []
+
+    def fake_quantize(w):
+        calls.append(w)
+        return (torch.full(w.shape, len(calls), dtype=torch.int8),
+                torch.full((w.size(0),), float(len(calls))))
+
+    monkeypatch.setattr(w8a8, "quantize_int8_per_channel", fake_quantize)
+    st = w8a8.Int8State()
+    w1 = torch.zeros(4, 8, dtype=torch.bfloat16)
+    q1, _ = st.get_weight(w1)
+    assert st.get_weight(w1)[0] is q1 and len(calls) == 1          # hit
+    alias = w1.detach()                                            # same address, shape, dtype, version
+    assert alias.data_ptr() == w1.data_ptr() and alias is not w1
+    assert st.lookup(alias) is None
+    q2, s2 = st.get_weight(alias)
+    assert len(calls) == 2 and int(q2[0, 0]) == 2 and float(s2[0]) == 2.0
+    assert st.lookup(w1) is None                                   # the slot now belongs to `alias`
+    alias.add_(1)                                                  # version bump
+    assert st.lookup(alias) is None
+    st.get_weight(alias)
+    assert len(calls) == 3
+    # an installed form (checkpoint load) obeys the same identity rule
+    w3 = torch.zeros(2, 8, dtype=torch.bfloat16)
+    st.put_weight(w3, torch.ones(2, 8, dtype=torch.int8), torch.ones(2))
+    assert st.lookup(w3) is not None and st.lookup(w3.detach()) is None
+    # entries of dead tensors are dropped on the next store
+    del w3
+    st.put_weight(w1, torch.ones(4, 8, dtype=torch.int8), torch.ones(4))
+    assert all(e[0]() is not None for e in st._weights.values())
