@@ -594,7 +594,9 @@ def rope_cache_write(qkv: torch.Tensor, freqs: torch.Tensor, positions: torch.Te
 
 
 def attn_decode_supported(n_heads: int, n_kv_heads: int, seq: int, head_dim: int) -> bool:
-    return head_dim == 128 and n_heads % n_kv_heads == 0 and (n_heads // n_kv_heads) * seq <= 8
+    """The shapes ``astrai_w8a8_attn_decode_bf16`` takes (the limits its entry point checks)."""
+    return (head_dim == 128 and n_kv_heads > 0 and n_heads % n_kv_heads == 0
+            and (n_heads // n_kv_heads) * seq <= 8 and n_heads <= 64)
 
 
 def attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, positions: torch.Tensor,
@@ -948,9 +950,19 @@ def mm_int8(a: torch.Tensor, b: torch.Tensor, sa: Optional[torch.Tensor],
     return out
 
 
-def mm_int8_rope_cache_supported(tokens: int, k: int, head_dim: int) -> bool:
-    """Shapes the fused q|k|v projection + rotary + cache-write kernel takes."""
-    return 0 < tokens <= 64 and k % 256 == 0 and head_dim % 4 == 0
+def mm_int8_rope_cache_supported(tokens: int, k: int, head_dim: int, n: int = 0) -> bool:
+    """Shapes the fused q|k|v projection + rotary + cache-write kernel takes (the limits
+    its entry point checks); ``n`` = rows of the q|k|v weight, when known."""
+    return 0 < tokens <= 64 and k % 256 == 0 and head_dim % 4 == 0 and n * k < 2 ** 31
+
+
+FUSED_ROW_MAX = 8192
+
+
+def fused_rows_supported(width: int) -> bool:
+    """Row widths the producers fused with the per-token quantizer take
+    (``add_rmsnorm_quantize_int8_rows``, ``silu_mul_quantize_int8_rows``)."""
+    return width % 8 == 0 and 0 <= width <= FUSED_ROW_MAX
 
 
 def mm_int8_rope_cache(a: torch.Tensor, wqkv: torch.Tensor, sa: torch.Tensor, sb: torch.Tensor,
@@ -969,8 +981,9 @@ def mm_int8_rope_cache(a: torch.Tensor, wqkv: torch.Tensor, sa: torch.Tensor, sb
     n = (n_heads + 2 * n_kv_heads) * head_dim
     if m != batch * seq or wqkv.size(0) != n or wqkv.size(1) != k:
         raise RuntimeError("a must be [batch*seq, K] and wqkv [(n_heads + 2 n_kv_heads) * head_dim, K]")
-    if not mm_int8_rope_cache_supported(m, k, head_dim):
-        raise RuntimeError("mm_int8_rope_cache: needs at most 64 tokens, K % 256 == 0, head_dim % 4 == 0")
+    if not mm_int8_rope_cache_supported(m, k, head_dim, n):
+        raise RuntimeError("mm_int8_rope_cache: needs at most 64 tokens, K % 256 == 0, head_dim % 4 == 0, "
+                           "a weight matrix under 2 GiB")
     sa = _check_vec(sa, a, m, "sa")
     sb = _check_vec(sb, a, n, "sb")
     if k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:

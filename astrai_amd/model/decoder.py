@@ -263,7 +263,7 @@ class DecoderBlock(nn.Module):
             aq, sa = I.quantize_int8_per_token(
                 att.core(qkv[..., :nq], qkv[..., nq:nq + nkv], qkv[..., nq + nkv:], rotary_emb, None,
                          positions, key_mask))
-        elif _cabi.mm_int8_rope_cache_supported(b * s, d, att.head_dim):
+        elif _cabi.mm_int8_rope_cache_supported(b * s, d, att.head_dim, f.wqkv.size(0)):
             # a few new tokens: the projection's epilogue rotates q and k and writes the cache
             q = _cabi.mm_int8_rope_cache(xq, f.wqkv, sx, f.sqkv, rotary_emb[0], positions,
                                          kv_cache.k[att.layer_id], kv_cache.v[att.layer_id],
@@ -348,8 +348,14 @@ def fuse_int8_weights(model: AutoRegressiveLM) -> int:
     int8 matrix each on the block. While ``w8a8.int8_autocast`` is on, blocks then take
     the fused path. Returns the number of int8 matrices held. Call again after
     changing weights."""
-    from astrai_amd.extension import w8a8
+    from astrai_amd.extension import _cabi, w8a8
 
+    cfg = model.config
+    for what, width in (("hidden_size", cfg.hidden_size), ("intermediate_size", cfg.intermediate_size)):
+        if not _cabi.fused_rows_supported(width):
+            raise ValueError(f"fuse_int8_weights: {what} {width} is outside what the fused producers take "
+                             f"(a multiple of 8, at most {_cabi.FUSED_ROW_MAX}); use the Linear-by-Linear "
+                             "int8 path (w8a8.prepare_int8_weights) for this model")
     state = w8a8.int8_state()
 
     def cat(*linears):

@@ -49,3 +49,59 @@ def test_argument_validation_needs_no_gpu():
     assert rc == 1 and b"out_scale" in lib.astrai_w8a8_last_error()
     rc = lib.astrai_w8a8_gemm_fp8_pt(8, 16, 16, 16, None, None, 16, 4, 4, 64, 0, 0, None)
     assert rc == 1 and b"aligned" in lib.astrai_w8a8_last_error()
+
+
+def test_shape_predicates_agree_with_the_entry_points():
+    """Just past each limit the Python predicate says no and the entry point returns
+    UNSUPPORTED (status 2) before anything touches the device; 16 stands for an
+    aligned non-null pointer that is never dereferenced."""
+    lib = _cabi.load()
+    assert lib is not None, _cabi.load_error()
+    P = 16
+
+    def decode(n_heads, n_kv, seq, hd):
+        return lib.astrai_w8a8_attn_decode_bf16(P, P, P, P, P, 1 << 30, P, None, None, 1, seq, n_heads, n_kv,
+                                                hd, 64, 1, 1.0, None)
+
+    for shape in ((128, 16, 1, 128), (16, 4, 3, 128), (16, 4, 1, 64)):   # > 64 heads, > 8 rows, head_dim
+        assert not _cabi.attn_decode_supported(*shape), shape
+        assert decode(*shape) == 2, (shape, lib.astrai_w8a8_last_error())
+    assert _cabi.attn_decode_supported(64, 8, 1, 128) and _cabi.attn_decode_supported(16, 4, 2, 128)
+
+    def prefill(n_heads, n_kv, hd):
+        return lib.astrai_w8a8_attn_prefill_bf16(P, P, P, P, P, 1, 8, n_heads, n_kv, hd, 64, 1.0, None)
+
+    for shape in ((16, 16, 128), (48, 3, 128), (16, 4, 64)):
+        assert not _cabi.attn_prefill_supported(*shape), shape
+        assert prefill(*shape) == 2, (shape, lib.astrai_w8a8_last_error())
+
+    def rope_gemm(tokens, k, hd, n_heads, n_kv):
+        return lib.astrai_w8a8_gemm_int8_ptpc_rope_cache(P, P, P, P, P, P, P, P, P, tokens, 1, n_heads, n_kv,
+                                                         hd, 64, k, None)
+
+    for tokens, k, hd, n_heads, n_kv in ((65, 256, 128, 4, 1), (8, 128, 128, 4, 1), (8, 256, 6, 4, 1),
+                                         (8, 1 << 16, 128, 200, 28)):        # last: 2 GiB weight
+        n = (n_heads + 2 * n_kv) * hd
+        assert not _cabi.mm_int8_rope_cache_supported(tokens, k, hd, n), (tokens, k, hd, n)
+        assert rope_gemm(tokens, k, hd, n_heads, n_kv) == 2, lib.astrai_w8a8_last_error()
+    assert _cabi.mm_int8_rope_cache_supported(64, 2048, 128, 3072)
+
+    for width in (8200, 12, 11008):
+        assert not _cabi.fused_rows_supported(width)
+        assert lib.astrai_w8a8_add_rmsnorm_quantize_int8_rows(P, None, P, 1e-5, None, None, P, P, 4, width,
+                                                              None) == 2
+        assert lib.astrai_w8a8_silu_mul_quantize_int8_rows(P, P, max(width, 16) + (-width) % 8, None, P, P, 4,
+                                                           width, None) == 2
+    assert _cabi.fused_rows_supported(8192) and _cabi.fused_rows_supported(5632)
+    header = open(os.path.join(ROOT, "astrai_amd", "csrc", "launchers.h")).read()
+    assert int(re.search(r"kFusedRowMax\s*=\s*(\d+)", header).group(1)) == _cabi.FUSED_ROW_MAX
+
+
+def test_fuse_int8_weights_refuses_widths_the_fused_producers_reject():
+    import pytest
+    import torch
+    from astrai_amd.model import AutoRegressiveLM, AutoRegressiveLMConfig, fuse_int8_weights
+    cfg = AutoRegressiveLMConfig(vocab_size=32, hidden_size=64, num_hidden_layers=1, num_attention_heads=2,
+                                 num_key_value_heads=1, intermediate_size=8200, max_position_embeddings=8)
+    with pytest.raises(ValueError, match="intermediate_size 8200"):
+        fuse_int8_weights(AutoRegressiveLM(cfg).to(torch.bfloat16))
