@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 
@@ -60,6 +61,36 @@ w8a8::GemmArgs pack(const void* a, const void* b, const float* sa, const float* 
     g.k = (int)k;
     g.out_kind = out_kind;
     return g;
+}
+
+// ---- library-owned scratch for the entry point that takes no workspace ----------
+// Every GPU the library runs on holds its own copy of this array, at its own address,
+// until the process ends. In host code the array's name is only a handle for
+// hipGetSymbolAddress: what kernels and copies get is the address that call returns
+// for the current device, looked up once per device and kept in scratch_addr.
+constexpr int64_t kScratchFloats = ASTRAI_W8A8_STATIC_SCRATCH_FLOATS;
+static __device__ __align__(256) float scratch[kScratchFloats];
+
+constexpr int kMaxDevices = 64;
+std::atomic<float*> scratch_addr[kMaxDevices];
+
+int scratch_of_current_device(const char* what, float** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess)
+        return fail(ASTRAI_W8A8_LAUNCH_FAILED, "%s: hipGetDevice: %s", what, hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices)
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "%s: device ordinal %d outside 0..%d", what, dev, kMaxDevices - 1);
+    float* p = scratch_addr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return fail(ASTRAI_W8A8_LAUNCH_FAILED, "%s: hipGetSymbolAddress(scratch): %s", what,
+                        hipGetErrorString(e));
+        scratch_addr[dev].store(p, std::memory_order_release);  // two threads racing store the same address
+    }
+    *out = p;
+    return ASTRAI_W8A8_OK;
 }
 
 }  // namespace
@@ -220,36 +251,67 @@ int64_t astrai_w8a8_attn_decode_workspace_floats(int64_t batch, int64_t n_kv_hea
     return w8a8::attn_decode_workspace_floats((int)batch, (int)n_kv_heads, (int)nsplit, (int)n_query_rows);
 }
 
+// shared by the two dense decode entries; `ws` is device memory of `ws_floats` floats
+static int attn_decode_common(const char* what, const void* q, const void* k_cache, const void* v_cache,
+                              const int64_t* positions, float* ws, int64_t ws_floats, bool ws_is_static,
+                              void* out, void* out_q, float* out_scale, int64_t batch, int64_t seq,
+                              int64_t n_heads, int64_t n_kv_heads, int64_t head_dim, int64_t max_len,
+                              int64_t nsplit, float scale, void* stream) {
+    if (!q || !k_cache || !v_cache || !positions || (!ws && !ws_is_static) || (!out && !out_q) ||
+        (out_q && !out_scale))
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: null pointer", what);
+    if (batch < 0 || seq < 0 || n_heads <= 0 || n_kv_heads <= 0 || max_len <= 0 || nsplit <= 0 ||
+        nsplit > 64 || batch > 65535 || n_heads % n_kv_heads)
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: bad dims", what);
+    if (head_dim != 128 || (n_heads / n_kv_heads) * seq > 8 || n_heads > 64)
+        return fail(ASTRAI_W8A8_UNSUPPORTED,
+                    "%s: needs head_dim 128, (n_heads / n_kv_heads) * seq <= 8, n_heads <= 64", what);
+    if (max_len * 256 >= ((int64_t)1 << 32))
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "%s: one head of the cache must stay under 4 GiB", what);
+    if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || (out && !aligned16(out)) ||
+        (out_q && !aligned16(out_q)))
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: pointers must be 16-byte aligned", what);
+    if (batch == 0 || seq == 0) return ASTRAI_W8A8_OK;
+    const int64_t need = w8a8::attn_decode_workspace_floats((int)batch, (int)n_kv_heads, (int)nsplit,
+                                                            (int)((n_heads / n_kv_heads) * seq));
+    if (ws_is_static) {
+        if (need > kScratchFloats)
+            return fail(ASTRAI_W8A8_UNSUPPORTED,
+                        "%s: batch * n_kv_heads * nsplit too large for the library's scratch array "
+                        "(%lld floats needed, %lld held); lower nsplit or call attn_decode_bf16 with a workspace",
+                        what, (long long)need, (long long)kScratchFloats);
+        if (int rc = scratch_of_current_device(what, &ws)) return rc;
+    } else if (ws_floats < need) {
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: workspace too small (%lld floats needed)", what,
+                    (long long)need);
+    }
+    w8a8::AttnDecodeArgs a{q, k_cache, v_cache, positions, ws, out, out_q, out_scale, (int)batch, (int)seq,
+                           (int)n_heads, (int)n_kv_heads, (int)head_dim, max_len, (int)nsplit, scale};
+    if (!w8a8::launch_attn_decode(a, static_cast<hipStream_t>(stream)))
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "%s: shape not supported", what);
+    return check_launch(what);
+}
+
 int astrai_w8a8_attn_decode_bf16(const void* q, const void* k_cache, const void* v_cache,
                                  const int64_t* positions, float* workspace, int64_t workspace_floats,
                                  void* out, void* out_q, float* out_scale, int64_t batch,
                                  int64_t seq, int64_t n_heads,
                                  int64_t n_kv_heads, int64_t head_dim, int64_t max_len,
                                  int64_t nsplit, float scale, void* stream) {
-    if (!q || !k_cache || !v_cache || !positions || !workspace || (!out && !out_q) || (out_q && !out_scale))
-        return fail(ASTRAI_W8A8_BAD_ARG, "attn_decode_bf16: null pointer");
-    if (batch < 0 || seq < 0 || n_heads <= 0 || n_kv_heads <= 0 || max_len <= 0 || nsplit <= 0 ||
-        nsplit > 64 || batch > 65535 || n_heads % n_kv_heads)
-        return fail(ASTRAI_W8A8_BAD_ARG, "attn_decode_bf16: bad dims");
-    if (head_dim != 128 || (n_heads / n_kv_heads) * seq > 8 || n_heads > 64)
-        return fail(ASTRAI_W8A8_UNSUPPORTED,
-                    "attn_decode_bf16: needs head_dim 128, (n_heads / n_kv_heads) * seq <= 8, n_heads <= 64");
-    if (max_len * 256 >= ((int64_t)1 << 32))
-        return fail(ASTRAI_W8A8_UNSUPPORTED, "attn_decode_bf16: one head of the cache must stay under 4 GiB");
-    if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || (out && !aligned16(out)) ||
-        (out_q && !aligned16(out_q)))
-        return fail(ASTRAI_W8A8_BAD_ARG, "attn_decode_bf16: pointers must be 16-byte aligned");
-    if (batch == 0 || seq == 0) return ASTRAI_W8A8_OK;
-    const int64_t need = w8a8::attn_decode_workspace_floats((int)batch, (int)n_kv_heads, (int)nsplit,
-                                                            (int)((n_heads / n_kv_heads) * seq));
-    if (workspace_floats < need)
-        return fail(ASTRAI_W8A8_BAD_ARG, "attn_decode_bf16: workspace too small (%lld floats needed)",
-                    (long long)need);
-    w8a8::AttnDecodeArgs a{q, k_cache, v_cache, positions, workspace, out, out_q, out_scale, (int)batch, (int)seq,
-                           (int)n_heads, (int)n_kv_heads, (int)head_dim, max_len, (int)nsplit, scale};
-    if (!w8a8::launch_attn_decode(a, static_cast<hipStream_t>(stream)))
-        return fail(ASTRAI_W8A8_UNSUPPORTED, "attn_decode_bf16: shape not supported");
-    return check_launch("attn_decode_bf16");
+    return attn_decode_common("attn_decode_bf16", q, k_cache, v_cache, positions, workspace, workspace_floats,
+                              false, out, out_q, out_scale, batch, seq, n_heads, n_kv_heads, head_dim,
+                              max_len, nsplit, scale, stream);
+}
+
+int astrai_w8a8_attn_decode_bf16_static_scratch(const void* q, const void* k_cache, const void* v_cache,
+                                                const int64_t* positions, void* out, void* out_q,
+                                                float* out_scale, int64_t batch, int64_t seq,
+                                                int64_t n_heads, int64_t n_kv_heads, int64_t head_dim,
+                                                int64_t max_len, int64_t nsplit, float scale,
+                                                void* stream) {
+    return attn_decode_common("attn_decode_bf16_static_scratch", q, k_cache, v_cache, positions, nullptr, 0,
+                              true, out, out_q, out_scale, batch, seq, n_heads, n_kv_heads, head_dim,
+                              max_len, nsplit, scale, stream);
 }
 
 int astrai_w8a8_attn_paged_decode_bf16(const void* q, const void* k_pool, const void* v_pool,

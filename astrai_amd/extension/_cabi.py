@@ -65,6 +65,8 @@ PROTOTYPES = {
     "astrai_w8a8_attn_decode_bf16": (
         [_P, _P, _P, _P, _P, _I64, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, ctypes.c_float, _P],
         _INT),
+    "astrai_w8a8_attn_decode_bf16_static_scratch": (
+        [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, ctypes.c_float, _P], _INT),
     "astrai_w8a8_quantize_bf16_fp8_block128_act": ([_P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_quantize_bf16_fp8_block128_weight": ([_P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_gemm_fp8_pt": ([_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _INT, _INT, _P], _INT),
@@ -641,6 +643,43 @@ def attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, p
             ws.data_ptr(), ws.numel(), _ptr(out), _ptr(oq), _ptr(os_), b, s, h, hkv, d, max_len, nsplit,
             float(scale), _stream(q)), lib)
     return (oq, os_) if quantized else out
+
+
+STATIC_SCRATCH_FLOATS = 1 << 20
+
+
+def attn_decode_static_scratch(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                               positions: torch.Tensor, out: Optional[torch.Tensor] = None,
+                               out_q: Optional[torch.Tensor] = None, out_scale: Optional[torch.Tensor] = None,
+                               scale: Optional[float] = None, nsplit: int = 1) -> None:
+    """:func:`attn_decode` for callers that must not allocate: the caller brings the outputs
+    (``out`` bf16 ``[batch, seq, n_heads*128]`` and / or ``out_q`` int8 with ``out_scale`` fp32
+    ``[batch*seq]``), the context splits' partial results go to the array the library holds in
+    static device memory (``STATIC_SCRATCH_FLOATS`` floats a GPU; larger requests are refused).
+    Nothing is allocated here or in the library. Calls that overlap on one GPU share that
+    array and race; calls ordered on one stream do not."""
+    lib = _require()
+    _gpu(q, "attn_decode_static_scratch")
+    if q.dim() != 4 or k_cache.dim() != 4 or k_cache.shape != v_cache.shape:
+        raise RuntimeError("q must be [B, H, S, D] and the caches [B, H_kv, max_len, D]")
+    for t, dt, name in ((q, torch.bfloat16, "q"), (k_cache, torch.bfloat16, "k_cache"),
+                        (v_cache, torch.bfloat16, "v_cache"), (positions, torch.int64, "positions"),
+                        (out, torch.bfloat16, "out"), (out_q, torch.int8, "out_q"),
+                        (out_scale, torch.float32, "out_scale")):
+        if t is not None and (t.dtype != dt or not t.is_contiguous() or t.device != q.device):
+            raise RuntimeError(f"{name} must be a contiguous {dt} tensor on q's device")
+    b, h, s, d = q.shape
+    hkv, max_len = k_cache.size(1), k_cache.size(2)
+    if k_cache.size(0) != b or k_cache.size(3) != d or positions.numel() != s:
+        raise RuntimeError("cache batch / head_dim or the number of positions do not match q")
+    if (out is not None and out.numel() != b * s * h * d) or (out_q is not None and (
+            out_q.numel() != b * s * h * d or out_scale is None or out_scale.numel() != b * s)):
+        raise RuntimeError("out / out_q must hold batch*seq rows of n_heads*head_dim, out_scale batch*seq steps")
+    with torch.cuda.device(q.device):
+        _check(lib.astrai_w8a8_attn_decode_bf16_static_scratch(
+            q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), positions.data_ptr(), _ptr(out), _ptr(out_q),
+            _ptr(out_scale), b, s, h, hkv, d, max_len, nsplit, float(d ** -0.5 if scale is None else scale),
+            _stream(q)), lib)
 
 
 def attn_paged_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,

@@ -203,6 +203,28 @@ int astrai_w8a8_attn_decode_bf16(const void* q_bf16, const void* k_cache_bf16, c
                                  int64_t nsplit, float scale, void* stream);
 
 /*
+ * attn_decode_bf16 for callers that cannot allocate device memory or bring a workspace
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * It has no counterpart in the reference. Same arguments, kernels and results as
+ * attn_decode_bf16 minus the workspace: the context splits' partial results go to an array
+ * of ASTRAI_W8A8_STATIC_SCRATCH_FLOATS floats (4 MiB) that the library holds in static device
+ * memory, one copy per GPU it runs on, until the process ends. Calls no hipMalloc / hipFree
+ * or any other allocating routine. Returns ASTRAI_W8A8_UNSUPPORTED when
+ * astrai_w8a8_attn_decode_workspace_floats(batch, n_kv_heads, nsplit, rows) exceeds the array.
+ * The array's device address is looked up on the first call on each device (make that call
+ * outside stream capture). Every call on a GPU shares that GPU's array: calls that overlap on
+ * one GPU (other streams, other threads) race; calls ordered on one stream do not. Nothing in
+ * the array has to be cleared between calls: every slot a call reads it has written itself.
+ */
+#define ASTRAI_W8A8_STATIC_SCRATCH_FLOATS (1 << 20)
+int astrai_w8a8_attn_decode_bf16_static_scratch(const void* q_bf16, const void* k_cache_bf16,
+                                                const void* v_cache_bf16, const int64_t* positions,
+                                                void* out_bf16, void* out_q, float* out_scale,
+                                                int64_t batch, int64_t seq, int64_t n_heads,
+                                                int64_t n_kv_heads, int64_t head_dim, int64_t max_len,
+                                                int64_t nsplit, float scale, void* stream);
+
+/*
  * The same decode attention over a token-granular paged cache. Replaces
  * attn_paged_decode (csrc/kernels/attention/paged_decode.cu:4-67, addressing policy
  * PagedKV in csrc/kernels/attention/layout_policies.cuh:174-232; Python wrapper
