@@ -30,27 +30,59 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 HEADLINE_TRAFFIC_MB = 134.5
 
 
-def _event_time_ms(fn, iters, warmup):
-    """Average duration of `fn` (launches on torch's current stream) over `iters`
-    back-to-back launches, by HIP events on that stream."""
+LAUNCHES_PER_BATCH = 50   # event-timed launches per batch
+TIMED_BATCHES = 7         # the reported duration is the median of this many batch averages
+MAX_WARM_BATCHES = 60     # warm-up ends when two consecutive batches agree within 2% (or here)
+
+
+def _timed_batch_ms(run_batch):
+    """Duration of `run_batch()` (which launches on torch's current stream) by HIP events
+    recorded on that stream."""
     import torch
 
-    for _ in range(warmup):
-        fn()
-    torch.cuda.synchronize()
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
     e0.record()
-    for _ in range(iters):
-        fn()
+    run_batch()
     e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1)
+
+
+def _protocol_us(run_batch, launches=LAUNCHES_PER_BATCH):
+    """The fixed timing protocol of every kernel figure in the JSON line, whatever --steps
+    and --warmup say: batches of `launches` back-to-back launches timed by HIP events;
+    warm-up batches until two consecutive ones agree within 2% (at least two, i.e. >= 100
+    launches); then the median of TIMED_BATCHES batch averages. Returns (microseconds per
+    launch, {protocol details})."""
+    import torch
+
     torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / iters
+    prev, warm = None, 0
+    while warm < MAX_WARM_BATCHES:
+        t = _timed_batch_ms(run_batch)
+        warm += 1
+        if prev is not None and abs(t - prev) <= 0.02 * prev:
+            break
+        prev = t
+    ts = sorted(_timed_batch_ms(run_batch) for _ in range(TIMED_BATCHES))
+    med = ts[len(ts) // 2]
+    return med * 1e3 / launches, {"launches_per_batch": launches, "timed_batches": TIMED_BATCHES,
+                                  "warm_batches": warm,
+                                  "batch_spread": round((ts[-1] - ts[0]) / med, 4)}
 
 
-def _graph_time_ms(launch, n_launch, replays, warm_replays=2):
-    """Average per-launch duration with the launches captured in one HIP graph
-    (removes host launch overhead for kernels of a few microseconds)."""
+def _kernel_us(fn):
+    """_protocol_us for a host-launched kernel `fn`."""
+    def batch():
+        for _ in range(LAUNCHES_PER_BATCH):
+            fn()
+    return _protocol_us(batch)[0]
+
+
+def _graph_us(launch, n_launch=LAUNCHES_PER_BATCH):
+    """_protocol_us with the batch captured in one HIP graph (`launch(i)` for i in
+    range(n_launch)): removes host launch overhead for kernels of a few microseconds."""
     import torch
 
     s = torch.cuda.Stream()
@@ -64,17 +96,7 @@ def _graph_time_ms(launch, n_launch, replays, warm_replays=2):
     with torch.cuda.graph(g):
         for i in range(n_launch):
             launch(i)
-    for _ in range(warm_replays):
-        g.replay()
-    torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(replays):
-        g.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / (replays * n_launch)
+    return _protocol_us(g.replay, n_launch)[0]
 
 
 def _bench_decoder(dev):
@@ -151,6 +173,110 @@ def _bench_decoder(dev):
     del model
     torch.cuda.empty_cache()
     return res
+
+
+def _cpu_decoder_baseline(layers=1, prefill_batch=8, decode_steps=8):
+    """BASELINE config 4 on the host CPU through the decoder oracle (every Linear the exact
+    int8 oracle, dense cache), on a bounded sample: a `layers`-layer model of the config-4
+    dimensions, the 512-token prefill of `prefill_batch` of the 32 sequences, then
+    `decode_steps` greedy steps of all 32 (the cache of the prefilled sequences repeated).
+    Rates are per token; the per-layer share (total minus the separately timed embedding +
+    final norm + lm_head share) is scaled to 24 layers."""
+    import torch
+    import torch.nn.functional as F
+
+    from astrai_amd.model import AutoRegressiveLM, AutoRegressiveLMConfig
+    from oracle import decoder_oracle as D
+
+    threads = _cpu_threads()
+    torch.set_num_threads(threads)
+    cfg = AutoRegressiveLMConfig(num_hidden_layers=layers)
+    full_layers = AutoRegressiveLMConfig().num_hidden_layers
+    torch.manual_seed(4)
+    model = AutoRegressiveLM(cfg).to(torch.bfloat16).eval()
+    sd = {k: v.detach() for k, v in model.state_dict().items()}
+    lin = D.int8_linear_fn(sd)
+    batch, prompt = 32, 512
+    ids = torch.randint(0, cfg.vocab_size, (batch, prompt), generator=torch.Generator().manual_seed(4))
+    ids = ids[:prefill_batch]
+    hd = cfg.hidden_size // cfg.num_attention_heads
+    kc = torch.zeros(layers, prefill_batch, cfg.num_key_value_heads, prompt + decode_steps, hd,
+                     dtype=torch.bfloat16)
+    vc = torch.zeros_like(kc)
+
+    def head(x_ids):   # what does not grow with the layer count
+        x = F.embedding(x_ids, sd["embed_tokens.weight"])
+        return lin(F.rms_norm(x, (cfg.hidden_size,), sd["norm.weight"], cfg.rms_norm_eps), "lm_head.weight")
+
+    with torch.no_grad():
+        D.forward_cached(sd, cfg, ids[:2, :64], lin, kc[:, :2], vc[:, :2], torch.arange(64))  # warm-up
+        t0 = time.perf_counter()
+        logits = D.forward_cached(sd, cfg, ids, lin, kc, vc, torch.arange(prompt))
+        t_pre = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        head(ids)
+        t_pre_head = time.perf_counter() - t0
+        rep = batch // prefill_batch
+        tok = logits[:, -1].argmax(-1).reshape(-1, 1).repeat(rep, 1)
+        kc, vc = kc.repeat(1, rep, 1, 1, 1), vc.repeat(1, rep, 1, 1, 1)
+        del logits
+        t0 = time.perf_counter()
+        for i in range(decode_steps):
+            lg = D.forward_cached(sd, cfg, tok, lin, kc, vc, torch.tensor([prompt + i]))
+            tok = lg[:, -1].argmax(-1).reshape(batch, 1)
+        t_dec = (time.perf_counter() - t0) / decode_steps
+        t0 = time.perf_counter()
+        for _ in range(decode_steps):
+            head(tok)
+        t_dec_head = (time.perf_counter() - t0) / decode_steps
+    scale = full_layers / layers
+    pre_full = (t_pre - t_pre_head) * scale + t_pre_head      # seconds for prefill_batch x 512 tokens
+    dec_full = (t_dec - t_dec_head) * scale + t_dec_head
+    return {"unit": "tokens/s", "cores": threads, "kind": "port",
+            "prefill_tokens_per_s": round(prefill_batch * prompt / pre_full, 1),
+            "decode_tokens_per_s": round(batch / dec_full, 1),
+            "decode_ms_per_step_extrapolated_24_layers": round(dec_full * 1e3, 1),
+            "measured": {"layers": layers, "prefill_sequences": prefill_batch, "prefill_s": round(t_pre, 2),
+                         "prefill_head_share_s": round(t_pre_head, 2), "decode_ms_per_step": round(t_dec * 1e3, 1),
+                         "decode_head_share_ms": round(t_dec_head * 1e3, 1)},
+            "sample": f"EXTRAPOLATED: a {layers}-layer model of the config-4 dimensions; prefill of {prefill_batch} "
+                      f"of the 32 x 512-token prompts and {decode_steps} decode steps of 32 sequences, timed once; "
+                      f"layer share x {scale:g} + embedding / lm_head share"}
+
+
+def _cpu_threads():
+    """Threads the CPU baselines run on: the box's CPU share (16 for one GPU), which
+    OMP_NUM_THREADS states there, never more than the logical CPUs present."""
+    n = os.cpu_count() or 1
+    try:
+        n = min(n, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    except ValueError:
+        n = min(n, 16)
+    return max(1, min(n, 16))
+
+
+def _host_info():
+    """Logical CPUs, physical cores (distinct (package, core id) pairs of /proc/cpuinfo) and
+    the CPU model of the host the CPU baselines ran on."""
+    info = {"logical_cpus": os.cpu_count()}
+    try:
+        pairs, model, phys, core = set(), None, None, None
+        for ln in open("/proc/cpuinfo"):
+            if ln.startswith("model name") and model is None:
+                model = ln.split(":", 1)[1].strip()
+            elif ln.startswith("physical id"):
+                phys = ln.split(":", 1)[1].strip()
+            elif ln.startswith("core id"):
+                core = ln.split(":", 1)[1].strip()
+            elif not ln.strip():
+                if phys is not None and core is not None:
+                    pairs.add((phys, core))
+                phys = core = None
+        info["physical_cores"] = len(pairs) or None
+        info["cpu_model"] = model
+    except OSError:
+        pass
+    return info
 
 
 def _measured_ceilings():
@@ -384,14 +510,22 @@ def main():
     flop = 2.0 * M * N * K
     value = flop / (ms_per_step * 1e-3) / 1e12
 
-    kern_ms = _event_time_ms(step, args.steps, 5)
-    achieved = flop / (kern_ms * 1e-3) / 1e12
+    def step_batch():
+        for _ in range(LAUNCHES_PER_BATCH):
+            step()
+
+    kern_us, proto = _protocol_us(step_batch)
+    achieved = flop / (kern_us * 1e-6) / 1e12
     roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP8_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP8_TFLOPS, 4),
-                "traffic": HEADLINE_TRAFFIC_MB, "traffic_unit": "MB per launch (rocprofv3 FETCH_SIZE + "
-                "WRITE_SIZE, calibrated on a plain copy; summary in profiles/gemm_fp8_wave128_4096cubed.txt)",
+                "traffic": HEADLINE_TRAFFIC_MB, "traffic_unit": "MB per launch; NOT measured in this run: "
+                "rocprofv3 FETCH_SIZE + WRITE_SIZE of this kernel, calibrated on a plain copy, from "
+                "profiles/gemm_fp8_wave128_4096cubed.txt",
                 "kernel": "gemm_wave128_kernel<Op32F8<e4m3>,per-tensor> (256x256x128, 4 waves)",
-                "avg_launch_us": round(kern_ms * 1e3, 2)}
+                "avg_launch_us": round(kern_us, 2),
+                "timing": {"what": "HIP events on the launch stream; median of batch averages after a warm-up "
+                                   "that ends when two consecutive batches agree within 2%; independent of "
+                                   "--steps / --warmup", **proto}}
     if "mfma_fp8_random_TFLOPs" in ceilings:
         # the same kernel against what this GPU's MFMA pipe sustains on random operand bits
         roofline["measured_ceiling"] = {
@@ -404,7 +538,7 @@ def main():
     if not args.no_cpu:
         from oracle import w8a8_oracle as O
 
-        cores = min(os.cpu_count() or 1, 16)
+        cores = _cpu_threads()
         torch.set_num_threads(cores)
         O.fp8_gemm(a8_cpu[:256], b8_cpu, sa, sb)  # warm-up
         trials = []
@@ -419,7 +553,20 @@ def main():
                                   "median of 3 after 1 warm-up", "ms": round(med * 1e3, 1)}
 
     extra = {}
+    cpu_more = {}
     if not args.no_extra:
+        def ms_of(fn):
+            return _kernel_us(fn) * 1e-3
+
+        def cpu_median_ms(fn, trials=3):
+            fn()  # warm-up
+            ts = []
+            for _ in range(trials):
+                t0 = time.perf_counter()
+                fn()
+                ts.append(time.perf_counter() - t0)
+            return sorted(ts)[len(ts) // 2] * 1e3
+
         # ---- int8 4096^3 through the tiled kernel
         ai = torch.randint(-127, 128, (M, K), dtype=torch.int8).to(dev)
         bi = torch.randint(-127, 128, (N, K), dtype=torch.int8).to(dev)
@@ -431,7 +578,7 @@ def main():
                                                        swi.data_ptr(), None, out.data_ptr(),
                                                        M, N, K, 0, stream))
 
-        ms = _event_time_ms(step_i8, 500, 300)
+        ms = ms_of(step_i8)
         tops = flop / (ms * 1e-3) / 1e12
         extra["int8_gemm_4096"] = {"us": round(ms * 1e3, 2), "TOP/s": round(tops, 1),
                                    "frac_mfma_peak": round(tops / PEAK_INT8_TOPS, 4)}
@@ -444,7 +591,7 @@ def main():
                                               sb_d.data_ptr(), None, bias.data_ptr(), out.data_ptr(),
                                               M, N, K, 0, 0, stream))
 
-        ms = _event_time_ms(step_bias, 500, 300)
+        ms = ms_of(step_bias)
         extra["fp8_gemm_4096_bias"] = {"us": round(ms * 1e3, 2),
                                        "TFLOP/s": round(flop / (ms * 1e-3) / 1e12, 1)}
         del ai, bi
@@ -457,7 +604,7 @@ def main():
             check(lib.astrai_w8a8_gemm_fp8_ptpc(a8.data_ptr(), b8.data_ptr(), sa_rows.data_ptr(),
                                                 sb_rows.data_ptr(), None, out.data_ptr(), M, N, K, 0, stream))
 
-        ms = _event_time_ms(step_rowcol, 500, 300)
+        ms = ms_of(step_rowcol)
         extra["fp8_gemm_4096_row_and_column_scales"] = {"us": round(ms * 1e3, 2),
                                                         "TFLOP/s": round(flop / (ms * 1e-3) / 1e12, 1)}
 
@@ -474,12 +621,12 @@ def main():
         def step_bwd():
             mod.linear_backward_fp8(gb16, xb16, wb16, [1, 1, 0], s_one, s_one, s_one, 0)
 
-        ms = _event_time_ms(step_bwd, 100, 30)
+        ms = ms_of(step_bwd)
 
         def step_qt():
             mod.quantize_transpose_bf16(gb16, s_one, 0, True, True)
 
-        ms_qt = _event_time_ms(step_qt, 200, 50)
+        ms_qt = ms_of(step_qt)
         extra["fp8_linear_backward_4096"] = {
             "us": round(ms * 1e3, 1), "TFLOP/s_two_gemms": round(2 * flop / (ms * 1e-3) / 1e12, 1),
             "quantize_transpose_us": round(ms_qt * 1e3, 2),
@@ -489,24 +636,28 @@ def main():
         import torch.nn.functional as F
         from astrai_amd.extension import fp8 as P
 
-        e2e = {"bf16_stock_us": round(_event_time_ms(lambda: F.linear(xb16, wb16), 100, 30) * 1e3, 1)}
+        e2e = {"bf16_stock_us": round(ms_of(lambda: F.linear(xb16, wb16)) * 1e3, 1)}
         for rname, recipe in (("dynamic", P.DynamicScaling()), ("delayed", P.DelayedScaling())):
             for cache in (False, True):
                 P.fp8_state().reset()
                 with P.fp8_autocast(True, recipe=recipe):
                     P.fp8_cache_weights(cache)
-                    ms = _event_time_ms(lambda: F.linear(xb16, wb16), 100, 30)
+                    ms = ms_of(lambda: F.linear(xb16, wb16))
                 e2e[f"{rname}{'_cached_weight' if cache else ''}_us"] = round(ms * 1e3, 1)
         P.fp8_state().reset()
         extra["fp8_linear_4096_through_dispatcher"] = e2e
         del gb16, xb16, wb16
 
-        # ---- config 3: block-scaled fp8 8192 x 2048 x 7168
+        # ---- config 3: block-scaled fp8 8192 x 2048 x 7168 on the seed-3 tensors (activation,
+        # weight, outlier mask drawn in this order; 1% of the weights x 20), quantized per
+        # 1x128 / 128x128 block by the device quantizers
         M3, N3, K3 = 8192, 2048, 7168
-        a3 = torch.randn(M3, K3, device=dev).clamp(-3, 3).to(torch.float8_e4m3fn)
-        b3 = torch.randn(N3, K3, device=dev).clamp(-3, 3).to(torch.float8_e4m3fn)
-        sa3 = torch.rand(M3, K3 // 128, device=dev) + 0.5
-        sb3 = torch.rand(N3 // 128, K3 // 128, device=dev) + 0.5
+        g3 = torch.Generator().manual_seed(3)
+        x3 = torch.randn(M3, K3, generator=g3).to(torch.bfloat16)
+        w3 = torch.randn(N3, K3, generator=g3) * 0.02
+        w3 = torch.where(torch.rand(N3, K3, generator=g3) < 0.01, w3 * 20.0, w3).to(torch.bfloat16)
+        a3, sa3 = _cabi.quantize_fp8_block128_act(x3.to(dev))
+        b3, sb3 = _cabi.quantize_fp8_block128_weight(w3.to(dev))
         out3 = torch.empty(M3, N3, device=dev, dtype=torch.bfloat16)
 
         def step_blk():
@@ -514,22 +665,42 @@ def main():
                                                     sb3.data_ptr(), None, out3.data_ptr(),
                                                     M3, N3, K3, stream))
 
-        ms = _event_time_ms(step_blk, 300, 150)
+        ms = ms_of(step_blk)
         f3 = 2.0 * M3 * N3 * K3
         extra["fp8_block128_8192x2048x7168"] = {
+            "data": "BASELINE config 3 (seed 3)",
             "us": round(ms * 1e3, 2), "TFLOP/s": round(f3 / (ms * 1e-3) / 1e12, 1),
             "frac_mfma_peak": round(f3 / (ms * 1e-3) / 1e12 / PEAK_FP8_TFLOPS, 4)}
-        del a3, b3, out3
+        if not args.no_cpu:
+            from oracle import w8a8_oracle as O
 
-        # ---- config 2: decode GEMV, weights rotated through a ring larger than the
-        # 256 MB Infinity Cache so that every launch streams from HBM
+            # CPU: the first 1024 activation rows (1/8 of the GEMM), scaled to the whole
+            rows = 1024
+            a3c, sa3c = a3[:rows].cpu(), sa3[:rows].cpu()
+            b3c, sb3c = b3.cpu(), sb3.cpu()
+            cms = cpu_median_ms(lambda: O.fp8_gemm_blockscaled(a3c, b3c, sa3c, sb3c))
+            cpu_more["config3_fp8_block128"] = {
+                "value": round(f3 * rows / M3 / (cms * 1e-3) / 1e12, 4), "unit": "TFLOP/s", "cores": _cpu_threads(),
+                "kind": "port", "ms_sample": round(cms, 1), "ms_whole_extrapolated": round(cms * M3 / rows, 1),
+                "sample": f"rows 0..{rows - 1} of the config-3 activation against the whole weight (1/8 of the "
+                          "GEMM: 56 K-block fp32 matmuls with the block steps applied), median of 3 after 1 warm-up"}
+            del a3c, b3c
+        del a3, b3, out3, x3, w3
+
+        # ---- config 2: decode GEMV on the seed-2 tensors (activation and weight quantized per
+        # token / per channel by the oracle's quantizer on the host), weights rotated through a
+        # ring of ten copies (451 MB) so that the 256 MB Infinity Cache cannot serve them
+        from oracle import w8a8_oracle as O2
+
         N2, K2 = 11008, 4096
-        ring = [torch.randint(-127, 128, (N2, K2), dtype=torch.int8, device=dev) for _ in range(10)]
-        sw2 = torch.rand(N2, device=dev) + 0.5
-        gemv = {}
+        x2_all, w2, _ = O2.make_inputs(2, 64, N2, K2)
+        wq2, sw2c = O2.int8_quantize_rows(w2)
+        ring = [wq2.to(dev).clone() for _ in range(10)]
+        sw2 = sw2c.reshape(-1).to(dev)
+        gemv, cpu_c2 = {}, {}
         for m in (1, 4, 16, 64):
-            x2 = torch.randint(-127, 128, (m, K2), dtype=torch.int8, device=dev)
-            sx2 = torch.rand(m, device=dev) + 0.5
+            xq2c, sx2c = O2.int8_quantize_rows(x2_all[:m])
+            x2, sx2 = xq2c.to(dev), sx2c.reshape(-1).to(dev)
             y2 = torch.empty(m, N2, device=dev, dtype=torch.bfloat16)
 
             def launch(i, x2=x2, sx2=sx2, y2=y2, m=m):
@@ -538,23 +709,32 @@ def main():
                     x2.data_ptr(), w.data_ptr(), sx2.data_ptr(), sw2.data_ptr(), None,
                     y2.data_ptr(), m, N2, K2, 0, torch.cuda.current_stream().cuda_stream))
 
-            ms = _graph_time_ms(launch, 40, 10)
+            us = _graph_us(launch)
             nbytes = N2 * K2 + m * K2 + 2 * m * N2 + 4 * N2 + 4 * m
-            gbs = nbytes / (ms * 1e-3) / 1e9
-            ms1 = _graph_time_ms(lambda i: launch(0), 40, 10)
-            gemv[f"M{m}"] = {"us": round(ms * 1e3, 2), "GB/s": round(gbs, 0),
+            gbs = nbytes / (us * 1e-6) / 1e9
+            us1 = _graph_us(lambda i: launch(0))
+            gemv[f"M{m}"] = {"us": round(us, 2), "GB/s": round(gbs, 0),
                              "frac_hbm_peak": round(gbs / PEAK_HBM_GBS, 4),
                              **({"frac_measured_stream": round(gbs / ceilings["hbm_stream_45MB_GBs"], 4)}
                                 if "hbm_stream_45MB_GBs" in ceilings else {}),
-                             "single_buffer_cache_resident_us": round(ms1 * 1e3, 2)}
-        extra["int8_gemv_11008x4096_hbm_ring"] = gemv
+                             "single_buffer_cache_resident_us": round(us1, 2)}
+            if not args.no_cpu:
+                cms = cpu_median_ms(lambda: O2.int8_gemm(xq2c, wq2, sx2c, sw2c), trials=5)
+                cpu_c2[f"M{m}"] = {"ms": round(cms, 2), "GB/s": round(nbytes / (cms * 1e-3) / 1e9, 1)}
+        extra["int8_gemv_11008x4096_hbm_ring"] = {"data": "BASELINE config 2 (seed 2)", **gemv}
+        if cpu_c2:
+            cpu_more["config2_int8_gemv"] = {
+                "unit": "GB/s of the same algorithmic bytes", "cores": _cpu_threads(), "kind": "port",
+                "sample": "the whole call at each M (exact int8 x int8 -> int32 matmul + scale epilogue -> bf16), "
+                          "median of 5 after 1 warm-up", **cpu_c2}
         del ring
 
-        # ---- config 0: 16 x 2048 x 2048 int8 linear (launch-latency bound)
-        x0 = torch.randint(-127, 128, (16, 2048), dtype=torch.int8, device=dev)
-        w0 = torch.randint(-127, 128, (2048, 2048), dtype=torch.int8, device=dev)
-        s0 = torch.rand(16, device=dev)
-        s1 = torch.rand(2048, device=dev)
+        # ---- config 0: 16 x 2048 x 2048 int8 linear (launch-latency bound), seed-0 tensors
+        xc, wc, _ = O2.make_inputs(0, 16, 2048, 2048)
+        wq0c, sw0c = O2.int8_quantize_rows(wc)
+        xq0c, sx0c = O2.int8_quantize_rows(xc)
+        x0, w0 = xq0c.to(dev), wq0c.to(dev)
+        s0, s1 = sx0c.reshape(-1).to(dev), sw0c.reshape(-1).to(dev)
         y0 = torch.empty(16, 2048, device=dev, dtype=torch.bfloat16)
 
         def launch0(i):
@@ -562,23 +742,22 @@ def main():
                                                  s1.data_ptr(), None, y0.data_ptr(), 16, 2048, 2048,
                                                  0, torch.cuda.current_stream().cuda_stream))
 
-        ms = _graph_time_ms(launch0, 40, 10)
-        extra["int8_config0_16x2048x2048"] = {"us": round(ms * 1e3, 2)}
+        extra["int8_config0_16x2048x2048"] = {"data": "BASELINE config 0 (seed 0)",
+                                              "us": round(_graph_us(launch0), 2)}
         if not args.no_cpu:
-            from oracle import w8a8_oracle as O
-
-            xc, wc, _ = O.make_inputs(0, 16, 2048, 2048)
-            wq, sw = O.int8_quantize_rows(wc)
-            O.int8_linear(xc, wq, sw)
-            ts = []
-            for _ in range(5):
-                t0 = time.perf_counter()
-                O.int8_linear(xc, wq, sw)
-                ts.append(time.perf_counter() - t0)
-            extra["int8_config0_16x2048x2048"]["cpu_oracle_ms"] = round(sorted(ts)[2] * 1e3, 2)
+            cms = cpu_median_ms(lambda: O2.int8_linear(xc, wq0c, sw0c), trials=5)
+            extra["int8_config0_16x2048x2048"]["cpu_oracle_ms"] = round(cms, 3)
+            cpu_more["config0_int8_linear"] = {
+                "value": round(cms, 3), "unit": "ms", "cores": _cpu_threads(), "kind": "port",
+                "sample": "the whole config-0 linear (per-token quantize, int32 matmul, scale -> bf16), "
+                          "median of 5 after 1 warm-up"}
 
     if not args.no_extra and not args.no_model:
         extra["decoder_config4_int8"] = _bench_decoder(dev)
+        if not args.no_cpu:
+            cpu_more["config4_decoder"] = _cpu_decoder_baseline()
+    if cpu_more:
+        extra["cpu_baselines"] = cpu_more
 
     line = {
         "metric": "W8A8 GEMM TFLOPS/TOPS + % MFMA peak; decode GEMV GB/s + % HBM peak (1 GPU)",
@@ -588,7 +767,7 @@ def main():
         "config": {"workload": "BASELINE config 1: fp8 e4m3fn per-tensor GEMM, M=N=K=4096, "
                                "fp32 accumulate, bf16 out, seed 1"},
         "roofline": roofline, "cpu_baseline": cpu_baseline, "extra": extra,
-        "host": {"cpu_count": os.cpu_count(), "torch": torch.__version__},
+        "host": {**_host_info(), "cpu_threads_used": _cpu_threads(), "torch": torch.__version__},
         "measured_ceilings": ceilings,
     }
     print(json.dumps(line))

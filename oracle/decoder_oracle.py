@@ -249,3 +249,34 @@ def forward(sd: Dict[str, torch.Tensor], cfg, input_ids: torch.Tensor,
         x = lin(up * F.silu(gate), p + "mlp.down.weight") + x
     hidden = F.rms_norm(x, (cfg.hidden_size,), sd["norm.weight"], cfg.rms_norm_eps)
     return lin(hidden, "lm_head.weight")
+
+
+def forward_cached(sd: Dict[str, torch.Tensor], cfg, input_ids: torch.Tensor,
+                   lin: Callable[[torch.Tensor, str], torch.Tensor], k_cache: torch.Tensor,
+                   v_cache: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+    """The same forward for a block of tokens at ``positions [S]`` with a dense KV cache
+    ``[layers, B, H_kv, max_len, D]`` (updated in place): the cached branch of
+    components/attention.py:19-85, i.e. :func:`rope_cache_write` then :func:`attn_cached` per
+    layer. A prefill followed by one-token calls reproduces :func:`forward` (the contract of
+    tests/module/test_model_forward.py:71-115)."""
+    b, s = input_ids.shape
+    nh, nkv = cfg.num_attention_heads, cfg.num_key_value_heads
+    hd = cfg.hidden_size // nh
+    x = F.embedding(input_ids, sd["embed_tokens.weight"])
+    table = rotary_table(hd, int(positions.max()) + 1, cfg.rope_theta)
+    fc = table.index_select(0, positions).unsqueeze(0)      # [1, S, hd/2, 2]
+    for i in range(cfg.num_hidden_layers):
+        p = f"layers.{i}."
+        h = F.rms_norm(x, (cfg.hidden_size,), sd[p + "input_norm.weight"], cfg.rms_norm_eps)
+        qkv = torch.cat([lin(h, p + "attention.q_proj.weight"), lin(h, p + "attention.k_proj.weight"),
+                         lin(h, p + "attention.v_proj.weight")], dim=-1)
+        q = rope_cache_write(qkv, fc, positions, k_cache[i], v_cache[i], nh, nkv, hd)
+        a = attn_cached(q, k_cache[i], v_cache[i], positions)
+        x = lin(a, p + "attention.o_proj.weight") + x
+        h = F.rms_norm(x, (cfg.hidden_size,), sd[p + "post_attention_norm.weight"], cfg.rms_norm_eps)
+        up = lin(h, p + "mlp.up.weight")
+        gate = lin(h, p + "mlp.gate.weight")
+        x = lin(up * F.silu(gate), p + "mlp.down.weight") + x
+    hidden = F.rms_norm(x, (cfg.hidden_size,), sd["norm.weight"], cfg.rms_norm_eps)
+    return lin(hidden, "lm_head.weight")
+

@@ -151,10 +151,22 @@ def int8_quantize_rows(x: torch.Tensor):
     return q, s
 
 
+def int8_acc_int32_matmul(xq: torch.Tensor, wq: torch.Tensor) -> torch.Tensor:
+    """Exact int32 accumulator ``xq @ wq^T`` as a plain int32 tensor matmul."""
+    return xq.to(torch.int32) @ wq.to(torch.int32).t()
+
+
 def int8_acc(xq: torch.Tensor, wq: torch.Tensor) -> torch.Tensor:
     """Exact int32 accumulator ``xq @ wq^T``. fp32 matmul of int8 values is not
-    exact once K*127^2 >= 2^24, so the integer matmul is used at every size."""
-    return xq.to(torch.int32) @ wq.to(torch.int32).t()
+    exact once K*127^2 >= 2^24, so an integer matmul is used at every size:
+    PyTorch's int8 x int8 -> int32 CPU routine (``torch._int_mm``), which takes any
+    shape and is ~200x faster than the int32 tensor matmul it is pinned against
+    (tests/test_oracle_gemm.py: equal to :func:`int8_acc_int32_matmul`, to the C loop
+    and to pure-Python integer loops, worst-case magnitudes included). That routine
+    returns garbage for K = 1 (torch 2.10 CPU), so short contractions keep the int32 matmul."""
+    if xq.dtype == torch.int8 and wq.dtype == torch.int8 and xq.size(-1) >= 16 and xq.numel() and wq.numel():
+        return torch._int_mm(xq.contiguous(), wq.contiguous().t())
+    return int8_acc_int32_matmul(xq, wq)
 
 
 def int8_gemm(xq, wq, sx, sw, bias=None):

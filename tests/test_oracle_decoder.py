@@ -75,6 +75,29 @@ def test_causality_and_prefill_decode_contract():
     torch.testing.assert_close(torch.cat([pre] + dec, 1).float(), whole.float(), atol=2e-2, rtol=2e-2)
 
 
+def test_oracle_cached_forward_reproduces_the_full_forward():
+    """forward_cached (prefill, then one token at a time, then a two-token block) against
+    forward with bf16 linears: same arithmetic up to the attention's rounding (SDPA in bf16
+    there, float32 softmax here), and the cache ends up holding every position."""
+    torch.manual_seed(5)
+    model = AutoRegressiveLM(CFG).to(torch.bfloat16).eval()
+    sd = {k: v.detach() for k, v in model.state_dict().items()}
+    hd = CFG.hidden_size // CFG.num_attention_heads
+    ids = torch.randint(0, CFG.vocab_size, (2, 11))
+    for lin in (D.bf16_linear_fn(sd), D.int8_linear_fn(sd)):
+        whole = D.forward(sd, CFG, ids, lin).float()
+        kc = torch.zeros(CFG.num_hidden_layers, 2, CFG.num_key_value_heads, 11, hd, dtype=torch.bfloat16)
+        vc = torch.zeros_like(kc)
+        parts = [D.forward_cached(sd, CFG, ids[:, :6], lin, kc, vc, torch.arange(6))]
+        parts += [D.forward_cached(sd, CFG, ids[:, t:t + 1], lin, kc, vc, torch.tensor([t])) for t in range(6, 9)]
+        parts += [D.forward_cached(sd, CFG, ids[:, 9:11], lin, kc, vc, torch.arange(9, 11))]
+        inc = torch.cat(parts, 1).float()
+        scale = whole.abs().max().item()
+        assert (inc - whole).abs().max().item() <= 0.03 * scale
+        assert torch.nn.functional.cosine_similarity(inc.flatten(), whole.flatten(), dim=0).item() > 0.999
+        assert (kc.float().abs().sum(dim=(0, 1, 2, 4)) > 0).all()
+
+
 def test_int8_path_tracks_bf16_path():
     torch.manual_seed(3)
     model = AutoRegressiveLM(CFG).to(torch.bfloat16).eval()

@@ -176,6 +176,29 @@ def test_int8_config0_fp32_matmul_would_not_be_exact_but_int_is():
     assert torch.equal(acc, (xq.double() @ wq.double().t()).to(torch.int32))
 
 
+def test_int8_acc_library_routine_equals_int32_matmul_and_c_loop():
+    """The accumulator goes through PyTorch's int8 CPU routine; pin it on ragged shapes, a
+    decode shape, a multi-tile shape and worst-case magnitudes (every product +-127^2, K = 4096:
+    |acc| = 66 M, no wrap) against the int32 tensor matmul and the C triple loop."""
+    g = torch.Generator().manual_seed(11)
+    for m, n, k in ((1, 5, 1), (4, 3, 1), (3, 5, 7), (2, 3, 15), (5, 4, 16), (17, 9, 33), (1, 300, 4096), (130, 257, 1000), (64, 96, 4096)):
+        a = torch.randint(-127, 128, (m, k), dtype=torch.int8, generator=g)
+        b = torch.randint(-127, 128, (n, k), dtype=torch.int8, generator=g)
+        got = O.int8_acc(a, b)
+        assert got.dtype == torch.int32 and torch.equal(got, O.int8_acc_int32_matmul(a, b)), (m, n, k)
+        if m * n * k <= 4_000_000:
+            assert np.array_equal(got.numpy(), c_oracle.int8_gemm_i32(a.numpy(), b.numpy())), (m, n, k)
+    a = torch.full((5, 4096), 127, dtype=torch.int8)
+    a[1::2] = -127
+    b = torch.full((7, 4096), -127, dtype=torch.int8)
+    b[::3] = 127
+    want = (a.double() @ b.double().t())
+    assert want.abs().max().item() == 127 * 127 * 4096
+    assert torch.equal(O.int8_acc(a, b), want.to(torch.int32))
+    # a strided view takes the same route
+    assert torch.equal(O.int8_acc(a[:, ::2], b[:, ::2]), O.int8_acc_int32_matmul(a[:, ::2], b[:, ::2]))
+
+
 # ---- 128-block scaled ----
 
 def test_block128_exact_small(golden):
