@@ -1,39 +1,44 @@
 // Skinny int8 W8A8 kernels for decode shapes (M <= 128): bandwidth-bound, the
-// weight matrix is streamed from HBM exactly once and the MFMA pipe is almost
-// idle -- speed is set by bytes in flight and by how whole the memory requests
-// are. The int32 partials of the waves that split K are summed through LDS
-// (integer addition is associative, so the split keeps the accumulator
-// bit-exact) and the first waves run the dequant epilogue.
+// weight matrix is streamed from HBM exactly once (with the streaming cache hint:
+// no line of it is used twice) and the MFMA pipe is almost idle -- speed is set by
+// whole-line requests, by a steady, modest number of bytes in flight per wave and by
+// how often the activation block is pulled out of L2 again. The int32 partials of
+// the waves that split K are summed through LDS (integer addition is associative,
+// so the split keeps the accumulator bit-exact) and the first waves run the dequant
+// epilogue.
 //
-//  * M = 1: gemv_int8_dot_kernel, one wave per four weight rows, whole 1 KiB row
+//  * M = 1: gemv_int8_dot_kernel, one wave per two weight rows, whole 1 KiB row
 //    pieces straight into registers and v_dot4 on the vector ALU -- no LDS, no
-//    barrier, every wave of the launch resident and loading at once.
-//  * 2 <= M <= 16: gemv_int8_lds_kernel, 16 rows per workgroup, weights through
-//    LDS in 1 KiB row pieces, every load of the workgroup issued at once.
-//  * 17 <= M <= 128: skinny_int8_kernel, up to 48 rows per workgroup so that the
-//    activation block is pulled from L2 by as few workgroups as possible.
-// Measured at N=11008, K=4096 (weights from HBM): M=1 10.4 us, M=2..16 11.0-13.4,
-// M=32 16.6, M=64 21.2 (the tiled GEMM kernel needs 29 us for any M <= 128).
+//    barrier, every wave of the launch resident.
+//  * 2 <= M <= 64: gemv_int8_rows_kernel (gemv_rows.cuh), about one workgroup per
+//    compute unit with an equal share of the rows, a rolling ring of loads per wave.
+//  * 65 <= M <= 128: skinny_int8_kernel, up to 48 rows per workgroup, weights through
+//    LDS by direct-to-LDS loads.
+// Measured at N=11008, K=4096 (weights from HBM, graph replay): M=1 8.6 us, M=2..16
+// 9.3-9.9, M=32 11.2, M=64 13.9.
 #include "gemm_tile.cuh"
+#include "gemv_rows.cuh"
 
 namespace w8a8 {
 
 namespace {
 
-// Single-token kernel (M = 1). A workgroup is one wave and owns R = 4 weight
-// rows; lane l holds bytes [16 l, 16 l + 16) of every 1 KiB K-step of its rows and
+// Single-token kernel (M = 1). A workgroup is one wave and owns R weight rows
+// (two, or four for a short matrix); lane l holds bytes [16 l, 16 l + 16) of every 1 KiB K-step of its rows and
 // of the token, so each load instruction moves one whole 1 KiB row piece (the
 // request pattern HBM and the address coalescer like best) and the matching
 // activation bytes sit in the same lane. The dot products run on the vector ALU
 // (v_dot4_i32_i8, exact int32), which frees the kernel of LDS, barriers and
-// operand shuffles: a wave needs ~60 registers, so the ~2750 waves of an
-// 11008-row matrix are all resident at once and the whole matrix is requested in
-// the first microsecond. Lane partials are summed across the wave at the end
-// (integer addition: the split over lanes keeps the accumulator bit-exact). The
-// vector ALU's dot4 rate carries one token comfortably, not several: from two
-// tokens on the MFMA kernel below is faster.
+// operand shuffles: a wave needs few registers, so the ~5500 waves of an
+// 11008-row matrix are all resident at once, each with four K-steps (8 KiB of
+// weights) in flight. Two rows per wave measured faster than four or eight (8.6 us
+// against 8.8 / 9.3 at 11008 x 4096, and the streaming hint is worth 1.2 us: 10.2 ->
+// 8.8). Lane partials are summed across the wave at the end (integer addition: the
+// split over lanes keeps the accumulator bit-exact). The vector ALU's dot4 rate
+// carries one token comfortably, not several: from two tokens on the MFMA kernel
+// is faster.
+template <int R>
 __global__ __launch_bounds__(64) void gemv_int8_dot_kernel(GemmArgs g) {
-    constexpr int R = 4;
     const int lane = threadIdx.x;
     const int n0 = blockIdx.x * R;
     const int K = g.k;
@@ -56,13 +61,14 @@ __global__ __launch_bounds__(64) void gemv_int8_dot_kernel(GemmArgs g) {
         if (g.bias) e_b = bf16_to_f32(static_cast<const uint16_t*>(g.bias)[en]);
     }
 
-    int acc[R] = {0, 0, 0, 0};
-#pragma unroll 2
+    int acc[R] = {};
+#pragma unroll(8 / R)
     for (int k0 = 0; k0 < K; k0 += 1024) {
         const bool in = k0 + lane * 16 < K;
         u32x4 wv[R];
 #pragma unroll
-        for (int r = 0; r < R; ++r) wv[r] = buf_load16(rw, in ? w_off[r] : kOutOfRange, (uint32_t)k0);
+        for (int r = 0; r < R; ++r)
+            wv[r] = buf_load16_aux<kAuxStream>(rw, in ? w_off[r] : kOutOfRange, (uint32_t)k0);
         const u32x4 xv = buf_load16(rx, in ? (uint32_t)(lane * 16) : kOutOfRange, (uint32_t)k0);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -96,128 +102,12 @@ __global__ __launch_bounds__(64) void gemv_int8_dot_kernel(GemmArgs g) {
     }
 }
 
-// Variant that streams the weights through LDS: every load instruction moves
-// 1 KiB of ONE weight row (64 lanes x 16 contiguous bytes) straight into LDS, so
-// HBM, L2 and the address coalescer all see whole 128-byte lines in order; the
-// MFMA operands (16 rows x 16 bytes per K-group) are then cut out of LDS, where
-// the strided access is free. A workgroup of four waves owns 16 weight rows, wave
-// w takes the 1 KiB K-steps w, w+4, ...; rows are laid down 1040 bytes apart so
-// that the 16 rows of an operand read fall in distinct banks.
-constexpr int kLdsRow = 1040;
-
-template <int MB>
-__global__ __launch_bounds__(256) void gemv_int8_lds_kernel(GemmArgs g) {
-    __shared__ __attribute__((aligned(16))) uint8_t wbuf[4][16 * kLdsRow];
-    __shared__ i32x4 red[4][MB][64];
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int lrow = lane & 15, lgrp = lane >> 4;
-    const int K = g.k;
-    const int nsteps = (K + 1023) >> 10;
-    const int n0 = blockIdx.x * 16;
-
-    const __amdgpu_buffer_rsrc_t rw = make_rsrc(g.b, (uint32_t)g.n * (uint32_t)K);
-    const __amdgpu_buffer_rsrc_t rx = make_rsrc(g.a, (uint32_t)g.m * (uint32_t)K);
-
-    // epilogue operands first: their latency hides under the weight stream
-    const int en = n0 + lgrp * 4;
-    f32x4 sw4 = {0.0f, 0.0f, 0.0f, 0.0f};
-    float sxv[MB];
-    if (g.out_kind != OUT_ACC && wave < MB) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            if (en + j < g.n) sw4[j] = g.sb[en + j];
-    }
-#pragma unroll
-    for (int b = 0; b < MB; ++b) {
-        const int m = b * 16 + lrow;
-        sxv[b] = (g.out_kind != OUT_ACC && m < g.m) ? g.sa[m] : 0.0f;
-    }
-
-    i32x4 acc[MB];
-#pragma unroll
-    for (int b = 0; b < MB; ++b) acc[b] = i32x4{0, 0, 0, 0};
-    uint8_t* const mine = wbuf[wave];
-
-    for (int s = wave; s < nsteps; s += 4) {
-        const uint32_t k0 = (uint32_t)s << 10;
-        // weights: 16 rows x 1 KiB, one instruction per row
-        const bool k_in = (int)(k0 + lane * 16) < K;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const uint32_t off = (uint32_t)(n0 + r) * (uint32_t)K + lane * 16;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                rw, (__attribute__((address_space(3))) void*)(mine + r * kLdsRow), 16,
-                k_in ? off : kOutOfRange, k0, 0, 0);
-        }
-        // activations: MFMA layout straight from L2 (they are a few KiB, shared by
-        // every workgroup)
-        u32x4 xf[MB][16];
-#pragma unroll
-        for (int b = 0; b < MB; ++b) {
-            const uint32_t xo = (uint32_t)(b * 16 + lrow) * (uint32_t)K + lgrp * 16;
-#pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                const bool in = (int)(k0 + j * 64 + lgrp * 16) < K;
-                xf[b][j] = buf_load16(rx, in ? xo + j * 64 : kOutOfRange, k0);
-            }
-        }
-        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the wave's own rows are in LDS
-#pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            const u32x4 wf = *reinterpret_cast<const u32x4*>(mine + lrow * kLdsRow + j * 64 + lgrp * 16);
-#pragma unroll
-            for (int b = 0; b < MB; ++b)
-                acc[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8((i32x4)wf, (i32x4)xf[b][j], acc[b], 0, 0, 0);
-        }
-    }
-
-#pragma unroll
-    for (int b = 0; b < MB; ++b) red[wave][b][lane] = acc[b];
-    __syncthreads();
-    if (wave < MB) {
-        const int b = wave;
-        const i32x4 sum = red[0][b][lane] + red[1][b][lane] + red[2][b][lane] + red[3][b][lane];
-        const int m = b * 16 + lrow;
-        if (m < g.m && en < g.n) {
-            const size_t o = (size_t)m * g.n + en;
-            if (g.out_kind == OUT_ACC) {
-                int* out = static_cast<int*>(g.out);
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    if (en + j < g.n) out[o + j] = sum[j];
-            } else {
-                const uint16_t* bias = static_cast<const uint16_t*>(g.bias);
-                float sx = 0.0f;
-#pragma unroll
-                for (int bb = 0; bb < MB; ++bb)
-                    if (bb == b) sx = sxv[bb];
-                float v[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    float f = (float)sum[j] * sx * sw4[j];
-                    if (bias && en + j < g.n) f += bf16_to_f32(bias[en + j]);
-                    v[j] = f;
-                }
-                uint16_t* out = static_cast<uint16_t*>(g.out);
-                if ((g.n & 3) == 0) {
-                    u32x2 pk;
-                    pk.x = pack_bf16x2(v[0], v[1]);
-                    pk.y = pack_bf16x2(v[2], v[3]);
-                    *reinterpret_cast<u32x2*>(out + o) = pk;
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        if (en + j < g.n) out[o + j] = f32_to_bf16(v[j]);
-                }
-            }
-        }
-    }
-}
-
 void launch_dot(const GemmArgs& g, hipStream_t stream) {
-    const int blocks = (g.n + 3) / 4;
-    gemv_int8_dot_kernel<<<dim3((unsigned)blocks), dim3(64), 0, stream>>>(g);
+    // a short matrix has too few rows to fill the chip with two-row waves' small windows
+    if (g.n < 4096)
+        gemv_int8_dot_kernel<4><<<dim3((unsigned)((g.n + 3) / 4)), dim3(64), 0, stream>>>(g);
+    else
+        gemv_int8_dot_kernel<2><<<dim3((unsigned)((g.n + 1) / 2)), dim3(64), 0, stream>>>(g);
 }
 
 // Skinny kernel for 2 <= M <= 128 (batched decode). The weight matrix is streamed
@@ -457,22 +347,8 @@ void launch_skinny(const GemmArgs& g, hipStream_t stream, const RopeCacheArgs& r
 
 // the q|k|v projection with rotary and cache write in the epilogue: up to 64 tokens
 template <int RG, int NW>
-void launch_skinny_rope_mb(const GemmArgs& g, const RopeCacheArgs& rc, hipStream_t stream) {
-    switch ((g.m + 15) / 16) {
-        case 1: launch_skinny<RG, 1, NW, true>(g, stream, rc); break;
-        case 2: launch_skinny<RG, 2, NW, true>(g, stream, rc); break;
-        case 3: launch_skinny<RG, 3, NW, true>(g, stream, rc); break;
-        default: launch_skinny<RG, 4, NW, true>(g, stream, rc); break;
-    }
-}
-
-template <int RG, int NW>
 void launch_skinny_mb(const GemmArgs& g, hipStream_t stream) {
     switch ((g.m + 15) / 16) {
-        case 1: launch_skinny<RG, 1, NW>(g, stream); break;
-        case 2: launch_skinny<RG, 2, NW>(g, stream); break;
-        case 3: launch_skinny<RG, 3, NW>(g, stream); break;
-        case 4: launch_skinny<RG, 4, NW>(g, stream); break;
         case 5: launch_skinny<RG, 5, NW>(g, stream); break;
         case 6: launch_skinny<RG, 6, NW>(g, stream); break;
         case 7: launch_skinny<RG, 7, NW>(g, stream); break;
@@ -493,10 +369,54 @@ void launch_skinny_auto(const GemmArgs& g, hipStream_t stream) {
     else launch_skinny_mb<1, 16>(g, stream);
 }
 
-template <int MB>
-void launch_lds(const GemmArgs& g, hipStream_t stream) {
-    const int blocks = (g.n + 15) / 16;
-    gemv_int8_lds_kernel<MB><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(g);
+// Rows kernel launch plan. The rows are dealt out over 256 x rounds workgroups, rounds
+// being the smallest count that keeps a workgroup's range within 48 rows (three MFMA
+// row groups); ranges are rounded up to four rows (one load instruction). Four waves
+// split K; a short matrix with a long K (one row group, K >= 4096) takes eight so that
+// enough bytes are in flight (2048 x 5632: 5.7 us against 6.6 at M = 16). Measured per
+// shape against deeper rings (IB = 2..4), fewer / more waves and one workgroup per
+// sixteen rows: this plan was the fastest or within 2% of it on every decoder shape.
+struct RowsPlan { int rows_per_wg, rg, nw, blocks; };
+
+RowsPlan plan_rows(const GemmArgs& g) {
+    RowsPlan p;
+    const int rounds = (g.n + 256 * 48 - 1) / (256 * 48);
+    const int wgs = 256 * rounds;
+    p.rows_per_wg = (((g.n + wgs - 1) / wgs) + 3) & ~3;
+    p.rg = (p.rows_per_wg + 15) / 16;
+    p.nw = (p.rg == 1 && g.k >= 4096) ? 8 : 4;
+    p.blocks = (g.n + p.rows_per_wg - 1) / p.rows_per_wg;
+    return p;
+}
+
+template <int RG, int MB, int NW, bool ROPE>
+void launch_rows_inst(const GemmArgs& g, const RopeCacheArgs& rc, const RowsPlan& p, hipStream_t stream) {
+    constexpr int lds_bytes = gemv_rows_lds_bytes<RG, MB, NW>();
+    static_assert(lds_bytes <= 160 * 1024, "patches and partials of all waves must fit in LDS");
+    auto kern = gemv_int8_rows_kernel<RG, MB, NW, 1, ROPE>;
+    static std::atomic<uint64_t> lds_allowed{0};
+    allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_allowed);
+    kern<<<dim3((unsigned)p.blocks), dim3(NW * 64), lds_bytes, stream>>>(g, rc, p.rows_per_wg);
+}
+
+template <int RG, int NW, bool ROPE>
+void launch_rows_mb(const GemmArgs& g, const RopeCacheArgs& rc, const RowsPlan& p, hipStream_t stream) {
+    switch ((g.m + 15) / 16) {
+        case 1: launch_rows_inst<RG, 1, NW, ROPE>(g, rc, p, stream); break;
+        case 2: launch_rows_inst<RG, 2, NW, ROPE>(g, rc, p, stream); break;
+        case 3: launch_rows_inst<RG, 3, NW, ROPE>(g, rc, p, stream); break;
+        default: launch_rows_inst<RG, 4, NW, ROPE>(g, rc, p, stream); break;
+    }
+}
+
+// M <= 64
+template <bool ROPE>
+void launch_rows(const GemmArgs& g, const RopeCacheArgs& rc, hipStream_t stream) {
+    const RowsPlan p = plan_rows(g);
+    if (p.rg == 3) launch_rows_mb<3, 4, ROPE>(g, rc, p, stream);
+    else if (p.rg == 2) launch_rows_mb<2, 4, ROPE>(g, rc, p, stream);
+    else if (p.nw == 8) launch_rows_mb<1, 8, ROPE>(g, rc, p, stream);
+    else launch_rows_mb<1, 4, ROPE>(g, rc, p, stream);
 }
 
 }  // namespace
@@ -506,13 +426,7 @@ bool launch_gemm_int8_rope_cache(const GemmArgs& g, const RopeCacheArgs& rc, hip
     if (g.out_kind != OUT_BF16 || g.bias != nullptr || (rc.head_dim & 3) != 0) return false;
     if (g.m != rc.batch * rc.seq || g.n != (rc.n_heads + 2 * rc.n_kv_heads) * rc.head_dim) return false;
     if ((int64_t)g.n * g.k >= ((int64_t)1 << 31)) return false;
-    // the same workgroup shapes as the plain skinny launch
-    const int nsteps = (g.k + 511) >> 9;
-    if ((g.n + 47) / 48 >= 192) launch_skinny_rope_mb<3, 4>(g, rc, stream);
-    else if ((g.n + 31) / 32 >= 192) launch_skinny_rope_mb<2, 4>(g, rc, stream);
-    else if (nsteps <= 4 || (g.n + 15) / 16 >= 512) launch_skinny_rope_mb<1, 4>(g, rc, stream);
-    else if (nsteps <= 8) launch_skinny_rope_mb<1, 8>(g, rc, stream);
-    else launch_skinny_rope_mb<1, 16>(g, rc, stream);
+    launch_rows<true>(g, rc, stream);
     return true;
 }
 
@@ -522,8 +436,8 @@ bool launch_gemv_int8(const GemmArgs& g, hipStream_t stream) {
     if ((int64_t)g.n * g.k >= lim) return false;
     if (g.m == 1)
         launch_dot(g, stream);
-    else if (g.m <= 16)
-        launch_lds<1>(g, stream);
+    else if (g.m <= 64)
+        launch_rows<false>(g, RopeCacheArgs{}, stream);
     else
         launch_skinny_auto(g, stream);
     return true;
