@@ -60,6 +60,7 @@ w8a8::GemmArgs pack(const void* a, const void* b, const float* sa, const float* 
     g.n = (int)n;
     g.k = (int)k;
     g.out_kind = out_kind;
+    g.row_max = nullptr;
     return g;
 }
 
@@ -199,9 +200,47 @@ int astrai_w8a8_silu_mul_quantize_int8_rows(const void* gate, const void* up, in
     if (!aligned16(gate) || !aligned16(up) || !aligned16(hq) || (h_out && !aligned16(h_out)))
         return fail(ASTRAI_W8A8_BAD_ARG, "silu_mul_quantize_int8_rows: pointers must be 16-byte aligned");
     if (rows == 0 || width == 0) return ASTRAI_W8A8_OK;
-    w8a8::launch_silu_mul_quantize_int8_rows(gate, up, ld, h_out, hq, s, rows, width,
+    w8a8::launch_silu_mul_quantize_int8_rows(gate, up, ld, 0, h_out, hq, s, rows, width,
                                              static_cast<hipStream_t>(stream));
     return check_launch("silu_mul_quantize_int8_rows");
+}
+
+int astrai_w8a8_silu_mul_quantize_int8_rows_blocked(const void* gu, int64_t ld, int64_t block,
+                                                    void* h_out, void* hq, float* s, int64_t rows,
+                                                    int64_t width, void* stream) {
+    const char* what = "silu_mul_quantize_int8_rows_blocked";
+    if (!gu || !hq || !s) return fail(ASTRAI_W8A8_BAD_ARG, "%s: null pointer", what);
+    if (rows < 0 || width < 0 || rows > 0x7fffffff || block <= 0 || ld < 2 * width)
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: bad dims", what);
+    if ((width & 7) != 0 || (ld & 7) != 0 || (block & 7) != 0 || width % block != 0 ||
+        width > w8a8::kFusedRowMax)
+        return fail(ASTRAI_W8A8_UNSUPPORTED,
+                    "%s: width, ld and block must be multiples of 8, width a multiple of block and at most 8192",
+                    what);
+    if (!aligned16(gu) || !aligned16(hq) || (h_out && !aligned16(h_out)))
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: pointers must be 16-byte aligned", what);
+    if (rows == 0 || width == 0) return ASTRAI_W8A8_OK;
+    w8a8::launch_silu_mul_quantize_int8_rows(gu, static_cast<const uint16_t*>(gu) + block, ld, block,
+                                             h_out, hq, s, rows, width,
+                                             static_cast<hipStream_t>(stream));
+    return check_launch(what);
+}
+
+int astrai_w8a8_quantize_int8_rows_pmax(const void* h, const float* row_max, int64_t pieces,
+                                        void* hq, float* s, int64_t rows, int64_t width,
+                                        void* stream) {
+    const char* what = "quantize_int8_rows_pmax";
+    if (!h || !row_max || !hq || !s) return fail(ASTRAI_W8A8_BAD_ARG, "%s: null pointer", what);
+    if (rows < 0 || width < 0 || pieces <= 0 || rows > 0x7fffffff)
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: bad dims", what);
+    if ((width & 7) != 0 || width > w8a8::kFusedRowMax)
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "%s: width must be a multiple of 8 and at most 8192", what);
+    if (!aligned16(h) || !aligned16(hq))
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: pointers must be 16-byte aligned", what);
+    if (rows == 0 || width == 0) return ASTRAI_W8A8_OK;
+    w8a8::launch_quantize_int8_rows_pmax(h, row_max, pieces, hq, s, rows, width,
+                                         static_cast<hipStream_t>(stream));
+    return check_launch(what);
 }
 
 int astrai_w8a8_rope_cache_write_bf16(const void* qkv, int64_t ld, const float* freqs,
@@ -657,6 +696,24 @@ int astrai_w8a8_gemm_int8_ptpc_rope_cache(const void* a, const void* b, const fl
                                  (int)batch, (int)seq, (int)n_heads, (int)n_kv_heads, (int)head_dim, max_len};
     if (!w8a8::launch_gemm_int8_rope_cache(g, rc, static_cast<hipStream_t>(stream)))
         return fail(ASTRAI_W8A8_UNSUPPORTED, "%s: shape not supported", what);
+    return check_launch(what);
+}
+
+int astrai_w8a8_gemm_int8_ptpc_swiglu(const void* a, const void* b, const float* sa, const float* sb,
+                                      void* h_out, float* row_max, int64_t m, int64_t n, int64_t k,
+                                      void* stream) {
+    const char* what = "gemm_int8_ptpc_swiglu";
+    if (int rc = int8_common(what, a, b, sa, sb, h_out, m, n, k, ASTRAI_W8A8_OUT_BF16)) return rc;
+    if (!row_max) return fail(ASTRAI_W8A8_BAD_ARG, "%s: null pointer", what);
+    if (n % 128)
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "%s: N (gate and up rows together) must be a multiple of 128", what);
+    if (m == 0 || n == 0) return ASTRAI_W8A8_OK;
+    w8a8::GemmArgs g = pack(a, b, sa, sb, nullptr, nullptr, h_out, m, n, k, w8a8::OUT_BF16);
+    g.row_max = row_max;
+    if (!w8a8::launch_gemm_int8_swiglu(g, static_cast<hipStream_t>(stream)))
+        return fail(ASTRAI_W8A8_UNSUPPORTED,
+                    "%s: needs at least 192 output tiles of 256 x 256, K a multiple of 128 and at least 256",
+                    what);
     return check_launch(what);
 }
 

@@ -21,4 +21,11 @@ bool launch_gemm_int8_tiled(const GemmArgs& g, hipStream_t stream) {
     return true;
 }
 
+bool launch_gemm_int8_swiglu(const GemmArgs& g, hipStream_t stream) {
+    if (!tiled_shape_ok(g) || !wave128_shape_ok(g) || (g.n & 127) != 0 || g.bias != nullptr || !g.row_max)
+        return false;
+    launch_wave128<Op32I8, SCALE_ROWCOL, EPI_SWIGLU>(g, stream);
+    return true;
+}
+
 }  // namespace w8a8

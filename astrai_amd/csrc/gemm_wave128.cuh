@@ -63,9 +63,18 @@ struct Wave128Cfg {
 __device__ constexpr int kReadIsW[8] = {1, 0, 1, 1, 1, 0, 0, 0};
 __device__ constexpr int kReadSub[8] = {0, 0, 1, 2, 3, 1, 2, 3};
 
-template <class Op, int ScaleKind>
+// silu(g) = g / (1 + exp(-g)) on the hardware's exp2 and reciprocal, the arithmetic of the
+// SwiGLU producer kernel (quantize.hip)
+__device__ __forceinline__ float silu_hw(float g) {
+    return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.44269504088896340736f));
+}
+
+enum : int { EPI_PLAIN = 0, EPI_SWIGLU = 1 };
+
+template <class Op, int ScaleKind, int Epi = EPI_PLAIN>
 __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmArgs g) {
     static_assert(ScaleKind != SCALE_BLOCK128, "block scales run on the ping-pong kernel");
+    static_assert(Epi == EPI_PLAIN || ScaleKind == SCALE_ROWCOL, "the SwiGLU epilogue is the int8 decoder's");
     PP_STAMP_INIT();
     using Cfg = Wave128Cfg;
     using Acc = typename Op::Acc;
@@ -279,6 +288,80 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
     // takes no part in the check. The stores are non-temporal (aux bit 1): the
     // 2 M N output bytes stream to memory while the epilogue still computes instead
     // of sitting dirty in L2 until the end-of-kernel write-back (-1.5 us at 4096^3).
+    if constexpr (Epi == EPI_SWIGLU) {
+        // The wave's 128 columns are 64 gate columns (sub-tiles 0, 1) and the 64 up columns
+        // (sub-tiles 2, 3) of the same 64 columns of h, so a lane holds every pair in its own
+        // registers. gate and up are rounded to bf16 as the plain epilogue would have stored
+        // them, then h = bf16(up * bf16(silu(gate))) -- the arithmetic of the SwiGLU producer
+        // kernel on the same rounded inputs. A pass is 32 rows x 64 columns of h (one 128-byte
+        // line per row) staged through wave-private LDS (144-byte rows) and stored as whole
+        // lines; the maximum of |h| over the wave's 64 columns goes to row_max[m, piece] (bf16
+        // magnitudes order like their bit patterns, so the maximum is taken on the packed bits).
+        constexpr int ROWB = 144, PASS_BYTES = 32 * ROWB;
+        uint8_t* const mine = lds + wave * (2 * PASS_BYTES);
+        const int rows_here = min(Cfg::BM, g.m - m0);
+        const int hw = g.n >> 1;                       // width of h
+        const uint32_t row_bytes = (uint32_t)hw * 2u;
+        const __amdgpu_buffer_rsrc_t rout =
+            make_rsrc(static_cast<uint16_t*>(g.out) + (size_t)m0 * hw, (uint32_t)rows_here * row_bytes);
+        const int nwv = n0 + wave_n * 128;             // first fused column of this wave
+        const int piece = nwv >> 7;                    // its 64-column piece of h
+        const int pieces = g.n >> 7;
+        f32x4 sw4[NI][4];
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int n = nwv + ni * 32 + q * 8 + lgrp * 4;
+                sw4[ni][q] = (n < g.n) ? *reinterpret_cast<const f32x4*>(g.sb + n) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+        const int r8 = lane >> 3, c8 = lane & 7;
+        const uint32_t lane_off = (nwv < g.n)
+            ? (uint32_t)(wave_m * 128 + r8) * row_bytes + (uint32_t)(piece * 64 + c8 * 8) * 2u
+            : kOutOfRange;
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi) {
+            uint8_t* const buf = mine + (mi & 1) * PASS_BYTES;
+            uint32_t mx = 0u;
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float gt[4], up[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+#pragma clang fp contract(off)
+                        gt[j] = (float)acc[ni][mi][4 * q + j] * sx[mi] * sw4[ni][q][j];
+                        up[j] = (float)acc[ni + 2][mi][4 * q + j] * sx[mi] * sw4[ni + 2][q][j];
+                    }
+                    u32x2 pk;
+#pragma unroll
+                    for (int p = 0; p < 2; ++p) {
+                        const uint32_t gb = pack_bf16x2(gt[2 * p], gt[2 * p + 1]);
+                        const uint32_t ub = pack_bf16x2(up[2 * p], up[2 * p + 1]);
+                        const uint32_t sb2 = pack_bf16x2(silu_hw(__uint_as_float(gb << 16)),
+                                                         silu_hw(__uint_as_float(gb & 0xffff0000u)));
+                        const uint32_t hb = pack_bf16x2(
+                            __uint_as_float(ub << 16) * __uint_as_float(sb2 << 16),
+                            __uint_as_float(ub & 0xffff0000u) * __uint_as_float(sb2 & 0xffff0000u));
+                        pk[p] = hb;
+                        const uint32_t mag = hb & 0x7fff7fffu;
+                        mx = max(mx, max(mag & 0xffffu, mag >> 16));
+                    }
+                    *reinterpret_cast<u32x2*>(buf + lrow * ROWB + (ni * 32 + q * 8 + lgrp * 4) * 2) = pk;
+                }
+            // the other half of the row's columns sits in lane ^ 32
+            mx = max(mx, (uint32_t)__shfl_xor((int)mx, 32, 64));
+            const int m = m0 + wave_m * 128 + mi * 32 + lrow;
+            if (lgrp == 0 && m < g.m && nwv < g.n) g.row_max[(size_t)m * pieces + piece] = __uint_as_float(mx << 16);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const u32x4 v = *reinterpret_cast<const u32x4*>(buf + (i * 8 + r8) * ROWB + c8 * 16);
+                __builtin_amdgcn_raw_buffer_store_b128(
+                    v, rout, lane_off + (uint32_t)(mi * 32 + i * 8) * row_bytes, 0, 2);
+            }
+        }
+    } else
     {
         constexpr int ROWB = Cfg::EPI_ROW_BYTES, PASS_BYTES = Cfg::EPI_PASS_BYTES;
         uint8_t* const mine = lds + wave * (2 * PASS_BYTES);
@@ -354,11 +437,11 @@ inline bool wave128_shape_ok(const GemmArgs& g) {
     return pingpong_shape_ok(g) && g.out_kind == OUT_BF16 && (g.n & 7) == 0 && g.n <= (1 << 22);
 }
 
-template <class Op, int ScaleKind>
+template <class Op, int ScaleKind, int Epi = EPI_PLAIN>
 inline void launch_wave128(const GemmArgs& g, hipStream_t stream) {
     using Cfg = Wave128Cfg;
     const int tiles = ((g.m + Cfg::BM - 1) / Cfg::BM) * ((g.n + Cfg::BN - 1) / Cfg::BN);
-    auto kern = gemm_wave128_kernel<Op, ScaleKind>;
+    auto kern = gemm_wave128_kernel<Op, ScaleKind, Epi>;
     static std::atomic<uint64_t> lds_allowed{0};
     allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::LDS_BYTES, lds_allowed);
     kern<<<dim3((unsigned)tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(g);

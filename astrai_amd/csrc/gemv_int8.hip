@@ -62,7 +62,8 @@ __global__ __launch_bounds__(64) void gemv_int8_dot_kernel(GemmArgs g) {
     }
 
     int acc[R] = {};
-#pragma unroll(8 / R)
+    constexpr int kSteps = 8 / R;  // K-steps in flight: 8 KiB of weights per wave
+#pragma unroll kSteps
     for (int k0 = 0; k0 < K; k0 += 1024) {
         const bool in = k0 + lane * 16 < K;
         u32x4 wv[R];

@@ -36,6 +36,7 @@ struct GemmArgs {
     void* out;            // [M,N]
     int m, n, k;
     int out_kind;
+    float* row_max = nullptr;  // SwiGLU epilogue only: fp32 [M, N/128] partial row maxima of |h|
 };
 
 // quantize.hip
@@ -58,9 +59,13 @@ constexpr int64_t kFusedRowMax = 8192;
 void launch_add_rmsnorm_quantize_int8_rows(const void* x, const void* res, const void* w, float eps,
                                            void* sum_out, void* y_out, void* xq, float* s,
                                            int64_t rows, int64_t k, hipStream_t stream);
-void launch_silu_mul_quantize_int8_rows(const void* gate, const void* up, int64_t ld, void* h_out,
-                                        void* hq, float* s, int64_t rows, int64_t width,
+// block > 0: gate and up columns come in pieces of `block` columns, 2 * block apart
+void launch_silu_mul_quantize_int8_rows(const void* gate, const void* up, int64_t ld, int64_t block,
+                                        void* h_out, void* hq, float* s, int64_t rows, int64_t width,
                                         hipStream_t stream);
+// per-row int8 of bf16 rows whose |maximum| is known as `pieces` partial maxima per row
+void launch_quantize_int8_rows_pmax(const void* h, const float* row_max, int64_t pieces, void* hq,
+                                    float* s, int64_t rows, int64_t width, hipStream_t stream);
 void launch_quantize_fp8_block128_act(const void* x, void* x8, float* sa, int64_t m,
                                       int64_t k, hipStream_t stream);
 void launch_quantize_fp8_block128_weight(const void* w, void* w8, float* sb, int64_t n,
@@ -187,6 +192,11 @@ bool launch_attn_rows(AttnRowsArgs a, hipStream_t stream);
 // Require k % 16 == 0 and m*k, n*k < 2^31 bytes; return false if the shape is
 // not accepted (the caller then uses the generic kernel).
 bool launch_gemm_int8_tiled(const GemmArgs& g, hipStream_t stream);
+// gate|up projection with the SwiGLU product in the epilogue. Weight rows come in blocks of
+// 128: 64 gate rows, then the 64 up rows of the same columns of h. g.out is h = bf16(up *
+// bf16(silu(gate))) [M, N/2], g.row_max[m, N/128] the maximum of |h| over each 64-column piece.
+// Large shapes only (those of the four-wave 256x256 kernel, N % 128 == 0, no bias); false otherwise.
+bool launch_gemm_int8_swiglu(const GemmArgs& g, hipStream_t stream);
 bool launch_gemm_fp8_tiled(const GemmArgs& g, int fmt, hipStream_t stream);
 // sa per activation row [M], sb per weight row [N], bf16 output
 bool launch_gemm_fp8_rowcol_tiled(const GemmArgs& g, int fmt, hipStream_t stream);

@@ -464,9 +464,12 @@ __device__ __forceinline__ float silu_f32(float g) {
 // h = bf16(up * bf16(silu(gate))), silu(g) = g / (1 + exp(-g)) in fp32: the bf16
 // arithmetic of ``up(x) * F.silu(gate(x))`` (model/components/mlp.py:41); then the
 // per-row int8 quantizer on h. gate and up rows are `ld` elements apart (they may
-// be the two halves of one fused gate|up GEMM output).
+// be the two halves of one fused gate|up GEMM output). With block > 0 the columns of
+// gate and of up come in pieces of `block` columns that lie 2 * block apart (a fused
+// output whose columns alternate between `block` gate and `block` up columns, `up`
+// pointing at the first up piece).
 __global__ __launch_bounds__(kThreads) void silu_mul_quantize_int8_rows_kernel(
-    const uint16_t* __restrict__ gate, const uint16_t* __restrict__ up, int64_t ld,
+    const uint16_t* __restrict__ gate, const uint16_t* __restrict__ up, int64_t ld, int64_t block,
     uint16_t* __restrict__ h_out, int8_t* __restrict__ hq, float* __restrict__ s, int64_t width) {
     __shared__ float slots[kThreads / kWave];
     const int64_t row = blockIdx.x;
@@ -478,8 +481,10 @@ __global__ __launch_bounds__(kThreads) void silu_mul_quantize_int8_rows_kernel(
         const int64_t i = threadIdx.x + (int64_t)c * kThreads;
         if (i < nvec) {
             float g[8];
-            unpack8(*reinterpret_cast<const u32x4*>(gate + row * ld + i * 8), g);
-            unpack8(*reinterpret_cast<const u32x4*>(up + row * ld + i * 8), v[c]);
+            const int64_t col = i * 8;
+            const int64_t src = block ? (col / block) * (2 * block) + col % block : col;
+            unpack8(*reinterpret_cast<const u32x4*>(gate + row * ld + src), g);
+            unpack8(*reinterpret_cast<const u32x4*>(up + row * ld + src), v[c]);
 #pragma unroll
             for (int j = 0; j < 8; ++j)
                 v[c][j] = round_bf16(v[c][j] * round_bf16(silu_f32(g[j])));
@@ -493,6 +498,37 @@ __global__ __launch_bounds__(kThreads) void silu_mul_quantize_int8_rows_kernel(
     for (int c = 0; c < kCache; ++c) {
         const int64_t i = threadIdx.x + (int64_t)c * kThreads;
         if (i < nvec) *reinterpret_cast<u32x2*>(hq + row * width + i * 8) = quant8_int8(v[c], step);
+    }
+}
+
+// Per-row int8 quantizer for rows whose maximum is already known in pieces: row_max holds
+// `pieces` partial maxima of |h| per row (written by the SwiGLU epilogue of the gate|up
+// GEMM), so the row is read once. Same codes and steps as quantize_int8_rows_kernel.
+__global__ __launch_bounds__(kThreads) void quantize_int8_rows_pmax_kernel(
+    const uint16_t* __restrict__ h, const float* __restrict__ row_max, int64_t pieces,
+    int8_t* __restrict__ hq, float* __restrict__ s, int64_t width) {
+    __shared__ float slots[kThreads / kWave];
+    const int64_t row = blockIdx.x;
+    const int64_t nvec = width >> 3;
+    // the row's data is requested before the maxima are reduced
+    u32x4 raw[kCache];
+#pragma unroll
+    for (int c = 0; c < kCache; ++c) {
+        const int64_t i = threadIdx.x + (int64_t)c * kThreads;
+        if (i < nvec) raw[c] = *reinterpret_cast<const u32x4*>(h + row * width + i * 8);
+    }
+    float local = 0.0f;
+    for (int64_t i = threadIdx.x; i < pieces; i += kThreads) local = fmaxf(local, row_max[row * pieces + i]);
+    const float step = fmaxf(block_max(local, slots), 1e-12f) / 127.0f;
+    if (threadIdx.x == 0) s[row] = step;
+#pragma unroll
+    for (int c = 0; c < kCache; ++c) {
+        const int64_t i = threadIdx.x + (int64_t)c * kThreads;
+        if (i < nvec) {
+            float v[8];
+            unpack8(raw[c], v);
+            *reinterpret_cast<u32x2*>(hq + row * width + i * 8) = quant8_int8(v, step);
+        }
     }
 }
 
@@ -618,13 +654,20 @@ void launch_add_rmsnorm_quantize_int8_rows(const void* x, const void* res, const
         static_cast<uint16_t*>(y_out), static_cast<int8_t*>(xq), s, k);
 }
 
-void launch_silu_mul_quantize_int8_rows(const void* gate, const void* up, int64_t ld, void* h_out,
-                                        void* hq, float* s, int64_t rows, int64_t width,
+void launch_silu_mul_quantize_int8_rows(const void* gate, const void* up, int64_t ld, int64_t block,
+                                        void* h_out, void* hq, float* s, int64_t rows, int64_t width,
                                         hipStream_t stream) {
     if (rows <= 0 || width <= 0) return;
     silu_mul_quantize_int8_rows_kernel<<<dim3((unsigned)rows), dim3(kThreads), 0, stream>>>(
-        static_cast<const uint16_t*>(gate), static_cast<const uint16_t*>(up), ld,
+        static_cast<const uint16_t*>(gate), static_cast<const uint16_t*>(up), ld, block,
         static_cast<uint16_t*>(h_out), static_cast<int8_t*>(hq), s, width);
+}
+
+void launch_quantize_int8_rows_pmax(const void* h, const float* row_max, int64_t pieces, void* hq,
+                                    float* s, int64_t rows, int64_t width, hipStream_t stream) {
+    if (rows <= 0 || width <= 0) return;
+    quantize_int8_rows_pmax_kernel<<<dim3((unsigned)rows), dim3(kThreads), 0, stream>>>(
+        static_cast<const uint16_t*>(h), row_max, pieces, static_cast<int8_t*>(hq), s, width);
 }
 
 void launch_quantize_fp8_block128_act(const void* x, void* x8, float* sa, int64_t m,

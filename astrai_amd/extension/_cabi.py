@@ -40,6 +40,9 @@ PROTOTYPES = {
     "astrai_w8a8_add_rmsnorm_quantize_int8_rows": (
         [_P, _P, _P, ctypes.c_float, _P, _P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_silu_mul_quantize_int8_rows": ([_P, _P, _I64, _P, _P, _P, _I64, _I64, _P], _INT),
+    "astrai_w8a8_gemm_int8_ptpc_swiglu": ([_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _INT),
+    "astrai_w8a8_quantize_int8_rows_pmax": ([_P, _P, _I64, _P, _P, _I64, _I64, _P], _INT),
+    "astrai_w8a8_silu_mul_quantize_int8_rows_blocked": ([_P, _I64, _I64, _P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_rope_cache_write_bf16": (
         [_P, _I64, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _P], _INT),
     "astrai_w8a8_attn_decode_workspace_floats": ([_I64, _I64, _I64, _I64], _I64),
@@ -987,6 +990,83 @@ def mm_int8(a: torch.Tensor, b: torch.Tensor, sa: Optional[torch.Tensor],
                 _check(fn(a_c.data_ptr(), b_c.data_ptr(), _ptr(sa), _ptr(sb), _ptr(bias),
                           out.data_ptr(), m, n, k, out_dtype, _stream(a)), lib)
     return out
+
+
+SWIGLU_BLOCK = 64
+
+
+def swiglu_block_rows(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """Rows of ``gate`` and ``up`` (``[W, ...]`` each, W a multiple of 64) in the order the
+    SwiGLU GEMM entry points take: blocks of 128 rows, 64 of gate then the 64 of up that
+    belong to the same columns of ``h``."""
+    w = gate.size(0)
+    if up.shape != gate.shape or w % SWIGLU_BLOCK:
+        raise RuntimeError("gate and up must have the same shape with a multiple of 64 rows")
+    rest = gate.shape[1:]
+    g = gate.reshape(w // SWIGLU_BLOCK, 1, SWIGLU_BLOCK, *rest)
+    u = up.reshape(w // SWIGLU_BLOCK, 1, SWIGLU_BLOCK, *rest)
+    return torch.cat((g, u), dim=1).reshape(2 * w, *rest).contiguous()
+
+
+def mm_int8_swiglu_fused_shape(m: int, n: int, k: int) -> bool:
+    """Shapes whose gate|up GEMM applies the SwiGLU product in its own epilogue (the limits
+    of ``astrai_w8a8_gemm_int8_ptpc_swiglu``); others run the GEMM and the blocked producer."""
+    tiles = ((m + 255) // 256) * ((n + 255) // 256)
+    return (tiles >= 192 and k >= 256 and k % 128 == 0 and n % 128 == 0 and n <= 1 << 22
+            and m * k < 2 ** 31 and n * k < 2 ** 31 and n // 2 <= FUSED_ROW_MAX)
+
+
+def mm_int8_swiglu(a: torch.Tensor, wgu: torch.Tensor, sa: torch.Tensor, sgu: torch.Tensor,
+                   want_h: bool = False, fused: Optional[bool] = None):
+    """``h = up * silu(gate)`` of the gate and up projections of ``a`` and its per-row int8
+    form, ``wgu`` / ``sgu`` being the int8 weight and its scales in :func:`swiglu_block_rows`
+    order. Returns ``(hq [M, W], s [M, 1], h or None)``, bit for bit what :func:`mm_int8` on
+    the unblocked weight followed by :func:`silu_mul_quantize_int8` gives. Large shapes run
+    the GEMM whose epilogue forms ``h`` and the row maxima piecewise, then the one-read
+    quantizer; others the plain GEMM and the producer that reads the blocked columns
+    (``fused`` forces one or the other)."""
+    lib = _require()
+    _gpu(a, "mm_int8_swiglu")
+    if a.dtype != torch.int8 or wgu.dtype != torch.int8 or a.dim() != 2 or wgu.dim() != 2:
+        raise RuntimeError("a and wgu must be 2D int8")
+    if a.size(1) != wgu.size(1) or a.device != wgu.device:
+        raise RuntimeError("inner dim or device mismatch")
+    m, k = a.shape
+    n = wgu.size(0)
+    if n % (2 * SWIGLU_BLOCK):
+        raise RuntimeError("wgu must hold blocks of 64 gate and 64 up rows")
+    w = n // 2
+    if not fused_rows_supported(w):
+        raise RuntimeError(f"h rows of {w} columns are outside what the quantizer takes")
+    if fused is None:
+        fused = mm_int8_swiglu_fused_shape(m, n, k)
+    if not fused:
+        gu = mm_int8(a, wgu, sa, sgu)
+        with torch.cuda.device(a.device):
+            hq = torch.empty((m, w), device=a.device, dtype=torch.int8)
+            s = torch.empty((m, 1), device=a.device, dtype=torch.float32)
+            h = torch.empty((m, w), device=a.device, dtype=torch.bfloat16) if want_h else None
+            if m:
+                _check(lib.astrai_w8a8_silu_mul_quantize_int8_rows_blocked(
+                    gu.data_ptr(), n, SWIGLU_BLOCK, _ptr(h), hq.data_ptr(), s.data_ptr(), m, w,
+                    _stream(a)), lib)
+        return hq, s, h
+    a_c, w_c = a.contiguous(), wgu.contiguous()
+    sa = _check_vec(sa, a, m, "sa")
+    sgu = _check_vec(sgu, a, n, "sgu")
+    pieces = n // 128
+    with torch.cuda.device(a.device):
+        h = torch.empty((m, w), device=a.device, dtype=torch.bfloat16)
+        row_max = torch.empty((m, pieces), device=a.device, dtype=torch.float32)
+        hq = torch.empty((m, w), device=a.device, dtype=torch.int8)
+        s = torch.empty((m, 1), device=a.device, dtype=torch.float32)
+        _check(lib.astrai_w8a8_gemm_int8_ptpc_swiglu(
+            a_c.data_ptr(), w_c.data_ptr(), sa.data_ptr(), sgu.data_ptr(), h.data_ptr(),
+            row_max.data_ptr(), m, n, k, _stream(a)), lib)
+        _check(lib.astrai_w8a8_quantize_int8_rows_pmax(
+            h.data_ptr(), row_max.data_ptr(), pieces, hq.data_ptr(), s.data_ptr(), m, w,
+            _stream(a)), lib)
+    return hq, s, (h if want_h else None)
 
 
 def mm_int8_rope_cache_supported(tokens: int, k: int, head_dim: int, n: int = 0) -> bool:

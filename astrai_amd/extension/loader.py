@@ -41,6 +41,8 @@ def _int8_mm_module() -> SimpleNamespace:
         mm_int8=_cabi.mm_int8,
         add_rmsnorm_quantize_int8=_cabi.add_rmsnorm_quantize_int8,
         silu_mul_quantize_int8=_cabi.silu_mul_quantize_int8,
+        mm_int8_swiglu=_cabi.mm_int8_swiglu,
+        swiglu_block_rows=_cabi.swiglu_block_rows,
     )
 
 

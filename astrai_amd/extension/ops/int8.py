@@ -11,6 +11,9 @@ scales as quantization steps.
   residual add, ``F.rms_norm`` and the per-token quantizer in one kernel
 - ``silu_mul_quantize_int8(gate, up) -> (hq, sh)``: ``up * silu(gate)`` and the
   per-token quantizer in one kernel
+- ``mm_int8_swiglu(xq, wgu, sx, sgu) -> (hq, sh)``: the gate and up projections (one weight
+  in ``swiglu_block_rows`` order), the SwiGLU product and the per-token quantizer; large
+  shapes form ``h`` in the GEMM's epilogue, gate|up never reaches memory
 """
 
 from typing import Optional
@@ -185,3 +188,36 @@ def rmsnorm_quantize_int8(x, weight, eps: float, res: Optional[torch.Tensor] = N
 
 def silu_mul_quantize_int8(gate, up):
     return int8_silu_mul_quantize(gate, up)
+
+
+@custom_op("custom::int8_mm_swiglu", mutates_args=())
+def int8_mm_swiglu(xq: torch.Tensor, wgu: torch.Tensor, sx: torch.Tensor,
+                   sgu: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """``h = up(x) * silu(gate(x))`` (astrai/model/components/mlp.py:40-43) from int8 ``xq
+    [M,K]`` and the blocked gate|up weight ``wgu [2W,K]``, per-token int8 of ``h``:
+    ``(hq int8 [M,W], s fp32 [M,1])``."""
+    _no_cpu("custom::int8_mm_swiglu")
+
+
+@int8_mm_swiglu.register_fake
+def _int8_mm_swiglu_fake(xq, wgu, sx, sgu):
+    m, w = xq.shape[0], wgu.shape[0] // 2
+    return (
+        torch.empty((m, w), device=xq.device, dtype=torch.int8),
+        torch.empty((m, 1), device=xq.device, dtype=torch.float32),
+    )
+
+
+@int8_mm_swiglu.register_kernel("cuda")
+def _int8_mm_swiglu_cuda(xq, wgu, sx, sgu):
+    hq, s, _ = _mod().mm_int8_swiglu(xq, wgu, sx, sgu, False)
+    return hq, s
+
+
+def mm_int8_swiglu(xq, wgu, sx, sgu):
+    return int8_mm_swiglu(xq, wgu, sx, sgu)
+
+
+def swiglu_block_rows(gate, up):
+    """Gate and up rows (weights or their scales) in the order ``mm_int8_swiglu`` takes."""
+    return _mod().swiglu_block_rows(gate, up)

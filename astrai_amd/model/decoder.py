@@ -276,9 +276,13 @@ class DecoderBlock(nn.Module):
         # h = attention + x, then its norm, quantized: one kernel
         hq, sh, h = I.rmsnorm_quantize_int8(o, self.post_attention_norm.weight,
                                             self.post_attention_norm.norm_eps, res=x)
-        gu = I.mm_int8(hq, f.wgu, sh, f.sgu)                 # [B*S, gate | up]
-        w = f.wgu.size(0) // 2
-        mq, sm = I.silu_mul_quantize_int8(gu[:, :w], gu[:, w:])
+        if f.gu_blocked:
+            # gate|up in 64-row blocks: a long block forms up * silu(gate) in the GEMM's epilogue
+            mq, sm = I.mm_int8_swiglu(hq, f.wgu, sh, f.sgu)
+        else:
+            gu = I.mm_int8(hq, f.wgu, sh, f.sgu)             # [B*S, gate | up]
+            w = f.wgu.size(0) // 2
+            mq, sm = I.silu_mul_quantize_int8(gu[:, :w], gu[:, w:])
         return h, I.mm_int8(mq, f.wdown, sm, f.sdown).reshape(b, s, d)
 
 
@@ -369,10 +373,15 @@ def fuse_int8_weights(model: AutoRegressiveLM) -> int:
         att, mlp = blk.attention, blk.mlp
         wqkv, sqkv = cat(att.q_proj, att.k_proj, att.v_proj)
         wo, so = cat(att.o_proj)
-        wgu, sgu = cat(mlp.gate, mlp.up)
+        gu_blocked = cfg.intermediate_size % _cabi.SWIGLU_BLOCK == 0
+        if gu_blocked:
+            (wg, sg), (wu, su) = state.get_weight(mlp.gate.weight), state.get_weight(mlp.up.weight)
+            wgu, sgu = _cabi.swiglu_block_rows(wg, wu), _cabi.swiglu_block_rows(sg, su)
+        else:
+            wgu, sgu = cat(mlp.gate, mlp.up)
         wdown, sdown = cat(mlp.down)
         blk.fused_int8 = SimpleNamespace(wqkv=wqkv, sqkv=sqkv, wo=wo, so=so, wgu=wgu, sgu=sgu,
-                                         wdown=wdown, sdown=sdown)
+                                         gu_blocked=gu_blocked, wdown=wdown, sdown=sdown)
         n += 4
     wlm, slm = cat(model.lm_head)
     model.fused_int8 = SimpleNamespace(wlm=wlm, slm=slm)

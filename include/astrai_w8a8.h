@@ -136,6 +136,39 @@ int astrai_w8a8_silu_mul_quantize_int8_rows(const void* gate_bf16, const void* u
                                             int64_t width, void* stream);
 
 /*
+ * The gate and up projections of MLP.forward (astrai/model/components/mlp.py:40-43) as one
+ * GEMM whose epilogue applies the SwiGLU product, so that the [rows, 2*width] gate|up
+ * matrix never reaches memory. The fused weight holds the rows of gate and up in blocks of
+ * 128: rows 128t .. 128t+63 are gate rows 64t .. 64t+63, rows 128t+64 .. 128t+127 the up
+ * rows of the same 64 columns of h (scales b likewise). Three entry points share that layout:
+ *
+ * gemm_int8_ptpc_swiglu: a int8 [M,K], b int8 [N,K] (N = 2*width, blocked as above), sa [M],
+ *   sb [N]. Writes h bf16 [M, N/2] with
+ *     gate = bf16(acc * sa[m] * sb[n_gate]), up = bf16(acc * sa[m] * sb[n_up])   (what
+ *     gemm_int8_ptpc would have stored), h = bf16(up * bf16(gate / (1 + exp(-gate))))
+ *   and row_max fp32 [M, N/128]: the maximum of |h| over each 64-column piece of the row.
+ *   Shapes of the large-tile kernel only (at least 192 output tiles of 256 x 256, K % 128 == 0,
+ *   K >= 256, N % 128 == 0); ASTRAI_W8A8_UNSUPPORTED otherwise -- then run gemm_int8_ptpc on
+ *   the same blocked weight and silu_mul_quantize_int8_rows_blocked on its output.
+ * quantize_int8_rows_pmax: the per-row int8 quantizer for rows whose maximum is known as
+ *   `pieces` partial maxima per row (row_max above): one read of h, same s and hq as
+ *   quantize_bf16_int8_rows. width % 8 == 0, width <= 8192.
+ * silu_mul_quantize_int8_rows_blocked: silu_mul_quantize_int8_rows on a [rows, ld >= 2*width]
+ *   gate|up matrix whose columns alternate between `block` gate and `block` up columns.
+ * Together (GEMM + quantizer, or GEMM + blocked producer) they give bit for bit the h, s and
+ * hq of gemm_int8_ptpc on an unblocked weight followed by silu_mul_quantize_int8_rows.
+ */
+int astrai_w8a8_gemm_int8_ptpc_swiglu(const void* a, const void* b, const float* sa, const float* sb,
+                                      void* h_out_bf16, float* row_max, int64_t m, int64_t n,
+                                      int64_t k, void* stream);
+int astrai_w8a8_quantize_int8_rows_pmax(const void* h_bf16, const float* row_max, int64_t pieces,
+                                        void* hq, float* s, int64_t rows, int64_t width,
+                                        void* stream);
+int astrai_w8a8_silu_mul_quantize_int8_rows_blocked(const void* gu_bf16, int64_t ld, int64_t block,
+                                                    void* h_out_bf16, void* hq, float* s,
+                                                    int64_t rows, int64_t width, void* stream);
+
+/*
  * Rotary embedding of q and k plus the KV-cache write of one decoder layer, one
  * pass over the (fused) q|k|v projection output. Replaces, between the
  * projections and the attention call of GQA.forward

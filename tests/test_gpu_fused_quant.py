@@ -88,3 +88,74 @@ def test_fused_producers_random_shape_sweep(C):
         test_add_rmsnorm_quantize(C, r(1, 70), 8 * r(1, 1025), bool(i % 2))
     for i in range(12):
         test_silu_mul_quantize(C, r(1, 70), 8 * r(1, 1025), bool(i % 2))
+
+
+def _swiglu_case(C, m, width, k, seed):
+    """int8 activations and the gate / up weights of one MLP; returns the device tensors and
+    what the unblocked chain (GEMM on gate|up, then the producer) gives."""
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randint(-127, 128, (m, k), generator=g, dtype=torch.int8).to(DEV)
+    wg = torch.randint(-127, 128, (width, k), generator=g, dtype=torch.int8).to(DEV)
+    wu = torch.randint(-127, 128, (width, k), generator=g, dtype=torch.int8).to(DEV)
+    # steps sized so that gate covers the range where silu bends (|gate| up to ~8)
+    sa = (torch.rand(m, generator=g) * 0.01 + 0.005).to(DEV)
+    sg = (torch.rand(width, generator=g) * 0.002 + 0.0005).to(DEV)
+    su = (torch.rand(width, generator=g) * 0.002 + 0.0005).to(DEV)
+    gu = C.mm_int8(a, torch.cat((wg, wu)), sa, torch.cat((sg, su)))
+    want = C.silu_mul_quantize_int8(gu[:, :width], gu[:, width:], want_h=True)
+    wgu = C.swiglu_block_rows(wg, wu)
+    sgu = C.swiglu_block_rows(sg, su)
+    return a, wgu, sa, sgu, gu, want
+
+
+def test_swiglu_block_rows_layout(C):
+    gate = torch.arange(128).reshape(128, 1).repeat(1, 2)
+    up = gate + 1000
+    b = C.swiglu_block_rows(gate, up)
+    assert b.shape == (256, 2)
+    assert b[:64, 0].tolist() == list(range(64)) and b[64:128, 0].tolist() == list(range(1000, 1064))
+    assert b[128:192, 0].tolist() == list(range(64, 128)) and b[192:, 0].tolist() == list(range(1064, 1128))
+
+
+@pytest.mark.parametrize("m,width,k", [(4096, 5632, 2048),    # config-4 MLP, 16 x 44 tiles
+                                       (3900, 3136, 512),     # ragged rows, last tile half wide (N = 49 * 128)
+                                       (8192, 2048, 256)])    # two slabs only
+def test_swiglu_gemm_epilogue_bit_equal(C, m, width, k):
+    """The gate|up GEMM with the SwiGLU product in its epilogue + the known-maximum quantizer
+    against the plain GEMM + producer kernel: h, codes and steps bit for bit; the row maxima
+    pieces are the maxima of |h| over 64 columns."""
+    print(f"case m={m} width={width} k={k}", flush=True)
+    assert C.mm_int8_swiglu_fused_shape(m, 2 * width, k)
+    a, wgu, sa, sgu, gu, (wq, ws, wh) = _swiglu_case(C, m, width, k, seed=m + width + k)
+    hq, s, h = C.mm_int8_swiglu(a, wgu, sa, sgu, want_h=True)
+    assert torch.equal(h.view(torch.int16), wh.view(torch.int16))
+    assert torch.equal(s, ws) and torch.equal(hq, wq)
+    # against the oracle's chain on the GEMM's own gate|up output (sampled rows: CPU time)
+    rows = torch.arange(0, m, max(1, m // 64))
+    oq, os_, oh = O.silu_mul_quantize_int8(gu[rows, :width].cpu(), gu[rows, width:].cpu())
+    assert_bf16_close(h[rows], oh, what="silu*up")
+    _codes_close(hq[rows], oq, s[rows], os_)
+
+
+@pytest.mark.parametrize("m,width,k", [(1, 5632, 2048), (16, 5632, 2048), (64, 5632, 2048), (200, 320, 256),
+                                       (1000, 5632, 2048)])
+def test_swiglu_blocked_producer_bit_equal(C, m, width, k):
+    """Shapes below the large-tile kernel: plain GEMM on the blocked weight + the producer
+    that reads blocked columns equals the unblocked chain bit for bit."""
+    print(f"case m={m} width={width} k={k}", flush=True)
+    assert not C.mm_int8_swiglu_fused_shape(m, 2 * width, k)
+    a, wgu, sa, sgu, gu, (wq, ws, wh) = _swiglu_case(C, m, width, k, seed=7 * m + width + k)
+    hq, s, h = C.mm_int8_swiglu(a, wgu, sa, sgu, want_h=True)
+    assert torch.equal(h.view(torch.int16), wh.view(torch.int16))
+    assert torch.equal(s, ws) and torch.equal(hq, wq)
+
+
+def test_swiglu_both_routes_agree_and_reject(C):
+    a, wgu, sa, sgu, gu, (wq, ws, wh) = _swiglu_case(C, 4096, 3072, 256, seed=99)
+    for fused in (True, False):
+        hq, s, h = C.mm_int8_swiglu(a, wgu, sa, sgu, want_h=True, fused=fused)
+        assert torch.equal(h.view(torch.int16), wh.view(torch.int16)) and torch.equal(hq, wq) and torch.equal(s, ws)
+    with pytest.raises(RuntimeError, match="192 output tiles"):
+        C.mm_int8_swiglu(a[:64], wgu, sa[:64], sgu, fused=True)
+    with pytest.raises(RuntimeError, match="blocks of 64"):
+        C.mm_int8_swiglu(a, wgu[:192], sa, sgu[:192])
