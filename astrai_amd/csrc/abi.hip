@@ -226,6 +226,45 @@ int astrai_w8a8_silu_mul_quantize_int8_rows_blocked(const void* gu, int64_t ld, 
     return check_launch(what);
 }
 
+int astrai_w8a8_add_rmsnorm_quantize_fp8_rows(const void* x, const void* res, const void* weight,
+                                              float eps, void* sum_out, void* y_out, void* x8,
+                                              const float* scale, float* amax, int64_t rows,
+                                              int64_t k, int fmt, void* stream) {
+    const char* what = "add_rmsnorm_quantize_fp8_rows";
+    if (!x || !weight || !x8 || !scale) return fail(ASTRAI_W8A8_BAD_ARG, "%s: null pointer", what);
+    if (rows < 0 || k < 0 || rows > 0x7fffffff) return fail(ASTRAI_W8A8_BAD_ARG, "%s: bad dims", what);
+    if (fmt != ASTRAI_W8A8_E4M3 && fmt != ASTRAI_W8A8_E5M2)
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: fmt must be 0 (e4m3) or 1 (e5m2)", what);
+    if ((k & 7) != 0 || k > w8a8::kFusedRowMax)
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "%s: K must be a multiple of 8 and at most 8192", what);
+    if (!aligned16(x) || !aligned16(weight) || !aligned16(x8) || (res && !aligned16(res)) ||
+        (sum_out && !aligned16(sum_out)) || (y_out && !aligned16(y_out)))
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: pointers must be 16-byte aligned", what);
+    if (rows == 0 || k == 0) return ASTRAI_W8A8_OK;
+    w8a8::launch_add_rmsnorm_quantize_fp8_rows(x, res, weight, eps, sum_out, y_out, x8, scale, amax,
+                                               rows, k, fmt, static_cast<hipStream_t>(stream));
+    return check_launch(what);
+}
+
+int astrai_w8a8_silu_mul_quantize_fp8_rows(const void* gate, const void* up, int64_t ld, void* h_out,
+                                           void* h8, const float* scale, float* amax, int64_t rows,
+                                           int64_t width, int fmt, void* stream) {
+    const char* what = "silu_mul_quantize_fp8_rows";
+    if (!gate || !up || !h8 || !scale) return fail(ASTRAI_W8A8_BAD_ARG, "%s: null pointer", what);
+    if (rows < 0 || width < 0 || rows > 0x7fffffff || ld < width)
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: bad dims", what);
+    if (fmt != ASTRAI_W8A8_E4M3 && fmt != ASTRAI_W8A8_E5M2)
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: fmt must be 0 (e4m3) or 1 (e5m2)", what);
+    if ((width & 7) != 0 || (ld & 7) != 0)
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "%s: width and ld must be multiples of 8", what);
+    if (!aligned16(gate) || !aligned16(up) || !aligned16(h8) || (h_out && !aligned16(h_out)))
+        return fail(ASTRAI_W8A8_BAD_ARG, "%s: pointers must be 16-byte aligned", what);
+    if (rows == 0 || width == 0) return ASTRAI_W8A8_OK;
+    w8a8::launch_silu_mul_quantize_fp8_rows(gate, up, ld, h_out, h8, scale, amax, rows, width, fmt,
+                                            static_cast<hipStream_t>(stream));
+    return check_launch(what);
+}
+
 int astrai_w8a8_quantize_int8_rows_pmax(const void* h, const float* row_max, int64_t pieces,
                                         void* hq, float* s, int64_t rows, int64_t width,
                                         void* stream) {

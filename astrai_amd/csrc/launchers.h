@@ -63,6 +63,14 @@ void launch_add_rmsnorm_quantize_int8_rows(const void* x, const void* res, const
 void launch_silu_mul_quantize_int8_rows(const void* gate, const void* up, int64_t ld, int64_t block,
                                         void* h_out, void* hq, float* s, int64_t rows, int64_t width,
                                         hipStream_t stream);
+// per-tensor fp8 twins (step known ahead; *amax = max(*amax, max |value|) when amax is given)
+void launch_add_rmsnorm_quantize_fp8_rows(const void* x, const void* res, const void* w, float eps,
+                                          void* sum_out, void* y_out, void* x8, const float* scale,
+                                          float* amax, int64_t rows, int64_t k, int fmt,
+                                          hipStream_t stream);
+void launch_silu_mul_quantize_fp8_rows(const void* gate, const void* up, int64_t ld, void* h_out,
+                                       void* h8, const float* scale, float* amax, int64_t rows,
+                                       int64_t width, int fmt, hipStream_t stream);
 // per-row int8 of bf16 rows whose |maximum| is known as `pieces` partial maxima per row
 void launch_quantize_int8_rows_pmax(const void* h, const float* row_max, int64_t pieces, void* hq,
                                     float* s, int64_t rows, int64_t width, hipStream_t stream);

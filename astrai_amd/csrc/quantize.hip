@@ -501,6 +501,85 @@ __global__ __launch_bounds__(kThreads) void silu_mul_quantize_int8_rows_kernel(
     }
 }
 
+// Per-tensor fp8 twins of the two producers above, for a Linear under delayed scaling: the
+// step is known before the tensor exists (astrai/extension/fp8.py:147-173), so the codes
+// are written in the pass that forms the values and the pass reports max |y| for the ring.
+// Same value arithmetic as the int8 producers, the quantizer of quantize_fp8_kernel.
+template <int Fmt>
+__global__ __launch_bounds__(kThreads) void add_rmsnorm_quantize_fp8_rows_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ res,
+    const uint16_t* __restrict__ w, float eps, uint16_t* __restrict__ sum_out,
+    uint16_t* __restrict__ y_out, uint8_t* __restrict__ x8, const float* __restrict__ scale,
+    float* __restrict__ amax, int64_t k) {
+    __shared__ float slots[kThreads / kWave];
+    const int64_t row = blockIdx.x;
+    const int64_t nvec = k >> 3;
+    const float step = *scale;
+    float v[kCache][8];
+    float ss = 0.0f;
+#pragma unroll
+    for (int c = 0; c < kCache; ++c) {
+        const int64_t i = threadIdx.x + (int64_t)c * kThreads;
+        if (i < nvec) {
+            unpack8(*reinterpret_cast<const u32x4*>(x + row * k + i * 8), v[c]);
+            if (res) {
+                float r[8];
+                unpack8(*reinterpret_cast<const u32x4*>(res + row * k + i * 8), r);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[c][j] = round_bf16(v[c][j] + r[j]);
+                if (sum_out) *reinterpret_cast<u32x4*>(sum_out + row * k + i * 8) = pack8(v[c]);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) ss += v[c][j] * v[c][j];
+        }
+    }
+    const float rstd = rsqrtf(block_sum(ss, slots) / (float)k + eps);
+    float local = 0.0f;
+#pragma unroll
+    for (int c = 0; c < kCache; ++c) {
+        const int64_t i = threadIdx.x + (int64_t)c * kThreads;
+        if (i < nvec) {
+            float g[8];
+            unpack8(*reinterpret_cast<const u32x4*>(w + i * 8), g);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[c][j] = round_bf16(g[j] * (rstd * v[c][j]));
+            local = fmaxf(local, amax8(v[c]));
+            if (y_out) *reinterpret_cast<u32x4*>(y_out + row * k + i * 8) = pack8(v[c]);
+            *reinterpret_cast<u32x2*>(x8 + row * k + i * 8) = quant8_fp8<Fmt>(v[c], step);
+        }
+    }
+    if (amax) {
+        const float m = block_max(local, slots);
+        if (threadIdx.x == 0) atomic_max_nonneg(amax, m);
+    }
+}
+
+template <int Fmt>
+__global__ __launch_bounds__(kThreads) void silu_mul_quantize_fp8_rows_kernel(
+    const uint16_t* __restrict__ gate, const uint16_t* __restrict__ up, int64_t ld,
+    uint16_t* __restrict__ h_out, uint8_t* __restrict__ h8, const float* __restrict__ scale,
+    float* __restrict__ amax, int64_t width) {
+    __shared__ float slots[kThreads / kWave];
+    const int64_t row = blockIdx.x;
+    const int64_t nvec = width >> 3;
+    const float step = *scale;
+    float local = 0.0f;
+    for (int64_t i = threadIdx.x; i < nvec; i += kThreads) {
+        float g[8], v[8];
+        unpack8(*reinterpret_cast<const u32x4*>(gate + row * ld + i * 8), g);
+        unpack8(*reinterpret_cast<const u32x4*>(up + row * ld + i * 8), v);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = round_bf16(v[j] * round_bf16(silu_f32(g[j])));
+        local = fmaxf(local, amax8(v));
+        if (h_out) *reinterpret_cast<u32x4*>(h_out + row * width + i * 8) = pack8(v);
+        *reinterpret_cast<u32x2*>(h8 + row * width + i * 8) = quant8_fp8<Fmt>(v, step);
+    }
+    if (amax) {
+        const float m = block_max(local, slots);
+        if (threadIdx.x == 0) atomic_max_nonneg(amax, m);
+    }
+}
+
 // Per-row int8 quantizer for rows whose maximum is already known in pieces: row_max holds
 // `pieces` partial maxima of |h| per row (written by the SwiGLU epilogue of the gate|up
 // GEMM), so the row is read once. Same codes and steps as quantize_int8_rows_kernel.
@@ -661,6 +740,28 @@ void launch_silu_mul_quantize_int8_rows(const void* gate, const void* up, int64_
     silu_mul_quantize_int8_rows_kernel<<<dim3((unsigned)rows), dim3(kThreads), 0, stream>>>(
         static_cast<const uint16_t*>(gate), static_cast<const uint16_t*>(up), ld, block,
         static_cast<uint16_t*>(h_out), static_cast<int8_t*>(hq), s, width);
+}
+
+void launch_add_rmsnorm_quantize_fp8_rows(const void* x, const void* res, const void* w, float eps,
+                                          void* sum_out, void* y_out, void* x8, const float* scale,
+                                          float* amax, int64_t rows, int64_t k, int fmt,
+                                          hipStream_t stream) {
+    if (rows <= 0 || k <= 0) return;
+    auto kern = fmt ? add_rmsnorm_quantize_fp8_rows_kernel<1> : add_rmsnorm_quantize_fp8_rows_kernel<0>;
+    kern<<<dim3((unsigned)rows), dim3(kThreads), 0, stream>>>(
+        static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(res),
+        static_cast<const uint16_t*>(w), eps, static_cast<uint16_t*>(sum_out),
+        static_cast<uint16_t*>(y_out), static_cast<uint8_t*>(x8), scale, amax, k);
+}
+
+void launch_silu_mul_quantize_fp8_rows(const void* gate, const void* up, int64_t ld, void* h_out,
+                                       void* h8, const float* scale, float* amax, int64_t rows,
+                                       int64_t width, int fmt, hipStream_t stream) {
+    if (rows <= 0 || width <= 0) return;
+    auto kern = fmt ? silu_mul_quantize_fp8_rows_kernel<1> : silu_mul_quantize_fp8_rows_kernel<0>;
+    kern<<<dim3((unsigned)rows), dim3(kThreads), 0, stream>>>(
+        static_cast<const uint16_t*>(gate), static_cast<const uint16_t*>(up), ld,
+        static_cast<uint16_t*>(h_out), static_cast<uint8_t*>(h8), scale, amax, width);
 }
 
 void launch_quantize_int8_rows_pmax(const void* h, const float* row_max, int64_t pieces, void* hq,

@@ -40,6 +40,9 @@ PROTOTYPES = {
     "astrai_w8a8_add_rmsnorm_quantize_int8_rows": (
         [_P, _P, _P, ctypes.c_float, _P, _P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_silu_mul_quantize_int8_rows": ([_P, _P, _I64, _P, _P, _P, _I64, _I64, _P], _INT),
+    "astrai_w8a8_add_rmsnorm_quantize_fp8_rows": (
+        [_P, _P, _P, ctypes.c_float, _P, _P, _P, _P, _P, _I64, _I64, _INT, _P], _INT),
+    "astrai_w8a8_silu_mul_quantize_fp8_rows": ([_P, _P, _I64, _P, _P, _P, _P, _I64, _I64, _INT, _P], _INT),
     "astrai_w8a8_gemm_int8_ptpc_swiglu": ([_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _INT),
     "astrai_w8a8_quantize_int8_rows_pmax": ([_P, _P, _I64, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_silu_mul_quantize_int8_rows_blocked": ([_P, _I64, _I64, _P, _P, _P, _I64, _I64, _P], _INT),
@@ -513,6 +516,76 @@ def silu_mul_quantize_int8(gate: torch.Tensor, up: torch.Tensor, want_h: bool = 
             g2.data_ptr(), u2.data_ptr(), ld, _ptr(h), hq.data_ptr(), s.data_ptr(), rows, w,
             _stream(gate)), lib)
     return hq, s, None if h is None else h.reshape(gate.shape)
+
+
+def _fp8_scale_amax(scale: torch.Tensor, amax: Optional[torch.Tensor], ref: torch.Tensor):
+    if not (scale.is_cuda and scale.device == ref.device and scale.dtype == torch.float32
+            and scale.numel() == 1):
+        raise RuntimeError("scale must be one CUDA float32 on the input device")
+    if amax is not None and not (amax.is_cuda and amax.device == ref.device
+                                 and amax.dtype == torch.float32 and amax.numel() == 1):
+        raise RuntimeError("amax must be one CUDA float32 on the input device")
+
+
+def add_rmsnorm_quantize_fp8(x: torch.Tensor, weight: torch.Tensor, eps: float, scale: torch.Tensor,
+                             res: Optional[torch.Tensor] = None, fmt: int = 0,
+                             amax: Optional[torch.Tensor] = None, want_y: bool = False):
+    """Per-tensor fp8 twin of :func:`add_rmsnorm_quantize_int8` for a step known ahead
+    (delayed scaling): ``(x8 [R,K] fp8, amax [1], t or None, y or None)``; ``amax`` (a zeroed
+    slot is made when none is given) ends as ``max(amax, max |y|)``."""
+    lib = _require()
+    _gpu(x, "add_rmsnorm_quantize_fp8")
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise RuntimeError("x and weight must be bf16")
+    k = x.size(-1)
+    if weight.numel() != k or weight.device != x.device:
+        raise RuntimeError("weight must be [K] on x's device")
+    _fp8_scale_amax(scale, amax, x)
+    x2 = x.reshape(-1, k).contiguous()
+    rows = x2.size(0)
+    r2 = None
+    if res is not None:
+        if res.shape != x.shape or res.dtype != torch.bfloat16 or res.device != x.device:
+            raise RuntimeError("res must match x in shape, dtype and device")
+        r2 = res.reshape(-1, k).contiguous()
+    with torch.cuda.device(x.device):
+        x8 = torch.empty((rows, k), device=x.device, dtype=_FP8[1 if fmt else 0])
+        if amax is None:
+            amax = torch.zeros(1, device=x.device, dtype=torch.float32)
+        t = torch.empty_like(x2) if r2 is not None else None
+        y = torch.empty_like(x2) if want_y else None
+        _check(lib.astrai_w8a8_add_rmsnorm_quantize_fp8_rows(
+            x2.data_ptr(), _ptr(r2), weight.contiguous().data_ptr(), float(eps), _ptr(t), _ptr(y),
+            x8.data_ptr(), scale.data_ptr(), amax.data_ptr(), rows, k, 1 if fmt else 0, _stream(x)), lib)
+    return (x8, amax, None if t is None else t.reshape(x.shape), None if y is None else y.reshape(x.shape))
+
+
+def silu_mul_quantize_fp8(gate: torch.Tensor, up: torch.Tensor, scale: torch.Tensor, fmt: int = 0,
+                          amax: Optional[torch.Tensor] = None, want_h: bool = False):
+    """Per-tensor fp8 twin of :func:`silu_mul_quantize_int8`: ``(h8 [R,W] fp8, amax [1], h or
+    None)``."""
+    lib = _require()
+    _gpu(gate, "silu_mul_quantize_fp8")
+    if gate.dtype != torch.bfloat16 or up.dtype != torch.bfloat16:
+        raise RuntimeError("gate and up must be bf16")
+    if gate.shape != up.shape or gate.device != up.device:
+        raise RuntimeError("gate and up must match in shape and device")
+    _fp8_scale_amax(scale, amax, gate)
+    w = gate.size(-1)
+    g2, u2 = gate.reshape(-1, w), up.reshape(-1, w)
+    if g2.stride(1) != 1 or u2.stride(1) != 1 or g2.stride(0) != u2.stride(0):
+        g2, u2 = g2.contiguous(), u2.contiguous()
+    rows = g2.size(0)
+    ld = g2.stride(0) if rows > 1 else max(w, g2.stride(0))
+    with torch.cuda.device(gate.device):
+        h8 = torch.empty((rows, w), device=gate.device, dtype=_FP8[1 if fmt else 0])
+        if amax is None:
+            amax = torch.zeros(1, device=gate.device, dtype=torch.float32)
+        h = torch.empty((rows, w), device=gate.device, dtype=torch.bfloat16) if want_h else None
+        _check(lib.astrai_w8a8_silu_mul_quantize_fp8_rows(
+            g2.data_ptr(), u2.data_ptr(), ld, _ptr(h), h8.data_ptr(), scale.data_ptr(), amax.data_ptr(),
+            rows, w, 1 if fmt else 0, _stream(gate)), lib)
+    return h8, amax, None if h is None else h.reshape(gate.shape)
 
 
 def rotary_emb(x: torch.Tensor, freqs_cis: torch.Tensor) -> torch.Tensor:

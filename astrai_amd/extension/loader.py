@@ -32,6 +32,8 @@ def _fp8_mm_module() -> SimpleNamespace:
         quantize_transpose_bf16=_cabi.quantize_transpose_bf16,
         amax_bf16=_cabi.amax_bf16,
         amax_ring_push=_cabi.amax_ring_push,
+        add_rmsnorm_quantize_fp8=_cabi.add_rmsnorm_quantize_fp8,
+        silu_mul_quantize_fp8=_cabi.silu_mul_quantize_fp8,
     )
 
 

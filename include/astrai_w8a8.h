@@ -136,6 +136,28 @@ int astrai_w8a8_silu_mul_quantize_int8_rows(const void* gate_bf16, const void* u
                                             int64_t width, void* stream);
 
 /*
+ * Per-tensor fp8 twins of the two producers, for Linear layers under the delayed-scaling
+ * recipe (astrai/extension/fp8.py:147-173: the step of this call is known before the
+ * activation exists; the call reports the maximum for the ring). Replace the same
+ * reference code as the int8 producers plus custom::fp8_quantize
+ * (astrai/extension/ops/fp8.py:60-82) on the activation.
+ *   t, y, h     as above (same bf16 arithmetic)
+ *   x8 / h8     = fp8(value / *scale), magnitudes clamped to the format's finite maximum
+ *                 (the quantizer of quantize_bf16_fp8), [rows, K] / [rows, width]
+ *   *amax       = max(*amax, max |value|) when amax is given (clear it before the first call)
+ * K % 8 == 0 and K <= 8192 for add_rmsnorm; width % 8 == 0, ld % 8 == 0 for silu_mul.
+ */
+int astrai_w8a8_add_rmsnorm_quantize_fp8_rows(const void* x_bf16, const void* res_bf16,
+                                              const void* weight_bf16, float eps,
+                                              void* sum_out_bf16, void* y_out_bf16, void* x8,
+                                              const float* scale, float* amax, int64_t rows,
+                                              int64_t k, int fmt, void* stream);
+int astrai_w8a8_silu_mul_quantize_fp8_rows(const void* gate_bf16, const void* up_bf16, int64_t ld,
+                                           void* h_out_bf16, void* h8, const float* scale,
+                                           float* amax, int64_t rows, int64_t width, int fmt,
+                                           void* stream);
+
+/*
  * The gate and up projections of MLP.forward (astrai/model/components/mlp.py:40-43) as one
  * GEMM whose epilogue applies the SwiGLU product, so that the [rows, 2*width] gate|up
  * matrix never reaches memory. The fused weight holds the rows of gate and up in blocks of

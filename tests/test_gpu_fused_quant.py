@@ -159,3 +159,47 @@ def test_swiglu_both_routes_agree_and_reject(C):
         C.mm_int8_swiglu(a[:64], wgu, sa[:64], sgu, fused=True)
     with pytest.raises(RuntimeError, match="blocks of 64"):
         C.mm_int8_swiglu(a, wgu[:192], sa, sgu[:192])
+
+
+@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("rows,k,with_res", [(32, 2048, True), (5, 8, False), (3, 8192, True), (300, 5632, False)])
+def test_add_rmsnorm_quantize_fp8(C, rows, k, with_res, fmt):
+    """Per-tensor fp8 twin: value part to the bf16 tolerance against the oracle's chain, the
+    codes and the maximum bit-exact against the oracle's fp8 quantizer on the kernel's own y."""
+    print(f"case rows={rows} k={k} res={with_res} fmt={fmt}", flush=True)
+    g = torch.Generator().manual_seed(rows * 131 + k + fmt)
+    x = torch.randn(rows, k, generator=g).to(torch.bfloat16)
+    res = (torch.randn(rows, k, generator=g) * 0.5).to(torch.bfloat16) if with_res else None
+    w = (1.0 + 0.1 * torch.randn(k, generator=g)).to(torch.bfloat16)
+    scale = torch.tensor([3.7 / (57344.0 if fmt else 448.0)])   # some values saturate
+    x8, amax, t, y = C.add_rmsnorm_quantize_fp8(x.to(DEV), w.to(DEV), 1e-5, scale.to(DEV),
+                                                res.to(DEV) if with_res else None, fmt=fmt, want_y=True)
+    _, _, wt, wy = O.add_rmsnorm_quantize_int8(x, w, 1e-5, res)
+    if with_res:
+        assert torch.equal(t.cpu().view(torch.int16), wt.view(torch.int16))
+    assert_bf16_close(y, wy, what="rmsnorm y")
+    o8, oamax = O.fp8_quantize_saturating(y.cpu(), scale, fmt)
+    assert torch.equal(x8.cpu().view(torch.uint8), o8.view(torch.uint8))
+    assert torch.equal(amax.cpu(), oamax)
+
+
+@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("rows,width,fused_buffer", [(32, 5632, True), (7, 8, False), (3, 11008, True)])
+def test_silu_mul_quantize_fp8(C, rows, width, fused_buffer, fmt):
+    print(f"case rows={rows} width={width} fused={fused_buffer} fmt={fmt}", flush=True)
+    g = torch.Generator().manual_seed(rows * 17 + width + fmt)
+    gu = (torch.randn(rows, 2 * width, generator=g) * 2.0).to(torch.bfloat16)
+    d = gu.to(DEV)
+    scale = torch.tensor([6.0 / (57344.0 if fmt else 448.0)])
+    gate, up = (d[:, :width], d[:, width:]) if fused_buffer else (d[:, :width].contiguous(), d[:, width:].contiguous())
+    prior = torch.tensor([0.25], device=DEV)    # the slot keeps a larger earlier maximum or grows
+    h8, amax, h = C.silu_mul_quantize_fp8(gate, up, scale.to(DEV), fmt=fmt, amax=prior, want_h=True)
+    _, _, wh = O.silu_mul_quantize_int8(gu[:, :width], gu[:, width:])
+    assert_bf16_close(h, wh, what="silu*up")
+    o8, oamax = O.fp8_quantize_saturating(h.cpu(), scale, fmt)
+    assert torch.equal(h8.cpu().view(torch.uint8), o8.view(torch.uint8))
+    assert torch.equal(amax.cpu(), torch.maximum(oamax, torch.tensor([0.25])))
+    # same h as the int8 producer forms
+    if width <= 8192:
+        _, _, hi = C.silu_mul_quantize_int8(gate, up, want_h=True)
+        assert torch.equal(h.view(torch.int16), hi.view(torch.int16))
