@@ -756,6 +756,14 @@ int astrai_w8a8_gemm_int8_ptpc_swiglu(const void* a, const void* b, const float*
     return check_launch(what);
 }
 
+int astrai_w8a8_mfma_probe(int kind, const void* a, const void* b, void* d_raw, void* stream) {
+    if (!a || !b || !d_raw) return fail(ASTRAI_W8A8_BAD_ARG, "mfma_probe: null pointer");
+    if (!aligned16(a) || !aligned16(b)) return fail(ASTRAI_W8A8_BAD_ARG, "mfma_probe: pointers must be 16-byte aligned");
+    if (!w8a8::launch_mfma_probe(kind, a, b, d_raw, static_cast<hipStream_t>(stream)))
+        return fail(ASTRAI_W8A8_BAD_ARG, "mfma_probe: kind must be 0..7");
+    return check_launch("mfma_probe");
+}
+
 int astrai_w8a8_gemm_int8_ptpc_tiled(const void* a, const void* b, const float* sa,
                                      const float* sb, const void* bias, void* out, int64_t m,
                                      int64_t n, int64_t k, int out_dtype, void* stream) {

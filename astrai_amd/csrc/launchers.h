@@ -220,4 +220,8 @@ bool launch_gemv_int8(const GemmArgs& g, hipStream_t stream);
 // in the epilogue (g.out unused; rc.qkv / rc.ld unused); false when the shape does not fit
 bool launch_gemm_int8_rope_cache(const GemmArgs& g, const RopeCacheArgs& rc, hipStream_t stream);
 
+// mfma_probe.hip: one instruction of MFMA shape `kind` on a zero accumulator, one wave;
+// d_raw[lane][reg] are the accumulator registers as they are (4 or 16 per lane)
+bool launch_mfma_probe(int kind, const void* a, const void* b, void* d_raw, hipStream_t stream);
+
 }  // namespace w8a8

@@ -43,6 +43,7 @@ PROTOTYPES = {
     "astrai_w8a8_add_rmsnorm_quantize_fp8_rows": (
         [_P, _P, _P, ctypes.c_float, _P, _P, _P, _P, _P, _I64, _I64, _INT, _P], _INT),
     "astrai_w8a8_silu_mul_quantize_fp8_rows": ([_P, _P, _I64, _P, _P, _P, _P, _I64, _I64, _INT, _P], _INT),
+    "astrai_w8a8_mfma_probe": ([_INT, _P, _P, _P, _P], _INT),
     "astrai_w8a8_gemm_int8_ptpc_swiglu": ([_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _INT),
     "astrai_w8a8_quantize_int8_rows_pmax": ([_P, _P, _I64, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_silu_mul_quantize_int8_rows_blocked": ([_P, _I64, _I64, _P, _P, _P, _I64, _I64, _P], _INT),
@@ -1063,6 +1064,22 @@ def mm_int8(a: torch.Tensor, b: torch.Tensor, sa: Optional[torch.Tensor],
                 _check(fn(a_c.data_ptr(), b_c.data_ptr(), _ptr(sa), _ptr(sb), _ptr(bias),
                           out.data_ptr(), m, n, k, out_dtype, _stream(a)), lib)
     return out
+
+
+def mfma_probe(kind: int, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """One MFMA of shape ``kind`` on a zero accumulator in one wave (test hook); returns the
+    raw accumulator registers ``[64, 4]`` or ``[64, 16]`` as int32 words."""
+    lib = _require()
+    _gpu(a, "mfma_probe")
+    rows, kbytes = {0: (16, 64), 1: (16, 128), 2: (16, 128), 3: (32, 32), 4: (32, 64), 5: (32, 64),
+                    6: (16, 64), 7: (32, 32)}[kind]
+    for t in (a, b):
+        if not t.is_contiguous() or t.numel() * t.element_size() != rows * kbytes or t.device != a.device:
+            raise RuntimeError(f"operands of kind {kind} are contiguous [{rows}] rows of {kbytes} bytes")
+    with torch.cuda.device(a.device):
+        d = torch.zeros((64, 4 if rows == 16 else 16), device=a.device, dtype=torch.int32)
+        _check(lib.astrai_w8a8_mfma_probe(kind, a.data_ptr(), b.data_ptr(), d.data_ptr(), _stream(a)), lib)
+    return d
 
 
 SWIGLU_BLOCK = 64

@@ -536,6 +536,22 @@ int astrai_w8a8_gemm_int8_ptpc_tiled(const void* a, const void* b, const float* 
                                      int64_t m, int64_t n, int64_t k, int out_dtype,
                                      void* stream);
 
+/*
+ * Test hook: ONE MFMA instruction on a zero accumulator in a single 64-lane wave, for
+ * known-answer tests of the lane layouts the kernels assume (what the reference checks
+ * with csrc/tests/fp8_mma_test.cu:81-145 for its mma.sync shape). Operands are row-major
+ * [R][K] matrices a (first operand) and b (second); lane l loads row l % R and the K bytes
+ * of K-group l / R exactly as the GEMM / attention kernels do; d_raw receives every lane's
+ * accumulator registers unpermuted, [64][4] (16-row shapes) or [64][16] (32-row shapes)
+ * 32-bit words. The kernels assume D = a * b^T with
+ *   16-row shapes: d_raw[l][j] = D[4 * (l / 16) + j][l % 16]
+ *   32-row shapes: d_raw[l][r] = D[8 * (r / 4) + 4 * (l / 32) + r % 4][l % 32]
+ * kind: 0 i32_16x16x64_i8 ([16][64] int8) | 1, 2 f32_16x16x128_f8f6f4 e4m3 / e5m2 ([16][128])
+ *     | 3 i32_32x32x32_i8 ([32][32]) | 4, 5 f32_32x32x64_f8f6f4 e4m3 / e5m2 ([32][64])
+ *     | 6 f32_16x16x32_bf16 ([16][32] bf16) | 7 f32_32x32x16_bf16 ([32][16] bf16)
+ */
+int astrai_w8a8_mfma_probe(int kind, const void* a, const void* b, void* d_raw, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
