@@ -1366,6 +1366,52 @@ def _token_major(t, layout):
     return (t.transpose(1, 2) if layout == BHLD else t).contiguous()
 
 
+def attn_cache_rows_supported(n_heads: int, n_kv_heads: int, head_dim: int) -> bool:
+    """Head shapes :func:`attn_cache_rows` takes (those of the general paged kernel)."""
+    return head_dim in (32, 64, 128, 256) and n_heads % n_kv_heads == 0 and n_heads // n_kv_heads <= 16
+
+
+def attn_cache_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                    positions: torch.Tensor) -> torch.Tensor:
+    """Attention of new tokens ``q [batch, n_heads, seq, head_dim]`` at ``positions [seq]``
+    (int64, on the device) against the dense head-major caches ``[batch, n_kv_heads, max_len,
+    head_dim]`` through the general paged kernel, for the head shapes the tuned dense kernels
+    do not take (head_dim 32 / 64 / 256, any grouping up to 16). Every (sequence, KV head) pair
+    is addressed as one sequence of a one-head pool -- the cache rows of a KV head are
+    contiguous -- with the pair's query heads as its heads; nothing of the cache is copied
+    and no length is read on the host. A row attends keys at positions <= its own. Returns
+    token-major ``[batch, seq, n_heads * head_dim]``."""
+    _gpu(q, "attn_cache_rows")
+    b, h, s, d = q.shape
+    hkv, max_len = k_cache.size(1), k_cache.size(2)
+    if not attn_cache_rows_supported(h, hkv, d):
+        raise RuntimeError(f"attn_cache_rows: head_dim {d} with {h} / {hkv} heads is not supported")
+    if k_cache.shape != (b, hkv, max_len, d) or v_cache.shape != k_cache.shape \
+            or not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise RuntimeError("attn_cache_rows: the caches must be contiguous [batch, n_kv_heads, max_len, head_dim]")
+    n_rep, pairs = h // hkv, b * hkv
+    with torch.cuda.device(q.device):
+        table, rows = _identity_paging(pairs, max_len, q.device)
+        key = ("ramp", pairs, str(q.device))
+        if key not in _index_cache:
+            _index_cache[key] = torch.arange(pairs + 1, dtype=torch.int32, device=q.device)
+        kv_indptr = _index_cache[key] * (positions.max() + 1).to(torch.int32)
+        k_pool, v_pool = k_cache.view(pairs * max_len, 1, d), v_cache.view(pairs * max_len, 1, d)
+        if s == 1:
+            out = attn_paged_decode(q.reshape(pairs, n_rep, d), k_pool, v_pool, table, rows, kv_indptr)
+            return out.reshape(b, 1, h * d)
+        key = ("sched", pairs, s, str(q.device))
+        if key not in _index_cache:
+            _index_cache[key] = paged_prefill_schedule([s] * pairs, q.device)
+        qo, tb, ti = _index_cache[key]
+        # rows of a pair token-major: [pair, seq, n_rep, head_dim]
+        q_tm = q.reshape(b, hkv, n_rep, s, d).transpose(2, 3).reshape(pairs * s, n_rep, d)
+        mask = (torch.arange(max_len, device=q.device)[None, :] <= positions[:, None])  # [seq, max_len]
+        out = attn_paged_prefill(q_tm, k_pool, v_pool, table, rows, kv_indptr, qo, tb, ti,
+                                 mask=mask[None, None].expand(pairs, 1, s, max_len))
+    return out.view(b, hkv, s, n_rep, d).permute(0, 2, 1, 3, 4).reshape(b, s, h * d)
+
+
 def attn_decode_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Optional[torch.Tensor] = None,
                     causal_offset: int = -1, scale: float = 0.0, layout: int = BHLD,
                     o_part_buf=None, ml_part_buf=None) -> torch.Tensor:

@@ -189,8 +189,9 @@ class GQA(nn.Module):
         cache: rotation, permutes and the cache write are one kernel. Returns the attention
         output already quantized per token, ``(int8 [B*S, dim], fp32 [B*S, 1])``: for a few new
         tokens straight out of the split-context attention kernel (mask from ``positions``,
-        token-major), for longer blocks the causal block kernel followed by the quantizer
-        (SDPA only for head layouts neither kernel takes)."""
+        token-major), for longer blocks the causal block kernel followed by the quantizer; other
+        head_dim / groupings run the general paged kernel over the same cache (SDPA only for
+        head layouts no kernel takes)."""
         from astrai_amd.extension import _cabi
         q = _cabi.rope_cache_write(qkv, rotary_emb[0], positions, kv_cache.k[self.layer_id],
                                    kv_cache.v[self.layer_id], self.n_heads, self.n_kv_heads,
@@ -210,6 +211,10 @@ class GQA(nn.Module):
             # causal block kernel: no mask tensor, no head expansion, token-major output
             return I.quantize_int8_per_token(
                 _cabi.attn_prefill(q, kv_cache.k[self.layer_id], kv_cache.v[self.layer_id], positions))
+        if _cabi.attn_cache_rows_supported(self.n_heads, self.n_kv_heads, self.head_dim):
+            # other head shapes: the general kernel over the same cache, addressed per KV head
+            return I.quantize_int8_per_token(
+                _cabi.attn_cache_rows(q, kv_cache.k[self.layer_id], kv_cache.v[self.layer_id], positions))
         out = self._attend_cache(q, kv_cache, key_mask)
         return I.quantize_int8_per_token(out.permute(0, 2, 1, 3).reshape(b, s, self.dim))
 
