@@ -482,7 +482,8 @@ def main():
         ring = [torch.randint(-127, 128, (gn, gk), dtype=torch.int8, device=dev) for _ in range(4)]
         gsw = torch.rand(gn, device=dev) + 0.5
         dst.copy_(src)
-        for gm in (1, 16):
+        gemv_ms = (1, 4, 16, 64)
+        for gm in gemv_ms:
             gx = torch.randint(-127, 128, (gm, gk), dtype=torch.int8, device=dev)
             gsx = torch.rand(gm, device=dev) + 0.5
             gy = torch.empty(gm, gn, device=dev, dtype=torch.bfloat16)
@@ -493,9 +494,10 @@ def main():
         print(json.dumps({"pmc_mode": True, "gemm_launches": 5, "copy_launches": 4,
                           "copy_bytes_each_way": 256 << 20,
                           "gemm_algorithmic_bytes": 2 * M * K + 2 * M * N,
-                          "gemv_launches": "4 at M=1 (dot kernel), then 4 at M=16 (LDS kernel), 11008x4096",
-                          "gemv_algorithmic_bytes": {"M1": gn * gk + gk + 2 * gn + 4 * gn + 4,
-                                                     "M16": gn * gk + 16 * gk + 32 * gn + 4 * gn + 64}}))
+                          "gemv_launches": "4 each at M = 1 (dot kernel), 4, 16, 64 (rows kernel), 11008x4096, "
+                                           "every launch on another 45 MB weight buffer",
+                          "gemv_algorithmic_bytes": {f"M{m}": gn * gk + m * gk + 2 * m * gn + 4 * gn + 4 * m
+                                                     for m in gemv_ms}}))
         return
 
     for _ in range(args.warmup):
