@@ -71,7 +71,13 @@ __device__ __forceinline__ float silu_hw(float g) {
 
 enum : int { EPI_PLAIN = 0, EPI_SWIGLU = 1 };
 
-template <class Op, int ScaleKind, int Epi = EPI_PLAIN>
+// Knock-outs for the phase microbenchmark (ubench/wave128_phases.hip): each bit removes one
+// class of instructions so that its share of the kernel's time -- issue slots and, under the
+// power cap, clock -- can be read off a timing. The library instantiates KO = 0 only; a
+// knocked-out kernel computes nothing meaningful.
+enum : int { KO_LDS_READS = 1, KO_LOADS = 2, KO_MFMA = 4, KO_STORES = 8 };
+
+template <class Op, int ScaleKind, int Epi = EPI_PLAIN, int KO = 0>
 __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmArgs g) {
     static_assert(ScaleKind != SCALE_BLOCK128, "block scales run on the ping-pong kernel");
     static_assert(Epi == EPI_PLAIN || ScaleKind == SCALE_ROWCOL, "the SwiGLU epilogue is the int8 decoder's");
@@ -192,11 +198,21 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
         for (int r = 0; r < 8; ++r) dma_x(r, rx1, 1, 128u);
 #pragma unroll
         for (int r = 0; r < 8; ++r) dma_w(r, rw1, 1, 128u);
-        wait_vmcnt<16>();  // slab 0
+        if constexpr (KO & KO_LOADS) {  // every stage holds operand bytes once and for all
+#pragma unroll
+            for (int r = 0; r < 8; ++r) dma_x(r, rx1, 2, 256u);
+            wait_vmcnt<0>();
+        } else {
+            wait_vmcnt<16>();  // slab 0
+        }
         __builtin_amdgcn_s_waitcnt(0xc07f);
         __syncthreads();
 #pragma unroll
         for (int r = 0; r < 16; ++r) read_one(r, 0, 0, 0, xf0, wf0);
+        if constexpr (KO & KO_LDS_READS) {  // both register sets hold operand bytes once and for all
+#pragma unroll
+            for (int r = 0; r < 16; ++r) read_one(r, 0, 0, 1, xf1, wf1);
+        }
     }
 
     // reads are spread over the first three quarters of a half's MFMAs so that the
@@ -223,11 +239,12 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < NM; ++i) {
-            mfma_one(i, xf0, wf0);
+            if constexpr (!(KO & KO_MFMA)) mfma_one(i, xf0, wf0);
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-                if ((r * kReadSpan) / 16 == i) read_one(r, xs, ws, 1, xf1, wf1);
-            if constexpr (LOADS) {
+                if constexpr (!(KO & KO_LDS_READS))
+                    if ((r * kReadSpan) / 16 == i) read_one(r, xs, ws, 1, xf1, wf1);
+            if constexpr (LOADS && !(KO & KO_LOADS)) {
 #pragma unroll
                 for (int d = 0; d < 8; ++d)
                     if ((d * NM) / 8 == i) dma_x(d, rx, xs2, k2);
@@ -239,7 +256,7 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
         // older -- and this wave is done reading slab k; after the barrier both
         // hold for every wave.
         PP_STAMP_INNER();
-        wait_vmcnt<LOADS ? 8 : 0>();
+        wait_vmcnt<(LOADS && !(KO & KO_LOADS)) ? 8 : 0>();
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
         PP_STAMP_INNER();
         phase_barrier();
@@ -251,11 +268,12 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < NM; ++i) {
-            mfma_one(i, xf1, wf1);
+            if constexpr (!(KO & KO_MFMA)) mfma_one(i, xf1, wf1);
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-                if ((r * kReadSpan) / 16 == i) read_one(r, xs1, ws ^ 1, 0, xf0, wf0);
-            if constexpr (LOADS) {
+                if constexpr (!(KO & KO_LDS_READS))
+                    if ((r * kReadSpan) / 16 == i) read_one(r, xs1, ws ^ 1, 0, xf0, wf0);
+            if constexpr (LOADS && !(KO & KO_LOADS)) {
 #pragma unroll
                 for (int d = 0; d < 8; ++d)
                     if ((d * NM) / 8 == i) dma_w(d, rw, ws, k2);
@@ -422,8 +440,9 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const u32x4 v = *reinterpret_cast<const u32x4*>(buf + (i * 4 + r4) * ROWB + c16 * 16);
-                __builtin_amdgcn_raw_buffer_store_b128(
-                    v, rout, lane_off + (uint32_t)(mi * 32 + i * 4) * row_bytes, 0, 2);
+                if constexpr (!(KO & KO_STORES))
+                    __builtin_amdgcn_raw_buffer_store_b128(
+                        v, rout, lane_off + (uint32_t)(mi * 32 + i * 4) * row_bytes, 0, 2);
             }
         }
     }
