@@ -434,7 +434,6 @@ __global__ __launch_bounds__(Cfg::THREADS) void gemm_pingpong_kernel(GemmArgs g)
             // loads; past the end it re-touches the last slab (an L2 hit)
             prefetch(min(k + kPrefetch, ksteps - 1));
             wait_lgkmcnt0();
-            PP_STAMP();
             // lower MFMA priority than group 1: if group 1's wave on this SIMD still
             // has MFMAs of the previous slab to issue it goes first (the hardware
             // otherwise favours this, older, wave and starves the other one)
@@ -442,13 +441,9 @@ __global__ __launch_bounds__(Cfg::THREADS) void gemm_pingpong_kernel(GemmArgs g)
             if constexpr (kBlk) compute_block();
             else compute();
             __builtin_amdgcn_s_setprio(0);
-            PP_STAMP();
             // the slab loads; the prefetch touch (if any) may stay in flight
             wait_vmcnt<kTouch>();
-            PP_STAMP();
             phase_barrier();  // B_{k+1}
-            PP_STAMP();
-            PP_STAMP();
             xs = (xs == 2) ? 0 : xs + 1;
         }
         phase_barrier();  // matches group 1's final barrier
@@ -463,23 +458,18 @@ __global__ __launch_bounds__(Cfg::THREADS) void gemm_pingpong_kernel(GemmArgs g)
             load_block_scales(k + 2);
             prefetch(min(k + 2 + kPrefetch, ksteps - 1));
             wait_lgkmcnt0();
-            PP_STAMP();
             // slab k+1 (issued one slab ago) must have landed; this slab's eight
             // loads and the two latest touches may stay in flight
             // (block scales: and this phase's two scale loads)
             if (more) wait_vmcnt<8 + 2 * kTouch + (kBlk ? 2 : 0)>();
             else wait_vmcnt<kTouch>();
-            PP_STAMP();
             phase_barrier();  // B_{k+1}
-            PP_STAMP();
-            PP_STAMP();
         };
         int xs = 0;  // k % 3
         if constexpr (kBlk) {
             // slab 0 has no predecessor to compute: kept out of the loop, whose MFMAs
             // are then unconditional (under "if (k > 0)" the compiler moved the second
             // half's multiplies out of the MFMA stream, behind the join)
-            PP_STAMP();
             memory_phase(0, 0);
             xs = 1;
         }
@@ -491,7 +481,6 @@ __global__ __launch_bounds__(Cfg::THREADS) void gemm_pingpong_kernel(GemmArgs g)
                 if (k > 0) compute();  // slab k-1
             }
             __builtin_amdgcn_s_setprio(0);
-            PP_STAMP();
             memory_phase(k, xs);
             xs = (xs == 2) ? 0 : xs + 1;
         }

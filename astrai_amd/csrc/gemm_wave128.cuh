@@ -31,14 +31,6 @@
 // c of row r at position c ^ (r & 7) ^ ((r >> 3) & 1); weight rows are the
 // first MFMA operand.
 #pragma once
-// per-phase timestamps inside the main loop perturb it (~100 cycles each): off
-// unless asked for; the stamps around the loop are always taken when timing is on
-#ifdef W128_INNER_STAMPS
-#define PP_STAMP_INNER() PP_STAMP()
-#else
-#define PP_STAMP_INNER()
-#endif
-
 #include "gemm_pingpong.cuh"
 
 namespace w8a8 {
@@ -235,7 +227,6 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
 
         // first half: MFMAs on F0, reads of (k, half 1) into F1, activation rows
         // of slab k+2 into the stage slab k-1 left at the previous barrier
-        PP_STAMP_INNER();
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < NM; ++i) {
@@ -255,12 +246,9 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
         // Slab k+1 has landed for this wave -- all but this half's eight loads are
         // older -- and this wave is done reading slab k; after the barrier both
         // hold for every wave.
-        PP_STAMP_INNER();
         wait_vmcnt<(LOADS && !(KO & KO_LOADS)) ? 8 : 0>();
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
-        PP_STAMP_INNER();
         phase_barrier();
-        PP_STAMP_INNER();
 
         // second half: MFMAs on F1, reads of (k+1, half 0) into F0 (stale bytes
         // after the last slab, never used), weight rows of slab k+2 into the stage

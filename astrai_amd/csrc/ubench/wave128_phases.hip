@@ -66,6 +66,81 @@ static unsigned char e4m3_of(float v) {
     return s | (unsigned char)((E << 3) | q);
 }
 
+// the eight-wave ping-pong kernel (block-scaled and per-tensor instances) with its stamps
+template <class Op, int SK, class Cfg>
+static float pingpong_us(const GemmArgs& g) {
+    auto kern = gemm_pingpong_kernel<Op, SK, Cfg>;
+    CK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
+    const int tiles = ((g.m + 255) / 256) * ((g.n + 255) / 256);
+    hipEvent_t e0, e1;
+    CK(hipEventCreate(&e0));
+    CK(hipEventCreate(&e1));
+    for (int i = 0; i < 200; ++i) kern<<<tiles, Cfg::THREADS, Cfg::LDS_BYTES, 0>>>(g);
+    CK(hipDeviceSynchronize());
+    std::vector<float> ts;
+    for (int rep = 0; rep < 7; ++rep) {
+        CK(hipEventRecord(e0));
+        for (int i = 0; i < 50; ++i) kern<<<tiles, Cfg::THREADS, Cfg::LDS_BYTES, 0>>>(g);
+        CK(hipEventRecord(e1));
+        CK(hipEventSynchronize(e1));
+        float ms;
+        CK(hipEventElapsedTime(&ms, e0, e1));
+        ts.push_back(ms * 20.0f);
+    }
+    std::sort(ts.begin(), ts.end());
+    return ts[3];
+}
+
+static void print_stamps(unsigned long long* dbg, int k, std::initializer_list<int> waves) {
+    std::vector<unsigned long long> hd(8 * 256);
+    CK(hipMemcpy(hd.data(), dbg, hd.size() * 8, hipMemcpyDeviceToHost));
+    for (int w : waves) {
+        const unsigned long long* t = &hd[w * 256];
+        printf("  wave %d: prologue %llu cycles, main loop %llu (%.0f per slab), epilogue %llu\n", w,
+               t[1] - t[0], t[2] - t[1], (double)(t[2] - t[1]) / (k / 128), t[3] - t[2]);
+    }
+}
+
+// config-3 shape: block-scaled instance against the per-tensor instance of the same kernel
+static void pingpong_section(unsigned long long* dbg) {
+    const int M = 8192, N = 2048, K = 7168;
+    void *a, *b, *out;
+    float* s;
+    CK(hipMalloc(&a, (size_t)M * K));
+    CK(hipMalloc(&b, (size_t)N * K));
+    CK(hipMalloc(&out, (size_t)M * N * 2));
+    CK(hipMalloc(&s, (size_t)4 * M * (K / 128)));
+    std::vector<float> ones((size_t)M * (K / 128), 1.0f);
+    CK(hipMemcpy(s, ones.data(), ones.size() * 4, hipMemcpyHostToDevice));
+    GemmArgs g{a, b, s, s, nullptr, nullptr, out, M, N, K, OUT_BF16};
+    for (int random = 0; random < 2; ++random) {
+        if (random) {
+            std::vector<unsigned char> ra((size_t)M * K), rb((size_t)N * K);
+            auto gauss = [] { float u = 0; for (int i = 0; i < 12; ++i) u += (float)rand() / RAND_MAX; return u - 6.0f; };
+            for (auto& x : ra) x = e4m3_of(gauss() * 448.0f / 4.5f);
+            for (auto& x : rb) x = e4m3_of(gauss() * 448.0f / 4.5f);
+            CK(hipMemcpy(a, ra.data(), ra.size(), hipMemcpyHostToDevice));
+            CK(hipMemcpy(b, rb.data(), rb.size(), hipMemcpyHostToDevice));
+        } else {
+            CK(hipMemset(a, 0, (size_t)M * K));
+            CK(hipMemset(b, 0, (size_t)N * K));
+        }
+        const double ops = 2.0 * M * N * (double)K;
+        float us = pingpong_us<Op32F8<0>, SCALE_BLOCK128, PingPongCfgBlock>(g);
+        printf("ping-pong kernel, 128-block scales, %s %dx%dx%d: %.2f us (%.0f Tops/s)\n",
+               random ? "normal operands" : "zeros", M, N, K, us, ops / us / 1e6);
+        if (!random) print_stamps(dbg, K, {0, 4});
+        us = pingpong_us<Op32F8<0>, SCALE_TENSOR, PingPongCfg>(g);
+        printf("ping-pong kernel, per-tensor scales, %s: %.2f us (%.0f Tops/s)\n",
+               random ? "normal operands" : "zeros", us, ops / us / 1e6);
+        if (!random) print_stamps(dbg, K, {0, 4});
+        us = time_us<Op32F8<0>, SCALE_TENSOR, 0>(g);
+        printf("four-wave kernel, per-tensor scales, %s: %.2f us (%.0f Tops/s)\n",
+               random ? "normal operands" : "zeros", us, ops / us / 1e6);
+    }
+    CK(hipFree(a)); CK(hipFree(b)); CK(hipFree(out)); CK(hipFree(s));
+}
+
 template <class Op, int SK>
 static void knockouts(const char* what, const GemmArgs& g) {
     const double ops = 2.0 * g.m * g.n * (double)g.k;
@@ -98,15 +173,9 @@ int main(int argc, char** argv) {
     CK(hipMemset(b, 0, (size_t)N * K));
     for (int which = 0; which < 2; ++which) {
         const float us = which ? time_us<Op32I8, SCALE_ROWCOL, 0>(g) : time_us<Op32F8<0>, SCALE_TENSOR, 0>(g);
-        std::vector<unsigned long long> hd(8 * 256);
-        CK(hipMemcpy(hd.data(), dbg, hd.size() * 8, hipMemcpyDeviceToHost));
         printf("%s zeros %dx%dx%d: %.2f us; stamps of workgroup 0 in shader clock cycles\n",
                which ? "int8" : "fp8", M, N, K, us);
-        for (int w : {0, 3}) {
-            const unsigned long long* t = &hd[w * 256];
-            printf("  wave %d: prologue %llu cycles, main loop %llu (%.0f per slab), epilogue %llu\n", w,
-                   t[1] - t[0], t[2] - t[1], (double)(t[2] - t[1]) / (K / 128), t[3] - t[2]);
-        }
+        print_stamps(dbg, K, {0, 3});
     }
     knockouts<Op32F8<0>, SCALE_TENSOR>("fp8 zeros", g);
     knockouts<Op32I8, SCALE_ROWCOL>("int8 zeros", g);
@@ -129,5 +198,6 @@ int main(int argc, char** argv) {
         CK(hipMemcpy(b, rb.data(), rb.size(), hipMemcpyHostToDevice));
     }
     knockouts<Op32I8, SCALE_ROWCOL>("int8 normal operands (amax at 4.5 sigma)", g);
+    pingpong_section(dbg);
     return 0;
 }
