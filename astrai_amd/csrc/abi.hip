@@ -725,16 +725,19 @@ int astrai_w8a8_gemm_int8_ptpc_rope_cache(const void* a, const void* b, const fl
         return fail(ASTRAI_W8A8_BAD_ARG, "%s: pointers must be 16-byte aligned", what);
     const int64_t m = batch * seq, n = (n_heads + 2 * n_kv_heads) * head_dim;
     if (m == 0) return ASTRAI_W8A8_OK;
-    if (m > 64 || k % 256 || head_dim % 4 || n * k >= ((int64_t)1 << 31))
-        return fail(ASTRAI_W8A8_UNSUPPORTED,
-                    "%s: needs batch * seq <= 64, K a multiple of 256, head_dim a multiple of 4 and a "
-                    "weight matrix under 2 GiB (got m=%lld k=%lld head_dim=%lld)",
-                    what, (long long)m, (long long)k, (long long)head_dim);
+    if (n * k >= ((int64_t)1 << 31) || m * k >= ((int64_t)1 << 31))
+        return fail(ASTRAI_W8A8_UNSUPPORTED, "%s: operands must stay under 2 GiB", what);
     const w8a8::GemmArgs g = pack(a, b, sa, sb, nullptr, nullptr, nullptr, m, n, k, w8a8::OUT_BF16);
     const w8a8::RopeCacheArgs rc{nullptr, 0, freqs, positions, q_out, k_cache, v_cache,
                                  (int)batch, (int)seq, (int)n_heads, (int)n_kv_heads, (int)head_dim, max_len};
-    if (!w8a8::launch_gemm_int8_rope_cache(g, rc, static_cast<hipStream_t>(stream)))
-        return fail(ASTRAI_W8A8_UNSUPPORTED, "%s: shape not supported", what);
+    const bool small = m <= 64 && k % 256 == 0 && head_dim % 4 == 0;
+    if (!(small && w8a8::launch_gemm_int8_rope_cache(g, rc, static_cast<hipStream_t>(stream))) &&
+        !w8a8::launch_gemm_int8_rope_cache_large(g, rc, static_cast<hipStream_t>(stream)))
+        return fail(ASTRAI_W8A8_UNSUPPORTED,
+                    "%s: needs either batch * seq <= 64 with K a multiple of 256 and head_dim a multiple of 4, "
+                    "or head_dim 128 with at least 192 output tiles of 256 x 256 and K a multiple of 128, at "
+                    "least 256 (got m=%lld k=%lld head_dim=%lld)",
+                    what, (long long)m, (long long)k, (long long)head_dim);
     return check_launch(what);
 }
 

@@ -28,4 +28,15 @@ bool launch_gemm_int8_swiglu(const GemmArgs& g, hipStream_t stream) {
     return true;
 }
 
+bool launch_gemm_int8_rope_cache_large(const GemmArgs& g, const RopeCacheArgs& rc, hipStream_t stream) {
+    if (!tiled_shape_ok(g) || !wave128_shape_ok(g) || (g.n & 127) != 0 || g.bias != nullptr) return false;
+    if (rc.head_dim != 128 || g.m >= (1 << 23) || g.m != rc.batch * rc.seq || g.n != (rc.n_heads + 2 * rc.n_kv_heads) * 128) return false;
+    // destinations are addressed with 32-bit byte offsets below the out-of-range marker
+    const int64_t lim = (int64_t)1 << 31;
+    if ((int64_t)g.m * rc.n_heads * 256 >= lim || (int64_t)rc.batch * rc.n_kv_heads * rc.max_len * 256 >= lim)
+        return false;
+    launch_wave128<Op32I8, SCALE_ROWCOL, EPI_ROPE>(g, stream, rc);
+    return true;
+}
+
 }  // namespace w8a8

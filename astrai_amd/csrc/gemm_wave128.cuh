@@ -61,7 +61,7 @@ __device__ __forceinline__ float silu_hw(float g) {
     return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.44269504088896340736f));
 }
 
-enum : int { EPI_PLAIN = 0, EPI_SWIGLU = 1 };
+enum : int { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_ROPE = 2 };
 
 // Knock-outs for the phase microbenchmark (ubench/wave128_phases.hip): each bit removes one
 // class of instructions so that its share of the kernel's time -- issue slots and, under the
@@ -70,9 +70,9 @@ enum : int { EPI_PLAIN = 0, EPI_SWIGLU = 1 };
 enum : int { KO_LDS_READS = 1, KO_LOADS = 2, KO_MFMA = 4, KO_STORES = 8 };
 
 template <class Op, int ScaleKind, int Epi = EPI_PLAIN, int KO = 0>
-__global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmArgs g) {
+__global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmArgs g, RopeCacheArgs rc) {
     static_assert(ScaleKind != SCALE_BLOCK128, "block scales run on the ping-pong kernel");
-    static_assert(Epi == EPI_PLAIN || ScaleKind == SCALE_ROWCOL, "the SwiGLU epilogue is the int8 decoder's");
+    static_assert(Epi == EPI_PLAIN || ScaleKind == SCALE_ROWCOL, "the SwiGLU and rotary epilogues are the int8 decoder's");
     PP_STAMP_INIT();
     using Cfg = Wave128Cfg;
     using Acc = typename Op::Acc;
@@ -294,6 +294,133 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
     // takes no part in the check. The stores are non-temporal (aux bit 1): the
     // 2 M N output bytes stream to memory while the epilogue still computes instead
     // of sitting dirty in L2 until the end-of-kernel write-back (-1.5 us at 4096^3).
+    if constexpr (Epi == EPI_ROPE) {
+        // The rows are the fused q|k|v projection of a decoder layer, head_dim 128: the 128
+        // columns of a wave tile are one head. The epilogue goes on where the separate rotary /
+        // cache-write kernel would start: the bf16-rounded value pairs of q and k are rotated
+        // (fp32 products and sums rounded one by one, one rounding to bf16 -- the arithmetic of
+        // rope_cache.hip on the same rounded inputs), a pass of 32 tokens x 128 dims is staged
+        // through LDS and leaves as whole 256-byte head rows: q to [batch, heads, seq, 128], k
+        // and v into the cache at the tokens' positions (a position outside the cache: nothing).
+        constexpr int ROWB = Cfg::EPI_ROW_BYTES, PASS_BYTES = Cfg::EPI_PASS_BYTES;
+        uint8_t* const mine = lds + wave * (2 * PASS_BYTES);
+        const int nwv = n0 + wave_n * 128;
+        const int hh = nwv >> 7;                         // head among q heads | k heads | v heads
+        const bool live_head = nwv < g.n;
+        const bool is_q = hh < rc.n_heads, rotate = hh < rc.n_heads + rc.n_kv_heads;
+        const int hk = hh - rc.n_heads - (rotate ? 0 : rc.n_kv_heads);
+        const int mw = m0 + wave_m * 128;                // first token of this wave
+        f32x4 sw4[NI][4];
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int n = nwv + ni * 32 + q * 8 + lgrp * 4;
+                sw4[ni][q] = (n < g.n) ? *reinterpret_cast<const f32x4*>(g.sb + n) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+        void* const dst_base = is_q ? rc.q_out : (rotate ? rc.k_cache : rc.v_cache);
+        const uint32_t dst_bytes = is_q ? (uint32_t)g.m * (uint32_t)rc.n_heads * 256u
+                                        : (uint32_t)rc.batch * (uint32_t)rc.n_kv_heads * (uint32_t)rc.max_len * 256u;
+        const __amdgpu_buffer_rsrc_t rout = make_rsrc(dst_base, live_head ? dst_bytes : 0u);
+        const int r4 = lane >> 4, c16 = lane & 15;
+        // One wave per SIMD: nothing hides a memory round trip inside the epilogue, so everything
+        // it reads is requested ahead of its use -- the destinations of all 32 rows this lane will
+        // store (cache slots: one lookup of the token's position each) now, the (cos, sin) pairs of
+        // a group of 32 columns two groups before the group that uses them.
+        // token index -> (sequence, token in sequence) without an integer division per row: the
+        // float quotient of m < 2^23 is off by at most one, which the remainder shows
+        const float inv_seq = 1.0f / (float)rc.seq;
+        auto split_token = [&](int m, int& bt, int& sq) {
+            bt = (int)((float)m * inv_seq);
+            sq = m - bt * rc.seq;
+            if (sq < 0) { --bt; sq += rc.seq; }
+            else if (sq >= rc.seq) { ++bt; sq -= rc.seq; }
+        };
+        uint32_t dst_off[MI][8];
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int m = mw + mi * 32 + i * 4 + r4;
+                int bt, sq;
+                split_token(m, bt, sq);
+                dst_off[mi][i] = kOutOfRange;
+                if (m < g.m) {
+                    if (is_q) {
+                        dst_off[mi][i] = (uint32_t)((bt * rc.n_heads + hh) * rc.seq + sq) * 256u + (uint32_t)c16 * 16u;
+                    } else {
+                        const int64_t pos = rc.positions[sq];
+                        if (pos >= 0 && pos < rc.max_len)
+                            dst_off[mi][i] = (uint32_t)((int64_t)(bt * rc.n_kv_heads + hk) * rc.max_len + pos) * 256u +
+                                             (uint32_t)c16 * 16u;
+                    }
+                }
+            }
+        // group gi = mi * NI + ni: the lane's token of pass mi, columns 32 ni .. 32 ni + 31
+        constexpr int kAhead = 2;
+        f32x4 cs[kAhead + 1][4];
+        const float* cs_row[MI];
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi) {
+            int bt, sq;
+            split_token(mw + mi * 32 + lrow, bt, sq);
+            cs_row[mi] = rc.freqs + ((int64_t)sq * 64 + (lgrp * 2)) * 2;
+        }
+        auto request_cs = [&](int gi) {
+            if (!rotate || gi >= MI * NI) return;
+            const int mi = gi / NI, ni = gi % NI;
+#pragma unroll
+            for (int q = 0; q < 4; ++q)  // d = 32 ni + 8 q + 4 lgrp: pair index d / 2
+                cs[gi % (kAhead + 1)][q] = *reinterpret_cast<const f32x4*>(cs_row[mi] + (ni * 16 + q * 4) * 2);
+        };
+#pragma unroll
+        for (int gi = 0; gi < kAhead; ++gi) request_cs(gi);
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi) {
+            uint8_t* const buf = mine + (mi & 1) * PASS_BYTES;
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni) {
+                const int gi = mi * NI + ni;
+                request_cs(gi + kAhead);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float v[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+#pragma clang fp contract(off)
+                        v[j] = (float)acc[ni][mi][4 * q + j] * sx[mi] * sw4[ni][q][j];
+                    }
+                    u32x2 pk;
+                    pk.x = pack_bf16x2(v[0], v[1]);
+                    pk.y = pack_bf16x2(v[2], v[3]);
+                    if (rotate) {
+                        const f32x4 c4 = cs[gi % (kAhead + 1)][q];
+                        const float x[4] = {__uint_as_float(pk.x << 16), __uint_as_float(pk.x & 0xffff0000u),
+                                            __uint_as_float(pk.y << 16), __uint_as_float(pk.y & 0xffff0000u)};
+                        float y[4];
+#pragma unroll
+                        for (int p = 0; p < 2; ++p) {
+#pragma clang fp contract(off)
+                            const float c = c4[2 * p], sn = c4[2 * p + 1];
+                            const float xe = x[2 * p], xo = x[2 * p + 1];
+                            const float a0 = xe * c, a1 = xo * sn, b0 = xe * sn, b1 = xo * c;
+                            y[2 * p] = a0 - a1;
+                            y[2 * p + 1] = b0 + b1;
+                        }
+                        pk.x = pack_bf16x2(y[0], y[1]);
+                        pk.y = pack_bf16x2(y[2], y[3]);
+                    }
+                    *reinterpret_cast<u32x2*>(buf + lrow * ROWB + (ni * 32 + q * 8 + lgrp * 4) * 2) = pk;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const u32x4 v = *reinterpret_cast<const u32x4*>(buf + (i * 4 + r4) * ROWB + c16 * 16);
+                __builtin_amdgcn_raw_buffer_store_b128(v, rout, dst_off[mi][i], 0, 0);
+            }
+        }
+    } else
     if constexpr (Epi == EPI_SWIGLU) {
         // The wave's 128 columns are 64 gate columns (sub-tiles 0, 1) and the 64 up columns
         // (sub-tiles 2, 3) of the same 64 columns of h, so a lane holds every pair in its own
@@ -445,13 +572,13 @@ inline bool wave128_shape_ok(const GemmArgs& g) {
 }
 
 template <class Op, int ScaleKind, int Epi = EPI_PLAIN>
-inline void launch_wave128(const GemmArgs& g, hipStream_t stream) {
+inline void launch_wave128(const GemmArgs& g, hipStream_t stream, const RopeCacheArgs& rc = RopeCacheArgs{}) {
     using Cfg = Wave128Cfg;
     const int tiles = ((g.m + Cfg::BM - 1) / Cfg::BM) * ((g.n + Cfg::BN - 1) / Cfg::BN);
     auto kern = gemm_wave128_kernel<Op, ScaleKind, Epi>;
     static std::atomic<uint64_t> lds_allowed{0};
     allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::LDS_BYTES, lds_allowed);
-    kern<<<dim3((unsigned)tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(g);
+    kern<<<dim3((unsigned)tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(g, rc);
 }
 
 }  // namespace w8a8

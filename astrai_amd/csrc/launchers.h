@@ -219,6 +219,9 @@ bool launch_gemv_int8(const GemmArgs& g, hipStream_t stream);
 // the fused q|k|v projection of up to 64 tokens with rotary embedding and KV-cache write
 // in the epilogue (g.out unused; rc.qkv / rc.ld unused); false when the shape does not fit
 bool launch_gemm_int8_rope_cache(const GemmArgs& g, const RopeCacheArgs& rc, hipStream_t stream);
+// gemm_int8.hip: the same for long blocks of tokens (prefill) on the large-tile kernel: head_dim 128,
+// at least 192 output tiles of 256 x 256, K % 128 == 0; false when the shape does not fit
+bool launch_gemm_int8_rope_cache_large(const GemmArgs& g, const RopeCacheArgs& rc, hipStream_t stream);
 
 // mfma_probe.hip: one instruction of MFMA shape `kind` on a zero accumulator, one wave;
 // d_raw[lane][reg] are the accumulator registers as they are (4 or 16 per lane)

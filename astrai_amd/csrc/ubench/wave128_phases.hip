@@ -35,12 +35,12 @@ static float time_us(const GemmArgs& g) {
     hipEvent_t e0, e1;
     CK(hipEventCreate(&e0));
     CK(hipEventCreate(&e1));
-    for (int i = 0; i < 300; ++i) kern<<<tiles, 256, Wave128Cfg::LDS_BYTES, 0>>>(g);
+    for (int i = 0; i < 300; ++i) kern<<<tiles, 256, Wave128Cfg::LDS_BYTES, 0>>>(g, RopeCacheArgs{});
     CK(hipDeviceSynchronize());
     std::vector<float> ts;
     for (int rep = 0; rep < 7; ++rep) {
         CK(hipEventRecord(e0));
-        for (int i = 0; i < 100; ++i) kern<<<tiles, 256, Wave128Cfg::LDS_BYTES, 0>>>(g);
+        for (int i = 0; i < 100; ++i) kern<<<tiles, 256, Wave128Cfg::LDS_BYTES, 0>>>(g, RopeCacheArgs{});
         CK(hipEventRecord(e1));
         CK(hipEventSynchronize(e1));
         float ms;

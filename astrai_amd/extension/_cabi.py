@@ -1159,10 +1159,20 @@ def mm_int8_swiglu(a: torch.Tensor, wgu: torch.Tensor, sa: torch.Tensor, sgu: to
     return hq, s, (h if want_h else None)
 
 
-def mm_int8_rope_cache_supported(tokens: int, k: int, head_dim: int, n: int = 0) -> bool:
-    """Shapes the fused q|k|v projection + rotary + cache-write kernel takes (the limits
-    its entry point checks); ``n`` = rows of the q|k|v weight, when known."""
-    return 0 < tokens <= 64 and k % 256 == 0 and head_dim % 4 == 0 and n * k < 2 ** 31
+def mm_int8_rope_cache_supported(tokens: int, k: int, head_dim: int, n: int = 0, batch: int = 0,
+                                 n_heads: int = 0, n_kv_heads: int = 0, max_len: int = 0) -> bool:
+    """Shapes the fused q|k|v projection + rotary + cache-write entry takes (the limits it
+    checks); ``n`` = rows of the q|k|v weight, when known. A few tokens (decode steps: at most
+    64, K % 256 == 0, head_dim % 4 == 0) run the row-range kernel; long blocks (prefill: head_dim
+    128, at least 192 output tiles of 256 x 256, K % 128 == 0, destinations under 2 GiB -- checked
+    when ``batch`` .. ``max_len`` are given) the large-tile GEMM with the same epilogue."""
+    if tokens <= 0 or n * k >= 2 ** 31 or tokens * k >= 2 ** 31:
+        return False
+    if tokens <= 64 and k % 256 == 0 and head_dim % 4 == 0:
+        return True
+    tiles = ((tokens + 255) // 256) * ((n + 255) // 256)
+    return (head_dim == 128 and n > 0 and n % 128 == 0 and tiles >= 192 and k >= 256 and k % 128 == 0
+            and tokens * n_heads * 256 < 2 ** 31 and batch * n_kv_heads * max_len * 256 < 2 ** 31)
 
 
 FUSED_ROW_MAX = 8192
@@ -1179,7 +1189,8 @@ def mm_int8_rope_cache(a: torch.Tensor, wqkv: torch.Tensor, sa: torch.Tensor, sb
                        v_cache: torch.Tensor, batch: int, seq: int, n_heads: int, n_kv_heads: int,
                        head_dim: int) -> torch.Tensor:
     """``mm_int8(a, wqkv, sa, sb)`` followed by :func:`rope_cache_write` on its output, as one
-    kernel and bit for bit the same: ``a`` int8 ``[batch*seq, K]`` (at most 64 rows), ``wqkv``
+    kernel and bit for bit the same: ``a`` int8 ``[batch*seq, K]`` (a few rows or a long block, see
+    :func:`mm_int8_rope_cache_supported`), ``wqkv``
     int8 ``[(n_heads + 2 n_kv_heads) * head_dim, K]``. Writes k and v into the caches at
     ``positions`` and returns the rotated q as ``[batch, n_heads, seq, head_dim]``."""
     lib = _require()
@@ -1190,9 +1201,10 @@ def mm_int8_rope_cache(a: torch.Tensor, wqkv: torch.Tensor, sa: torch.Tensor, sb
     n = (n_heads + 2 * n_kv_heads) * head_dim
     if m != batch * seq or wqkv.size(0) != n or wqkv.size(1) != k:
         raise RuntimeError("a must be [batch*seq, K] and wqkv [(n_heads + 2 n_kv_heads) * head_dim, K]")
-    if not mm_int8_rope_cache_supported(m, k, head_dim, n):
-        raise RuntimeError("mm_int8_rope_cache: needs at most 64 tokens, K % 256 == 0, head_dim % 4 == 0, "
-                           "a weight matrix under 2 GiB")
+    if not mm_int8_rope_cache_supported(m, k, head_dim, n, batch, n_heads, n_kv_heads, k_cache.size(2)):
+        raise RuntimeError("mm_int8_rope_cache: needs at most 64 tokens with K % 256 == 0 and head_dim % 4 == 0, "
+                           "or head_dim 128 with at least 192 output tiles of 256 x 256 and K % 128 == 0; "
+                           "operands and destinations under 2 GiB")
     sa = _check_vec(sa, a, m, "sa")
     sb = _check_vec(sb, a, n, "sb")
     if k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:

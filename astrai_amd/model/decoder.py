@@ -268,8 +268,10 @@ class DecoderBlock(nn.Module):
             aq, sa = I.quantize_int8_per_token(
                 att.core(qkv[..., :nq], qkv[..., nq:nq + nkv], qkv[..., nq + nkv:], rotary_emb, None,
                          positions, key_mask))
-        elif _cabi.mm_int8_rope_cache_supported(b * s, d, att.head_dim, f.wqkv.size(0)):
-            # a few new tokens: the projection's epilogue rotates q and k and writes the cache
+        elif _cabi.mm_int8_rope_cache_supported(b * s, d, att.head_dim, f.wqkv.size(0), b, att.n_heads,
+                                                att.n_kv_heads, kv_cache.max_len):
+            # a few new tokens, or a long block at head_dim 128: the projection's epilogue rotates q
+            # and k and writes the cache
             q = _cabi.mm_int8_rope_cache(xq, f.wqkv, sx, f.sqkv, rotary_emb[0], positions,
                                          kv_cache.k[att.layer_id], kv_cache.v[att.layer_id],
                                          b, s, att.n_heads, att.n_kv_heads, att.head_dim)

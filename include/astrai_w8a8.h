@@ -507,17 +507,19 @@ int astrai_w8a8_gemv_int8_ptpc(const void* a, const void* b, const float* sa,
                                void* stream);
 
 /*
- * The fused q|k|v projection of a decoder layer for a few new tokens
- * (batch * seq <= 64), with what follows it in the reference done in the GEMM's
- * epilogue: the rotary embedding of q and k (astrai/extension/backend/rotary.py:25-33),
+ * The fused q|k|v projection of a decoder layer with what follows it in the reference done
+ * in the GEMM's epilogue: the rotary embedding of q and k (astrai/extension/backend/rotary.py:25-33),
  * the permutes and the KV-cache write (astrai/model/components/attention.py:19-85).
  * Equal, bit for bit, to astrai_w8a8_gemm_int8_ptpc (bf16 out, no bias) followed by
  * astrai_w8a8_rope_cache_write_bf16 on its output:
  *   a int8 [batch*seq, K] with sa fp32 [batch*seq]; b int8 [(n_heads + 2 n_kv_heads) * head_dim, K]
  *   (rows: q heads | k heads | v heads) with sb fp32 per row; freqs, positions, q_out,
  *   k_cache, v_cache as for astrai_w8a8_rope_cache_write_bf16.
- * Needs K % 256 == 0 and head_dim % 4 == 0; ASTRAI_W8A8_UNSUPPORTED otherwise (run the two
- * calls instead).
+ * Two shape classes: a few new tokens (decode steps: batch * seq <= 64, K % 256 == 0,
+ * head_dim % 4 == 0; the row-range kernel) and long blocks (prefill: head_dim == 128, at least
+ * 192 output tiles of 256 x 256, K % 128 == 0, K >= 256, q_out and each cache under 2 GiB; the
+ * large-tile GEMM, one head per 128-column wave tile). ASTRAI_W8A8_UNSUPPORTED otherwise (run
+ * the two calls instead).
  */
 int astrai_w8a8_gemm_int8_ptpc_rope_cache(const void* a, const void* b, const float* sa,
                                           const float* sb, const float* freqs,

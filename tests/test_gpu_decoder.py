@@ -293,7 +293,9 @@ def test_config4_dimensions_fused_cached_graph_properties(monkeypatch):
         cache = DenseKVCache(cfg, b, p + steps, DEV, torch.bfloat16)
         pre = gm(ids[:, :p], cache, torch.arange(p, device=DEV))["logits"]
         c = spy.take()
-        assert c["attn_prefill"] == 2 and c["rope_cache_write"] == 2 and c["sdpa"] == 0, c
+        # 16,384 new tokens: the projection GEMM rotates and writes the cache in its epilogue
+        assert c["attn_prefill"] == 2 and c["mm_int8_rope_cache"] == 2 and c["rope_cache_write"] == 0 \
+            and c["sdpa"] == 0, c
         dec = [gm(ids[:, t:t + 1], cache, torch.tensor([t], device=DEV))["logits"] for t in range(p, p + steps)]
         c = spy.take()
         assert c["attn_decode"] == 2 * steps and c["mm_int8_rope_cache"] == 2 * steps and c["sdpa"] == 0, c

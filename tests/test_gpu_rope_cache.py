@@ -70,6 +70,9 @@ def test_rope_cache_write_rejects_bad_arguments():
     (4, 16, 2, 1, 16, 40, 256),        # 64 rows: the largest the fused kernel takes
     (5, 1, 8, 8, 32, 16, 1024),        # no grouping, 16-row workgroups of eight waves
     (2, 3, 96, 8, 128, 16, 256),       # a wide projection: 48-row workgroups
+    (32, 512, 16, 4, 128, 640, 2048),  # config-4 prefill: the large-tile GEMM with the same epilogue
+    (3, 700, 32, 8, 128, 1000, 256),   # ragged token count (2100 rows, last tile partly empty), two slabs
+    (5, 413, 40, 4, 128, 500, 384),    # 2065 rows, N = 48 heads, three slabs
 ])
 def test_projection_with_rotary_epilogue_equals_the_two_kernels(b, s, h, hkv, d, max_len, k):
     """The fused q|k|v projection + rotary + cache write against the int8 GEMM followed by
@@ -91,7 +94,7 @@ def test_projection_with_rotary_epilogue_equals_the_two_kernels(b, s, h, hkv, d,
     k1, v1, k2, v2 = kc.to(DEV), vc.to(DEV), kc.to(DEV), vc.to(DEV)
     qkv = _cabi.mm_int8(a, w, sa, sb).reshape(b, s, n)
     q_want = _cabi.rope_cache_write(qkv, freqs, pos, k1, v1, h, hkv, d)
-    assert _cabi.mm_int8_rope_cache_supported(b * s, k, d)
+    assert _cabi.mm_int8_rope_cache_supported(b * s, k, d, n, b, h, hkv, max_len)
     q_got = _cabi.mm_int8_rope_cache(a, w, sa, sb, freqs, pos, k2, v2, b, s, h, hkv, d)
     for name, got, want in (("q", q_got, q_want), ("k_cache", k2, k1), ("v_cache", v2, v1)):
         assert torch.equal(got.view(torch.int16), want.view(torch.int16)), name
