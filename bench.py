@@ -689,6 +689,32 @@ def main():
             del a3c, b3c
         del a3, b3, out3, x3, w3
 
+        # ---- config-4 prefill MLP entry: gate|up projection + SwiGLU + per-token int8, as one GEMM
+        # with the product in its epilogue + the one-read quantizer, against GEMM + producer kernel
+        Mg, Wg, Kg = 32 * 512, 5632, 2048
+        gsw = torch.Generator().manual_seed(4)
+        xg = torch.randn(Mg, Kg, generator=gsw).to(torch.bfloat16).to(dev)
+        wgate = (torch.randn(Wg, Kg, generator=gsw) * 0.02).to(torch.bfloat16).to(dev)
+        wup = (torch.randn(Wg, Kg, generator=gsw) * 0.02).to(torch.bfloat16).to(dev)
+        xq, sxq = _cabi.quantize_int8_rows(xg)
+        (wgq, sgq), (wuq, suq) = _cabi.quantize_int8_rows(wgate), _cabi.quantize_int8_rows(wup)
+        sxq, sgq, suq = sxq.reshape(-1), sgq.reshape(-1), suq.reshape(-1)
+        wcat, scat = torch.cat((wgq, wuq)), torch.cat((sgq, suq))
+        wblk, sblk = _cabi.swiglu_block_rows(wgq, wuq), _cabi.swiglu_block_rows(sgq, suq)
+
+        def step_chain():
+            gu = _cabi.mm_int8(xq, wcat, sxq, scat)
+            _cabi.silu_mul_quantize_int8(gu[:, :Wg], gu[:, Wg:])
+
+        ms_chain = ms_of(step_chain)
+        ms_fused = ms_of(lambda: _cabi.mm_int8_swiglu(xq, wblk, sxq, sblk, fused=True))
+        extra["int8_gate_up_swiglu_16384x11264x2048"] = {
+            "data": "config-4 prefill shape, N(0,1) activations, N(0,0.02) weights, seed 4",
+            "gemm_plus_producer_us": round(ms_chain * 1e3, 1),
+            "swiglu_epilogue_gemm_plus_quantizer_us": round(ms_fused * 1e3, 1),
+            "TOP/s_of_the_fused_pair": round(2.0 * Mg * 2 * Wg * Kg / (ms_fused * 1e-3) / 1e12, 1)}
+        del xg, wgate, wup, xq, wgq, wuq, wcat, wblk
+
         # ---- config 2: decode GEMV on the seed-2 tensors (activation and weight quantized per
         # token / per channel by the oracle's quantizer on the host), weights rotated through a
         # ring of ten copies (451 MB) so that the 256 MB Infinity Cache cannot serve them
