@@ -214,7 +214,7 @@ bool launch_gemm_fp8_block128_tiled(const GemmArgs& g, hipStream_t stream);
 void launch_gemm_generic(const GemmArgs& g, int op /*0=i8,1=e4m3,2=e5m2*/, int scale_kind,
                          hipStream_t stream);
 
-// gemv_int8.hip: skinny int8 kernel, m <= 64, k % 256 == 0.
+// gemv_int8.hip: decode-shape int8 kernels (one token: dot kernel; 2..128 tokens: row-range kernel), k % 256 == 0.
 bool launch_gemv_int8(const GemmArgs& g, hipStream_t stream);
 // the fused q|k|v projection of up to 64 tokens with rotary embedding and KV-cache write
 // in the epilogue (g.out unused; rc.qkv / rc.ld unused); false when the shape does not fit
