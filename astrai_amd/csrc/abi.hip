@@ -692,6 +692,32 @@ int astrai_w8a8_gemm_int8_ptpc(const void* a, const void* b, const float* sa, co
     return check_launch("gemm_int8_ptpc");
 }
 
+int astrai_w8a8_gemm_int8_ptpc_resid(const void* a, const void* b, const float* sa, const float* sb,
+                                     const void* bias, const void* resid, void* out, int64_t m,
+                                     int64_t n, int64_t k, void* stream) {
+    const char* what = "gemm_int8_ptpc_resid";
+    if (int rc = int8_common(what, a, b, sa, sb, out, m, n, k, ASTRAI_W8A8_OUT_BF16)) return rc;
+    if (!resid) return fail(ASTRAI_W8A8_BAD_ARG, "%s: null residual pointer", what);
+    if (!aligned16(resid)) return fail(ASTRAI_W8A8_BAD_ARG, "%s: resid must be 16-byte aligned", what);
+    if (m == 0 || n == 0) return ASTRAI_W8A8_OK;
+    {
+        const auto lo = reinterpret_cast<uintptr_t>(out), ro = reinterpret_cast<uintptr_t>(resid);
+        const uintptr_t bytes = (uintptr_t)m * (uintptr_t)n * 2u;
+        if (lo < ro + bytes && ro < lo + bytes)
+            return fail(ASTRAI_W8A8_BAD_ARG, "%s: out overlaps resid", what);
+    }
+    auto s = static_cast<hipStream_t>(stream);
+    w8a8::GemmArgs g = pack(a, b, sa, sb, nullptr, bias, out, m, n, k, ASTRAI_W8A8_OUT_BF16);
+    g.resid = resid;
+    if (w8a8::launch_gemm_int8_resid(g, s)) return check_launch(what);
+    // shapes without a fused epilogue: the plain product, then the addition in place
+    g.resid = nullptr;
+    if (!(m <= 128 && w8a8::launch_gemv_int8(g, s)) && !w8a8::launch_gemm_int8_tiled(g, s))
+        w8a8::launch_gemm_generic(g, 0, w8a8::SCALE_ROWCOL, s);
+    w8a8::launch_add_bf16(out, resid, out, m * n, s);
+    return check_launch(what);
+}
+
 int astrai_w8a8_gemv_int8_ptpc(const void* a, const void* b, const float* sa, const float* sb,
                                const void* bias, void* out, int64_t m, int64_t n, int64_t k,
                                int out_dtype, void* stream) {

@@ -28,6 +28,14 @@ bool launch_gemm_int8_swiglu(const GemmArgs& g, hipStream_t stream) {
     return true;
 }
 
+bool launch_gemm_int8_resid(const GemmArgs& g, hipStream_t stream) {
+    if (!g.resid || g.out_kind != OUT_BF16) return false;
+    if (g.m <= 128 && launch_gemv_int8(g, stream)) return true;
+    if (!tiled_shape_ok(g) || !wave128_shape_ok(g) || g.bias != nullptr) return false;
+    launch_wave128<Op32I8, SCALE_ROWCOL, EPI_RESID>(g, stream);
+    return true;
+}
+
 bool launch_gemm_int8_rope_cache_large(const GemmArgs& g, const RopeCacheArgs& rc, hipStream_t stream) {
     if (!tiled_shape_ok(g) || !wave128_shape_ok(g) || (g.n & 127) != 0 || g.bias != nullptr) return false;
     if (rc.head_dim != 128 || g.m >= (1 << 23) || g.m != rc.batch * rc.seq || g.n != (rc.n_heads + 2 * rc.n_kv_heads) * 128) return false;

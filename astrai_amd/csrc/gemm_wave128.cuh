@@ -61,7 +61,7 @@ __device__ __forceinline__ float silu_hw(float g) {
     return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.44269504088896340736f));
 }
 
-enum : int { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_ROPE = 2 };
+enum : int { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_ROPE = 2, EPI_RESID = 3 };
 
 // Knock-outs for the phase microbenchmark (ubench/wave128_phases.hip): each bit removes one
 // class of instructions so that its share of the kernel's time -- issue slots and, under the
@@ -72,7 +72,7 @@ enum : int { KO_LDS_READS = 1, KO_LOADS = 2, KO_MFMA = 4, KO_STORES = 8 };
 template <class Op, int ScaleKind, int Epi = EPI_PLAIN, int KO = 0>
 __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmArgs g, RopeCacheArgs rc) {
     static_assert(ScaleKind != SCALE_BLOCK128, "block scales run on the ping-pong kernel");
-    static_assert(Epi == EPI_PLAIN || ScaleKind == SCALE_ROWCOL, "the SwiGLU and rotary epilogues are the int8 decoder's");
+    static_assert(Epi == EPI_PLAIN || ScaleKind == SCALE_ROWCOL, "the SwiGLU, rotary and residual epilogues are the int8 decoder's");
     PP_STAMP_INIT();
     using Cfg = Wave128Cfg;
     using Acc = typename Op::Acc;
@@ -516,7 +516,8 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
                 if (n < g.n) {
                     if constexpr (ScaleKind == SCALE_ROWCOL)
                         sw4[ni][q] = *reinterpret_cast<const f32x4*>(g.sb + n);
-                    if (bias) braw[ni][q] = *reinterpret_cast<const u32x2*>(bias + n);
+                    if constexpr (Epi != EPI_RESID)   // (no bias with the residual epilogue: registers)
+                        if (bias) braw[ni][q] = *reinterpret_cast<const u32x2*>(bias + n);
                 }
             }
         const int r4 = lane >> 4, c16 = lane & 15;
@@ -524,6 +525,18 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
         const uint32_t lane_off = (nst < g.n)
             ? (uint32_t)(wave_m * 128 + r4) * row_bytes + (uint32_t)nst * 2u
             : kOutOfRange;
+        // EPI_RESID: the residual rows of this tile, addressed like the output
+        [[maybe_unused]] const __amdgpu_buffer_rsrc_t rres = make_rsrc(
+            static_cast<const uint16_t*>(Epi == EPI_RESID ? g.resid : g.out) + (size_t)m0 * g.n,
+            (uint32_t)rows_here * row_bytes);
+        // the eight residual pieces of a pass live in a ring: each is requested again for the
+        // next pass as soon as it has been used, a whole pass ahead of its use
+        [[maybe_unused]] u32x4 rr[8];
+        if constexpr (Epi == EPI_RESID) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                rr[i] = buf_load16(rres, lane_off + (uint32_t)(i * 4) * row_bytes, 0);
+        }
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi) {
             uint8_t* const buf = mine + (mi & 1) * PASS_BYTES;
@@ -532,7 +545,7 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     const int nl = ni * 32 + q * 8 + lgrp * 4;
-                    const u32x2 raw = braw[ni][q];
+                    const u32x2 raw = Epi == EPI_RESID ? u32x2{0u, 0u} : braw[ni][q];
                     const f32x4 b4 = {__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u),
                                       __uint_as_float(raw.y << 16), __uint_as_float(raw.y & 0xffff0000u)};
                     float v[4];
@@ -554,7 +567,18 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmA
                 }
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const u32x4 v = *reinterpret_cast<const u32x4*>(buf + (i * 4 + r4) * ROWB + c16 * 16);
+                u32x4 v = *reinterpret_cast<const u32x4*>(buf + (i * 4 + r4) * ROWB + c16 * 16);
+                if constexpr (Epi == EPI_RESID) {
+                    // bf16(y + residual) on the rounded y, element by element
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t y2 = v[e], r2 = rr[i][e];
+                        v[e] = pack_bf16x2(__uint_as_float(y2 << 16) + __uint_as_float(r2 << 16),
+                                           __uint_as_float(y2 & 0xffff0000u) + __uint_as_float(r2 & 0xffff0000u));
+                    }
+                    if (mi + 1 < MI)
+                        rr[i] = buf_load16(rres, lane_off + (uint32_t)((mi + 1) * 32 + i * 4) * row_bytes, 0);
+                }
                 if constexpr (!(KO & KO_STORES))
                     __builtin_amdgcn_raw_buffer_store_b128(
                         v, rout, lane_off + (uint32_t)(mi * 32 + i * 4) * row_bytes, 0, 2);

@@ -183,7 +183,9 @@ bool launch_gemv_int8(const GemmArgs& g, hipStream_t stream) {
     if (g.m <= 0 || g.m > 128 || g.n <= 0 || g.k <= 0 || (g.k & 255) != 0) return false;
     const int64_t lim = (int64_t)1 << 31;
     if ((int64_t)g.n * g.k >= lim) return false;
-    if (g.m == 1)
+    // the residual epilogue is the row-range kernel's, on whole 8-byte pieces of bf16 rows
+    if (g.resid && ((g.n & 3) != 0 || g.out_kind != OUT_BF16)) return false;
+    if (g.m == 1 && !g.resid)
         launch_dot(g, stream);
     else
         launch_rows<false>(g, RopeCacheArgs{}, stream);

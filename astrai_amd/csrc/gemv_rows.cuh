@@ -70,6 +70,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_int8_rows_kernel(GemmArgs g, Rop
     // requested now so that their latency hides under the weight stream
     constexpr int TASKS = (RG * MB + NW - 1) / NW;
     float e_sx[TASKS], e_sw[TASKS][4], e_b[TASKS][4];
+    u32x2 e_res[TASKS];   // four bf16 of the residual row (g.resid given: N % 4 == 0, bf16 output)
 #pragma unroll
     for (int ti = 0; ti < TASKS; ++ti) {
         const int t = wave + ti * NW;
@@ -77,6 +78,9 @@ __global__ __launch_bounds__(NW * 64) void gemv_int8_rows_kernel(GemmArgs g, Rop
         const int en = r0 + (t / MB) * 16 + lgrp * 4;
         const bool live = t < RG * MB && g.out_kind != OUT_ACC;
         e_sx[ti] = (live && m < g.m) ? g.sa[m] : 0.0f;
+        e_res[ti] = (g.resid && live && m < g.m && en < r1)
+            ? *reinterpret_cast<const u32x2*>(static_cast<const uint16_t*>(g.resid) + (size_t)m * g.n + en)
+            : u32x2{0u, 0u};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const bool in = live && en + j < r1;
@@ -250,6 +254,13 @@ __global__ __launch_bounds__(NW * 64) void gemv_int8_rows_kernel(GemmArgs g, Rop
             u32x2 pk;
             pk.x = pack_bf16x2(v[0], v[1]);
             pk.y = pack_bf16x2(v[2], v[3]);
+            if (g.resid) {   // bf16(y + residual) on the rounded y
+                const u32x2 r = e_res[ti];
+                pk.x = pack_bf16x2(__uint_as_float(pk.x << 16) + __uint_as_float(r.x << 16),
+                                   __uint_as_float(pk.x & 0xffff0000u) + __uint_as_float(r.x & 0xffff0000u));
+                pk.y = pack_bf16x2(__uint_as_float(pk.y << 16) + __uint_as_float(r.y << 16),
+                                   __uint_as_float(pk.y & 0xffff0000u) + __uint_as_float(r.y & 0xffff0000u));
+            }
             *reinterpret_cast<u32x2*>(out + o) = pk;
         } else {
 #pragma unroll

@@ -37,6 +37,7 @@ struct GemmArgs {
     int m, n, k;
     int out_kind;
     float* row_max = nullptr;  // SwiGLU epilogue only: fp32 [M, N/128] partial row maxima of |h|
+    const void* resid = nullptr;  // residual epilogue only: bf16 [M,N]; out = bf16(bf16(y) + resid)
 };
 
 // quantize.hip
@@ -205,6 +206,13 @@ bool launch_gemm_int8_tiled(const GemmArgs& g, hipStream_t stream);
 // bf16(silu(gate))) [M, N/2], g.row_max[m, N/128] the maximum of |h| over each 64-column piece.
 // Large shapes only (those of the four-wave 256x256 kernel, N % 128 == 0, no bias); false otherwise.
 bool launch_gemm_int8_swiglu(const GemmArgs& g, hipStream_t stream);
+// a projection whose output is added to the residual stream in the epilogue:
+// g.out = bf16(bf16(dequantized product + bias) + g.resid), the bf16 arithmetic of `linear(x) + residual`.
+// Row-range kernel for up to 128 tokens (K % 256 == 0), four-wave 256x256 kernel for the large
+// shapes it takes; false otherwise (the caller runs the plain GEMM and an addition pass).
+bool launch_gemm_int8_resid(const GemmArgs& g, hipStream_t stream);
+// out = bf16(y + resid) over `total` bf16 elements; out may be y
+void launch_add_bf16(const void* y, const void* resid, void* out, int64_t total, hipStream_t stream);
 bool launch_gemm_fp8_tiled(const GemmArgs& g, int fmt, hipStream_t stream);
 // sa per activation row [M], sb per weight row [N], bf16 output
 bool launch_gemm_fp8_rowcol_tiled(const GemmArgs& g, int fmt, hipStream_t stream);

@@ -45,6 +45,7 @@ PROTOTYPES = {
     "astrai_w8a8_silu_mul_quantize_fp8_rows": ([_P, _P, _I64, _P, _P, _P, _P, _I64, _I64, _INT, _P], _INT),
     "astrai_w8a8_mfma_probe": ([_INT, _P, _P, _P, _P], _INT),
     "astrai_w8a8_gemm_int8_ptpc_swiglu": ([_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _INT),
+    "astrai_w8a8_gemm_int8_ptpc_resid": ([_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _P], _INT),
     "astrai_w8a8_quantize_int8_rows_pmax": ([_P, _P, _I64, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_silu_mul_quantize_int8_rows_blocked": ([_P, _I64, _I64, _P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_rope_cache_write_bf16": (
@@ -1063,6 +1064,50 @@ def mm_int8(a: torch.Tensor, b: torch.Tensor, sa: Optional[torch.Tensor],
             else:
                 _check(fn(a_c.data_ptr(), b_c.data_ptr(), _ptr(sa), _ptr(sb), _ptr(bias),
                           out.data_ptr(), m, n, k, out_dtype, _stream(a)), lib)
+    return out
+
+
+def mm_int8_resid(a: torch.Tensor, b: torch.Tensor, sa: torch.Tensor, sb: torch.Tensor,
+                  resid: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``mm_int8(a, b, sa, sb, bias) + resid`` in bf16 arithmetic, the addition done in the
+    GEMM's epilogue where the shape has one (``attn_output + x`` / ``mlp_output + x`` of
+    astrai/model/components/decoder_block.py:67,70). ``resid`` bf16 ``[M, N]``; returns a new
+    bf16 ``[M, N]`` tensor, bit for bit the two separate operations."""
+    lib = _require()
+    _gpu(a, "mm_int8_resid")
+    _gpu(b, "mm_int8_resid")
+    if a.dtype != torch.int8 or b.dtype != torch.int8:
+        raise RuntimeError("a and b must be int8")
+    if a.dim() != 2 or b.dim() != 2:
+        raise RuntimeError("a and b must be 2D")
+    if a.device != b.device:
+        raise RuntimeError("a and b must be on the same device")
+    if a.size(1) != b.size(1):
+        raise RuntimeError("inner dim mismatch")
+    a_c, b_c = a.contiguous(), b.contiguous()
+    m, k = a_c.shape
+    n = b_c.size(0)
+    sa = _check_vec(sa, a, m, "sa")
+    sb = _check_vec(sb, a, n, "sb")
+    if not (resid.is_cuda and resid.device == a.device and resid.dtype == torch.bfloat16
+            and resid.numel() == m * n):
+        raise RuntimeError("resid must be CUDA bf16 with M*N elements")
+    resid_c = resid.contiguous()
+    if bias is not None:
+        if not (bias.is_cuda and bias.device == a.device and bias.dtype == torch.bfloat16
+                and bias.numel() == n):
+            raise RuntimeError("bias must be CUDA bf16 with shape [N]")
+        bias = bias.contiguous()
+    with torch.cuda.device(a.device):
+        out = torch.empty((m, n), device=a.device, dtype=torch.bfloat16)
+        if m and n:
+            if k == 0:
+                out.copy_(resid_c.reshape(m, n) if bias is None
+                          else (bias.reshape(1, n).expand(m, n) + resid_c.reshape(m, n)))
+            else:
+                _check(lib.astrai_w8a8_gemm_int8_ptpc_resid(
+                    a_c.data_ptr(), b_c.data_ptr(), _ptr(sa), _ptr(sb), _ptr(bias), resid_c.data_ptr(),
+                    out.data_ptr(), m, n, k, _stream(a)), lib)
     return out
 
 

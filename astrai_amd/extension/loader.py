@@ -44,6 +44,7 @@ def _int8_mm_module() -> SimpleNamespace:
         add_rmsnorm_quantize_int8=_cabi.add_rmsnorm_quantize_int8,
         silu_mul_quantize_int8=_cabi.silu_mul_quantize_int8,
         mm_int8_swiglu=_cabi.mm_int8_swiglu,
+        mm_int8_resid=_cabi.mm_int8_resid,
         swiglu_block_rows=_cabi.swiglu_block_rows,
     )
 

@@ -106,6 +106,28 @@ def mm_int8(xq, wq, sx, sw, bias: Optional[torch.Tensor] = None) -> torch.Tensor
     return int8_gemm(xq, wq, sx, sw, bias)
 
 
+@custom_op("custom::int8_gemm_resid", mutates_args=())
+def int8_gemm_resid(xq: torch.Tensor, wq: torch.Tensor, sx: torch.Tensor, sw: torch.Tensor,
+                    resid: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``int8_gemm(xq, wq, sx, sw, bias) + resid`` in bf16 arithmetic: a projection whose
+    output joins the residual stream (astrai/model/components/decoder_block.py:67,70)."""
+    _no_cpu("custom::int8_gemm_resid")
+
+
+@int8_gemm_resid.register_fake
+def _int8_gemm_resid_fake(xq, wq, sx, sw, resid, bias=None):
+    return torch.empty((xq.shape[0], wq.shape[0]), device=xq.device, dtype=torch.bfloat16)
+
+
+@int8_gemm_resid.register_kernel("cuda")
+def _int8_gemm_resid_cuda(xq, wq, sx, sw, resid, bias=None):
+    return _mod().mm_int8_resid(xq, wq, sx, sw, resid, bias)
+
+
+def mm_int8_resid(xq, wq, sx, sw, resid, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    return int8_gemm_resid(xq, wq, sx, sw, resid, bias)
+
+
 def mm_int8_acc(xq: torch.Tensor, wq: torch.Tensor, kernel: str = "auto") -> torch.Tensor:
     """Raw int32 accumulator ``xq @ wq^T`` from the named kernel (auto / gemv / tiled)."""
     if xq.dtype != torch.int8 or wq.dtype != torch.int8:

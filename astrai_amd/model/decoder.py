@@ -245,23 +245,19 @@ class DecoderBlock(nn.Module):
 
     def forward(self, x, rotary_emb, kv_cache, positions, key_mask):
         if self.fused_int8 is not None and _fused_int8_active(x):
-            h, out = self._forward_fused_int8(x, None, rotary_emb, kv_cache, positions, key_mask)
-            return h + out
+            return self._forward_fused_int8(x, rotary_emb, kv_cache, positions, key_mask)
         x = self.attention(self.input_norm(x), rotary_emb, kv_cache, positions, key_mask) + x
         return self.mlp(self.post_attention_norm(x)) + x
 
-    def _forward_fused_int8(self, x, pending, rotary_emb, kv_cache, positions, key_mask):
-        """``x`` plus the not yet added residual branch ``pending`` (``None`` for the first
-        block) is the block input; returns ``(h, mlp_out)`` whose sum is the block output -- the
-        add is left to the next norm kernel, which also has to read both."""
+    def _forward_fused_int8(self, x, rotary_emb, kv_cache, positions, key_mask):
+        """The block on int8 projections with fused producers and epilogues: each norm is one
+        kernel with the per-token quantizer, and the output and down projections add the
+        residual stream in their epilogues (``attn_output + x``, ``mlp_output + x``)."""
         from astrai_amd.extension import _cabi
         from astrai_amd.extension.ops import int8 as I
         f, att = self.fused_int8, self.attention
         b, s, d = x.shape
-        xq, sx, xsum = I.rmsnorm_quantize_int8(x, self.input_norm.weight, self.input_norm.norm_eps,
-                                               res=pending)
-        if xsum is not None:
-            x = xsum
+        xq, sx, _ = I.rmsnorm_quantize_int8(x, self.input_norm.weight, self.input_norm.norm_eps)
         if kv_cache is None:
             qkv = I.mm_int8(xq, f.wqkv, sx, f.sqkv).reshape(b, s, -1)
             nq, nkv = att.n_heads * att.head_dim, att.n_kv_heads * att.head_dim
@@ -279,10 +275,9 @@ class DecoderBlock(nn.Module):
         else:
             qkv = I.mm_int8(xq, f.wqkv, sx, f.sqkv).reshape(b, s, -1)
             aq, sa = att.core_fused_qkv(qkv, rotary_emb, kv_cache, positions, key_mask)
-        o = I.mm_int8(aq, f.wo, sa, f.so).reshape(b, s, d)
-        # h = attention + x, then its norm, quantized: one kernel
-        hq, sh, h = I.rmsnorm_quantize_int8(o, self.post_attention_norm.weight,
-                                            self.post_attention_norm.norm_eps, res=x)
+        h = I.mm_int8_resid(aq, f.wo, sa, f.so, x.reshape(b * s, d)).reshape(b, s, d)   # attention + x
+        hq, sh, _ = I.rmsnorm_quantize_int8(h, self.post_attention_norm.weight,
+                                            self.post_attention_norm.norm_eps)
         if f.gu_blocked:
             # gate|up in 64-row blocks: a long block forms up * silu(gate) in the GEMM's epilogue
             mq, sm = I.mm_int8_swiglu(hq, f.wgu, sh, f.sgu)
@@ -290,7 +285,7 @@ class DecoderBlock(nn.Module):
             gu = I.mm_int8(hq, f.wgu, sh, f.sgu)             # [B*S, gate | up]
             w = f.wgu.size(0) // 2
             mq, sm = I.silu_mul_quantize_int8(gu[:, :w], gu[:, w:])
-        return h, I.mm_int8(mq, f.wdown, sm, f.sdown).reshape(b, s, d)
+        return I.mm_int8_resid(mq, f.wdown, sm, f.sdown, h.reshape(b * s, d)).reshape(b, s, d)   # mlp + h
 
 
 class AutoRegressiveLM(nn.Module):
@@ -334,11 +329,10 @@ class AutoRegressiveLM(nn.Module):
         if self.fused_int8 is not None and _fused_int8_active(x):
             from astrai_amd.extension import _cabi
             from astrai_amd.extension.ops import int8 as I
-            pending = None  # residual branch not yet added to x: the next norm kernel adds it
             for layer in self.layers:
-                x, pending = layer._forward_fused_int8(x, pending, rotary, kv_cache, positions, key_mask)
+                x = layer._forward_fused_int8(x, rotary, kv_cache, positions, key_mask)
             hq, sh, _, hidden = _cabi.add_rmsnorm_quantize_int8(x, self.norm.weight, self.norm.norm_eps,
-                                                                pending, True)
+                                                                None, True)
             logits = I.mm_int8(hq, self.fused_int8.wlm, sh, self.fused_int8.slm).reshape(b, s, -1)
             return {"logits": logits, "hidden_states": hidden}
         for layer in self.layers:

@@ -191,6 +191,19 @@ int astrai_w8a8_silu_mul_quantize_int8_rows_blocked(const void* gu_bf16, int64_t
                                                     int64_t rows, int64_t width, void* stream);
 
 /*
+ * A projection whose output joins the residual stream, `attn_output + x` and
+ * `mlp_output + x` of DecoderBlock.forward (astrai/model/components/decoder_block.py:67,70),
+ * as one kernel: out[m,n] = bf16(bf16(acc * sa[m] * sb[n] + bias[n]) + resid[m,n]), bit for
+ * bit gemm_int8_ptpc followed by the bf16 addition. resid bf16 [M,N], 16-byte aligned; out
+ * must not overlap it. The addition runs in the GEMM's epilogue for up to 128 tokens with
+ * K % 256 == 0 and N % 4 == 0 and for the shapes of the large-tile kernel; other shapes take
+ * the plain product and an addition pass.
+ */
+int astrai_w8a8_gemm_int8_ptpc_resid(const void* a, const void* b, const float* sa, const float* sb,
+                                     const void* bias_bf16, const void* resid_bf16, void* out_bf16,
+                                     int64_t m, int64_t n, int64_t k, void* stream);
+
+/*
  * Rotary embedding of q and k plus the KV-cache write of one decoder layer, one
  * pass over the (fused) q|k|v projection output. Replaces, between the
  * projections and the attention call of GQA.forward

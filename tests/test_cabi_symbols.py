@@ -49,6 +49,13 @@ def test_argument_validation_needs_no_gpu():
     assert rc == 1 and b"out_scale" in lib.astrai_w8a8_last_error()
     rc = lib.astrai_w8a8_gemm_fp8_pt(8, 16, 16, 16, None, None, 16, 4, 4, 64, 0, 0, None)
     assert rc == 1 and b"aligned" in lib.astrai_w8a8_last_error()
+    # the residual entry: residual required, aligned, and apart from the output
+    rc = lib.astrai_w8a8_gemm_int8_ptpc_resid(16, 16, 16, 16, None, None, 4096, 4, 4, 64, None)
+    assert rc == 1 and b"residual" in lib.astrai_w8a8_last_error()
+    rc = lib.astrai_w8a8_gemm_int8_ptpc_resid(16, 16, 16, 16, None, 4100, 8192, 4, 4, 64, None)
+    assert rc == 1 and b"aligned" in lib.astrai_w8a8_last_error()
+    rc = lib.astrai_w8a8_gemm_int8_ptpc_resid(16, 16, 16, 16, None, 4096, 4112, 4, 4, 64, None)
+    assert rc == 1 and b"overlaps" in lib.astrai_w8a8_last_error()
 
 
 def test_shape_predicates_agree_with_the_entry_points():

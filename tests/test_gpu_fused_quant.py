@@ -29,7 +29,11 @@ def _codes_close(got, want, s_got, s_want):
 
 
 @pytest.mark.parametrize("rows,k,with_res", [(32, 2048, True), (32, 2048, False), (1, 2048, True),
-                                             (5, 8, True), (3, 8192, False), (17, 5632, True)])
+                                             (5, 8, True), (3, 8192, False), (17, 5632, True),
+                                             # long blocks without a residual: one wave per row
+                                             (2048, 2048, False), (513, 4096, False), (1000, 264, False),
+                                             (4099, 512, False), (600, 1024, False), (700, 4104, False),
+                                             (2048, 2048, True)])
 def test_add_rmsnorm_quantize(C, rows, k, with_res):
     print(f"case rows={rows} k={k} res={with_res}", flush=True)
     g = torch.Generator().manual_seed(rows * 131 + k)
@@ -203,3 +207,61 @@ def test_silu_mul_quantize_fp8(C, rows, width, fused_buffer, fmt):
     if width <= 8192:
         _, _, hi = C.silu_mul_quantize_int8(gate, up, want_h=True)
         assert torch.equal(h.view(torch.int16), hi.view(torch.int16))
+
+
+# ---- projections whose output joins the residual stream -----------------------------------------
+
+@pytest.mark.parametrize("m,n,k,bias", [
+    (32, 2048, 2048, False),     # config-4 output projection at a decode step (row-range kernel)
+    (32, 2048, 5632, False),     # config-4 down projection
+    (1, 2048, 2048, False), (2, 44, 256, True), (17, 3072, 512, True), (64, 2048, 2048, False),
+    (100, 1028, 256, False), (128, 2048, 2048, True),
+    (16384, 2048, 2048, False),  # config-4 output projection at prefill (large-tile kernel, 64 x 8 tiles)
+    (4096, 2048, 5632, False),   # down projection, 16 x 8 tiles = 128 < 192: plain GEMM + addition pass
+    (12500, 4096, 256, True),    # large-tile kernel, ragged rows, bias
+    (200, 100, 48, True), (3, 7, 16, False), (129, 2050, 256, False),   # shapes without a fused epilogue
+])
+def test_mm_int8_resid_bit_equal(C, m, n, k, bias):
+    """``mm_int8`` + residual in one entry point against the GEMM followed by the bf16 addition
+    (what ``attn_output + x`` computes on bf16 tensors): bit for bit, every route; the GEMM
+    itself is checked against the oracle on sampled rows."""
+    print(f"case m={m} n={n} k={k} bias={bias}", flush=True)
+    g = torch.Generator().manual_seed(m * 7 + n * 3 + k)
+    a = torch.randint(-127, 128, (m, k), generator=g, dtype=torch.int8).to(DEV)
+    w = torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int8).to(DEV)
+    sa = (torch.rand(m, generator=g) * 0.01 + 0.005).to(DEV)
+    sw = (torch.rand(n, generator=g) * 0.002 + 0.0005).to(DEV)
+    b = torch.randn(n, generator=g).bfloat16().to(DEV) if bias else None
+    # residual of the product's own magnitude, so that the sum's rounding matters
+    r = (torch.randn(m, n, generator=g) * (0.3 * k ** 0.5)).bfloat16().to(DEV)
+    y = C.mm_int8(a, w, sa, sw, b)
+    want = y + r
+    got = C.mm_int8_resid(a, w, sa, sw, r, b)
+    assert got.data_ptr() != r.data_ptr()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    rows = torch.arange(0, m, max(1, m // 32))
+    oy = O.int8_gemm(a[rows].cpu(), w.cpu(), sa[rows].cpu(), sw.cpu(), None if b is None else b.cpu())
+    assert_bf16_close(got[rows], (oy.float() + r[rows].cpu().float()).bfloat16(), what="product + residual")
+
+
+def test_mm_int8_resid_rejects(C):
+    a = torch.zeros(8, 256, dtype=torch.int8, device=DEV)
+    w = torch.zeros(16, 256, dtype=torch.int8, device=DEV)
+    sa, sw = torch.ones(8, device=DEV), torch.ones(16, device=DEV)
+    with pytest.raises(RuntimeError, match="resid"):
+        C.mm_int8_resid(a, w, sa, sw, torch.zeros(8, 15, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(RuntimeError, match="resid"):
+        C.mm_int8_resid(a, w, sa, sw, torch.zeros(8, 16, dtype=torch.float32, device=DEV))
+    # through the C entry point: the output may not overlap the residual
+    lib = C.load()
+    r = torch.zeros(8, 16, dtype=torch.bfloat16, device=DEV)
+    rc = lib.astrai_w8a8_gemm_int8_ptpc_resid(a.data_ptr(), w.data_ptr(), sa.data_ptr(), sw.data_ptr(), None,
+                                              r.data_ptr(), r.data_ptr(), 8, 16, 256, None)
+    assert rc != 0 and b"overlaps" in lib.astrai_w8a8_last_error()
+    rc = lib.astrai_w8a8_gemm_int8_ptpc_resid(a.data_ptr(), w.data_ptr(), sa.data_ptr(), sw.data_ptr(), None,
+                                              None, r.data_ptr(), 8, 16, 256, None)
+    assert rc != 0 and b"residual" in lib.astrai_w8a8_last_error()
+    # k == 0: the product is empty, the residual passes through
+    r = torch.randn(8, 16, device=DEV).bfloat16()
+    out = C.mm_int8_resid(a[:, :0], w[:, :0], sa, sw, r)
+    assert torch.equal(out, r)

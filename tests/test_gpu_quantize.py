@@ -107,7 +107,10 @@ def test_fp8_quantize_transposed_codes(C, shape, fmt):
     assert torch.equal(_codes(only_t), _codes(x8t))
 
 
-@pytest.mark.parametrize("rows,k", [(1, 8), (3, 24), (16, 2048), (5, 33), (2, 9000), (7, 16384), (64, 4096), (0, 32)])
+@pytest.mark.parametrize("rows,k", [(1, 8), (3, 24), (16, 2048), (5, 33), (2, 9000), (7, 16384), (64, 4096), (0, 32),
+                                    # long blocks: one wave per row up to K = 4096
+                                    (16384, 2048), (513, 4096), (1000, 264), (4099, 8), (600, 1032), (700, 4104),
+                                    (512, 36)])
 def test_int8_rows_bit_exact(C, rows, k):
     print(f"case rows={rows} k={k}", flush=True)
     g = torch.Generator().manual_seed(rows * 31 + k)
