@@ -216,6 +216,7 @@ def test_silu_mul_quantize_fp8(C, rows, width, fused_buffer, fmt):
     (32, 2048, 5632, False),     # config-4 down projection
     (1, 2048, 2048, False), (2, 44, 256, True), (17, 3072, 512, True), (64, 2048, 2048, False),
     (100, 1028, 256, False), (128, 2048, 2048, True),
+    (48, 11008, 256, True), (64, 8192, 512, False),   # 33..64 tokens on long row ranges
     (16384, 2048, 2048, False),  # config-4 output projection at prefill (large-tile kernel, 64 x 8 tiles)
     (4096, 2048, 5632, False),   # down projection, 16 x 8 tiles = 128 < 192: plain GEMM + addition pass
     (12500, 4096, 256, True),    # large-tile kernel, ragged rows, bias

@@ -73,7 +73,9 @@ def test_golden_integer_cases_including_worst_case_magnitude(C, golden):
 
 @pytest.mark.parametrize("kernel", ["tiled", "gemv"])
 @pytest.mark.parametrize("m", [1, 2, 4, 16, 17, 33, 64, 65, 100, 128])
-@pytest.mark.parametrize("n,k", [(11008, 4096), (1000, 512), (40, 256), (3072, 2048), (2048, 5632), (200, 11008)])
+@pytest.mark.parametrize("n,k", [(11008, 4096), (1000, 512), (40, 256), (3072, 2048), (2048, 5632), (200, 11008),
+                                 # row ranges of 17..32 and 33..48 rows, ragged N
+                                 (8192, 512), (5000, 256), (10001, 768)])
 def test_skinny_shapes_both_kernels_bit_exact(C, kernel, m, n, k):
     """Decode shapes through the wave-split skinny kernel and through the tiled
     kernel: the split-K integer sums must equal the single-pass ones."""
@@ -85,7 +87,8 @@ def test_skinny_shapes_both_kernels_bit_exact(C, kernel, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(2, 11008, 4096), (32, 3072, 2048), (48, 11264, 2048), (128, 2048, 5632),
-                                   (5, 1001, 768)])
+                                   (5, 1001, 768), (64, 11008, 4096), (64, 8192, 512), (40, 10001, 768),
+                                   (33, 5000, 256)])
 def test_skinny_bf16_epilogue_bit_exact(C, m, n, k):
     """The skinny kernel's dequant epilogue (scales, bias, one rounding; ragged N
     takes the scalar stores) against the oracle's elementwise fp32 formula."""
