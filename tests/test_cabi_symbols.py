@@ -112,3 +112,13 @@ def test_fuse_int8_weights_refuses_widths_the_fused_producers_reject():
                                  num_key_value_heads=1, intermediate_size=8200, max_position_embeddings=8)
     with pytest.raises(ValueError, match="intermediate_size 8200"):
         fuse_int8_weights(AutoRegressiveLM(cfg).to(torch.bfloat16))
+
+
+def test_decode_attention_split_plan():
+    """A few hundred workgroups, at most eight splits, none shorter than ~192 keys of the longest context."""
+    assert _cabi.decode_nsplit(128, 640) == 3      # config 4: 32 sequences x 4 KV heads, 512 + 128 tokens
+    assert _cabi.decode_nsplit(8, 640) == 3
+    assert _cabi.decode_nsplit(8, 2048) == 8
+    assert _cabi.decode_nsplit(256, 4096) == 1
+    assert _cabi.decode_nsplit(1, 64) == 1
+    assert _cabi.decode_nsplit(0, 0) == 1
