@@ -1032,14 +1032,11 @@ _INT8_ENTRY = {
 }
 
 
-def mm_int8(a: torch.Tensor, b: torch.Tensor, sa: Optional[torch.Tensor],
-            sb: Optional[torch.Tensor], bias: Optional[torch.Tensor] = None,
-            out_dtype: int = 0, kernel: str = "auto") -> torch.Tensor:
-    """int8 NT GEMM. ``out_dtype`` 0: ``bf16(acc*sa[m]*sb[n] (+bias))``; 2: raw int32
-    accumulator. ``kernel`` names the entry point: auto / gemv / tiled."""
-    lib = _require()
-    _gpu(a, "mm_int8")
-    _gpu(b, "mm_int8")
+def _int8_operands(a, b, sa, sb, bias, need_scales: bool, what: str):
+    """The checks every int8 NT GEMM wrapper makes on its operands; returns contiguous operands,
+    checked scale vectors and bias, and ``(m, n, k)``."""
+    _gpu(a, what)
+    _gpu(b, what)
     if a.dtype != torch.int8 or b.dtype != torch.int8:
         raise RuntimeError("a and b must be int8")
     if a.dim() != 2 or b.dim() != 2:
@@ -1048,12 +1045,10 @@ def mm_int8(a: torch.Tensor, b: torch.Tensor, sa: Optional[torch.Tensor],
         raise RuntimeError("a and b must be on the same device")
     if a.size(1) != b.size(1):
         raise RuntimeError("inner dim mismatch")
-    if out_dtype not in (OUT_BF16, OUT_ACC):
-        raise RuntimeError("out_dtype must be 0 (bf16) or 2 (int32 accumulator)")
     a_c, b_c = a.contiguous(), b.contiguous()
     m, k = a_c.shape
     n = b_c.size(0)
-    if out_dtype == OUT_BF16:
+    if need_scales:
         if sa is None or sb is None:
             raise RuntimeError("bf16 output requires sa and sb")
         sa = _check_vec(sa, a, m, "sa")
@@ -1063,6 +1058,18 @@ def mm_int8(a: torch.Tensor, b: torch.Tensor, sa: Optional[torch.Tensor],
                 and bias.numel() == n):
             raise RuntimeError("bias must be CUDA bf16 with shape [N]")
         bias = bias.contiguous()
+    return a_c, b_c, sa, sb, bias, m, n, k
+
+
+def mm_int8(a: torch.Tensor, b: torch.Tensor, sa: Optional[torch.Tensor],
+            sb: Optional[torch.Tensor], bias: Optional[torch.Tensor] = None,
+            out_dtype: int = 0, kernel: str = "auto") -> torch.Tensor:
+    """int8 NT GEMM. ``out_dtype`` 0: ``bf16(acc*sa[m]*sb[n] (+bias))``; 2: raw int32
+    accumulator. ``kernel`` names the entry point: auto / gemv / tiled."""
+    lib = _require()
+    if out_dtype not in (OUT_BF16, OUT_ACC):
+        raise RuntimeError("out_dtype must be 0 (bf16) or 2 (int32 accumulator)")
+    a_c, b_c, sa, sb, bias, m, n, k = _int8_operands(a, b, sa, sb, bias, out_dtype == OUT_BF16, "mm_int8")
     fn = getattr(lib, _INT8_ENTRY[kernel])
     with torch.cuda.device(a.device):
         out = torch.empty((m, n), device=a.device,
@@ -1083,30 +1090,11 @@ def mm_int8_resid(a: torch.Tensor, b: torch.Tensor, sa: torch.Tensor, sb: torch.
     astrai/model/components/decoder_block.py:67,70). ``resid`` bf16 ``[M, N]``; returns a new
     bf16 ``[M, N]`` tensor, bit for bit the two separate operations."""
     lib = _require()
-    _gpu(a, "mm_int8_resid")
-    _gpu(b, "mm_int8_resid")
-    if a.dtype != torch.int8 or b.dtype != torch.int8:
-        raise RuntimeError("a and b must be int8")
-    if a.dim() != 2 or b.dim() != 2:
-        raise RuntimeError("a and b must be 2D")
-    if a.device != b.device:
-        raise RuntimeError("a and b must be on the same device")
-    if a.size(1) != b.size(1):
-        raise RuntimeError("inner dim mismatch")
-    a_c, b_c = a.contiguous(), b.contiguous()
-    m, k = a_c.shape
-    n = b_c.size(0)
-    sa = _check_vec(sa, a, m, "sa")
-    sb = _check_vec(sb, a, n, "sb")
+    a_c, b_c, sa, sb, bias, m, n, k = _int8_operands(a, b, sa, sb, bias, True, "mm_int8_resid")
     if not (resid.is_cuda and resid.device == a.device and resid.dtype == torch.bfloat16
             and resid.numel() == m * n):
         raise RuntimeError("resid must be CUDA bf16 with M*N elements")
     resid_c = resid.contiguous()
-    if bias is not None:
-        if not (bias.is_cuda and bias.device == a.device and bias.dtype == torch.bfloat16
-                and bias.numel() == n):
-            raise RuntimeError("bias must be CUDA bf16 with shape [N]")
-        bias = bias.contiguous()
     with torch.cuda.device(a.device):
         out = torch.empty((m, n), device=a.device, dtype=torch.bfloat16)
         if m and n:

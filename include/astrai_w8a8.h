@@ -501,8 +501,8 @@ int astrai_w8a8_gemm_fp8_block128(const void* a8, const void* b8, const float* s
  *   acc[m,n] = sum_k a[m,k] * b[n,k]              exact int32
  *   OUT_BF16: out = bf16(float(acc) * sa[m] * sb[n] + bias[n])
  *   OUT_ACC : out = acc as int32 (bit-exact parity surface)
- * Picks the skinny kernel for M <= 128 when the shape allows it, the tiled MFMA
- * kernel otherwise.
+ * Picks a decode kernel for M <= 128 when K % 256 == 0 (one token: a dot-product kernel;
+ * 2..128 tokens: the row-range MFMA kernel), the tiled MFMA kernels otherwise.
  */
 int astrai_w8a8_gemm_int8_ptpc(const void* a, const void* b, const float* sa,
                                const float* sb, const void* bias_bf16, void* out,
@@ -510,7 +510,7 @@ int astrai_w8a8_gemm_int8_ptpc(const void* a, const void* b, const float* sa,
                                void* stream);
 
 /*
- * The skinny (decode) int8 kernel on its own: same contract as
+ * The decode int8 kernels on their own: same contract as
  * astrai_w8a8_gemm_int8_ptpc but requires M <= 128 and K % 256 == 0, and
  * returns ASTRAI_W8A8_UNSUPPORTED otherwise.
  */
@@ -543,7 +543,7 @@ int astrai_w8a8_gemm_int8_ptpc_rope_cache(const void* a, const void* b, const fl
                                           void* stream);
 
 /*
- * The tiled MFMA int8 kernel on its own (no skinny dispatch), for tests and
+ * The tiled MFMA int8 kernels on their own (no decode-kernel dispatch), for tests and
  * benchmarks that must name the kernel they measure.
  */
 int astrai_w8a8_gemm_int8_ptpc_tiled(const void* a, const void* b, const float* sa,

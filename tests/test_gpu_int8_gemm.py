@@ -38,7 +38,7 @@ def test_int32_accumulator_bit_exact(C, m, n, k):
 
 def test_random_shape_sweep_default_dispatch_bit_exact(C):
     """Sixty seeded random shapes through the default entry point, whichever kernel
-    it picks (single-token, skinny, tiled, generic): accumulators bit-exact, and the
+    it picks (single-token, row-range, tiled, generic): accumulators bit-exact, and the
     scaled bf16 output bit-equal to the oracle's elementwise epilogue."""
     g = torch.Generator().manual_seed(20240)
     for i in range(60):
@@ -46,7 +46,7 @@ def test_random_shape_sweep_default_dispatch_bit_exact(C):
         n = int(torch.randint(1, 701, (1,), generator=g))
         k = int(torch.randint(1, 1201, (1,), generator=g))
         if i % 3 == 0:
-            k = (k + 255) // 256 * 256   # the skinny kernels need K % 256 == 0
+            k = (k + 255) // 256 * 256   # the decode kernels need K % 256 == 0
         if i % 4 == 0:
             m = 1 + i % 40
         print(f"case {i}: m={m} n={n} k={k}", flush=True)
@@ -77,7 +77,7 @@ def test_golden_integer_cases_including_worst_case_magnitude(C, golden):
                                  # row ranges of 17..32 and 33..48 rows, ragged N
                                  (8192, 512), (5000, 256), (10001, 768)])
 def test_skinny_shapes_both_kernels_bit_exact(C, kernel, m, n, k):
-    """Decode shapes through the wave-split skinny kernel and through the tiled
+    """Decode shapes through the wave-split row-range kernel and through the tiled
     kernel: the split-K integer sums must equal the single-pass ones."""
     print(f"case kernel={kernel} m={m} n={n} k={k}", flush=True)
     g = torch.Generator().manual_seed(m + n + k)
@@ -90,7 +90,7 @@ def test_skinny_shapes_both_kernels_bit_exact(C, kernel, m, n, k):
                                    (5, 1001, 768), (64, 11008, 4096), (64, 8192, 512), (40, 10001, 768),
                                    (33, 5000, 256)])
 def test_skinny_bf16_epilogue_bit_exact(C, m, n, k):
-    """The skinny kernel's dequant epilogue (scales, bias, one rounding; ragged N
+    """The row-range kernel's dequant epilogue (scales, bias, one rounding; ragged N
     takes the scalar stores) against the oracle's elementwise fp32 formula."""
     print(f"case m={m} n={n} k={k}", flush=True)
     g = torch.Generator().manual_seed(m * 7 + n + k)
