@@ -59,6 +59,10 @@ def test_random_shape_sweep_default_dispatch_bit_exact(C):
         out = C.mm_int8(a.to(DEV), b.to(DEV), sa.to(DEV), sb.to(DEV), None, 0).cpu()
         ref = (want.float() * sa[:, None] * sb[None, :]).to(torch.bfloat16)
         assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), (m, n, k)
+        # the same product joined to a residual stream in the epilogue (or by the addition pass)
+        r = (torch.randn(m, n, generator=g) * float(ref.float().abs().mean() + 1e-3)).to(torch.bfloat16)
+        fused = C.mm_int8_resid(a.to(DEV), b.to(DEV), sa.to(DEV), sb.to(DEV), r.to(DEV)).cpu()
+        assert torch.equal(fused.view(torch.int16), (ref + r).view(torch.int16)), (m, n, k)
 
 
 def test_golden_integer_cases_including_worst_case_magnitude(C, golden):
