@@ -144,14 +144,14 @@ class GQA(nn.Module):
         self.o_proj = Linear(dim, dim, init_std=0.02 / (2 * n_layers) ** 0.5)
 
     def forward(self, x: Tensor, rotary_emb: Tensor, kv_cache: Optional[DenseKVCache],
-                positions: Optional[Tensor], key_mask: Optional[Tensor]) -> Tensor:
+                positions: Optional[Tensor], key_mask: Optional["_KeyMask"]) -> Tensor:
         out = self.core(self.q_proj(x), self.k_proj(x), self.v_proj(x), rotary_emb, kv_cache,
                         positions, key_mask)
         return self.o_proj(out)
 
     def core(self, q: Tensor, k: Tensor, v: Tensor, rotary_emb: Tensor,
              kv_cache: Optional[DenseKVCache], positions: Optional[Tensor],
-             key_mask: Optional[Tensor]) -> Tensor:
+             key_mask: Optional["_KeyMask"]) -> Tensor:
         """Everything between the q/k/v projections and ``o_proj``: ``[B, S, *]`` in,
         ``[B, S, dim]`` out."""
         b, s = q.shape[0], q.shape[1]
@@ -174,17 +174,17 @@ class GQA(nn.Module):
             out = self._attend_cache(q, kv_cache, key_mask)
         return out.permute(0, 2, 1, 3).reshape(b, s, self.dim)
 
-    def _attend_cache(self, q: Tensor, kv_cache: DenseKVCache, key_mask: Tensor) -> Tensor:
-        """``q [B, H, S, D]`` against the layer's cache; ``key_mask`` is ``[1, 1, n_rep*S, max_len]``
-        (the block's mask repeated once per query head of a KV group)."""
+    def _attend_cache(self, q: Tensor, kv_cache: DenseKVCache, key_mask: "_KeyMask") -> Tensor:
+        """``q [B, H, S, D]`` against the layer's cache under the block's mask (``key_mask.get()``:
+        ``[1, 1, n_rep*S, max_len]``, one copy per query head of a KV group)."""
         b, _, s, _ = q.shape
         qf = q.reshape(b, self.n_kv_heads, self.n_rep * s, self.head_dim)
         out = F.scaled_dot_product_attention(qf, kv_cache.k[self.layer_id],
-                                             kv_cache.v[self.layer_id], attn_mask=key_mask)
+                                             kv_cache.v[self.layer_id], attn_mask=key_mask.get())
         return out.reshape(b, self.n_heads, s, self.head_dim)
 
     def core_fused_qkv(self, qkv: Tensor, rotary_emb: Tensor, kv_cache: DenseKVCache,
-                       positions: Tensor, key_mask: Tensor):
+                       positions: Tensor, key_mask: "_KeyMask"):
         """Same as :meth:`core` for a fused ``q|k|v`` projection ``[B, S, (H + 2 H_kv) D]`` with a
         cache: rotation, permutes and the cache write are one kernel. Returns the attention
         output already quantized per token, ``(int8 [B*S, dim], fp32 [B*S, 1])``: for a few new
@@ -198,7 +198,7 @@ class GQA(nn.Module):
                                    self.head_dim)
         return self.attend_rotated(q, kv_cache, positions, key_mask)
 
-    def attend_rotated(self, q: Tensor, kv_cache: DenseKVCache, positions: Tensor, key_mask: Tensor):
+    def attend_rotated(self, q: Tensor, kv_cache: DenseKVCache, positions: Tensor, key_mask: "_KeyMask"):
         """The attention of :meth:`core_fused_qkv` for an already rotated ``q [B, H, S, D]``
         whose keys and values are in the cache."""
         from astrai_amd.extension import _cabi
@@ -217,6 +217,25 @@ class GQA(nn.Module):
                 _cabi.attn_cache_rows(q, kv_cache.k[self.layer_id], kv_cache.v[self.layer_id], positions))
         out = self._attend_cache(q, kv_cache, key_mask)
         return I.quantize_int8_per_token(out.permute(0, 2, 1, 3).reshape(b, s, self.dim))
+
+
+class _KeyMask:
+    """The mask of a block of new tokens against the cache, ``key position <= token position``,
+    built on first use and shared by the layers of one forward: the HIP attention kernels take
+    ``positions`` themselves, so a model on those never builds it (three small launches a step)."""
+
+    def __init__(self, positions: Tensor, max_len: int, n_rep: int):
+        self.positions, self.max_len, self.n_rep = positions, max_len, n_rep
+        self._mask: Optional[Tensor] = None
+
+    def get(self) -> Tensor:
+        if self._mask is None:
+            key_pos = torch.arange(self.max_len, device=self.positions.device)
+            mask = (key_pos[None, :] <= self.positions[:, None])[None, None]  # [1,1,seq,max_len]
+            if self.n_rep > 1:  # one copy per query head of a KV group, made once for all layers
+                mask = mask.repeat(1, 1, self.n_rep, 1)
+            self._mask = mask
+        return self._mask
 
 
 class MLP(nn.Module):
@@ -321,11 +340,8 @@ class AutoRegressiveLM(nn.Module):
         rotary = self.freqs_cis.index_select(0, positions).unsqueeze(0).float()
         key_mask = None
         if kv_cache is not None:
-            key_pos = torch.arange(kv_cache.max_len, device=input_ids.device)
-            key_mask = (key_pos[None, :] <= positions[:, None])[None, None]  # [1,1,seq,max_len]
-            n_rep = self.config.num_attention_heads // self.config.num_key_value_heads
-            if n_rep > 1:  # one copy per query head of a KV group, made once for all layers
-                key_mask = key_mask.repeat(1, 1, n_rep, 1)
+            key_mask = _KeyMask(positions, kv_cache.max_len,
+                                self.config.num_attention_heads // self.config.num_key_value_heads)
         if self.fused_int8 is not None and _fused_int8_active(x):
             from astrai_amd.extension import _cabi
             from astrai_amd.extension.ops import int8 as I
