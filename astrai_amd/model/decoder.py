@@ -202,21 +202,20 @@ class GQA(nn.Module):
         """The attention of :meth:`core_fused_qkv` for an already rotated ``q [B, H, S, D]``
         whose keys and values are in the cache."""
         from astrai_amd.extension import _cabi
-        from astrai_amd.extension.ops import int8 as I
         b, _, s, _ = q.shape
         if _cabi.attn_decode_supported(self.n_heads, self.n_kv_heads, s, self.head_dim):
             return _cabi.attn_decode(q, kv_cache.k[self.layer_id], kv_cache.v[self.layer_id], positions,
                                      quantized=True)
         if _cabi.attn_prefill_supported(self.n_heads, self.n_kv_heads, self.head_dim):
             # causal block kernel: no mask tensor, no head expansion, token-major output
-            return I.quantize_int8_per_token(
+            return _cabi.quantize_int8_rows(
                 _cabi.attn_prefill(q, kv_cache.k[self.layer_id], kv_cache.v[self.layer_id], positions))
         if _cabi.attn_cache_rows_supported(self.n_heads, self.n_kv_heads, self.head_dim):
             # other head shapes: the general kernel over the same cache, addressed per KV head
-            return I.quantize_int8_per_token(
+            return _cabi.quantize_int8_rows(
                 _cabi.attn_cache_rows(q, kv_cache.k[self.layer_id], kv_cache.v[self.layer_id], positions))
         out = self._attend_cache(q, kv_cache, key_mask)
-        return I.quantize_int8_per_token(out.permute(0, 2, 1, 3).reshape(b, s, self.dim))
+        return _cabi.quantize_int8_rows(out.permute(0, 2, 1, 3).reshape(b, s, self.dim))
 
 
 class _KeyMask:
@@ -272,15 +271,16 @@ class DecoderBlock(nn.Module):
         """The block on int8 projections with fused producers and epilogues: each norm is one
         kernel with the per-token quantizer, and the output and down projections add the
         residual stream in their epilogues (``attn_output + x``, ``mlp_output + x``)."""
+        # (the C-ABI wrappers directly: a dispatcher round trip per call is what an eager decode step,
+        # ~220 launches of a few microseconds each, would otherwise spend most of its time in)
         from astrai_amd.extension import _cabi
-        from astrai_amd.extension.ops import int8 as I
         f, att = self.fused_int8, self.attention
         b, s, d = x.shape
-        xq, sx, _ = I.rmsnorm_quantize_int8(x, self.input_norm.weight, self.input_norm.norm_eps)
+        xq, sx, _, _ = _cabi.add_rmsnorm_quantize_int8(x, self.input_norm.weight, self.input_norm.norm_eps)
         if kv_cache is None:
-            qkv = I.mm_int8(xq, f.wqkv, sx, f.sqkv).reshape(b, s, -1)
+            qkv = _cabi.mm_int8(xq, f.wqkv, sx, f.sqkv).reshape(b, s, -1)
             nq, nkv = att.n_heads * att.head_dim, att.n_kv_heads * att.head_dim
-            aq, sa = I.quantize_int8_per_token(
+            aq, sa = _cabi.quantize_int8_rows(
                 att.core(qkv[..., :nq], qkv[..., nq:nq + nkv], qkv[..., nq + nkv:], rotary_emb, None,
                          positions, key_mask))
         elif _cabi.mm_int8_rope_cache_supported(b * s, d, att.head_dim, f.wqkv.size(0), b, att.n_heads,
@@ -292,19 +292,19 @@ class DecoderBlock(nn.Module):
                                          b, s, att.n_heads, att.n_kv_heads, att.head_dim)
             aq, sa = att.attend_rotated(q, kv_cache, positions, key_mask)
         else:
-            qkv = I.mm_int8(xq, f.wqkv, sx, f.sqkv).reshape(b, s, -1)
+            qkv = _cabi.mm_int8(xq, f.wqkv, sx, f.sqkv).reshape(b, s, -1)
             aq, sa = att.core_fused_qkv(qkv, rotary_emb, kv_cache, positions, key_mask)
-        h = I.mm_int8_resid(aq, f.wo, sa, f.so, x.reshape(b * s, d)).reshape(b, s, d)   # attention + x
-        hq, sh, _ = I.rmsnorm_quantize_int8(h, self.post_attention_norm.weight,
-                                            self.post_attention_norm.norm_eps)
+        h = _cabi.mm_int8_resid(aq, f.wo, sa, f.so, x.reshape(b * s, d)).reshape(b, s, d)   # attention + x
+        hq, sh, _, _ = _cabi.add_rmsnorm_quantize_int8(h, self.post_attention_norm.weight,
+                                                       self.post_attention_norm.norm_eps)
         if f.gu_blocked:
             # gate|up in 64-row blocks: a long block forms up * silu(gate) in the GEMM's epilogue
-            mq, sm = I.mm_int8_swiglu(hq, f.wgu, sh, f.sgu)
+            mq, sm, _ = _cabi.mm_int8_swiglu(hq, f.wgu, sh, f.sgu)
         else:
-            gu = I.mm_int8(hq, f.wgu, sh, f.sgu)             # [B*S, gate | up]
+            gu = _cabi.mm_int8(hq, f.wgu, sh, f.sgu)             # [B*S, gate | up]
             w = f.wgu.size(0) // 2
-            mq, sm = I.silu_mul_quantize_int8(gu[:, :w], gu[:, w:])
-        return I.mm_int8_resid(mq, f.wdown, sm, f.sdown, h.reshape(b * s, d)).reshape(b, s, d)   # mlp + h
+            mq, sm, _ = _cabi.silu_mul_quantize_int8(gu[:, :w], gu[:, w:])
+        return _cabi.mm_int8_resid(mq, f.wdown, sm, f.sdown, h.reshape(b * s, d)).reshape(b, s, d)   # mlp + h
 
 
 class AutoRegressiveLM(nn.Module):
@@ -344,12 +344,11 @@ class AutoRegressiveLM(nn.Module):
                                 self.config.num_attention_heads // self.config.num_key_value_heads)
         if self.fused_int8 is not None and _fused_int8_active(x):
             from astrai_amd.extension import _cabi
-            from astrai_amd.extension.ops import int8 as I
             for layer in self.layers:
                 x = layer._forward_fused_int8(x, rotary, kv_cache, positions, key_mask)
             hq, sh, _, hidden = _cabi.add_rmsnorm_quantize_int8(x, self.norm.weight, self.norm.norm_eps,
                                                                 None, True)
-            logits = I.mm_int8(hq, self.fused_int8.wlm, sh, self.fused_int8.slm).reshape(b, s, -1)
+            logits = _cabi.mm_int8(hq, self.fused_int8.wlm, sh, self.fused_int8.slm).reshape(b, s, -1)
             return {"logits": logits, "hidden_states": hidden}
         for layer in self.layers:
             x = layer(x, rotary, kv_cache, positions, key_mask)
