@@ -137,8 +137,35 @@ def _check(rc: int, lib: ctypes.CDLL) -> None:
         raise RuntimeError(f"astrai_w8a8 error {rc}: {msg}")
 
 
+try:  # the raw handle of the current stream without building a Stream object (a microsecond per call saved)
+    from torch._C import _cuda_getCurrentRawStream as _raw_stream
+except ImportError:  # pragma: no cover
+    _raw_stream = None
+
+
 def _stream(t: torch.Tensor) -> int:
+    if _raw_stream is not None:
+        return _raw_stream(t.device.index if t.device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on_device(dev: torch.device):
+    """``torch.cuda.device(dev)``, or nothing when ``dev`` is the current device already (every
+    call of a single-GPU process): the guard object costs more than a launch on the decode path."""
+    if dev.index is None or dev.index == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(dev)
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
@@ -181,7 +208,7 @@ def quantize_bf16(x: torch.Tensor, scale: torch.Tensor, fmt: int):
         raise RuntimeError("x must be bf16")
     _check_scale(scale, x, "scale")
     x_c = x.contiguous()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         x8 = torch.empty_like(x_c, dtype=torch.float8_e5m2 if fmt else torch.float8_e4m3fn)
         amax = torch.zeros(1, device=x.device, dtype=torch.float32)
         if x_c.numel():
@@ -234,7 +261,7 @@ def mm_fp8(a: torch.Tensor, b: torch.Tensor, sa: torch.Tensor, sb: torch.Tensor,
                 and bias.numel() == n):
             raise RuntimeError("bias must be CUDA bf16 with shape [N]")
         bias = bias.contiguous()
-    with torch.cuda.device(a.device):
+    with _on_device(a.device):
         out = torch.empty((m, n), device=a.device,
                           dtype=torch.float8_e4m3fn if out_dtype else torch.bfloat16)
         if m and n:
@@ -262,7 +289,7 @@ def mm_fp8_acc(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     a_c, b_c = a.contiguous(), b.contiguous()
     m, k = a_c.shape
     n = b_c.size(0)
-    with torch.cuda.device(a.device):
+    with _on_device(a.device):
         out = torch.empty((m, n), device=a.device, dtype=torch.float32)
         _check(lib.astrai_w8a8_gemm_fp8_pt(
             a_c.data_ptr(), b_c.data_ptr(), None, None, None, None, out.data_ptr(), m, n, k,
@@ -323,7 +350,7 @@ def amax_bf16(x: torch.Tensor) -> torch.Tensor:
     if x.dtype != torch.bfloat16:
         raise RuntimeError("x must be bf16")
     x_c = x.contiguous()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         amax = torch.zeros(1, device=x.device, dtype=torch.float32)
         if x_c.numel():
             _check(lib.astrai_w8a8_amax_bf16(x_c.data_ptr(), amax.data_ptr(), x_c.numel(),
@@ -343,7 +370,7 @@ def amax_ring_push(hist: torch.Tensor, idx: int, amax: torch.Tensor, scale: torc
             raise RuntimeError(f"{name} must be a contiguous float32 tensor on the ring's device")
     if amax.numel() != 1 or scale.numel() != 1:
         raise RuntimeError("amax and scale must have one element")
-    with torch.cuda.device(hist.device):
+    with _on_device(hist.device):
         _check(lib.astrai_w8a8_amax_ring_push(hist.data_ptr(), hist.numel(), int(idx),
                                              amax.data_ptr(), scale.data_ptr(), float(fmax),
                                              float(pow2_margin), _stream(hist)), lib)
@@ -362,7 +389,7 @@ def quantize_transpose_bf16(x: torch.Tensor, scale: torch.Tensor, fmt: int,
     x_c = x.contiguous()
     rows, cols = x_c.shape
     f8 = torch.float8_e5m2 if fmt else torch.float8_e4m3fn
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         x8 = torch.empty((rows, cols), device=x.device, dtype=f8) if want_rowmajor else None
         x8t = torch.empty((cols, rows), device=x.device, dtype=f8)
         amax = torch.zeros(1, device=x.device, dtype=torch.float32)
@@ -410,7 +437,7 @@ def linear_backward_fp8(g, x, w, masks, sg, sw, sx, fmt: int):
         raise RuntimeError("backward shape mismatch")
     for t, name in ((sg, "sg"), (sw, "sw"), (sx, "sx")):
         _check_scale(t, g, name)
-    with torch.cuda.device(g.device):
+    with _on_device(g.device):
         grad_input = torch.empty(x.shape, device=x.device, dtype=x.dtype)
         grad_weight = torch.empty((n, k), device=w.device, dtype=w.dtype)
         grad_bias = torch.empty(0, device=g.device, dtype=g.dtype)
@@ -453,7 +480,7 @@ def quantize_int8_rows(x: torch.Tensor):
     k = x.size(-1)
     x2 = x.reshape(-1, k).contiguous()
     rows = x2.size(0)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         xq = torch.empty((rows, k), device=x.device, dtype=torch.int8)
         s = torch.empty((rows, 1), device=x.device, dtype=torch.float32)
         if rows and k:
@@ -482,7 +509,7 @@ def add_rmsnorm_quantize_int8(x: torch.Tensor, weight: torch.Tensor, eps: float,
         if res.shape != x.shape or res.dtype != torch.bfloat16 or res.device != x.device:
             raise RuntimeError("res must match x in shape, dtype and device")
         r2 = res.reshape(-1, k).contiguous()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         xq = torch.empty((rows, k), device=x.device, dtype=torch.int8)
         s = torch.empty((rows, 1), device=x.device, dtype=torch.float32)
         t = torch.empty_like(x2) if r2 is not None else None
@@ -510,7 +537,7 @@ def silu_mul_quantize_int8(gate: torch.Tensor, up: torch.Tensor, want_h: bool = 
         g2, u2 = g2.contiguous(), u2.contiguous()
     rows = g2.size(0)
     ld = g2.stride(0) if rows > 1 else max(w, g2.stride(0))
-    with torch.cuda.device(gate.device):
+    with _on_device(gate.device):
         hq = torch.empty((rows, w), device=gate.device, dtype=torch.int8)
         s = torch.empty((rows, 1), device=gate.device, dtype=torch.float32)
         h = torch.empty((rows, w), device=gate.device, dtype=torch.bfloat16) if want_h else None
@@ -550,7 +577,7 @@ def add_rmsnorm_quantize_fp8(x: torch.Tensor, weight: torch.Tensor, eps: float, 
         if res.shape != x.shape or res.dtype != torch.bfloat16 or res.device != x.device:
             raise RuntimeError("res must match x in shape, dtype and device")
         r2 = res.reshape(-1, k).contiguous()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         x8 = torch.empty((rows, k), device=x.device, dtype=_FP8[1 if fmt else 0])
         if amax is None:
             amax = torch.zeros(1, device=x.device, dtype=torch.float32)
@@ -579,7 +606,7 @@ def silu_mul_quantize_fp8(gate: torch.Tensor, up: torch.Tensor, scale: torch.Ten
         g2, u2 = g2.contiguous(), u2.contiguous()
     rows = g2.size(0)
     ld = g2.stride(0) if rows > 1 else max(w, g2.stride(0))
-    with torch.cuda.device(gate.device):
+    with _on_device(gate.device):
         h8 = torch.empty((rows, w), device=gate.device, dtype=_FP8[1 if fmt else 0])
         if amax is None:
             amax = torch.zeros(1, device=gate.device, dtype=torch.float32)
@@ -624,7 +651,7 @@ def rotary_emb(x: torch.Tensor, freqs_cis: torch.Tensor) -> torch.Tensor:
         raise RuntimeError("freqs_cis dim/2 mismatch")
     if freqs_cis.size(-1) != 2:
         raise RuntimeError("freqs_cis last dim must be 2 [cos, sin]")
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         out = torch.empty_like(x)
         if x.numel():
             _check(lib.astrai_w8a8_rotary_emb_bf16(x.data_ptr(), freqs_cis.data_ptr(), out.data_ptr(),
@@ -664,7 +691,7 @@ def rope_cache_write(qkv: torch.Tensor, freqs: torch.Tensor, positions: torch.Te
     for t in (freqs, positions, k_cache, v_cache):
         if t.device != qkv.device:
             raise RuntimeError("all tensors must be on qkv's device")
-    with torch.cuda.device(qkv.device):
+    with _on_device(qkv.device):
         q_out = torch.empty((b, n_heads, s, head_dim), device=qkv.device, dtype=torch.bfloat16)
         _check(lib.astrai_w8a8_rope_cache_write_bf16(
             q2.data_ptr(), ld, freqs.contiguous().data_ptr(), positions.contiguous().data_ptr(),
@@ -716,7 +743,7 @@ def attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, p
     if nsplit <= 0:
         nsplit = decode_nsplit(b * hkv, max_len)
     nq = (h // hkv) * s
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         need = lib.astrai_w8a8_attn_decode_workspace_floats(b, hkv, nsplit, nq)
         ws = torch.empty(max(need, 1), device=q.device, dtype=torch.float32)
         out = oq = os_ = None
@@ -762,7 +789,7 @@ def attn_decode_static_scratch(q: torch.Tensor, k_cache: torch.Tensor, v_cache: 
     if (out is not None and out.numel() != b * s * h * d) or (out_q is not None and (
             out_q.numel() != b * s * h * d or out_scale is None or out_scale.numel() != b * s)):
         raise RuntimeError("out / out_q must hold batch*seq rows of n_heads*head_dim, out_scale batch*seq steps")
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         _check(lib.astrai_w8a8_attn_decode_bf16_static_scratch(
             q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), positions.data_ptr(), _ptr(out), _ptr(out_q),
             _ptr(out_scale), b, s, h, hkv, d, max_len, nsplit, float(d ** -0.5 if scale is None else scale),
@@ -824,7 +851,7 @@ def attn_paged_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     user_nsplit = nsplit > 0
     if nsplit <= 0:
         nsplit = decode_nsplit(b * hkv, req_to_token.size(1))
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         if new_k is not None:
             if new_k.shape != (b, hkv, d) or new_v.shape != (b, hkv, d):
                 raise RuntimeError("new K/V shape mismatch")
@@ -957,7 +984,7 @@ def attn_paged_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Te
     tensors = [t.contiguous() for t, _ in ints]
     if scale is None or scale <= 0.0:
         scale = d ** -0.5
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         # (rows that no tile of the schedule covers are left unwritten, as by the reference)
         out = torch.empty((total_q, h, d), device=q.device, dtype=torch.bfloat16)
         if total_q == 0 or q_tile_to_batch.numel() == 0:
@@ -1017,7 +1044,7 @@ def attn_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
         raise RuntimeError("n_heads must be a multiple of n_kv_heads")
     if scale is None:
         scale = d ** -0.5
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         out = torch.empty((b, s, h * d), device=q.device, dtype=torch.bfloat16)
         _check(lib.astrai_w8a8_attn_prefill_bf16(
             q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), positions.contiguous().data_ptr(),
@@ -1071,7 +1098,7 @@ def mm_int8(a: torch.Tensor, b: torch.Tensor, sa: Optional[torch.Tensor],
         raise RuntimeError("out_dtype must be 0 (bf16) or 2 (int32 accumulator)")
     a_c, b_c, sa, sb, bias, m, n, k = _int8_operands(a, b, sa, sb, bias, out_dtype == OUT_BF16, "mm_int8")
     fn = getattr(lib, _INT8_ENTRY[kernel])
-    with torch.cuda.device(a.device):
+    with _on_device(a.device):
         out = torch.empty((m, n), device=a.device,
                           dtype=torch.int32 if out_dtype == OUT_ACC else torch.bfloat16)
         if m and n:
@@ -1095,7 +1122,7 @@ def mm_int8_resid(a: torch.Tensor, b: torch.Tensor, sa: torch.Tensor, sb: torch.
             and resid.numel() == m * n):
         raise RuntimeError("resid must be CUDA bf16 with M*N elements")
     resid_c = resid.contiguous()
-    with torch.cuda.device(a.device):
+    with _on_device(a.device):
         out = torch.empty((m, n), device=a.device, dtype=torch.bfloat16)
         if m and n:
             if k == 0:
@@ -1118,7 +1145,7 @@ def mfma_probe(kind: int, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     for t in (a, b):
         if not t.is_contiguous() or t.numel() * t.element_size() != rows * kbytes or t.device != a.device:
             raise RuntimeError(f"operands of kind {kind} are contiguous [{rows}] rows of {kbytes} bytes")
-    with torch.cuda.device(a.device):
+    with _on_device(a.device):
         d = torch.zeros((64, 4 if rows == 16 else 16), device=a.device, dtype=torch.int32)
         _check(lib.astrai_w8a8_mfma_probe(kind, a.data_ptr(), b.data_ptr(), d.data_ptr(), _stream(a)), lib)
     return d
@@ -1174,7 +1201,7 @@ def mm_int8_swiglu(a: torch.Tensor, wgu: torch.Tensor, sa: torch.Tensor, sgu: to
         fused = mm_int8_swiglu_fused_shape(m, n, k)
     if not fused:
         gu = mm_int8(a, wgu, sa, sgu)
-        with torch.cuda.device(a.device):
+        with _on_device(a.device):
             hq = torch.empty((m, w), device=a.device, dtype=torch.int8)
             s = torch.empty((m, 1), device=a.device, dtype=torch.float32)
             h = torch.empty((m, w), device=a.device, dtype=torch.bfloat16) if want_h else None
@@ -1187,7 +1214,7 @@ def mm_int8_swiglu(a: torch.Tensor, wgu: torch.Tensor, sa: torch.Tensor, sgu: to
     sa = _check_vec(sa, a, m, "sa")
     sgu = _check_vec(sgu, a, n, "sgu")
     pieces = n // 128
-    with torch.cuda.device(a.device):
+    with _on_device(a.device):
         h = torch.empty((m, w), device=a.device, dtype=torch.bfloat16)
         row_max = torch.empty((m, pieces), device=a.device, dtype=torch.float32)
         hq = torch.empty((m, w), device=a.device, dtype=torch.int8)
@@ -1263,7 +1290,7 @@ def mm_int8_rope_cache(a: torch.Tensor, wqkv: torch.Tensor, sa: torch.Tensor, sb
         if t.device != a.device:
             raise RuntimeError("all tensors must be on a's device")
     a_c, w_c = a.contiguous(), wqkv.contiguous()
-    with torch.cuda.device(a.device):
+    with _on_device(a.device):
         q_out = torch.empty((batch, n_heads, seq, head_dim), device=a.device, dtype=torch.bfloat16)
         _check(lib.astrai_w8a8_gemm_int8_ptpc_rope_cache(
             a_c.data_ptr(), w_c.data_ptr(), sa.data_ptr(), sb.data_ptr(), freqs.contiguous().data_ptr(),
@@ -1282,7 +1309,7 @@ def quantize_fp8_block128_act(x: torch.Tensor):
     if k % 128:
         raise RuntimeError("K must be a multiple of 128")
     x_c = x.contiguous()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         x8 = torch.empty((m, k), device=x.device, dtype=torch.float8_e4m3fn)
         sa = torch.empty((m, k // 128), device=x.device, dtype=torch.float32)
         if m and k:
@@ -1301,7 +1328,7 @@ def quantize_fp8_block128_weight(w: torch.Tensor):
     if k % 128:
         raise RuntimeError("K must be a multiple of 128")
     w_c = w.contiguous()
-    with torch.cuda.device(w.device):
+    with _on_device(w.device):
         w8 = torch.empty((n, k), device=w.device, dtype=torch.float8_e4m3fn)
         sb = torch.empty(((n + 127) // 128, k // 128), device=w.device, dtype=torch.float32)
         if n and k:
@@ -1335,7 +1362,7 @@ def mm_fp8_block128(a: torch.Tensor, b: torch.Tensor, sa: torch.Tensor, sb: torc
                 and bias.numel() == n):
             raise RuntimeError("bias must be CUDA bf16 with shape [N]")
         bias = bias.contiguous()
-    with torch.cuda.device(a.device):
+    with _on_device(a.device):
         out = torch.empty((m, n), device=a.device, dtype=torch.bfloat16)
         if m and n:
             _check(lib.astrai_w8a8_gemm_fp8_block128(
@@ -1444,7 +1471,7 @@ def attn_cache_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             or not (k_cache.is_contiguous() and v_cache.is_contiguous()):
         raise RuntimeError("attn_cache_rows: the caches must be contiguous [batch, n_kv_heads, max_len, head_dim]")
     n_rep, pairs = h // hkv, b * hkv
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         table, rows = _identity_paging(pairs, max_len, q.device)
         key = ("ramp", pairs, str(q.device))
         if key not in _index_cache:
@@ -1483,7 +1510,7 @@ def attn_decode_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Opt
     if d not in (32, 64, 128, 256) or h // hkv > 16:
         raise RuntimeError("attn_decode needs head_dim in (32, 64, 128, 256) and n_heads / n_kv_heads <= 16")
     attend = kv_len if causal_offset < 0 else min(kv_len, causal_offset + 1)
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         if kv_len == 0 or b == 0:
             return torch.zeros_like(q)
         if layout == BHLD and m4 is None and k.is_contiguous() and v.is_contiguous() and d == 128 and h <= 64 \
@@ -1524,7 +1551,7 @@ def attn_prefill_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Op
     m4 = _dense_mask(mask, b, q_len, kv_len, h)
     if d not in (32, 64, 128, 256) or h // hkv > 16:
         raise RuntimeError("attn_prefill needs head_dim in (32, 64, 128, 256) and n_heads / n_kv_heads <= 16")
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         if kv_len == 0 or b == 0 or q_len == 0:
             return torch.zeros_like(q)
         rows_i = torch.arange(q_len, dtype=torch.int64, device=q.device)
