@@ -266,3 +266,6 @@ def test_mm_int8_resid_rejects(C):
     r = torch.randn(8, 16, device=DEV).bfloat16()
     out = C.mm_int8_resid(a[:, :0], w[:, :0], sa, sw, r)
     assert torch.equal(out, r)
+    # no rows: nothing to launch
+    out = C.mm_int8_resid(a[:0], w, sa[:0], sw, r[:0])
+    assert out.shape == (0, 16)
