@@ -1,9 +1,11 @@
 // fp8 (OCP e4m3fn / e5m2) MFMA GEMMs, per-tensor scales (optional bias, bf16 /
 // e4m3 / fp32 output) or one scale per activation row and per weight row (bf16 output). Large shapes run v_mfma_f32_32x32x64_f8f6f4 on 256x256
 // tiles: the four-wave 128x128-register-tile kernel for bf16 output, the
-// eight-wave ping-pong kernel for the other outputs; the generic tiled kernel
-// takes everything else.
+// eight-wave ping-pong kernel for the other outputs; bf16 shapes with too few of
+// those tiles for the chip run 128x128 tiles of the same instruction; the generic
+// tiled kernel takes everything else.
 #include "gemm_wave128.cuh"
+#include "gemm_mid128.cuh"
 #include "gemm_tile.cuh"
 
 namespace w8a8 {
@@ -15,6 +17,7 @@ void launch_for(const GemmArgs& g, hipStream_t stream) {
     if (wave128_shape_ok(g)) return launch_wave128<Op32F8<Fmt>, ScaleKind>(g, stream);
 #endif
     if (pingpong_shape_ok(g)) return launch_pingpong<Op32F8<Fmt>, ScaleKind>(g, stream);
+    if (mid128_shape_ok(g)) return launch_mid128<Op32F8<Fmt>, ScaleKind>(g, stream);
     launch_tiled_auto<OpF8<Fmt>, ScaleKind>(g, stream);
 }
 }  // namespace

@@ -1,8 +1,10 @@
 // int8 x int8 -> int32 MFMA GEMMs, per-token x per-channel dequant epilogue.
 // Large shapes run v_mfma_i32_32x32x32_i8 on 256x256 tiles: the four-wave
 // 128x128-register-tile kernel for bf16 output, the eight-wave ping-pong kernel
-// for int32 output; the generic tiled kernel takes everything else.
+// for int32 output; shapes with too few of those tiles for the chip run 128x128
+// tiles of the same instruction; the generic tiled kernel takes everything else.
 #include "gemm_wave128.cuh"
+#include "gemm_mid128.cuh"
 #include "gemm_tile.cuh"
 
 namespace w8a8 {
@@ -16,6 +18,8 @@ bool launch_gemm_int8_tiled(const GemmArgs& g, hipStream_t stream) {
 #endif
     if (pingpong_shape_ok(g))
         launch_pingpong<Op32I8, SCALE_ROWCOL>(g, stream);
+    else if (mid128_shape_ok(g))
+        launch_mid128<Op32I8, SCALE_ROWCOL>(g, stream);
     else
         launch_tiled_auto<OpI8, SCALE_ROWCOL>(g, stream);
     return true;

@@ -233,7 +233,8 @@ def test_config1_sampled_rows_at_full_size(ops):
     (17, 9, 33, 0, False),          # any-shape kernel (K % 16 != 0)
     (130, 200, 384, 0, True),       # small tiles
     (257, 513, 1024, 1, False),     # e5m2
-    (1024, 1536, 512, 0, True),     # 128x128 tiles
+    (1024, 1536, 512, 0, True),     # 128x128 tiles of the generic kernel
+    (2048, 1536, 512, 1, True),     # 128x128 tiles, mid-size kernel
     (4096, 4096, 256, 0, False),    # 256x256 tiles, four-wave kernel
     (3841, 4100, 640, 0, True),     # 256x256 tiles, N % 8 != 0: ping-pong kernel
 ])
@@ -372,7 +373,10 @@ def test_block128_large_kernel_wide_scale_range(m, n, k):
 
 @pytest.mark.parametrize("m,n,k,bias", [(3900, 4104, 1152, True),    # N % 8 == 0: four-wave kernel
                                         (3841, 4100, 640, False),   # N % 8 != 0: ping-pong kernel
-                                        (4096, 3848, 256, False)])  # shortest K the big kernels take
+                                        (4096, 3848, 256, False),   # shortest K the big kernels take
+                                        (1700, 2056, 384, True),    # 14 x 17 tiles of 128 x 128: mid-size kernel
+                                        (1793, 1798, 256, False),   # the same, N % 4 != 0: element stores
+                                        (2048, 2048, 2048, False)])
 def test_large_ragged_tiles_with_guard_rows(m, n, k, bias):
     """Edge tiles of the large-shape kernels: rows past M / columns past N must
     read as zero and must not be written. The call goes through the C ABI into

@@ -172,7 +172,11 @@ def test_full_size_linearity_property(C):
 
 @pytest.mark.parametrize("m,n,k,out_dtype", [(3900, 4104, 1152, 0),   # bf16, N % 8 == 0: four-wave kernel
                                              (3841, 4100, 640, 0),    # bf16, N % 8 != 0: ping-pong kernel
-                                             (3900, 4104, 384, 2)])   # int32 accumulator: ping-pong kernel
+                                             (3900, 4104, 384, 2),    # int32 accumulator: ping-pong kernel
+                                             (1700, 2052, 384, 0),    # 14 x 17 tiles of 128 x 128: mid-size kernel
+                                             (1793, 1798, 256, 0),    # the same, N % 4 != 0: element stores
+                                             (2048, 3072, 2048, 0),   # a 2048-token block of the config-4 q|k|v projection
+                                             (512, 11264, 2048, 0)])  # a 512-token block of its gate|up projection (4 x 88 tiles)
 def test_large_ragged_tiles_with_guard_rows(C, m, n, k, out_dtype):
     """Edge tiles of the large-shape kernels: bit-exact int32 (or the bf16
     epilogue of it) on the first / tile-boundary / last rows and the last columns,
