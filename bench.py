@@ -446,9 +446,21 @@ def main():
                                                     None, y3.data_ptr(), 8192, 2048, 7168, stream))
             check(lib.astrai_w8a8_gemm_fp8_pt(a8.data_ptr(), b8.data_ptr(), one.data_ptr(), one.data_ptr(),
                                               one.data_ptr(), None, y8.data_ptr(), 4096, 4096, 4096, 0, 1, stream))
+        # token blocks between decode and full prefill on the config-4 projections (128 x 128 tiles)
+        mids = []
+        for (mm, nn, kk) in ((2048, 3072, 2048), (2048, 2048, 5632), (1024, 11264, 2048)):
+            mx = (torch.randn(mm, kk, device=dev) * 32).clamp(-127, 127).round().to(torch.int8)
+            mw = (torch.randn(nn, kk, device=dev) * 32).clamp(-127, 127).round().to(torch.int8)
+            mids.append((mx, mw, torch.rand(mm, device=dev) + 0.5, torch.rand(nn, device=dev) + 0.5,
+                         torch.empty(mm, nn, device=dev, dtype=torch.bfloat16), mm, nn, kk))
+        for _ in range(20):
+            for (mx, mw, msx, msw, my, mm, nn, kk) in mids:
+                check(lib.astrai_w8a8_gemm_int8_ptpc(mx.data_ptr(), mw.data_ptr(), msx.data_ptr(), msw.data_ptr(),
+                                                     None, my.data_ptr(), mm, nn, kk, 0, stream))
         torch.cuda.synchronize()
         print(json.dumps({"trace_gemms": "20 launches each: int8 4096^3 per-token x per-channel (bf16 out), fp8 "
-                                         "128-block 8192x2048x7168 on config-3 data, fp8 4096^3 with e4m3 output"}))
+                                         "128-block 8192x2048x7168 on config-3 data, fp8 4096^3 with e4m3 output; "
+                                         "then int8 2048x3072x2048, 2048x2048x5632, 1024x11264x2048 (mid-size kernel)"}))
         return
 
     # ---------------- headline: config 1, fp8 per-tensor 4096^3 ----------------
@@ -714,6 +726,22 @@ def main():
             "swiglu_epilogue_gemm_plus_quantizer_us": round(ms_fused * 1e3, 1),
             "TOP/s_of_the_fused_pair": round(2.0 * Mg * 2 * Wg * Kg / (ms_fused * 1e-3) / 1e12, 1)}
         del xg, wgate, wup, xq, wgq, wuq, wcat, wblk
+
+        # ---- token blocks between decode and full prefill on the config-4 projections: too few
+        # 256 x 256 tiles for the chip, 128 x 128 tiles instead (N(0, 32) codes, per-token x per-channel)
+        mid = {}
+        for (mm, nn, kk) in ((2048, 3072, 2048), (2048, 2048, 5632), (1024, 11264, 2048)):
+            mx = (torch.randn(mm, kk, device=dev) * 32).clamp(-127, 127).round().to(torch.int8)
+            mw = (torch.randn(nn, kk, device=dev) * 32).clamp(-127, 127).round().to(torch.int8)
+            msx, msw = torch.rand(mm, device=dev) + 0.5, torch.rand(nn, device=dev) + 0.5
+            my = torch.empty(mm, nn, device=dev, dtype=torch.bfloat16)
+            ms_mid = ms_of(lambda: check(lib.astrai_w8a8_gemm_int8_ptpc(
+                mx.data_ptr(), mw.data_ptr(), msx.data_ptr(), msw.data_ptr(), None, my.data_ptr(), mm, nn, kk, 0,
+                stream)))
+            mid[f"{mm}x{nn}x{kk}"] = {"us": round(ms_mid * 1e3, 2),
+                                      "TOP/s": round(2.0 * mm * nn * kk / (ms_mid * 1e-3) / 1e12, 1)}
+            del mx, mw, my
+        extra["int8_gemm_token_blocks_128x128_tiles"] = mid
 
         # ---- config 2: decode GEMV on the seed-2 tensors (activation and weight quantized per
         # token / per channel by the oracle's quantizer on the host), weights rotated through a
