@@ -3,10 +3,11 @@
 // idle (2048 x 3072: 96 tiles for 256 compute units) and what counts is having every
 // compute unit busy, not the last percent of operand reuse.
 //
-// 128 x 128 output tiles, four waves of 64 x 64 (2 x 2 MFMA 32x32 sub-tiles, 64 accumulator
+// 128 x 128 output tiles, eight waves of 64 x 32 (two MFMA 32x32 sub-tiles, 32 accumulator
 // registers), K in 128-byte slabs through two LDS stages of 32 KiB filled by direct-to-LDS
-// loads: 64 KiB and ~130 registers per workgroup, so two or three workgroups share a compute
-// unit and cover each other's barriers and memory waits -- no hand-pinned schedule here. LDS
+// loads: 64 KiB per workgroup and ~95 registers per wave, so two workgroups -- four waves per
+// SIMD -- share a compute unit and cover each other's barriers and memory waits; no hand-pinned
+// schedule here (four waves of 64 x 64 measured 2-4% slower on the decoder's shapes). LDS
 // layout of a slab, fragment reads and accumulator layout are those of the large-tile
 // kernels (gemm_pingpong.cuh): 128 activation rows then 128 weight rows of 128 bytes, chunk
 // c of row r at position c ^ (r & 7) ^ ((r >> 3) & 1); weight rows are the first MFMA operand.
@@ -17,15 +18,15 @@ namespace w8a8 {
 
 struct Mid128Cfg {
     static constexpr int BM = 128, BN = 128, BK = 128;
-    static constexpr int THREADS = 256;
-    static constexpr int MI = 2, NI = 2;                 // 32-row sub-tiles per wave: 64 m x 64 n
+    static constexpr int THREADS = 512;
+    static constexpr int MI = 2, NI = 1;                 // 32-row sub-tiles per wave: 64 m x 32 n
     static constexpr int OPERAND_BYTES = 128 * BK;       // one operand's slab: 16 KiB
     static constexpr int STAGE_BYTES = 2 * OPERAND_BYTES;
     static constexpr int LDS_BYTES = 2 * STAGE_BYTES;    // 64 KiB
 };
 
 template <class Op, int ScaleKind>
-__global__ __launch_bounds__(Mid128Cfg::THREADS, 2) void gemm_mid128_kernel(GemmArgs g) {
+__global__ __launch_bounds__(Mid128Cfg::THREADS) void gemm_mid128_kernel(GemmArgs g) {
     using Cfg = Mid128Cfg;
     using Acc = typename Op::Acc;
     constexpr int MI = Cfg::MI, NI = Cfg::NI;
@@ -33,7 +34,7 @@ __global__ __launch_bounds__(Mid128Cfg::THREADS, 2) void gemm_mid128_kernel(Gemm
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int wave_m = wave & 1, wave_n = wave >> 1;
+    const int wave_m = wave & 1, wave_n = wave >> 1;   // 2 x 4 waves
     const int lrow = lane & 31, lgrp = lane >> 5;
 
     const int tiles_m = (g.m + Cfg::BM - 1) / Cfg::BM;
@@ -46,7 +47,7 @@ __global__ __launch_bounds__(Mid128Cfg::THREADS, 2) void gemm_mid128_kernel(Gemm
     // epilogue operands, requested now
     const EpilogueScalars es = load_epilogue_scalars<ScaleKind>(g);
     [[maybe_unused]] const float s_tensor = es.sa * es.sb;
-    const int mw = m0 + wave_m * 64, nw = n0 + wave_n * 64;
+    const int mw = m0 + wave_m * 64, nw = n0 + wave_n * 32;
     float sx[MI];
     f32x4 sw4[NI][4], b4[NI][4];
     const uint16_t* bias = static_cast<const uint16_t*>(g.bias);
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(Mid128Cfg::THREADS, 2) void gemm_mid128_kernel(Gemm
                 }
             }
 
-    // ---- direct-to-LDS load plan: wave w fills rows 32w .. 32w+31 of both operands, 8 rows per
+    // ---- direct-to-LDS load plan: wave w fills rows 16w .. 16w+15 of both operands, 8 rows per
     // instruction. Lane l lands at row l>>3, position l&7 of its 1 KiB block and fetches logical
     // chunk (l&7) ^ f(row): c0 for even instructions, c0 ^ 1 for odd ones. Rows past M / N are
     // past the buffer's num_records and read as zero.
@@ -82,21 +83,21 @@ __global__ __launch_bounds__(Mid128Cfg::THREADS, 2) void gemm_mid128_kernel(Gemm
     uint32_t x_off[2], w_off[2];
     {
         const int c0 = (lane & 7) ^ (lane >> 3);
-        const uint32_t xr = (uint32_t)(m0 + wave * 32 + (lane >> 3)) * (uint32_t)K;
-        const uint32_t wr = (uint32_t)(n0 + wave * 32 + (lane >> 3)) * (uint32_t)K;
+        const uint32_t xr = (uint32_t)(m0 + wave * 16 + (lane >> 3)) * (uint32_t)K;
+        const uint32_t wr = (uint32_t)(n0 + wave * 16 + (lane >> 3)) * (uint32_t)K;
         x_off[0] = xr + (uint32_t)c0 * 16;
         x_off[1] = xr + (uint32_t)(c0 ^ 1) * 16;
         w_off[0] = wr + (uint32_t)c0 * 16;
         w_off[1] = wr + (uint32_t)(c0 ^ 1) * 16;
     }
     const uint32_t row8 = 8u * (uint32_t)K;
-    uint8_t* const dma_base = lds + wave * (32 * 128);
+    uint8_t* const dma_base = lds + wave * (16 * 128);
     auto issue = [&](int stage, uint32_t k0) {
         uint8_t* const dst = dma_base + stage * Cfg::STAGE_BYTES;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) lds_dma16(rx, dst + r * 1024, x_off[r & 1] + (uint32_t)r * row8, k0);
+        for (int r = 0; r < 2; ++r) lds_dma16(rx, dst + r * 1024, x_off[r & 1] + (uint32_t)r * row8, k0);
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
+        for (int r = 0; r < 2; ++r)
             lds_dma16(rw, dst + Cfg::OPERAND_BYTES + r * 1024, w_off[r & 1] + (uint32_t)r * row8, k0);
     };
 
@@ -108,7 +109,7 @@ __global__ __launch_bounds__(Mid128Cfg::THREADS, 2) void gemm_mid128_kernel(Gemm
         for (int j = 0; j < 4; ++j) frag_off[j] = lrow * 128 + (((4 * lgrp + j) ^ sw) << 4);
     }
     const int x_rd = (wave_m * 64) * 128;
-    const int w_rd = Cfg::OPERAND_BYTES + (wave_n * 64) * 128;
+    const int w_rd = Cfg::OPERAND_BYTES + (wave_n * 32) * 128;
 
     Acc acc[NI][MI];
 #pragma unroll
@@ -145,7 +146,7 @@ __global__ __launch_bounds__(Mid128Cfg::THREADS, 2) void gemm_mid128_kernel(Gemm
     for (int k = 0; k < ksteps; ++k) {
         if (k + 1 < ksteps) {
             issue((k + 1) & 1, (uint32_t)(k + 1) << 7);
-            wait_vmcnt<8>();   // the eight loads of slab k are older than those just issued
+            wait_vmcnt<4>();   // the four loads of slab k are older than those just issued
         } else {
             wait_vmcnt<0>();
         }
