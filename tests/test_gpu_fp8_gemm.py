@@ -198,6 +198,30 @@ def test_mm_fp8_both_formats_tile_edges(ops, fmt, m, n, k):
     assert_bf16_close(out, O.fp8_gemm(a8, b8, sa, sb), what=f"mm_fp8 {name}")
 
 
+@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("m,n,k", [(300, 520, 1032), (64, 1024, 1288), (513, 257, 2047)])
+def test_mm_fp8_k_not_in_16_byte_pieces_zero_padded(ops, fmt, m, n, k):
+    """K % 16 != 0 on a product large enough for the wrapper to zero-pad the rows for the tuned
+    kernels: zero codes add nothing, the result stays within the GEMM's tolerance of the oracle."""
+    from astrai_amd.extension import _cabi
+    print(f"case fmt={fmt} m={m} n={n} k={k}", flush=True)
+    assert k % 16 and m * n * k >= _cabi._PAD_K_MIN_MACS
+    a, b, _ = O.make_inputs(1, m, n, k, w_std=1.0)
+    name = "e5m2" if fmt else "e4m3"
+    sa, sb = O.dynamic_scale(a, name).reshape(1), O.dynamic_scale(b, name).reshape(1)
+    a8, _ = O.fp8_quantize(a, sa, fmt)
+    b8, _ = O.fp8_quantize(b, sb, fmt)
+    ad, bd = a8.to(DEV), b8.to(DEV)
+    pa, pb, kp = _cabi._pad_k(ad, bd)
+    assert kp % 128 == 0 and pa.dtype == ad.dtype and pa.shape == (m, kp) and pb.shape == (n, kp)
+    assert torch.equal(pa[:, :k].view(torch.uint8), ad.view(torch.uint8)) and not pa[:, k:].view(torch.uint8).any()
+    out = ops.mm_fp8(ad, bd, sa.to(DEV), sb.to(DEV))
+    assert_bf16_close(out, O.fp8_gemm(a8, b8, sa, sb), what=f"mm_fp8 {name} padded K")
+    sa_r = (torch.rand(m, 1, generator=torch.Generator().manual_seed(k)) * 0.5 + 0.5) * sa
+    out = ops.mm_fp8(ad, bd, sa_r.to(DEV), sb.to(DEV))
+    assert_bf16_close(out, O.fp8_gemm(a8, b8, sa_r, sb), what=f"mm_fp8 {name} padded K, row scales")
+
+
 def test_mm_fp8_rejects_bad_arguments(ops):
     a8 = torch.zeros(4, 16, dtype=torch.float8_e4m3fn, device=DEV)
     b5 = torch.zeros(4, 16, dtype=torch.float8_e5m2, device=DEV)

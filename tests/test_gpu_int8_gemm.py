@@ -65,6 +65,32 @@ def test_random_shape_sweep_default_dispatch_bit_exact(C):
         assert torch.equal(fused.view(torch.int16), (ref + r).view(torch.int16)), (m, n, k)
 
 
+@pytest.mark.parametrize("m,n,k", [(300, 520, 1032), (64, 1024, 1288), (1, 2048, 8200), (513, 257, 2047)])
+def test_k_not_in_16_byte_pieces_zero_padded_bit_exact(C, m, n, k):
+    """K % 16 != 0 on a product large enough for the wrapper to zero-pad the rows for the tuned
+    kernels: accumulators, the scaled output and the residual form stay bit-exact, and the
+    caller's tensors are untouched."""
+    print(f"case m={m} n={n} k={k}", flush=True)
+    assert k % 16 and m * n * k >= C._PAD_K_MIN_MACS
+    g = torch.Generator().manual_seed(m + n + k)
+    a, b = _rand_i8(g, m, k), _rand_i8(g, n, k)
+    ad, bd = a.to(DEV), b.to(DEV)
+    padded = C._pad_k(ad, bd)
+    assert padded[2] % 128 == 0 and padded[0].shape == (m, padded[2]) and padded[1].shape == (n, padded[2])
+    assert torch.equal(padded[0][:, :k], ad) and not padded[0][:, k:].any() and not padded[1][:, k:].any()
+    want = O.int8_acc(a, b)
+    assert torch.equal(C.mm_int8(ad, bd, None, None, None, 2).cpu(), want)
+    sa = torch.rand(m, generator=g) * 0.02 + 0.001
+    sb = torch.rand(n, generator=g) * 0.02 + 0.001
+    ref = (want.float() * sa[:, None] * sb[None, :]).to(torch.bfloat16)
+    out = C.mm_int8(ad, bd, sa.to(DEV), sb.to(DEV), None, 0).cpu()
+    assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+    r = torch.randn(m, n, generator=g).to(torch.bfloat16)
+    fused = C.mm_int8_resid(ad, bd, sa.to(DEV), sb.to(DEV), r.to(DEV)).cpu()
+    assert torch.equal(fused.view(torch.int16), (ref + r).view(torch.int16))
+    assert torch.equal(ad.cpu(), a) and torch.equal(bd.cpu(), b)
+
+
 def test_golden_integer_cases_including_worst_case_magnitude(C, golden):
     for c in golden("int8_small.json")["gemm"]:
         a = torch.tensor(c["a"], dtype=torch.int8)
