@@ -630,7 +630,7 @@ int astrai_w8a8_gemm_fp8_pt(const void* a8, const void* b8, const float* sa, con
     if (k == 0) return fail(ASTRAI_W8A8_UNSUPPORTED, "gemm_fp8_pt: K must be >= 1");
     auto s = static_cast<hipStream_t>(stream);
     const w8a8::GemmArgs g = pack(a8, b8, sa, sb, out_scale, bias, out, m, n, k, out_dtype);
-    if (!w8a8::launch_gemm_fp8_tiled(g, fmt, s))
+    if (!w8a8::launch_gemv_fp8(g, fmt, w8a8::SCALE_TENSOR, s) && !w8a8::launch_gemm_fp8_tiled(g, fmt, s))
         w8a8::launch_gemm_generic(g, fmt ? 2 : 1, w8a8::SCALE_TENSOR, s);
     return check_launch("gemm_fp8_pt");
 }
@@ -646,7 +646,7 @@ int astrai_w8a8_gemm_fp8_ptpc(const void* a8, const void* b8, const float* sa, c
     if (k == 0) return fail(ASTRAI_W8A8_UNSUPPORTED, "gemm_fp8_ptpc: K must be >= 1");
     auto s = static_cast<hipStream_t>(stream);
     const w8a8::GemmArgs g = pack(a8, b8, sa, sb, nullptr, bias, out, m, n, k, w8a8::OUT_BF16);
-    if (!w8a8::launch_gemm_fp8_rowcol_tiled(g, fmt, s))
+    if (!w8a8::launch_gemv_fp8(g, fmt, w8a8::SCALE_ROWCOL, s) && !w8a8::launch_gemm_fp8_rowcol_tiled(g, fmt, s))
         w8a8::launch_gemm_generic(g, fmt ? 2 : 1, w8a8::SCALE_ROWCOL, s);
     return check_launch("gemm_fp8_ptpc");
 }

@@ -1,4 +1,4 @@
-// Batched-decode int8 W8A8 kernel (2 <= M <= 128 tokens): bandwidth-bound. The weight
+// Batched-decode W8A8 kernel (int8: 2 <= M <= 128 tokens; fp8: 1 <= M <= 64): bandwidth-bound. The weight
 // matrix is streamed from HBM exactly once with the streaming cache hint; what decides the
 // time besides that stream is how often the activation block X[M,K] is pulled out of
 // L2 again (every workgroup that owns weight rows over all of K needs all of it), how
@@ -21,6 +21,9 @@
 //  * int32 partials of the waves are summed through LDS (integer addition: the split
 //    keeps the accumulator bit-exact), then the dequant epilogue, optionally continued
 //    by rotary embedding and the KV-cache write for a fused q|k|v projection.
+//  * fp8 operands take the same route with v_mfma_f32_16x16x128_f8f6f4 on pairs of operand
+//    registers (any K order inside an item is a valid contraction); the waves' fp32 partials
+//    are added in wave order, so a result does not change from launch to launch.
 #pragma once
 
 #include "common.cuh"
@@ -48,8 +51,24 @@ __device__ __forceinline__ void to_operand_order(uint8_t* patch, int lane, const
         out[j] = *reinterpret_cast<const u32x4*>(patch + lrow * 256 + (((4 * j + lgrp) ^ lrow) << 4));
 }
 
-template <int RG, int MB, int NW, int IB, bool ROPE>
-__global__ __launch_bounds__(NW * 64) void gemv_int8_rows_kernel(GemmArgs g, RopeCacheArgs rc, int rows_per_wg) {
+struct RowsOpI8 {
+    using Acc = i32x4;
+    using AccScalar = int;
+    static constexpr bool kIsInt = true;
+};
+template <int Fmt>  // 0 = e4m3fn, 1 = e5m2
+struct RowsOpF8 {
+    using Acc = f32x4;
+    using AccScalar = float;
+    static constexpr bool kIsInt = false;
+    static constexpr int kFmt = Fmt;
+};
+
+// `rowcol`: one step per token and per weight row (always so for int8); else one per tensor
+template <class Op, int RG, int MB, int NW, int IB, bool ROPE>
+__device__ __forceinline__ void gemv_rows_body(const GemmArgs& g, const RopeCacheArgs& rc, int rows_per_wg,
+                                               bool rowcol) {
+    using Acc = typename Op::Acc;
     constexpr int PATCH = 8192;                     // per wave: 4 KiB weights + 4 KiB activations
     constexpr int RED = RG * MB * 1024;             // per wave: its partial accumulators
     constexpr int WAVE_LDS = PATCH > RED ? PATCH : RED;
@@ -77,14 +96,14 @@ __global__ __launch_bounds__(NW * 64) void gemv_int8_rows_kernel(GemmArgs g, Rop
         const int m = (t % MB) * 16 + lrow;
         const int en = r0 + (t / MB) * 16 + lgrp * 4;
         const bool live = t < RG * MB && g.out_kind != OUT_ACC;
-        e_sx[ti] = (live && m < g.m) ? g.sa[m] : 0.0f;
+        e_sx[ti] = (live && m < g.m) ? (rowcol ? g.sa[m] : g.sa[0] * g.sb[0]) : 0.0f;
         e_res[ti] = (g.resid && live && m < g.m && en < r1)
             ? *reinterpret_cast<const u32x2*>(static_cast<const uint16_t*>(g.resid) + (size_t)m * g.n + en)
             : u32x2{0u, 0u};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const bool in = live && en + j < r1;
-            e_sw[ti][j] = in ? g.sb[en + j] : 0.0f;
+            e_sw[ti][j] = in ? (rowcol ? g.sb[en + j] : 1.0f) : 0.0f;
             e_b[ti][j] = (in && g.bias) ? bf16_to_f32(static_cast<const uint16_t*>(g.bias)[en + j]) : 0.0f;
         }
     }
@@ -110,11 +129,11 @@ __global__ __launch_bounds__(NW * 64) void gemv_int8_rows_kernel(GemmArgs g, Rop
         }
     }
 
-    i32x4 acc[RG][MB];
+    Acc acc[RG][MB];
 #pragma unroll
     for (int r = 0; r < RG; ++r)
 #pragma unroll
-        for (int b = 0; b < MB; ++b) acc[r][b] = i32x4{0, 0, 0, 0};
+        for (int b = 0; b < MB; ++b) acc[r][b] = Acc{0, 0, 0, 0};
 
     uint8_t* const wpatch = smem + wave * WAVE_LDS;
     uint8_t* const xpatch = wpatch + 4096;
@@ -164,12 +183,21 @@ __global__ __launch_bounds__(NW * 64) void gemv_int8_rows_kernel(GemmArgs g, Rop
                 } else {
                     u32x4 wf[4];
                     to_operand_order(wpatch, lane, ring[t][s], wf);
+                    if constexpr (Op::kIsInt) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
+                        for (int j = 0; j < 4; ++j)
 #pragma unroll
-                        for (int b = 0; b < MB; ++b)
-                            acc[s < MB ? 0 : s - MB][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
-                                (i32x4)wf[j], (i32x4)xf[b][j], acc[s < MB ? 0 : s - MB][b], 0, 0, 0);
+                            for (int b = 0; b < MB; ++b)
+                                acc[s < MB ? 0 : s - MB][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
+                                    (i32x4)wf[j], (i32x4)xf[b][j], acc[s < MB ? 0 : s - MB][b], 0, 0, 0);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; j += 2)
+#pragma unroll
+                            for (int b = 0; b < MB; ++b)
+                                acc[s < MB ? 0 : s - MB][b] = OpF8<Op::kFmt>::mma(
+                                    wf[j], wf[j + 1], xf[b][j], xf[b][j + 1], acc[s < MB ? 0 : s - MB][b]);
+                    }
                 }
                 issue(ring[t][s], ib + t + IB, s);
                 __builtin_amdgcn_sched_barrier(0);
@@ -179,7 +207,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_int8_rows_kernel(GemmArgs g, Rop
 
     // sum the waves' partials through LDS (the patches are free now)
     __syncthreads();
-    i32x4* const red = reinterpret_cast<i32x4*>(smem);  // [NW] x WAVE_LDS bytes
+    Acc* const red = reinterpret_cast<Acc*>(smem);  // [NW] x WAVE_LDS bytes
 #pragma unroll
     for (int r = 0; r < RG; ++r)
 #pragma unroll
@@ -189,7 +217,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_int8_rows_kernel(GemmArgs g, Rop
     for (int ti = 0; ti < TASKS; ++ti) {
         const int t = wave + ti * NW;
         if (t >= RG * MB) break;
-        i32x4 sum = red[t * 64 + lane];
+        Acc sum = red[t * 64 + lane];
 #pragma unroll
         for (int w = 1; w < NW; ++w) sum += red[w * (WAVE_LDS / 16) + t * 64 + lane];
         const int r = t / MB, b = t % MB;
@@ -198,7 +226,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_int8_rows_kernel(GemmArgs g, Rop
         if (m >= g.m || en >= r1) continue;
         const size_t o = (size_t)m * g.n + en;
         if (g.out_kind == OUT_ACC) {
-            int* out = static_cast<int*>(g.out);
+            typename Op::AccScalar* out = static_cast<typename Op::AccScalar*>(g.out);
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 if (en + j < r1) out[o + j] = sum[j];
@@ -209,6 +237,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_int8_rows_kernel(GemmArgs g, Rop
         for (int j = 0; j < 4; ++j) {
             // product and bias add rounded separately (no fused multiply-add): the
             // int8 epilogue is specified as elementwise fp32 on the exact integer
+            // (per-tensor fp8: e_sx is the product of the two steps, e_sw is 1)
 #pragma clang fp contract(off)
             const float f = (float)sum[j] * e_sx[ti] * e_sw[ti][j];
             v[j] = f + e_b[ti][j];
@@ -268,6 +297,16 @@ __global__ __launch_bounds__(NW * 64) void gemv_int8_rows_kernel(GemmArgs g, Rop
                 if (en + j < r1) out[o + j] = f32_to_bf16(v[j]);
         }
     }
+}
+
+template <int RG, int MB, int NW, int IB, bool ROPE>
+__global__ __launch_bounds__(NW * 64) void gemv_int8_rows_kernel(GemmArgs g, RopeCacheArgs rc, int rows_per_wg) {
+    gemv_rows_body<RowsOpI8, RG, MB, NW, IB, ROPE>(g, rc, rows_per_wg, true);
+}
+
+template <int Fmt, int RG, int MB, int NW>
+__global__ __launch_bounds__(NW * 64) void gemv_fp8_rows_kernel(GemmArgs g, int rows_per_wg, int rowcol) {
+    gemv_rows_body<RowsOpF8<Fmt>, RG, MB, NW, 1, false>(g, RopeCacheArgs{}, rows_per_wg, rowcol != 0);
 }
 
 template <int RG, int MB, int NW>

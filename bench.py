@@ -502,12 +502,22 @@ def main():
             for w in ring:
                 check(lib.astrai_w8a8_gemv_int8_ptpc(gx.data_ptr(), w.data_ptr(), gsx.data_ptr(), gsw.data_ptr(),
                                                      None, gy.data_ptr(), gm, gn, gk, 0, stream))
+        # the same four buffers read as e4m3fn codes by the fp8 instance of the row-range kernel
+        # (arbitrary bytes, NaN codes included: only time and traffic are of interest here)
+        one = torch.ones(1, device=dev)
+        for gm in gemv_ms:
+            gx8 = torch.randint(-127, 128, (gm, gk), dtype=torch.int8, device=dev)
+            gy = torch.empty(gm, gn, device=dev, dtype=torch.bfloat16)
+            for w in ring:
+                check(lib.astrai_w8a8_gemm_fp8_pt(gx8.data_ptr(), w.data_ptr(), one.data_ptr(), one.data_ptr(),
+                                                  None, None, gy.data_ptr(), gm, gn, gk, 0, 0, stream))
         torch.cuda.synchronize()
         print(json.dumps({"pmc_mode": True, "gemm_launches": 5, "copy_launches": 4,
                           "copy_bytes_each_way": 256 << 20,
                           "gemm_algorithmic_bytes": 2 * M * K + 2 * M * N,
                           "gemv_launches": "4 each at M = 1 (dot kernel), 4, 16, 64 (rows kernel), 11008x4096, "
-                                           "every launch on another 45 MB weight buffer",
+                                           "every launch on another 45 MB weight buffer; then the same 16 launches "
+                                           "of the fp8 rows kernel",
                           "gemv_algorithmic_bytes": {f"M{m}": gn * gk + m * gk + 2 * m * gn + 4 * gn + 4 * m
                                                      for m in gemv_ms}}))
         return
@@ -784,6 +794,33 @@ def main():
                 "sample": "the whole call at each M (exact int8 x int8 -> int32 matmul + scale epilogue -> bf16), "
                           "median of 5 after 1 warm-up", **cpu_c2}
         del ring
+
+        # ---- the same shape with fp8 e4m3fn operands and per-tensor steps (seed-2 tensors, the
+        # oracle's quantizer): the row-range decode kernel on the fp8 MFMA, same weight ring
+        sw8 = O2.dynamic_scale(w2).reshape(1)
+        w8c, _ = O2.fp8_quantize(w2, sw8, 0)
+        ring8 = [w8c.to(dev).clone() for _ in range(10)]
+        sw8d = sw8.to(dev)
+        gemv8 = {}
+        for m in (1, 4, 16, 64):
+            sx8 = O2.dynamic_scale(x2_all[:m]).reshape(1)
+            x8c, _ = O2.fp8_quantize(x2_all[:m], sx8, 0)
+            x8, sx8d = x8c.to(dev), sx8.to(dev)
+            y8 = torch.empty(m, N2, device=dev, dtype=torch.bfloat16)
+
+            def launch8(i, x8=x8, sx8d=sx8d, y8=y8, m=m):
+                check(lib.astrai_w8a8_gemm_fp8_pt(
+                    x8.data_ptr(), ring8[i % len(ring8)].data_ptr(), sx8d.data_ptr(), sw8d.data_ptr(), None,
+                    None, y8.data_ptr(), m, N2, K2, 0, 0, torch.cuda.current_stream().cuda_stream))
+
+            us = _graph_us(launch8)
+            nbytes = N2 * K2 + m * K2 + 2 * m * N2 + 8
+            gbs = nbytes / (us * 1e-6) / 1e9
+            gemv8[f"M{m}"] = {"us": round(us, 2), "GB/s": round(gbs, 0),
+                              "frac_hbm_peak": round(gbs / PEAK_HBM_GBS, 4)}
+        extra["fp8_gemv_11008x4096_hbm_ring"] = {"data": "BASELINE config 2 tensors (seed 2) as e4m3fn, per-tensor steps",
+                                                 **gemv8}
+        del ring8
 
         # ---- config 0: 16 x 2048 x 2048 int8 linear (launch-latency bound), seed-0 tensors
         xc, wc, _ = O2.make_inputs(0, 16, 2048, 2048)

@@ -222,6 +222,38 @@ def test_mm_fp8_k_not_in_16_byte_pieces_zero_padded(ops, fmt, m, n, k):
     assert_bf16_close(out, O.fp8_gemm(a8, b8, sa_r, sb), what=f"mm_fp8 {name} padded K, row scales")
 
 
+@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("m,n,k", [(1, 11008, 4096), (4, 11008, 4096), (16, 3072, 2048), (33, 2048, 5632),
+                                   (64, 11008, 4096), (7, 1001, 512), (48, 130, 256), (17, 6144, 2048)])
+def test_mm_fp8_decode_shapes_row_range_kernel(ops, fmt, m, n, k):
+    """At most 64 activation rows with K % 256 == 0: the row-range decode kernel on fp8 operands
+    (weights streamed once, fp32 partials of the waves added in a fixed order). Per-tensor steps
+    with and without bias, one step per row and column, and the raw fp32 accumulator."""
+    from astrai_amd.extension import _cabi
+    print(f"case fmt={fmt} m={m} n={n} k={k}", flush=True)
+    g = torch.Generator().manual_seed(11 * m + 5 * n + k + fmt)
+    dt = torch.float8_e5m2 if fmt else torch.float8_e4m3fn
+    a8 = (torch.randn(m, k, generator=g) * 1.5).to(dt)
+    b8 = (torch.randn(n, k, generator=g) * 1.5).to(dt)
+    sa, sb = torch.tensor([0.37]), torch.tensor([0.011])
+    ad, bd = a8.to(DEV), b8.to(DEV)
+    out = ops.mm_fp8(ad, bd, sa.to(DEV), sb.to(DEV))
+    assert_bf16_close(out, O.fp8_gemm(a8, b8, sa, sb), what="decode rows, per tensor")
+    bias = torch.randn(n, generator=g).to(torch.bfloat16)
+    out = _cabi.mm_fp8(ad, bd, sa.to(DEV), sb.to(DEV), 0, None, bias.to(DEV))
+    assert_bf16_close(out, O.fp8_gemm_bias(a8, b8, sa, sb, bias), what="decode rows, bias")
+    sa_r = torch.exp2(torch.rand(m, 1, generator=g) * 6.0 - 3.0)
+    sb_r = torch.exp2(torch.rand(n, generator=g) * 6.0 - 3.0)
+    out = _cabi.mm_fp8(ad, bd, sa_r.to(DEV), sb_r.to(DEV), 0, None, bias.to(DEV))
+    assert_bf16_close(out, O.fp8_gemm_bias(a8, b8, sa_r, sb_r, bias), what="decode rows, row/column steps")
+    acc = _cabi.mm_fp8_acc(ad, bd).cpu()
+    want = a8.double() @ b8.double().t()
+    bound = (a8.double().abs() @ b8.double().abs().t()) * 2.0 ** -16 + 1e-30
+    assert acc.dtype == torch.float32 and bool(((acc.double() - want).abs() <= bound).all())
+    # the same call twice gives the same bits (the waves' partials are added in a fixed order)
+    assert torch.equal(acc, _cabi.mm_fp8_acc(ad, bd).cpu())
+
+
 def test_mm_fp8_rejects_bad_arguments(ops):
     a8 = torch.zeros(4, 16, dtype=torch.float8_e4m3fn, device=DEV)
     b5 = torch.zeros(4, 16, dtype=torch.float8_e5m2, device=DEV)
