@@ -168,7 +168,7 @@ void launch_rows(const GemmArgs& g, const RopeCacheArgs& rc, hipStream_t stream)
     else launch_rows_mb<1, 4, ROPE>(g, rc, p, stream);
 }
 
-// fp8: the same plan; at most 64 tokens (four token groups), bf16 or fp32-accumulator output
+// fp8: the same plan and the same token-group instances; bf16 or fp32-accumulator output
 template <int Fmt, int RG, int MB, int NW>
 void launch_rows_fp8_inst(const GemmArgs& g, const RowsPlan& p, bool rowcol, hipStream_t stream) {
     constexpr int lds_bytes = gemv_rows_lds_bytes<RG, MB, NW>();
@@ -184,7 +184,12 @@ void launch_rows_fp8_mb(const GemmArgs& g, const RowsPlan& p, bool rowcol, hipSt
         case 1: launch_rows_fp8_inst<Fmt, RG, 1, NW>(g, p, rowcol, stream); break;
         case 2: launch_rows_fp8_inst<Fmt, RG, 2, NW>(g, p, rowcol, stream); break;
         case 3: launch_rows_fp8_inst<Fmt, RG, 3, NW>(g, p, rowcol, stream); break;
-        default: launch_rows_fp8_inst<Fmt, RG, 4, NW>(g, p, rowcol, stream); break;
+        case 4: launch_rows_fp8_inst<Fmt, RG, 4, NW>(g, p, rowcol, stream); break;
+        default:
+            if constexpr (NW == 8) launch_rows_fp8_inst<Fmt, RG, 4, NW>(g, p, rowcol, stream);  // at most 64 tokens there
+            else if ((g.m + 15) / 16 <= 6) launch_rows_fp8_inst<Fmt, RG, 6, NW>(g, p, rowcol, stream);
+            else launch_rows_fp8_inst<Fmt, RG, 8, NW>(g, p, rowcol, stream);
+            break;
     }
 }
 
@@ -193,14 +198,14 @@ void launch_rows_fp8(const GemmArgs& g, bool rowcol, hipStream_t stream) {
     const RowsPlan p = plan_rows(g);
     if (p.rg == 3) launch_rows_fp8_mb<Fmt, 3, 4>(g, p, rowcol, stream);
     else if (p.rg == 2) launch_rows_fp8_mb<Fmt, 2, 4>(g, p, rowcol, stream);
-    else if (p.nw == 8) launch_rows_fp8_mb<Fmt, 1, 8>(g, p, rowcol, stream);
+    else if (p.nw == 8 && g.m <= 64) launch_rows_fp8_mb<Fmt, 1, 8>(g, p, rowcol, stream);
     else launch_rows_fp8_mb<Fmt, 1, 4>(g, p, rowcol, stream);
 }
 
 }  // namespace
 
 bool launch_gemv_fp8(const GemmArgs& g, int fmt, int scale_kind, hipStream_t stream) {
-    if (g.m <= 0 || g.m > 64 || g.n <= 0 || g.k <= 0 || (g.k & 255) != 0) return false;
+    if (g.m <= 0 || g.m > 128 || g.n <= 0 || g.k <= 0 || (g.k & 255) != 0) return false;
     if ((int64_t)g.n * g.k >= ((int64_t)1 << 31)) return false;
     if (g.out_kind != OUT_BF16 && g.out_kind != OUT_ACC) return false;
     if (scale_kind != SCALE_TENSOR && scale_kind != SCALE_ROWCOL) return false;

@@ -1,4 +1,4 @@
-// Batched-decode W8A8 kernel (int8: 2 <= M <= 128 tokens; fp8: 1 <= M <= 64): bandwidth-bound. The weight
+// Batched-decode W8A8 kernel (int8: 2 <= M <= 128 tokens; fp8: 1 <= M <= 128): bandwidth-bound. The weight
 // matrix is streamed from HBM exactly once with the streaming cache hint; what decides the
 // time besides that stream is how often the activation block X[M,K] is pulled out of
 // L2 again (every workgroup that owns weight rows over all of K needs all of it), how

@@ -224,7 +224,7 @@ void launch_gemm_generic(const GemmArgs& g, int op /*0=i8,1=e4m3,2=e5m2*/, int s
 
 // gemv_int8.hip: decode-shape int8 kernels (one token: dot kernel; 2..128 tokens: row-range kernel), k % 256 == 0.
 bool launch_gemv_int8(const GemmArgs& g, hipStream_t stream);
-// the row-range kernel on fp8 operands: at most 64 tokens, k % 256 == 0, bf16 or fp32-accumulator
+// the row-range kernel on fp8 operands: at most 128 tokens, k % 256 == 0, bf16 or fp32-accumulator
 // output, per-tensor or per-row / per-column steps; false when the shape does not fit
 bool launch_gemv_fp8(const GemmArgs& g, int fmt /*0=e4m3,1=e5m2*/, int scale_kind, hipStream_t stream);
 // the fused q|k|v projection of up to 64 tokens with rotary embedding and KV-cache write

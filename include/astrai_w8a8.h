@@ -467,7 +467,7 @@ int astrai_w8a8_quantize_bf16_fp8_block128_weight(const void* w_bf16, void* w8, 
  *   OUT_BF16: out = bf16(acc * *sa * *sb + bias[n])   (bias bf16 [N] or NULL; one rounding)
  *   OUT_E4M3: out = sat_e4m3(acc * *sa * *sb * *out_scale)   (bias must be NULL)
  *   OUT_ACC : out = acc as fp32 (parity/debug surface; scales ignored)
- * a8 and b8 share `fmt`. At most 64 rows of `a8` with K % 256 == 0 (decode steps; bf16 or
+ * a8 and b8 share `fmt`. At most 128 rows of `a8` with K % 256 == 0 (decode steps; bf16 or
  * accumulator output) run on the weight-streaming row-range kernel, as the int8 decode shapes do.
  * Any M, N, K >= 1 is accepted; the MFMA kernels fetch rows in 16-byte
  * pieces, so K % 16 != 0 (this and every other GEMM entry of this header) takes a plain any-shape

@@ -224,9 +224,10 @@ def test_mm_fp8_k_not_in_16_byte_pieces_zero_padded(ops, fmt, m, n, k):
 
 @pytest.mark.parametrize("fmt", [0, 1])
 @pytest.mark.parametrize("m,n,k", [(1, 11008, 4096), (4, 11008, 4096), (16, 3072, 2048), (33, 2048, 5632),
-                                   (64, 11008, 4096), (7, 1001, 512), (48, 130, 256), (17, 6144, 2048)])
+                                   (64, 11008, 4096), (7, 1001, 512), (48, 130, 256), (17, 6144, 2048),
+                                   (65, 3072, 2048), (96, 11008, 4096), (128, 2048, 5632), (113, 777, 768)])
 def test_mm_fp8_decode_shapes_row_range_kernel(ops, fmt, m, n, k):
-    """At most 64 activation rows with K % 256 == 0: the row-range decode kernel on fp8 operands
+    """At most 128 activation rows with K % 256 == 0: the row-range decode kernel on fp8 operands
     (weights streamed once, fp32 partials of the waves added in a fixed order). Per-tensor steps
     with and without bias, one step per row and column, and the raw fp32 accumulator."""
     from astrai_amd.extension import _cabi
