@@ -197,14 +197,16 @@ __global__ __launch_bounds__(Mid128Cfg::THREADS) void gemm_mid128_kernel(GemmArg
     }
 }
 
-// bf16 output, K in whole slabs, and a shape this tile size suits: at least 192 tiles of 128 x 128
-// (below that the 64 x 64 tiles of the generic kernel spread the work further and win: 512 x 3072 x
-// 2048 13.2 against 15.1 us, 1024 x 2048 x 2048 13.3 against 14.9 us; from 192 tiles on this kernel
-// does: 1024 x 3072 x 2048 16.0 against 23.6 us, 2048 x 3072 x 2048 22.9 against 30.7 us)
+// bf16 output, K in whole slabs, and a shape this tile size suits: at least 140 tiles of 128 x 128
+// (below that the 64 x 64 tiles of the generic kernel spread the work further and win or draw: 512 x
+// 3072 x 2048 13.2 against 15.1 us, 1024 x 2048 x 2048 13.3 against 14.9 us, 512 x 4096 x 4096 (128
+// tiles) 22.5 against 22.3 us; from there on this kernel wins: 768 x 3072 x 2048 (144 tiles) 14.2
+// against 16.4 us, 256 x 11008 x 4096 (172) 23.7 against 28.6 us, 1024 x 3072 x 2048 16.0 against
+// 23.6 us, 2048 x 3072 x 2048 22.9 against 30.7 us)
 inline bool mid128_shape_ok(const GemmArgs& g) {
     if (!tiled_shape_ok(g) || (g.k & 127) != 0 || g.k < 128 || g.out_kind != OUT_BF16) return false;
     const int64_t tiles = (int64_t)((g.m + 127) / 128) * ((g.n + 127) / 128);
-    return tiles >= 192;
+    return tiles >= 140;
 }
 
 template <class Op, int ScaleKind>
