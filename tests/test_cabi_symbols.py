@@ -122,3 +122,33 @@ def test_decode_attention_split_plan():
     assert _cabi.decode_nsplit(256, 4096) == 1
     assert _cabi.decode_nsplit(1, 64) == 1
     assert _cabi.decode_nsplit(0, 0) == 1
+
+
+def test_k_padding_plan_of_the_wrappers():
+    """Which products the wrappers re-lay with zero codes (K % 16 != 0 and at least 2^24
+    multiply-adds) and to which K; values and the zero tail, on CPU tensors."""
+    import torch
+
+    a = torch.randint(-127, 128, (300, 1032), dtype=torch.int8)
+    b = torch.randint(-127, 128, (520, 1032), dtype=torch.int8)
+    pa, pb, kp = _cabi._pad_k(a, b)
+    assert kp == 1152 and pa.shape == (300, kp) and pb.shape == (520, kp) and pa.dtype == torch.int8
+    assert torch.equal(pa[:, :1032], a) and not pa[:, 1032:].any() and not pb[:, 1032:].any()
+    assert _cabi._pad_k(a[:64], b)[2] == 1280          # decode kernels take whole 256-byte items
+    assert _cabi._pad_k(a[:, :1024].contiguous(), b[:, :1024].contiguous())[0].shape == (300, 1024)  # K % 16 == 0
+    assert _cabi._pad_k(a[:8], b[:8])[2] == 1032        # too small to repay the copies
+    f = torch.randn(300, 1032).to(torch.float8_e4m3fn)
+    pf = _cabi._pad_k(f, b.view(torch.float8_e4m3fn))[0]
+    assert pf.dtype == torch.float8_e4m3fn and torch.equal(pf[:, :1032].view(torch.uint8), f.view(torch.uint8))
+    assert not pf[:, 1032:].view(torch.uint8).any()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0 and "--gpus 1" in r.stderr and not r.stdout.strip()
