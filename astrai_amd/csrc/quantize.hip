@@ -451,6 +451,14 @@ __global__ __launch_bounds__(kThreads) void add_rmsnorm_quantize_int8_rows_kerne
     const int64_t row = blockIdx.x;
     const int64_t nvec = k >> 3;
     float v[kCache][8];
+    // the norm weights are requested with the row, not after the reduction's barrier (a load does
+    // not move across it by itself, and its latency would then sit in the middle of the chain)
+    u32x4 wr[kCache];
+#pragma unroll
+    for (int c = 0; c < kCache; ++c) {
+        const int64_t i = threadIdx.x + (int64_t)c * kThreads;
+        wr[c] = i < nvec ? *reinterpret_cast<const u32x4*>(w + i * 8) : u32x4{0u, 0u, 0u, 0u};
+    }
     float ss = 0.0f;
 #pragma unroll
     for (int c = 0; c < kCache; ++c) {
@@ -475,7 +483,7 @@ __global__ __launch_bounds__(kThreads) void add_rmsnorm_quantize_int8_rows_kerne
         const int64_t i = threadIdx.x + (int64_t)c * kThreads;
         if (i < nvec) {
             float g[8];
-            unpack8(*reinterpret_cast<const u32x4*>(w + i * 8), g);
+            unpack8(wr[c], g);
 #pragma unroll
             for (int j = 0; j < 8; ++j) v[c][j] = g[j] * (rstd * v[c][j]);
             const u32x4 packed = round8_bf16(v[c]);
