@@ -55,11 +55,12 @@ __global__ __launch_bounds__(64) void gemv_int8_dot_kernel(GemmArgs g) {
     // first so that their latency hides under the weight stream
     const int en = n0 + lane;
     const bool writer = lane < R && en < g.n;
-    float e_sx = 0.0f, e_sw = 0.0f, e_b = 0.0f;
+    float e_sx = 0.0f, e_sw = 0.0f, e_b = 0.0f, e_r = 0.0f;
     if (writer && g.out_kind != OUT_ACC) {
         e_sx = g.sa[0];
         e_sw = g.sb[en];
         if (g.bias) e_b = bf16_to_f32(static_cast<const uint16_t*>(g.bias)[en]);
+        if (g.resid) e_r = bf16_to_f32(static_cast<const uint16_t*>(g.resid)[en]);
     }
 
     int acc[R] = {};
@@ -99,7 +100,9 @@ __global__ __launch_bounds__(64) void gemv_int8_dot_kernel(GemmArgs g) {
             // int8 epilogue is specified as elementwise fp32 on the exact integer
 #pragma clang fp contract(off)
             const float scaled = (float)mine * e_sx * e_sw;
-            static_cast<uint16_t*>(g.out)[en] = f32_to_bf16(scaled + e_b);
+            uint16_t y = f32_to_bf16(scaled + e_b);
+            if (g.resid) y = f32_to_bf16(bf16_to_f32(y) + e_r);   // bf16(y + residual) on the rounded y
+            static_cast<uint16_t*>(g.out)[en] = y;
         }
     }
 }
@@ -228,9 +231,10 @@ bool launch_gemv_int8(const GemmArgs& g, hipStream_t stream) {
     if (g.m <= 0 || g.m > 128 || g.n <= 0 || g.k <= 0 || (g.k & 255) != 0) return false;
     const int64_t lim = (int64_t)1 << 31;
     if ((int64_t)g.n * g.k >= lim) return false;
-    // the residual epilogue is the row-range kernel's, on whole 8-byte pieces of bf16 rows
-    if (g.resid && ((g.n & 3) != 0 || g.out_kind != OUT_BF16)) return false;
-    if (g.m == 1 && !g.resid)
+    // the row-range kernel's residual epilogue works on whole 8-byte pieces of bf16 rows
+    if (g.resid && g.out_kind != OUT_BF16) return false;
+    if (g.resid && g.m > 1 && (g.n & 3) != 0) return false;
+    if (g.m == 1)
         launch_dot(g, stream);
     else
         launch_rows<false>(g, RopeCacheArgs{}, stream);

@@ -214,7 +214,8 @@ def test_silu_mul_quantize_fp8(C, rows, width, fused_buffer, fmt):
 @pytest.mark.parametrize("m,n,k,bias", [
     (32, 2048, 2048, False),     # config-4 output projection at a decode step (row-range kernel)
     (32, 2048, 5632, False),     # config-4 down projection
-    (1, 2048, 2048, False), (2, 44, 256, True), (17, 3072, 512, True), (64, 2048, 2048, False),
+    (1, 2048, 2048, False), (1, 2049, 5632, True), (1, 11008, 4096, False), (1, 3, 256, True),   # one token: dot kernel
+    (2, 44, 256, True), (17, 3072, 512, True), (64, 2048, 2048, False),
     (100, 1028, 256, False), (128, 2048, 2048, True),
     (48, 11008, 256, True), (64, 8192, 512, False),   # 33..64 tokens on long row ranges
     (16384, 2048, 2048, False),  # config-4 output projection at prefill (large-tile kernel, 64 x 8 tiles)
