@@ -522,6 +522,15 @@ def main():
                                                      for m in gemv_ms}}))
         return
 
+    flop = 2.0 * M * N * K
+    # the kernel's own time first (fixed protocol, see `roofline.timing`), so that the driver's
+    # --warmup / --steps below find the GPU at its working clocks, not coming out of idle
+    def step_batch():
+        for _ in range(LAUNCHES_PER_BATCH):
+            step()
+
+    kern_us, proto = _protocol_us(step_batch)
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -531,14 +540,8 @@ def main():
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
-    flop = 2.0 * M * N * K
     value = flop / (ms_per_step * 1e-3) / 1e12
 
-    def step_batch():
-        for _ in range(LAUNCHES_PER_BATCH):
-            step()
-
-    kern_us, proto = _protocol_us(step_batch)
     achieved = flop / (kern_us * 1e-6) / 1e12
     roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_FP8_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP8_TFLOPS, 4),
@@ -549,7 +552,7 @@ def main():
                 "avg_launch_us": round(kern_us, 2),
                 "timing": {"what": "HIP events on the launch stream; median of batch averages after a warm-up "
                                    "that ends when two consecutive batches agree within 2%; independent of "
-                                   "--steps / --warmup", **proto}}
+                                   "--steps / --warmup, and run before them", **proto}}
     if "mfma_fp8_random_TFLOPs" in ceilings:
         # the same kernel against what this GPU's MFMA pipe sustains on random operand bits
         roofline["measured_ceiling"] = {
