@@ -14,7 +14,15 @@ namespace {
 template <int Fmt, int ScaleKind>
 void launch_for(const GemmArgs& g, hipStream_t stream) {
 #ifndef W8A8_NO_WAVE128
-    if (wave128_shape_ok(g)) return launch_wave128<Op32F8<Fmt>, ScaleKind>(g, stream);
+    if (wave128_shape_ok(g)) {
+        if (const int r = ragged_tail_rows(g)) {
+            GemmArgs head, tail;
+            split_rows(g, r, ScaleKind == SCALE_ROWCOL, head, tail);
+            if (wave128_shape_ok(head) && launch_gemv_fp8(tail, Fmt, ScaleKind, stream))   // (disjoint rows: either order)
+                return launch_wave128<Op32F8<Fmt>, ScaleKind>(head, stream);
+        }
+        return launch_wave128<Op32F8<Fmt>, ScaleKind>(g, stream);
+    }
 #endif
     if (pingpong_shape_ok(g)) return launch_pingpong<Op32F8<Fmt>, ScaleKind>(g, stream);
     if (mid128_shape_ok(g)) return launch_mid128<Op32F8<Fmt>, ScaleKind>(g, stream);

@@ -12,9 +12,17 @@ namespace w8a8 {
 bool launch_gemm_int8_tiled(const GemmArgs& g, hipStream_t stream) {
     if (!tiled_shape_ok(g)) return false;
 #ifndef W8A8_NO_WAVE128
-    if (wave128_shape_ok(g))
+    if (wave128_shape_ok(g)) {
+        if (const int r = ragged_tail_rows(g)) {
+            GemmArgs head, tail;
+            split_rows(g, r, true, head, tail);
+            if (wave128_shape_ok(head) && launch_gemv_int8(tail, stream)) {   // (disjoint rows: either order)
+                launch_wave128<Op32I8, SCALE_ROWCOL>(head, stream);
+                return true;
+            }
+        }
         launch_wave128<Op32I8, SCALE_ROWCOL>(g, stream);
-    else
+    } else
 #endif
     if (pingpong_shape_ok(g))
         launch_pingpong<Op32I8, SCALE_ROWCOL>(g, stream);
@@ -36,6 +44,14 @@ bool launch_gemm_int8_resid(const GemmArgs& g, hipStream_t stream) {
     if (!g.resid || g.out_kind != OUT_BF16) return false;
     if (g.m <= 128 && launch_gemv_int8(g, stream)) return true;
     if (!tiled_shape_ok(g) || !wave128_shape_ok(g) || g.bias != nullptr) return false;
+    if (const int r = ragged_tail_rows(g)) {
+        GemmArgs head, tail;
+        split_rows(g, r, true, head, tail);
+        if (wave128_shape_ok(head) && launch_gemv_int8(tail, stream)) {
+            launch_wave128<Op32I8, SCALE_ROWCOL, EPI_RESID>(head, stream);
+            return true;
+        }
+    }
     launch_wave128<Op32I8, SCALE_ROWCOL, EPI_RESID>(g, stream);
     return true;
 }

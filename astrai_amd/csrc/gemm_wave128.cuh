@@ -595,6 +595,33 @@ inline bool wave128_shape_ok(const GemmArgs& g) {
     return pingpong_shape_ok(g) && g.out_kind == OUT_BF16 && (g.n & 7) == 0 && g.n <= (1 << 22);
 }
 
+// A token count a little above a multiple of 256 (M = 256 q + r, 0 < r <= 128) can cost the
+// large-tile kernel a whole extra round of workgroups for r rows (4100 x 4096 x 4096: 272 tiles on
+// 256 compute units, 96 us against 69 us at 4096 rows). When it does, and the weight-streaming
+// decode kernel takes the shape, those rows are better served by it in a launch of their own
+// (70 us for the two). Returns r then, else 0.
+inline int ragged_tail_rows(const GemmArgs& g) {
+    const int r = g.m & 255;
+    if (r == 0 || r > 128 || g.m < 256 || (g.k & 255) != 0) return 0;
+    const int64_t tn = (g.n + 255) / 256;
+    const int64_t full = (int64_t)((g.m + 255) / 256) * tn, cut = (int64_t)(g.m / 256) * tn;
+    return (full + 255) / 256 > (cut + 255) / 256 ? r : 0;
+}
+
+// the first m - r rows and the last r rows of a product as calls of their own (bf16 output;
+// `rowcol`: sa holds one step per row)
+inline void split_rows(const GemmArgs& g, int r, bool rowcol, GemmArgs& head, GemmArgs& tail) {
+    head = g;
+    head.m = g.m - r;
+    tail = g;
+    tail.m = r;
+    const size_t row0 = (size_t)head.m;
+    tail.a = static_cast<const uint8_t*>(g.a) + row0 * (size_t)g.k;
+    if (rowcol) tail.sa = g.sa + row0;
+    tail.out = static_cast<uint8_t*>(g.out) + row0 * (size_t)g.n * 2;
+    if (g.resid) tail.resid = static_cast<const uint8_t*>(g.resid) + row0 * (size_t)g.n * 2;
+}
+
 template <class Op, int ScaleKind, int Epi = EPI_PLAIN>
 inline void launch_wave128(const GemmArgs& g, hipStream_t stream, const RopeCacheArgs& rc = RopeCacheArgs{}) {
     using Cfg = Wave128Cfg;

@@ -255,6 +255,31 @@ def test_mm_fp8_decode_shapes_row_range_kernel(ops, fmt, m, n, k):
     assert torch.equal(acc, _cabi.mm_fp8_acc(ad, bd).cpu())
 
 
+@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("m,n,k", [(4100, 4096, 512), (4224, 4096, 256)])
+def test_mm_fp8_token_tail_past_a_round_of_large_tiles(ops, fmt, m, n, k):
+    """The last few rows of a block that would cost the large-tile kernel a round of their own run
+    on the decode kernel in a second launch: rows either side of the seam against the oracle, per
+    tensor with bias and with row / column steps."""
+    from astrai_amd.extension import _cabi
+    print(f"case fmt={fmt} m={m} n={n} k={k}", flush=True)
+    g = torch.Generator().manual_seed(m + n + k + fmt)
+    dt = torch.float8_e5m2 if fmt else torch.float8_e4m3fn
+    a8 = (torch.randn(m, k, generator=g) * 1.5).to(dt)
+    b8 = (torch.randn(n, k, generator=g) * 1.5).to(dt)
+    bias = torch.randn(n, generator=g).to(torch.bfloat16)
+    sa, sb = torch.tensor([0.37]), torch.tensor([0.011])
+    cut = m - m % 256
+    rows = torch.cat([torch.arange(0, 5), torch.arange(cut - 6, m)])
+    ad, bd = a8.to(DEV), b8.to(DEV)
+    out = _cabi.mm_fp8(ad, bd, sa.to(DEV), sb.to(DEV), 0, None, bias.to(DEV))[rows.to(DEV)]
+    assert_bf16_close(out, O.fp8_gemm_bias(a8[rows], b8, sa, sb, bias), what="tail rows, per tensor")
+    sa_r = torch.exp2(torch.rand(m, 1, generator=g) * 6.0 - 3.0)
+    sb_r = torch.exp2(torch.rand(n, generator=g) * 6.0 - 3.0)
+    out = _cabi.mm_fp8(ad, bd, sa_r.to(DEV), sb_r.to(DEV), 0, None, None)[rows.to(DEV)]
+    assert_bf16_close(out, O.fp8_gemm_bias(a8[rows], b8, sa_r[rows], sb_r, None), what="tail rows, row/column steps")
+
+
 def test_mm_fp8_rejects_bad_arguments(ops):
     a8 = torch.zeros(4, 16, dtype=torch.float8_e4m3fn, device=DEV)
     b5 = torch.zeros(4, 16, dtype=torch.float8_e5m2, device=DEV)

@@ -91,6 +91,33 @@ def test_k_not_in_16_byte_pieces_zero_padded_bit_exact(C, m, n, k):
     assert torch.equal(ad.cpu(), a) and torch.equal(bd.cpu(), b)
 
 
+@pytest.mark.parametrize("m,n,k", [(4100, 4096, 512), (4224, 4096, 256), (4097, 4104, 768), (8200, 2048, 512)])
+def test_token_tail_past_a_round_of_large_tiles_bit_exact(C, m, n, k):
+    """A few rows more than whole 256-row tiles that would cost the large-tile kernel a round of
+    their own go to the decode kernel in a second launch: the seam must not show -- bf16 output
+    bit-equal to the oracle's epilogue on sampled rows either side of it, with bias and as the
+    residual form."""
+    print(f"case m={m} n={n} k={k}", flush=True)
+    g = torch.Generator().manual_seed(m + n + k)
+    a, b = _rand_i8(g, m, k), _rand_i8(g, n, k)
+    sa = torch.rand(m, generator=g) * 0.02 + 0.001
+    sb = torch.rand(n, generator=g) * 0.02 + 0.001
+    bias = torch.randn(n, generator=g).to(torch.bfloat16)
+    cut = m - m % 256
+    rows = torch.cat([torch.arange(0, 5), torch.arange(cut - 6, m)])
+    acc = O.int8_acc(a[rows], b).float()
+    ad, bd, sad, sbd = a.to(DEV), b.to(DEV), sa.to(DEV), sb.to(DEV)
+    out = C.mm_int8(ad, bd, sad, sbd, None, 0)[rows.to(DEV)].cpu()
+    ref = (acc * sa[rows, None] * sb[None, :]).to(torch.bfloat16)
+    assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+    out = C.mm_int8(ad, bd, sad, sbd, bias.to(DEV), 0)[rows.to(DEV)].cpu()
+    refb = (acc * sa[rows, None] * sb[None, :] + bias.float()).to(torch.bfloat16)
+    assert torch.equal(out.view(torch.int16), refb.view(torch.int16))
+    r = torch.randn(m, n, generator=g).to(torch.bfloat16)
+    fused = C.mm_int8_resid(ad, bd, sad, sbd, r.to(DEV))[rows.to(DEV)].cpu()
+    assert torch.equal(fused.view(torch.int16), (ref + r[rows]).view(torch.int16))
+
+
 def test_golden_integer_cases_including_worst_case_magnitude(C, golden):
     for c in golden("int8_small.json")["gemm"]:
         a = torch.tensor(c["a"], dtype=torch.int8)
