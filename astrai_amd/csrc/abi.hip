@@ -662,7 +662,7 @@ int astrai_w8a8_gemm_fp8_block128(const void* a8, const void* b8, const float* s
     auto s = static_cast<hipStream_t>(stream);
     const w8a8::GemmArgs g =
         pack(a8, b8, sa, sb, nullptr, bias, out, m, n, k, w8a8::OUT_BF16);
-    if (!w8a8::launch_gemm_fp8_block128_tiled(g, s))
+    if (!w8a8::launch_gemv_fp8_block128(g, s) && !w8a8::launch_gemm_fp8_block128_tiled(g, s))
         w8a8::launch_gemm_generic(g, 1, w8a8::SCALE_BLOCK128, s);
     return check_launch("gemm_fp8_block128");
 }

@@ -205,7 +205,38 @@ void launch_rows_fp8(const GemmArgs& g, bool rowcol, hipStream_t stream) {
     else launch_rows_fp8_mb<Fmt, 1, 4>(g, p, rowcol, stream);
 }
 
+template <int RG, int MB, int NW>
+void launch_rows_fp8_block_inst(const GemmArgs& g, const RowsPlan& p, hipStream_t stream) {
+    constexpr int lds_bytes = gemv_rows_lds_bytes<RG, MB, NW>();
+    auto kern = gemv_fp8_block128_rows_kernel<RG, MB, NW>;
+    static std::atomic<uint64_t> lds_allowed{0};
+    allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_allowed);
+    kern<<<dim3((unsigned)p.blocks), dim3(NW * 64), lds_bytes, stream>>>(g, p.rows_per_wg);
+}
+
+template <int RG, int NW>
+void launch_rows_fp8_block_mb(const GemmArgs& g, const RowsPlan& p, hipStream_t stream) {
+    switch ((g.m + 15) / 16) {
+        case 1: launch_rows_fp8_block_inst<RG, 1, NW>(g, p, stream); break;
+        case 2: launch_rows_fp8_block_inst<RG, 2, NW>(g, p, stream); break;
+        case 3: launch_rows_fp8_block_inst<RG, 3, NW>(g, p, stream); break;
+        default: launch_rows_fp8_block_inst<RG, 4, NW>(g, p, stream); break;
+    }
+}
+
 }  // namespace
+
+bool launch_gemv_fp8_block128(const GemmArgs& g, hipStream_t stream) {
+    if (g.m <= 0 || g.m > 64 || g.n <= 0 || g.k <= 0 || (g.k & 255) != 0) return false;
+    if ((int64_t)g.n * g.k >= ((int64_t)1 << 31)) return false;
+    if (g.out_kind != OUT_BF16 || g.resid || g.row_max) return false;
+    const RowsPlan p = plan_rows(g);
+    if (p.rg == 3) launch_rows_fp8_block_mb<3, 4>(g, p, stream);
+    else if (p.rg == 2) launch_rows_fp8_block_mb<2, 4>(g, p, stream);
+    else if (p.nw == 8) launch_rows_fp8_block_mb<1, 8>(g, p, stream);
+    else launch_rows_fp8_block_mb<1, 4>(g, p, stream);
+    return true;
+}
 
 bool launch_gemv_fp8(const GemmArgs& g, int fmt, int scale_kind, hipStream_t stream) {
     if (g.m <= 0 || g.m > 128 || g.n <= 0 || g.k <= 0 || (g.k & 255) != 0) return false;

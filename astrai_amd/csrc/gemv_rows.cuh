@@ -64,6 +64,19 @@ struct RowsOpF8 {
     static constexpr int kFmt = Fmt;
 };
 
+// e4m3fn with one step per 1 x 128 K-group of the activations and per 128 x 128 block of the weights
+// (sa [M, K/128], sb [ceil(N/128), K/128]): each 128-byte half of an item is one K-block, its
+// MFMA result is scaled by the two steps before it joins the accumulator
+struct RowsOpF8Block {
+    using Acc = f32x4;
+    using AccScalar = float;
+    static constexpr bool kIsInt = false;
+    static constexpr int kFmt = 0;
+    static constexpr bool kBlock = true;
+};
+template <class Op, class = void> struct rows_op_block { static constexpr bool value = false; };
+template <class Op> struct rows_op_block<Op, decltype((void)Op::kBlock)> { static constexpr bool value = Op::kBlock; };
+
 // `rowcol`: one step per token and per weight row (always so for int8); else one per tensor
 template <class Op, int RG, int MB, int NW, int IB, bool ROPE>
 __device__ __forceinline__ void gemv_rows_body(const GemmArgs& g, const RopeCacheArgs& rc, int rows_per_wg,
@@ -96,14 +109,16 @@ __device__ __forceinline__ void gemv_rows_body(const GemmArgs& g, const RopeCach
         const int m = (t % MB) * 16 + lrow;
         const int en = r0 + (t / MB) * 16 + lgrp * 4;
         const bool live = t < RG * MB && g.out_kind != OUT_ACC;
-        e_sx[ti] = (live && m < g.m) ? (rowcol ? g.sa[m] : g.sa[0] * g.sb[0]) : 0.0f;
+        if constexpr (rows_op_block<Op>::value) e_sx[ti] = (live && m < g.m) ? 1.0f : 0.0f;   // steps applied per K-block
+        else e_sx[ti] = (live && m < g.m) ? (rowcol ? g.sa[m] : g.sa[0] * g.sb[0]) : 0.0f;
         e_res[ti] = (g.resid && live && m < g.m && en < r1)
             ? *reinterpret_cast<const u32x2*>(static_cast<const uint16_t*>(g.resid) + (size_t)m * g.n + en)
             : u32x2{0u, 0u};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const bool in = live && en + j < r1;
-            e_sw[ti][j] = in ? (rowcol ? g.sb[en + j] : 1.0f) : 0.0f;
+            if constexpr (rows_op_block<Op>::value) e_sw[ti][j] = in ? 1.0f : 0.0f;
+            else e_sw[ti][j] = in ? (rowcol ? g.sb[en + j] : 1.0f) : 0.0f;
             e_b[ti][j] = (in && g.bias) ? bf16_to_f32(static_cast<const uint16_t*>(g.bias)[en + j]) : 0.0f;
         }
     }
@@ -151,6 +166,24 @@ __device__ __forceinline__ void gemv_rows_body(const GemmArgs& g, const RopeCach
     // window each).
     constexpr int P = MB + RG;
     u32x4 ring[IB][P][4];
+    // block steps of an item's two K-blocks, per unit: activations' for token s * 16 + lrow, weights'
+    // for the 128-row block of rows r0 + (s - MB) * 16 + 4 * lgrp .. + 3 (requested with the unit)
+    [[maybe_unused]] f32x2 steps[IB][P];
+    [[maybe_unused]] const int kblocks = K >> 7;
+    auto issue_steps = [&](f32x2& dst, int item, int s) {
+        if constexpr (rows_op_block<Op>::value) {
+            dst = f32x2{0.0f, 0.0f};
+            if (item < i1) {
+                if (s < MB) {
+                    const int m = s * 16 + lrow;
+                    if (m < g.m) dst = *reinterpret_cast<const f32x2*>(g.sa + (size_t)m * kblocks + 2 * item);
+                } else {
+                    const int row = r0 + (s - MB) * 16 + 4 * lgrp;
+                    if (row < r1) dst = *reinterpret_cast<const f32x2*>(g.sb + (size_t)(row >> 7) * kblocks + 2 * item);
+                }
+            }
+        }
+    };
     auto issue = [&](u32x4 (&dst)[4], int item, int s) {
         const bool live = item < i1;
         const uint32_t k0 = (uint32_t)item << 8;
@@ -170,16 +203,21 @@ __device__ __forceinline__ void gemv_rows_body(const GemmArgs& g, const RopeCach
 #pragma unroll
     for (int t = 0; t < IB; ++t)
 #pragma unroll
-        for (int s = 0; s < P; ++s) issue(ring[t][s], i0 + t, s);
+        for (int s = 0; s < P; ++s) {
+            issue(ring[t][s], i0 + t, s);
+            issue_steps(steps[t][s], i0 + t, s);
+        }
 
     for (int ib = i0; ib < i1; ib += IB) {
 #pragma unroll
         for (int t = 0; t < IB; ++t) {
             u32x4 xf[MB][4];
+            [[maybe_unused]] f32x2 xs[MB];
 #pragma unroll
             for (int s = 0; s < P; ++s) {
                 if (s < MB) {
                     to_operand_order(xpatch, lane, ring[t][s], xf[s < MB ? s : 0]);
+                    if constexpr (rows_op_block<Op>::value) xs[s < MB ? s : 0] = steps[t][s];
                 } else {
                     u32x4 wf[4];
                     to_operand_order(wpatch, lane, ring[t][s], wf);
@@ -190,6 +228,18 @@ __device__ __forceinline__ void gemv_rows_body(const GemmArgs& g, const RopeCach
                             for (int b = 0; b < MB; ++b)
                                 acc[s < MB ? 0 : s - MB][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
                                     (i32x4)wf[j], (i32x4)xf[b][j], acc[s < MB ? 0 : s - MB][b], 0, 0, 0);
+                    } else if constexpr (rows_op_block<Op>::value) {
+                        const f32x2 ws = steps[t][s];
+#pragma unroll
+                        for (int j = 0; j < 4; j += 2)
+#pragma unroll
+                            for (int b = 0; b < MB; ++b) {
+                                const f32x4 part = OpF8<0>::mma(wf[j], wf[j + 1], xf[b][j], xf[b][j + 1],
+                                                                f32x4{0.0f, 0.0f, 0.0f, 0.0f});
+                                const float sc = xs[b][j >> 1] * ws[j >> 1];
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) acc[s < MB ? 0 : s - MB][b][e] += part[e] * sc;
+                            }
                     } else {
 #pragma unroll
                         for (int j = 0; j < 4; j += 2)
@@ -200,6 +250,7 @@ __device__ __forceinline__ void gemv_rows_body(const GemmArgs& g, const RopeCach
                     }
                 }
                 issue(ring[t][s], ib + t + IB, s);
+                issue_steps(steps[t][s], ib + t + IB, s);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -307,6 +358,11 @@ __global__ __launch_bounds__(NW * 64) void gemv_int8_rows_kernel(GemmArgs g, Rop
 template <int Fmt, int RG, int MB, int NW>
 __global__ __launch_bounds__(NW * 64) void gemv_fp8_rows_kernel(GemmArgs g, int rows_per_wg, int rowcol) {
     gemv_rows_body<RowsOpF8<Fmt>, RG, MB, NW, 1, false>(g, RopeCacheArgs{}, rows_per_wg, rowcol != 0);
+}
+
+template <int RG, int MB, int NW>
+__global__ __launch_bounds__(NW * 64) void gemv_fp8_block128_rows_kernel(GemmArgs g, int rows_per_wg) {
+    gemv_rows_body<RowsOpF8Block, RG, MB, NW, 1, false>(g, RopeCacheArgs{}, rows_per_wg, false);
 }
 
 template <int RG, int MB, int NW>

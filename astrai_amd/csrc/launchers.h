@@ -227,6 +227,9 @@ bool launch_gemv_int8(const GemmArgs& g, hipStream_t stream);
 // the row-range kernel on fp8 operands: at most 128 tokens, k % 256 == 0, bf16 or fp32-accumulator
 // output, per-tensor or per-row / per-column steps; false when the shape does not fit
 bool launch_gemv_fp8(const GemmArgs& g, int fmt /*0=e4m3,1=e5m2*/, int scale_kind, hipStream_t stream);
+// the same kernel on e4m3fn operands with 128-block steps (sa [M, K/128], sb [ceil(N/128), K/128]):
+// at most 64 tokens, k % 256 == 0, bf16 output
+bool launch_gemv_fp8_block128(const GemmArgs& g, hipStream_t stream);
 // the fused q|k|v projection of up to 64 tokens with rotary embedding and KV-cache write
 // in the epilogue (g.out unused; rc.qkv / rc.ld unused); false when the shape does not fit
 bool launch_gemm_int8_rope_cache(const GemmArgs& g, const RopeCacheArgs& rc, hipStream_t stream);

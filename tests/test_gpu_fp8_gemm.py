@@ -393,6 +393,25 @@ def test_block128_gemm_small(m, n, k):
     assert_bf16_close(out, O.fp8_gemm_blockscaled(x8, w8, sa, sb), what="block128")
 
 
+@pytest.mark.parametrize("m,n,k,bias", [(1, 2048, 7168, False), (16, 2048, 7168, True), (64, 11008, 4096, False),
+                                        (33, 130, 256, True), (4, 7168, 2048, False), (48, 1001, 512, True),
+                                        (7, 2052, 5632, False)])
+def test_block128_decode_shapes_row_range_kernel(m, n, k, bias):
+    """At most 64 activation rows with K % 256 == 0: the block-scaled instance of the row-range
+    decode kernel (each 128-byte half of an item is one K-block, scaled before it is accumulated),
+    wide scale ranges (outliers in 1% of the weights), ragged N, weight blocks cut by workgroup ranges."""
+    from astrai_amd.extension.ops import fp8_block as blk
+    print(f"case m={m} n={n} k={k} bias={bias}", flush=True)
+    x, w, b = O.make_inputs(3, m, n, k, outlier_p=0.01, bias=bias)
+    x8, sa = O.fp8_quantize_act_block128(x)
+    w8, sb = O.fp8_quantize_weight_block128(w)
+    bd = b.to(DEV) if bias else None
+    out = blk.mm_fp8_blockscaled(x8.to(DEV), w8.to(DEV), sa.to(DEV), sb.to(DEV), bd)
+    assert_bf16_close(out, O.fp8_gemm_blockscaled(x8, w8, sa, sb, b if bias else None), what="block128 decode rows")
+    again = blk.mm_fp8_blockscaled(x8.to(DEV), w8.to(DEV), sa.to(DEV), sb.to(DEV), bd)
+    assert torch.equal(out.view(torch.int16), again.view(torch.int16))    # fixed summation order
+
+
 def test_block128_golden_exact_rationals(golden):
     from astrai_amd.extension.ops import fp8_block as blk
     for c in golden("fp8_gemm_small.json")["block128"]:
