@@ -496,7 +496,7 @@ int astrai_w8a8_gemm_fp8_ptpc(const void* a8, const void* b8, const float* sa,
  * Pre-quantized e4m3fn GEMM with 128-block scales. No counterpart in the
  * reference. K must be a multiple of 128.
  *   out[m,n] = bf16( sum_kb (sum_{k in kb} a8[m,k]*b8[n,k]) * sa[m,kb] * sb[n/128,kb] + bias[n] )
-  * At most 64 rows of `a8` with K % 256 == 0 (decode steps) run on the weight-streaming row-range
+ * At most 64 rows of `a8` with K % 256 == 0 (decode steps) run on the weight-streaming row-range
  * kernel, as the per-tensor decode shapes do.
  */
 int astrai_w8a8_gemm_fp8_block128(const void* a8, const void* b8, const float* sa,
