@@ -1,9 +1,11 @@
 // e4m3fn MFMA GEMM with 128-block scales (1x128 activation groups, 128x128
 // weight blocks): the 256x256 ping-pong kernel for large shapes (a K slab is
 // exactly one scale block; the promotion runs in place on the accumulators),
-// the generic tiled kernel otherwise (one 16x16x128 MFMA per scale block,
-// partial product promoted with sa[m,kb] * sb[n/128,kb]).
+// 128x128 tiles of the same instruction for mid-size shapes (a slab's product scaled before it
+// joins the accumulator), the generic tiled kernel otherwise (one 16x16x128 MFMA per scale
+// block, partial product promoted with sa[m,kb] * sb[n/128,kb]).
 #include "gemm_pingpong.cuh"
+#include "gemm_mid128.cuh"
 #include "gemm_tile.cuh"
 
 namespace w8a8 {
@@ -17,7 +19,9 @@ bool launch_gemm_fp8_block128_tiled(const GemmArgs& g, hipStream_t stream) {
     // the 256x256 configuration of the generic tiled kernel runs out of registers
     // with the per-block promotion; 128x128 and 64x64 do not
     const int64_t tiles128 = (int64_t)((g.m + 127) / 128) * ((g.n + 127) / 128);
-    if (tiles128 >= 192)
+    if (mid128_shape_ok(g))   // blocks of a few hundred to a few thousand tokens: 128 x 128 tiles of the 32x32x64 MFMA
+        launch_mid128<Op32F8<0>, SCALE_BLOCK128>(g, stream);
+    else if (tiles128 >= 192)
         launch_tiled<OpF8<0>, CfgMid, SCALE_BLOCK128>(g, stream);
     else
         launch_tiled<OpF8<0>, CfgSmall, SCALE_BLOCK128>(g, stream);

@@ -26,7 +26,7 @@ struct Mid128Cfg {
 };
 
 template <class Op, int ScaleKind>
-__global__ __launch_bounds__(Mid128Cfg::THREADS) void gemm_mid128_kernel(GemmArgs g) {
+__global__ __launch_bounds__(Mid128Cfg::THREADS, 4) void gemm_mid128_kernel(GemmArgs g) {
     using Cfg = Mid128Cfg;
     using Acc = typename Op::Acc;
     constexpr int MI = Cfg::MI, NI = Cfg::NI;
@@ -70,7 +70,9 @@ __global__ __launch_bounds__(Mid128Cfg::THREADS) void gemm_mid128_kernel(GemmArg
                 b4[ni][q][j] = 0.0f;
                 if (n < g.n) {
                     if constexpr (ScaleKind == SCALE_ROWCOL) sw4[ni][q][j] = g.sb[n];
-                    if (bias) b4[ni][q][j] = bf16_to_f32(bias[n]);
+                    // (the block-scaled instance needs its registers in the loop and fetches the bias at the end)
+                    if constexpr (ScaleKind != SCALE_BLOCK128)
+                        if (bias) b4[ni][q][j] = bf16_to_f32(bias[n]);
                 }
             }
 
@@ -119,6 +121,24 @@ __global__ __launch_bounds__(Mid128Cfg::THREADS) void gemm_mid128_kernel(GemmArg
 #pragma unroll
             for (int j = 0; j < 16; ++j) acc[ni][mi][j] = 0;
 
+    // ---- 128-block scales: a slab is exactly one K-block. The slab's product is formed in a
+    // temporary and joins the accumulator scaled by the activation rows' and the weight block's
+    // steps (the tile's 128 columns lie in one weight block); the steps of slab k + 1 are requested
+    // while slab k is computed.
+    [[maybe_unused]] float blk_sa[MI], blk_sa_next[MI];
+    [[maybe_unused]] float blk_sb = 0.0f, blk_sb_next = 0.0f;
+    [[maybe_unused]] const int kblocks = K >> 7;
+    auto request_steps = [&](int kb) {
+        if constexpr (ScaleKind == SCALE_BLOCK128) {
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi) {
+                const int m = mw + mi * 32 + lrow;
+                blk_sa_next[mi] = (m < g.m && kb < kblocks) ? g.sa[(size_t)m * kblocks + kb] : 0.0f;
+            }
+            blk_sb_next = kb < kblocks ? g.sb[(size_t)(n0 >> 7) * kblocks + kb] : 0.0f;
+        }
+    };
+
     auto compute = [&](int stage) {
         const uint8_t* const base = lds + stage * Cfg::STAGE_BYTES;
         u32x4 xf[MI][4], wf[NI][4];
@@ -132,18 +152,40 @@ __global__ __launch_bounds__(Mid128Cfg::THREADS) void gemm_mid128_kernel(GemmArg
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 xf[mi][j] = *reinterpret_cast<const u32x4*>(base + x_rd + mi * 4096 + frag_off[j]);
-#pragma unroll
-        for (int q = 0; q < Op::STEPS; ++q)
+        if constexpr (ScaleKind == SCALE_BLOCK128) {
 #pragma unroll
             for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-                for (int ni = 0; ni < NI; ++ni) acc[ni][mi] = Op::mma_step(q, wf[ni], xf[mi], acc[ni][mi]);
+                for (int ni = 0; ni < NI; ++ni) {
+                    Acc part;
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) part[j] = 0;
+#pragma unroll
+                    for (int q = 0; q < Op::STEPS; ++q) part = Op::mma_step(q, wf[ni], xf[mi], part);
+                    const float sc = blk_sa[mi] * blk_sb;
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) acc[ni][mi][j] += part[j] * sc;
+                }
+        } else {
+#pragma unroll
+            for (int q = 0; q < Op::STEPS; ++q)
+#pragma unroll
+                for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni) acc[ni][mi] = Op::mma_step(q, wf[ni], xf[mi], acc[ni][mi]);
+        }
     };
 
     // ---- main loop: slab k+1 in flight while slab k is read; a barrier before a stage is
     // read (every wave's part has landed) and one before it is filled again
+    request_steps(0);
     issue(0, 0u);
     for (int k = 0; k < ksteps; ++k) {
+        if constexpr (ScaleKind == SCALE_BLOCK128) {
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi) blk_sa[mi] = blk_sa_next[mi];
+            blk_sb = blk_sb_next;
+        }
         if (k + 1 < ksteps) {
             issue((k + 1) & 1, (uint32_t)(k + 1) << 7);
             wait_vmcnt<4>();   // the four loads of slab k are older than those just issued
@@ -151,6 +193,9 @@ __global__ __launch_bounds__(Mid128Cfg::THREADS) void gemm_mid128_kernel(GemmArg
             wait_vmcnt<0>();
         }
         phase_barrier();
+        // (after the wait: the next slab's steps are then older than the slab loads of the following
+        // iteration, whose wait they pass without holding it up -- a compute phase has gone by)
+        request_steps(k + 1);
         compute(k & 1);
         wait_lgkmcnt0();
         phase_barrier();
@@ -174,7 +219,9 @@ __global__ __launch_bounds__(Mid128Cfg::THREADS) void gemm_mid128_kernel(GemmArg
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const float f = (float)acc[ni][mi][4 * q + j];
-                    if constexpr (ScaleKind == SCALE_TENSOR) {
+                    if constexpr (ScaleKind == SCALE_BLOCK128) {
+                        v[j] = f + ((bias && n + j < g.n) ? bf16_to_f32(bias[n + j]) : 0.0f);
+                    } else if constexpr (ScaleKind == SCALE_TENSOR) {
                         v[j] = f * s_tensor + b4[ni][q][j];
                     } else {
 #pragma clang fp contract(off)

@@ -412,6 +412,21 @@ def test_block128_decode_shapes_row_range_kernel(m, n, k, bias):
     assert torch.equal(out.view(torch.int16), again.view(torch.int16))    # fixed summation order
 
 
+@pytest.mark.parametrize("m,n,k,bias", [(1536, 1536, 512, False), (1100, 2050, 384, True), (2048, 1280, 1024, True),
+                                        (1793, 1798, 256, False)])
+def test_block128_mid_size_tiles(m, n, k, bias):
+    """Shapes with at least 140 tiles of 128 x 128 but too few of 256 x 256: the block-scaled instance of
+    the mid-size kernel (a slab = one K-block, scaled before it joins the accumulator); ragged rows
+    and columns, outliers in 1% of the weights for a wide scale range."""
+    from astrai_amd.extension.ops import fp8_block as blk
+    print(f"case m={m} n={n} k={k} bias={bias}", flush=True)
+    x, w, b = O.make_inputs(3, m, n, k, outlier_p=0.01, bias=bias)
+    x8, sa = O.fp8_quantize_act_block128(x)
+    w8, sb = O.fp8_quantize_weight_block128(w)
+    out = blk.mm_fp8_blockscaled(x8.to(DEV), w8.to(DEV), sa.to(DEV), sb.to(DEV), b.to(DEV) if bias else None)
+    assert_bf16_close(out, O.fp8_gemm_blockscaled(x8, w8, sa, sb, b if bias else None), what="block128 mid-size")
+
+
 def test_block128_golden_exact_rationals(golden):
     from astrai_amd.extension.ops import fp8_block as blk
     for c in golden("fp8_gemm_small.json")["block128"]:
