@@ -457,10 +457,30 @@ def main():
             for (mx, mw, msx, msw, my, mm, nn, kk) in mids:
                 check(lib.astrai_w8a8_gemm_int8_ptpc(mx.data_ptr(), mw.data_ptr(), msx.data_ptr(), msw.data_ptr(),
                                                      None, my.data_ptr(), mm, nn, kk, 0, stream))
+        # block-scaled shapes below the large-tile kernel: a mid-size block of tokens and a decode step on
+        # config-3-like weights; then an int8 product with four token rows past whole 256-row tiles
+        xb = torch.randn(1024, 4096, device=dev).to(torch.bfloat16)
+        wb = torch.randn(11008, 4096, device=dev).to(torch.bfloat16) * 0.02
+        ab, sab = _cabi.quantize_fp8_block128_act(xb)
+        bb, sbb = _cabi.quantize_fp8_block128_weight(wb)
+        yb = torch.empty(1024, 11008, device=dev, dtype=torch.bfloat16)
+        a3d, sa3d = a3[:16].contiguous(), sa3[:16].contiguous()
+        xt = torch.randint(-127, 128, (4100, 4096), dtype=torch.int8, device=dev)
+        sxt = torch.rand(4100, device=dev) + 0.5
+        yt = torch.empty(4100, 4096, device=dev, dtype=torch.bfloat16)
+        for _ in range(20):
+            check(lib.astrai_w8a8_gemm_fp8_block128(ab.data_ptr(), bb.data_ptr(), sab.data_ptr(), sbb.data_ptr(),
+                                                    None, yb.data_ptr(), 1024, 11008, 4096, stream))
+            check(lib.astrai_w8a8_gemm_fp8_block128(a3d.data_ptr(), b3.data_ptr(), sa3d.data_ptr(), sb3.data_ptr(),
+                                                    None, y3.data_ptr(), 16, 2048, 7168, stream))
+            check(lib.astrai_w8a8_gemm_int8_ptpc(xt.data_ptr(), wq.data_ptr(), sxt.data_ptr(), sw.data_ptr(), None,
+                                                 yt.data_ptr(), 4100, 4096, 4096, 0, stream))
         torch.cuda.synchronize()
         print(json.dumps({"trace_gemms": "20 launches each: int8 4096^3 per-token x per-channel (bf16 out), fp8 "
                                          "128-block 8192x2048x7168 on config-3 data, fp8 4096^3 with e4m3 output; "
-                                         "then int8 2048x3072x2048, 2048x2048x5632, 1024x11264x2048 (mid-size kernel)"}))
+                                         "then int8 2048x3072x2048, 2048x2048x5632, 1024x11264x2048 (mid-size kernel); "
+                                         "then block-scaled 1024x11008x4096 (mid-size kernel) and 16x2048x7168 "
+                                         "(row-range kernel), and int8 4100x4096x4096 (large tiles + a four-row tail)"}))
         return
 
     # ---------------- headline: config 1, fp8 per-tensor 4096^3 ----------------
