@@ -530,9 +530,15 @@ __device__ __forceinline__ float silu_f32(float g) {
 // gate and of up come in pieces of `block` columns that lie 2 * block apart (a fused
 // output whose columns alternate between `block` gate and `block` up columns, `up`
 // pointing at the first up piece).
-__global__ __launch_bounds__(kThreads) void silu_mul_quantize_int8_rows_kernel(
+// T threads per row: 256 with up to four pieces a thread, or -- for the few rows of a decode step,
+// where the row's chain of loads, exponentials and reductions is all there is to wait for -- 1024
+// with one piece each (the maximum does not depend on who holds which piece: same bits).
+template <int T>
+__global__ __launch_bounds__(T) void silu_mul_quantize_int8_rows_kernel(
     const uint16_t* __restrict__ gate, const uint16_t* __restrict__ up, int64_t ld, int64_t block,
     uint16_t* __restrict__ h_out, int8_t* __restrict__ hq, float* __restrict__ s, int64_t width) {
+    constexpr int kThreads = T;
+    constexpr int kCache = w8a8::kCache * 256 / T;
     __shared__ float slots[kThreads / kWave];
     const int64_t row = blockIdx.x;
     const int64_t nvec = width >> 3;
@@ -554,7 +560,7 @@ __global__ __launch_bounds__(kThreads) void silu_mul_quantize_int8_rows_kernel(
             if (h_out) *reinterpret_cast<u32x4*>(h_out + row * width + i * 8) = pack8(v[c]);
         }
     }
-    const float step = fmaxf(block_max(local, slots), 1e-12f) / 127.0f;
+    const float step = fmaxf(block_max_t<T>(local, slots), 1e-12f) / 127.0f;
     if (threadIdx.x == 0) s[row] = step;
 #pragma unroll
     for (int c = 0; c < kCache; ++c) {
@@ -817,9 +823,14 @@ void launch_silu_mul_quantize_int8_rows(const void* gate, const void* up, int64_
                                         void* h_out, void* hq, float* s, int64_t rows, int64_t width,
                                         hipStream_t stream) {
     if (rows <= 0 || width <= 0) return;
-    silu_mul_quantize_int8_rows_kernel<<<dim3((unsigned)rows), dim3(kThreads), 0, stream>>>(
-        static_cast<const uint16_t*>(gate), static_cast<const uint16_t*>(up), ld, block,
-        static_cast<uint16_t*>(h_out), static_cast<int8_t*>(hq), s, width);
+    if (rows <= 64)
+        silu_mul_quantize_int8_rows_kernel<1024><<<dim3((unsigned)rows), dim3(1024), 0, stream>>>(
+            static_cast<const uint16_t*>(gate), static_cast<const uint16_t*>(up), ld, block,
+            static_cast<uint16_t*>(h_out), static_cast<int8_t*>(hq), s, width);
+    else
+        silu_mul_quantize_int8_rows_kernel<256><<<dim3((unsigned)rows), dim3(256), 0, stream>>>(
+            static_cast<const uint16_t*>(gate), static_cast<const uint16_t*>(up), ld, block,
+            static_cast<uint16_t*>(h_out), static_cast<int8_t*>(hq), s, width);
 }
 
 void launch_add_rmsnorm_quantize_fp8_rows(const void* x, const void* res, const void* w, float eps,

@@ -74,6 +74,20 @@ __device__ __forceinline__ float block_max(float v, float* slots) {
     return r;
 }
 
+// the same for a workgroup of T threads
+template <int T>
+__device__ __forceinline__ float block_max_t(float v, float* slots) {
+    v = wave_max(v);
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) slots[wave] = v;
+    __syncthreads();
+    float r = slots[0];
+#pragma unroll
+    for (int w = 1; w < T / kWave; ++w) r = fmaxf(r, slots[w]);
+    __syncthreads();
+    return r;
+}
+
 // block-wide sum of a per-thread value; result valid in every thread
 __device__ __forceinline__ float block_sum(float v, float* slots) {
 #pragma unroll
