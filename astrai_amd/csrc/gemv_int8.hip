@@ -118,8 +118,9 @@ void launch_dot(const GemmArgs& g, hipStream_t stream) {
 // Rows kernel launch plan. The rows are dealt out over 256 x rounds workgroups, rounds
 // being the smallest count that keeps a workgroup's range within 48 rows (three MFMA
 // row groups); ranges are rounded up to four rows (one load instruction). Four waves
-// split K; a short matrix with a long K (one row group, K >= 4096) takes eight so that
-// enough bytes are in flight (2048 x 5632: 5.7 us against 6.6 at M = 16). Measured per
+// split K; a short matrix (one row group) with K >= 2048 takes eight so that enough bytes
+// are in flight (2048 x 5632: 5.7 us against 6.6 at M = 16; at K = 2048 the decoder's q|k|v
+// and output projections gain 0.15 us each inside the decode step). Measured per
 // shape against deeper rings (IB = 2..4), fewer / more waves and one workgroup per
 // sixteen rows: this plan was the fastest or within 2% of it on every decoder shape.
 struct RowsPlan { int rows_per_wg, rg, nw, blocks; };
@@ -130,7 +131,7 @@ RowsPlan plan_rows(const GemmArgs& g) {
     const int wgs = 256 * rounds;
     p.rows_per_wg = (((g.n + wgs - 1) / wgs) + 3) & ~3;
     p.rg = (p.rows_per_wg + 15) / 16;
-    p.nw = (p.rg == 1 && g.k >= 4096) ? 8 : 4;
+    p.nw = (p.rg == 1 && g.k >= 2048) ? 8 : 4;
     p.blocks = (g.n + p.rows_per_wg - 1) / p.rows_per_wg;
     return p;
 }
