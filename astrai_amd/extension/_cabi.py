@@ -733,11 +733,13 @@ def attn_decode_supported(n_heads: int, n_kv_heads: int, seq: int, head_dim: int
 
 def decode_nsplit(pairs: int, max_keys: int) -> int:
     """Context splits of the decode attention kernel for ``pairs`` (sequence, KV head) pairs whose
-    contexts hold at most ``max_keys`` keys: a few hundred workgroups, but no more than eight
-    splits and no split shorter than ~192 keys of the longest possible context -- every split
-    adds to the merge and to the launch (measured, 16 / 4 heads: 2 sequences x 520 keys 11.7 us
-    with 3 splits against 15.5 us with 16; 32 x 520 keys 14.7 us with 3 against 18.9 us with 1)."""
-    return max(1, min(8, 384 // max(1, pairs), max_keys // 192))
+    contexts hold at most ``max_keys`` keys: up to 512 workgroups (two whole rounds of the 256
+    compute units: 32 sequences x 4 KV heads run 4 splits, 1.352 ms a decode step, against 1.366 ms
+    with 3 -- 1.5 workgroups per compute unit -- and 1.359 ms with 2), but no more than eight
+    splits and no split shorter than ~160 keys of the longest possible context -- every split
+    adds to the merge and to the launch (16 / 4 heads, 2 sequences x 520 keys: 11.7 us with 3
+    splits against 15.5 us with 16; 32 x 520 keys: 18.9 us with 1)."""
+    return max(1, min(8, 512 // max(1, pairs), max_keys // 160))
 
 
 def attn_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, positions: torch.Tensor,

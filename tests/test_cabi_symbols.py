@@ -115,11 +115,12 @@ def test_fuse_int8_weights_refuses_widths_the_fused_producers_reject():
 
 
 def test_decode_attention_split_plan():
-    """A few hundred workgroups, at most eight splits, none shorter than ~192 keys of the longest context."""
-    assert _cabi.decode_nsplit(128, 640) == 3      # config 4: 32 sequences x 4 KV heads, 512 + 128 tokens
-    assert _cabi.decode_nsplit(8, 640) == 3
+    """Up to 512 workgroups, at most eight splits, none shorter than ~160 keys of the longest context."""
+    assert _cabi.decode_nsplit(128, 640) == 4      # config 4: 32 sequences x 4 KV heads, 512 + 128 tokens
+    assert _cabi.decode_nsplit(8, 640) == 4
+    assert _cabi.decode_nsplit(256, 640) == 2
     assert _cabi.decode_nsplit(8, 2048) == 8
-    assert _cabi.decode_nsplit(256, 4096) == 1
+    assert _cabi.decode_nsplit(256, 4096) == 2 and _cabi.decode_nsplit(1024, 4096) == 1
     assert _cabi.decode_nsplit(1, 64) == 1
     assert _cabi.decode_nsplit(0, 0) == 1
 
