@@ -596,3 +596,43 @@ def test_fp8_mfma_accumulator_deviation_from_exact_sum(m, n, k):
     assert rel.max().item() < 2.0 ** -17
     assert rel.pow(2).mean().sqrt().item() < 2.0 ** -19
     assert vs_result < 2e-4
+
+
+def test_graph_replay_of_decode_and_two_launch_products_equals_eager():
+    """The fp8 decode kernels (per-tensor and 128-block steps) and a product that runs as two
+    launches (large tiles + a token tail on the decode kernel), captured in one graph: every
+    replay, with eager work and new inputs in between, gives the eager call's bits."""
+    from astrai_amd.extension import _cabi
+    g = torch.Generator().manual_seed(77)
+    w8 = (torch.randn(3072, 2048, generator=g) * 1.5).to(torch.float8_e4m3fn).to(DEV)
+    x8 = (torch.randn(8, 2048, generator=g) * 1.5).to(torch.float8_e4m3fn).to(DEV)
+    sa, sb = torch.tensor([0.3], device=DEV), torch.tensor([0.02], device=DEV)
+    xb = torch.randn(16, 2048, generator=g).to(torch.bfloat16).to(DEV)
+    wb8, sbb = _cabi.quantize_fp8_block128_weight((torch.randn(1024, 2048, generator=g) * 0.02).to(torch.bfloat16).to(DEV))
+    big = torch.randint(-127, 128, (4100, 512), generator=g, dtype=torch.int8).to(DEV)
+    wbig = torch.randint(-127, 128, (4096, 512), generator=g, dtype=torch.int8).to(DEV)
+    sbig, swbig = (torch.rand(4100, generator=g) * 0.01).to(DEV), (torch.rand(4096, generator=g) * 0.01).to(DEV)
+
+    def run():
+        xb8, sab = _cabi.quantize_fp8_block128_act(xb)
+        return (_cabi.mm_fp8(x8, w8, sa, sb), _cabi.mm_fp8_block128(xb8, wb8, sab, sbb),
+                _cabi.mm_int8(big, wbig, sbig, swbig))
+
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        for _ in range(2):
+            run()
+    torch.cuda.current_stream().wait_stream(s)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = run()
+    for i in range(3):
+        x8.copy_((torch.randn(8, 2048, generator=g) * 1.5).to(torch.float8_e4m3fn))
+        xb.copy_(torch.randn(16, 2048, generator=g).to(torch.bfloat16))
+        big.copy_(torch.randint(-127, 128, (4100, 512), generator=g, dtype=torch.int8))
+        graph.replay()
+        torch.cuda.synchronize()
+        want = run()
+        for got, ref in zip(outs, want):
+            assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), i
