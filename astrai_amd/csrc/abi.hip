@@ -800,7 +800,7 @@ int astrai_w8a8_gemm_int8_ptpc_tiled(const void* a, const void* b, const float* 
         return rc;
     if (m == 0 || n == 0) return ASTRAI_W8A8_OK;
     const w8a8::GemmArgs g = pack(a, b, sa, sb, nullptr, bias, out, m, n, k, out_dtype);
-    if (!w8a8::launch_gemm_int8_tiled(g, static_cast<hipStream_t>(stream)))
+    if (!w8a8::launch_gemm_int8_tiled(g, static_cast<hipStream_t>(stream), false))
         return fail(ASTRAI_W8A8_UNSUPPORTED,
                     "gemm_int8_ptpc_tiled: needs K %% 16 == 0 and operands under 2 GiB");
     return check_launch("gemm_int8_ptpc_tiled");

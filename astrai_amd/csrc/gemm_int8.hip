@@ -9,11 +9,11 @@
 
 namespace w8a8 {
 
-bool launch_gemm_int8_tiled(const GemmArgs& g, hipStream_t stream) {
+bool launch_gemm_int8_tiled(const GemmArgs& g, hipStream_t stream, bool tail_on_decode_kernel) {
     if (!tiled_shape_ok(g)) return false;
 #ifndef W8A8_NO_WAVE128
     if (wave128_shape_ok(g)) {
-        if (const int r = ragged_tail_rows(g)) {
+        if (const int r = tail_on_decode_kernel ? ragged_tail_rows(g) : 0) {
             GemmArgs head, tail;
             split_rows(g, r, true, head, tail);
             if (wave128_shape_ok(head) && launch_gemv_int8(tail, stream)) {   // (disjoint rows: either order)

@@ -200,7 +200,9 @@ bool launch_attn_rows(AttnRowsArgs a, hipStream_t stream);
 // gemm_int8.hip / gemm_fp8.hip / gemm_fp8_block.hip: tiled MFMA kernels.
 // Require k % 16 == 0 and m*k, n*k < 2^31 bytes; return false if the shape is
 // not accepted (the caller then uses the generic kernel).
-bool launch_gemm_int8_tiled(const GemmArgs& g, hipStream_t stream);
+// `tail_on_decode_kernel`: a token tail that would cost the large-tile kernel a round of its own may
+// run on the decode kernel in a second launch (false: the tiled kernels only)
+bool launch_gemm_int8_tiled(const GemmArgs& g, hipStream_t stream, bool tail_on_decode_kernel = true);
 // gate|up projection with the SwiGLU product in the epilogue. Weight rows come in blocks of
 // 128: 64 gate rows, then the 64 up rows of the same columns of h. g.out is h = bf16(up *
 // bf16(silu(gate))) [M, N/2], g.row_max[m, N/128] the maximum of |h| over each 64-column piece.

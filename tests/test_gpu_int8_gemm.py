@@ -116,6 +116,9 @@ def test_token_tail_past_a_round_of_large_tiles_bit_exact(C, m, n, k):
     r = torch.randn(m, n, generator=g).to(torch.bfloat16)
     fused = C.mm_int8_resid(ad, bd, sad, sbd, r.to(DEV))[rows.to(DEV)].cpu()
     assert torch.equal(fused.view(torch.int16), (ref + r[rows]).view(torch.int16))
+    # the entry that names the tiled kernels runs the whole product on them: the same bits
+    tiled = C.mm_int8(ad, bd, sad, sbd, None, 0, kernel="tiled")[rows.to(DEV)].cpu()
+    assert torch.equal(tiled.view(torch.int16), ref.view(torch.int16))
 
 
 def test_golden_integer_cases_including_worst_case_magnitude(C, golden):
