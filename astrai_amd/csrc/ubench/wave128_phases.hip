@@ -9,6 +9,7 @@
 // Build: make -C astrai_amd/csrc ubench     Run: astrai_amd/csrc/ubench/wave128_phases [M N K]
 #define W8A8_PP_TIMING 1
 #include "../gemm_wave128.cuh"
+#include "../gemm_wave128_q16.cuh"
 
 #include <algorithm>
 #include <cmath>
@@ -41,6 +42,31 @@ static float time_us(const GemmArgs& g) {
     for (int rep = 0; rep < 7; ++rep) {
         CK(hipEventRecord(e0));
         for (int i = 0; i < 100; ++i) kern<<<tiles, 256, Wave128Cfg::LDS_BYTES, 0>>>(g, RopeCacheArgs{});
+        CK(hipEventRecord(e1));
+        CK(hipEventSynchronize(e1));
+        float ms;
+        CK(hipEventElapsedTime(&ms, e0, e1));
+        ts.push_back(ms * 10.0f);
+    }
+    std::sort(ts.begin(), ts.end());
+    return ts[3];
+}
+
+// the 16x16x128 instance of the four-wave kernel (fp8 only)
+template <int SK, int KO>
+static float time_q16_us(const GemmArgs& g) {
+    auto kern = gemm_wave128_q16_kernel<0, SK, KO>;
+    CK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Wave128Cfg::LDS_BYTES));
+    const int tiles = ((g.m + 255) / 256) * ((g.n + 255) / 256);
+    hipEvent_t e0, e1;
+    CK(hipEventCreate(&e0));
+    CK(hipEventCreate(&e1));
+    for (int i = 0; i < 300; ++i) kern<<<tiles, 256, Wave128Cfg::LDS_BYTES, 0>>>(g);
+    CK(hipDeviceSynchronize());
+    std::vector<float> ts;
+    for (int rep = 0; rep < 7; ++rep) {
+        CK(hipEventRecord(e0));
+        for (int i = 0; i < 100; ++i) kern<<<tiles, 256, Wave128Cfg::LDS_BYTES, 0>>>(g);
         CK(hipEventRecord(e1));
         CK(hipEventSynchronize(e1));
         float ms;
@@ -153,6 +179,18 @@ static void knockouts(const char* what, const GemmArgs& g) {
     printf("  without MFMAs                  %.2f us\n", time_us<Op, SK, KO_MFMA>(g));
 }
 
+template <int SK>
+static void knockouts_q16(const char* what, const GemmArgs& g) {
+    const double ops = 2.0 * g.m * g.n * (double)g.k;
+    const float base = time_q16_us<SK, 0>(g);
+    printf("%s, 16x16x128 instance: whole kernel %.2f us (%.0f Tops/s)\n", what, base, ops / base / 1e6);
+    printf("  without LDS operand reads      %.2f us\n", time_q16_us<SK, KO_LDS_READS>(g));
+    printf("  without global->LDS loads      %.2f us\n", time_q16_us<SK, KO_LOADS>(g));
+    printf("  without either                 %.2f us\n", time_q16_us<SK, KO_LDS_READS | KO_LOADS>(g));
+    printf("  without output stores          %.2f us\n", time_q16_us<SK, KO_STORES>(g));
+    printf("  without MFMAs                  %.2f us\n", time_q16_us<SK, KO_MFMA>(g));
+}
+
 int main(int argc, char** argv) {
     int M = 4096, N = 4096, K = 4096;
     if (argc > 3) { M = atoi(argv[1]); N = atoi(argv[2]); K = atoi(argv[3]); }
@@ -177,7 +215,13 @@ int main(int argc, char** argv) {
                which ? "int8" : "fp8", M, N, K, us);
         print_stamps(dbg, K, {0, 3});
     }
+    {
+        const float us = time_q16_us<SCALE_TENSOR, 0>(g);
+        printf("fp8 16x16x128 instance zeros %dx%dx%d: %.2f us; stamps of workgroup 0 in shader clock cycles\n", M, N, K, us);
+        print_stamps(dbg, K, {0, 3});
+    }
     knockouts<Op32F8<0>, SCALE_TENSOR>("fp8 zeros", g);
+    knockouts_q16<SCALE_TENSOR>("fp8 zeros", g);
     knockouts<Op32I8, SCALE_ROWCOL>("int8 zeros", g);
 
     {
@@ -189,6 +233,11 @@ int main(int argc, char** argv) {
         CK(hipMemcpy(b, rb.data(), rb.size(), hipMemcpyHostToDevice));
     }
     knockouts<Op32F8<0>, SCALE_TENSOR>("fp8 normal operands (amax at 4.5 sigma)", g);
+    knockouts_q16<SCALE_TENSOR>("fp8 normal operands (amax at 4.5 sigma)", g);
+    // the two instances in alternation on the same operands
+    for (int rep = 0; rep < 3; ++rep)
+        printf("alternating, normal operands: 32x32x64 %.2f us, 16x16x128 %.2f us\n",
+               time_us<Op32F8<0>, SCALE_TENSOR, 0>(g), time_q16_us<SCALE_TENSOR, 0>(g));
     {
         std::vector<signed char> ra((size_t)M * K), rb((size_t)N * K);
         auto gauss = [] { float u = 0; for (int i = 0; i < 12; ++i) u += (float)rand() / RAND_MAX; return u - 6.0f; };

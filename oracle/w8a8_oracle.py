@@ -156,17 +156,30 @@ def int8_acc_int32_matmul(xq: torch.Tensor, wq: torch.Tensor) -> torch.Tensor:
     return xq.to(torch.int32) @ wq.to(torch.int32).t()
 
 
-def int8_acc(xq: torch.Tensor, wq: torch.Tensor) -> torch.Tensor:
-    """Exact int32 accumulator ``xq @ wq^T``. fp32 matmul of int8 values is not
-    exact once K*127^2 >= 2^24, so an integer matmul is used at every size:
-    PyTorch's int8 x int8 -> int32 CPU routine (``torch._int_mm``), which takes any
-    shape and is ~200x faster than the int32 tensor matmul it is pinned against
-    (tests/test_oracle_gemm.py: equal to :func:`int8_acc_int32_matmul`, to the C loop
-    and to pure-Python integer loops, worst-case magnitudes included). That routine
-    returns garbage for K = 1 (torch 2.10 CPU), so short contractions keep the int32 matmul."""
-    if xq.dtype == torch.int8 and wq.dtype == torch.int8 and xq.size(-1) >= 16 and xq.numel() and wq.numel():
-        return torch._int_mm(xq.contiguous(), wq.contiguous().t())
-    return int8_acc_int32_matmul(xq, wq)
+def int8_acc(xq: torch.Tensor, wq: torch.Tensor, fast: bool = False) -> torch.Tensor:
+    """Exact int32 accumulator ``xq @ wq^T``. fp32 matmul of int8 values is not exact once
+    K*127^2 >= 2^24, so the default is arithmetic that is exact by construction: the int32
+    tensor matmul for small products and, for large ones, a float64 matmul -- every partial
+    sum is an integer of magnitude <= K*127^2 < 2^53, so each double addition is exact in
+    any order the BLAS chooses (0.8 s at 4096^3 on eight cores).
+
+    ``fast=True`` (timing legs only) takes PyTorch's int8 x int8 -> int32 CPU routine,
+    ``torch._int_mm``: ~15x faster, private, and known to return garbage for K = 1; every
+    such call re-computes a random subset of rows with the int32 matmul and raises on a
+    mismatch, and short contractions never reach it."""
+    if not (xq.numel() and wq.numel()):
+        return int8_acc_int32_matmul(xq, wq)
+    m, k, n = xq.size(0), xq.size(-1), wq.size(0)
+    if fast and xq.dtype == torch.int8 and wq.dtype == torch.int8 and k >= 16:
+        out = torch._int_mm(xq.contiguous(), wq.contiguous().t())
+        rows = torch.randint(0, m, (min(m, 4),))
+        if not torch.equal(out[rows], int8_acc_int32_matmul(xq[rows], wq)):
+            raise RuntimeError(f"torch._int_mm disagrees with the int32 matmul at {m}x{n}x{k}")
+        return out
+    if m * n * k <= (1 << 24):
+        return int8_acc_int32_matmul(xq, wq)
+    assert k * 127 * 127 < (1 << 53)
+    return (xq.double() @ wq.double().t()).to(torch.int32)
 
 
 def int8_gemm(xq, wq, sx, sw, bias=None):

@@ -209,9 +209,10 @@ def test_linear_forward_int8_end_to_end_matches_oracle(C):
 
 
 def test_full_size_linearity_property(C):
-    """At 4096^3 the oracle is too slow for a full check: use exactness of the
-    integer ring instead -- acc(a1+a2, b) == acc(a1, b) + acc(a2, b) with operands
-    kept inside int8, plus a sampled row block against the oracle."""
+    """4096^3: every one of the 4096 x 4096 int32 accumulators against the exact oracle
+    (all 16 x 16 tiles of the launch, so a tile at a wrong coordinate or a K slab dropped
+    in one tile fails), and exactness of the integer ring on top --
+    acc(a1+a2, b) == acc(a1, b) + acc(a2, b) with operands kept inside int8."""
     g = torch.Generator().manual_seed(5)
     m = n = k = 4096
     a1 = torch.randint(-63, 64, (m, k), generator=g, dtype=torch.int8)
@@ -222,8 +223,12 @@ def test_full_size_linearity_property(C):
     p1 = C.mm_int8(a1.to(DEV), bd, None, None, None, 2, "tiled")
     p2 = C.mm_int8(a2.to(DEV), bd, None, None, None, 2, "tiled")
     assert torch.equal(s, p1 + p2)
-    rows = torch.tensor([0, 1, 255, 256, 2047, 4095])
-    assert torch.equal(p1.cpu()[rows], O.int8_acc(a1[rows], b))
+    assert torch.equal(p1.cpu(), O.int8_acc(a1, b))
+    # the bf16 epilogue of the four-wave kernel on the same product, every element
+    sx = torch.rand(m, generator=g) + 0.5
+    sw = (torch.rand(n, generator=g) + 0.5) * 1e-3
+    y = C.mm_int8(a1.to(DEV), bd, sx.to(DEV), sw.to(DEV), None, 0, "tiled")
+    assert torch.equal(y.cpu().view(torch.int16), O.int8_gemm(a1, b, sx, sw).view(torch.int16))
 
 
 @pytest.mark.parametrize("m,n,k,out_dtype", [(3900, 4104, 1152, 0),   # bf16, N % 8 == 0: four-wave kernel

@@ -176,42 +176,46 @@ def test_int8_config0_fp32_matmul_would_not_be_exact_but_int_is():
     assert torch.equal(acc, (xq.double() @ wq.double().t()).to(torch.int32))
 
 
-def test_int8_acc_library_routine_equals_int32_matmul_and_c_loop():
-    """The accumulator goes through PyTorch's int8 CPU routine; pin it on ragged shapes, a
-    decode shape, a multi-tile shape and worst-case magnitudes (every product +-127^2, K = 4096:
-    |acc| = 66 M, no wrap) against the int32 tensor matmul and the C triple loop."""
+def test_int8_acc_every_route_equals_int32_matmul_and_c_loop():
+    """The accumulator's three routes (int32 matmul, exact float64 matmul, and the opt-in
+    library int8 routine with its sampled self-check) on ragged shapes, a decode shape, a
+    multi-tile shape and worst-case magnitudes (every product +-127^2, K = 4096: |acc| = 66 M,
+    no wrap) against the int32 tensor matmul and the C triple loop."""
     g = torch.Generator().manual_seed(11)
     for m, n, k in ((1, 5, 1), (4, 3, 1), (3, 5, 7), (2, 3, 15), (5, 4, 16), (17, 9, 33), (1, 300, 4096), (130, 257, 1000), (64, 96, 4096)):
         a = torch.randint(-127, 128, (m, k), dtype=torch.int8, generator=g)
         b = torch.randint(-127, 128, (n, k), dtype=torch.int8, generator=g)
-        got = O.int8_acc(a, b)
-        assert got.dtype == torch.int32 and torch.equal(got, O.int8_acc_int32_matmul(a, b)), (m, n, k)
+        want = O.int8_acc_int32_matmul(a, b)
+        for fast in (False, True):
+            got = O.int8_acc(a, b, fast=fast)
+            assert got.dtype == torch.int32 and torch.equal(got, want), (m, n, k, fast)
         if m * n * k <= 4_000_000:
-            assert np.array_equal(got.numpy(), c_oracle.int8_gemm_i32(a.numpy(), b.numpy())), (m, n, k)
+            assert np.array_equal(want.numpy(), c_oracle.int8_gemm_i32(a.numpy(), b.numpy())), (m, n, k)
     a = torch.full((5, 4096), 127, dtype=torch.int8)
     a[1::2] = -127
     b = torch.full((7, 4096), -127, dtype=torch.int8)
     b[::3] = 127
-    want = (a.double() @ b.double().t())
+    want = O.int8_acc_int32_matmul(a, b)
     assert want.abs().max().item() == 127 * 127 * 4096
-    assert torch.equal(O.int8_acc(a, b), want.to(torch.int32))
-    # a strided view takes the same route
+    assert torch.equal(O.int8_acc(a, b), want) and torch.equal(O.int8_acc(a, b, fast=True), want)
+    # the float64 route (products too large for the int32 matmul's time) on worst-case magnitudes
+    a = torch.full((300, 4096), 127, dtype=torch.int8)
+    a[1::2] = -127
+    b = torch.full((260, 4096), -127, dtype=torch.int8)
+    b[::3] = 127
+    assert 300 * 260 * 4096 > (1 << 24)
+    assert torch.equal(O.int8_acc(a, b), O.int8_acc_int32_matmul(a, b))
+    # a strided view takes the same routes
     assert torch.equal(O.int8_acc(a[:, ::2], b[:, ::2]), O.int8_acc_int32_matmul(a[:, ::2], b[:, ::2]))
 
 
-# ---- 128-block scaled ----
-
-def test_block128_exact_small(golden):
-    for c in golden("fp8_gemm_small.json")["block128"]:
-        a8 = torch.tensor(c["a"], dtype=torch.uint8).view(torch.float8_e4m3fn)
-        b8 = torch.tensor(c["b"], dtype=torch.uint8).view(torch.float8_e4m3fn)
-        sa, sb = torch.tensor(c["sa"]), torch.tensor(c["sb"])
-        exact = torch.tensor(c["exact"], dtype=torch.float64)
-        out = O.fp8_gemm_blockscaled(a8, b8, sa, sb)
-        scale = exact.abs().max().item()
-        assert (out.double() - exact).abs().max().item() <= 2 ** -8 * scale
-        cc = c_oracle.fp8_gemm_block128_f32(np.array(c["a"]), np.array(c["b"]), sa.numpy(), sb.numpy())
-        assert np.abs(cc - exact.numpy()).max() <= 1e-5 * scale
+def test_int8_acc_fast_route_raises_on_a_wrong_library_result(monkeypatch):
+    a = torch.randint(-127, 128, (8, 64), dtype=torch.int8)
+    b = torch.randint(-127, 128, (8, 64), dtype=torch.int8)
+    real = torch._int_mm
+    monkeypatch.setattr(torch, "_int_mm", lambda x, y: real(x, y) + 1)
+    with pytest.raises(RuntimeError, match="disagrees"):
+        O.int8_acc(a, b, fast=True)
 
 
 def test_block128_reduces_to_per_tensor_when_scales_equal():
