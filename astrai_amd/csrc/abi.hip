@@ -96,11 +96,17 @@ int scratch_of_current_device(const char* what, float** out) {
 
 }  // namespace
 
+namespace w8a8 {
+thread_local const char* g_last_kernel = "";
+}
+
 extern "C" {
 
 int astrai_w8a8_abi_version(void) { return ASTRAI_W8A8_ABI_VERSION; }
 
 const char* astrai_w8a8_last_error(void) { return g_err; }
+
+const char* astrai_w8a8_last_kernel(void) { return w8a8::g_last_kernel; }
 
 int astrai_w8a8_quantize_bf16_fp8(const void* x, void* x8, const float* scale, float* amax,
                                   int64_t total, int fmt, void* stream) {

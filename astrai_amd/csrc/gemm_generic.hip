@@ -67,6 +67,7 @@ template <class Op, int ScaleKind>
 void launch(const GemmArgs& g, hipStream_t stream) {
     const int64_t tiles = (int64_t)((g.m + 15) / 16) * ((g.n + 15) / 16);
     const int64_t blocks = (tiles + 3) / 4;
+    note_kernel("generic");
     gemm_generic_kernel<Op, ScaleKind><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(g);
 }
 

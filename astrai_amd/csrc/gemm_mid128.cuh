@@ -263,6 +263,7 @@ inline void launch_mid128(const GemmArgs& g, hipStream_t stream) {
     auto kern = gemm_mid128_kernel<Op, ScaleKind>;
     static std::atomic<uint64_t> lds_allowed{0};
     allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::LDS_BYTES, lds_allowed);
+    note_kernel(ScaleKind == SCALE_BLOCK128 ? "mid128_block128" : "mid128");
     kern<<<dim3((unsigned)tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(g);
 }
 

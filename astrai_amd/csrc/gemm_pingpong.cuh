@@ -591,6 +591,7 @@ inline void launch_pingpong(const GemmArgs& g, hipStream_t stream) {
     auto kern = gemm_pingpong_kernel<Op, ScaleKind, Cfg>;
     static std::atomic<uint64_t> lds_allowed{0};
     allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::LDS_BYTES, lds_allowed);
+    note_kernel(ScaleKind == SCALE_BLOCK128 ? "pingpong_block128" : "pingpong");
     kern<<<dim3((unsigned)tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(g);
 }
 

@@ -309,6 +309,7 @@ inline void launch_tiled(const GemmArgs& g, hipStream_t stream) {
     auto kern = gemm_tiled_kernel<Op, Cfg, ScaleKind>;
     static std::atomic<uint64_t> lds_allowed{0};
     allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::LDS_BYTES, lds_allowed);
+    note_kernel(Cfg::BM == 256 ? "tiled_256" : Cfg::BM == 128 ? "tiled_128" : "tiled_64");
     kern<<<dim3((unsigned)tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(g);
 }
 

@@ -629,6 +629,7 @@ inline void launch_wave128(const GemmArgs& g, hipStream_t stream, const RopeCach
     auto kern = gemm_wave128_kernel<Op, ScaleKind, Epi>;
     static std::atomic<uint64_t> lds_allowed{0};
     allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::LDS_BYTES, lds_allowed);
+    note_kernel(Epi == EPI_SWIGLU ? "wave128_swiglu" : Epi == EPI_ROPE ? "wave128_rope" : Epi == EPI_RESID ? "wave128_resid" : "wave128");
     kern<<<dim3((unsigned)tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(g, rc);
 }
 

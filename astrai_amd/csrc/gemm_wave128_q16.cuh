@@ -320,6 +320,7 @@ inline void launch_wave128_q16(const GemmArgs& g, hipStream_t stream) {
     auto kern = gemm_wave128_q16_kernel<Fmt, ScaleKind>;
     static std::atomic<uint64_t> lds_allowed{0};
     allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::LDS_BYTES, lds_allowed);
+    note_kernel("wave128_q16");
     kern<<<dim3((unsigned)tiles), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(g);
 }
 

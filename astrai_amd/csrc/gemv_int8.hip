@@ -108,6 +108,7 @@ __global__ __launch_bounds__(64) void gemv_int8_dot_kernel(GemmArgs g) {
 }
 
 void launch_dot(const GemmArgs& g, hipStream_t stream) {
+    note_kernel("gemv_dot");
     // a short matrix has too few rows to fill the chip with two-row waves' small windows
     if (g.n < 4096)
         gemv_int8_dot_kernel<4><<<dim3((unsigned)((g.n + 3) / 4)), dim3(64), 0, stream>>>(g);
@@ -143,6 +144,7 @@ void launch_rows_inst(const GemmArgs& g, const RopeCacheArgs& rc, const RowsPlan
     auto kern = gemv_int8_rows_kernel<RG, MB, NW, 1, ROPE>;
     static std::atomic<uint64_t> lds_allowed{0};
     allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_allowed);
+    note_kernel(ROPE ? "gemv_rows_rope" : "gemv_rows");
     kern<<<dim3((unsigned)p.blocks), dim3(NW * 64), lds_bytes, stream>>>(g, rc, p.rows_per_wg);
 }
 
@@ -179,6 +181,7 @@ void launch_rows_fp8_inst(const GemmArgs& g, const RowsPlan& p, bool rowcol, hip
     auto kern = gemv_fp8_rows_kernel<Fmt, RG, MB, NW>;
     static std::atomic<uint64_t> lds_allowed{0};
     allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_allowed);
+    note_kernel("gemv_rows_fp8");
     kern<<<dim3((unsigned)p.blocks), dim3(NW * 64), lds_bytes, stream>>>(g, p.rows_per_wg, rowcol ? 1 : 0);
 }
 
@@ -212,6 +215,7 @@ void launch_rows_fp8_block_inst(const GemmArgs& g, const RowsPlan& p, hipStream_
     auto kern = gemv_fp8_block128_rows_kernel<RG, MB, NW>;
     static std::atomic<uint64_t> lds_allowed{0};
     allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_allowed);
+    note_kernel("gemv_rows_fp8_block128");
     kern<<<dim3((unsigned)p.blocks), dim3(NW * 64), lds_bytes, stream>>>(g, p.rows_per_wg);
 }
 

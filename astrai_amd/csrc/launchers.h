@@ -23,6 +23,12 @@ inline void allow_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_
     if (known) done.fetch_or(bit, std::memory_order_release);
 }
 
+// Diagnostic: every GEMM launcher leaves the family name of the kernel it launched here (per
+// host thread); astrai_w8a8_last_kernel() reads it back. A product sent out as two launches
+// (whole 256-row tiles + a ragged tail on the decode kernel) reports the tile kernel.
+extern thread_local const char* g_last_kernel;
+inline void note_kernel(const char* name) { g_last_kernel = name; }
+
 enum OutKind : int { OUT_BF16 = 0, OUT_E4M3 = 1, OUT_ACC = 2 };
 enum ScaleKind : int { SCALE_TENSOR = 0, SCALE_ROWCOL = 1, SCALE_BLOCK128 = 2 };
 

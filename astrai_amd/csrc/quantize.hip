@@ -1,8 +1,9 @@
 // bf16 -> fp8 / int8 quantization kernels for gfx950.
 //
 // All kernels are bandwidth-bound elementwise passes: 16-byte loads (8 bf16 per
-// lane), IEEE fp32 division by the step (the CPU kernel's arithmetic,
-// astrai/extension/ops/fp8.py:80), hardware RNE conversion, 8-byte stores.
+// lane), the correctly rounded fp32 quotient by the step (the CPU kernel's arithmetic,
+// astrai/extension/ops/fp8.py:80; formed without a division sequence per element where the
+// step is shared, see quant8_fp8), hardware RNE conversion, 8-byte stores.
 #include "common.cuh"
 #include "launchers.h"
 #include "row_ops.cuh"
@@ -13,13 +14,65 @@ namespace {
 
 constexpr int kThreads = kRowThreads;
 
+// Eight saturating fp8 codes of RN32(f / step), the oracle's arithmetic: an IEEE division per
+// element and a NaN-preserving clamp.
 template <int Fmt>
-__device__ __forceinline__ u32x2 quant8_fp8(const float (&f)[8], float step) {
+__device__ __forceinline__ u32x2 quant8_fp8_div(const float (&f)[8], float step) {
     u32x2 o;
     o.x = cvt_pk_fp8<Fmt>(f[0] / step, f[1] / step) |
           (cvt_pk_fp8<Fmt>(f[2] / step, f[3] / step) << 16);
     o.y = cvt_pk_fp8<Fmt>(f[4] / step, f[5] / step) |
           (cvt_pk_fp8<Fmt>(f[6] / step, f[7] / step) << 16);
+    return o;
+}
+
+// The same eight codes without eight IEEE division sequences (a quantizer is otherwise bound by
+// them: ~11 of its ~18 vector instructions per element). The step is shared by the tensor, so
+// the correctly rounded reciprocal inv = RN(1 / step) is formed once, and per element
+//   q0 = f * inv,  e0 = fma(-q0, step, f),  q1 = fma(e0, inv, q0)     (q1: RN of t + 2^-22 ulp,
+//   e1 = fma(-q1, step, f),  q = fma(e1, inv, q1)                      a faithful quotient)
+// is the correctly rounded quotient RN32(f / step): Markstein's theorem -- a faithful quotient
+// corrected once with its exact remainder and the correctly rounded reciprocal rounds
+// correctly, unless the divisor's significand is all ones. The remainders are exact unless they
+// underflow, which needs |f| < 2^-102: a zero code for every step >= 2^-60. So steps outside
+// [2^-60, 2^60] or with an all-ones significand take the division throughout, and so do lanes
+// whose quotient is not finite (infinite or NaN inputs, products that overflow), which also
+// keeps NaN out of the clamp below.
+template <int Fmt>
+__device__ __forceinline__ u32x2 quant8_fp8(const float (&f)[8], float step) {
+    constexpr float lim = Fmt ? 57344.0f : 448.0f;
+    const float inv = 1.0f / step;
+    const bool step_ok = step >= 0x1p-60f && step <= 0x1p60f && (__float_as_uint(step) & 0x7fffffu) != 0x7fffffu;
+    float q[8];
+    bool finite = true;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float q0 = f[j] * inv;
+        const float e0 = __builtin_fmaf(-q0, step, f[j]);
+        const float q1 = __builtin_fmaf(e0, inv, q0);
+        const float e1 = __builtin_fmaf(-q1, step, f[j]);
+        // (a zero quotient takes the sign of f, as the division gives it: the corrections add
+        // +0 to a -0; everywhere else the sign bit is already f's, the step being positive)
+        q[j] = __uint_as_float(__float_as_uint(__builtin_fmaf(e1, inv, q1)) | (__float_as_uint(f[j]) & 0x80000000u));
+        finite = finite && fabsf(q[j]) < __builtin_inff();
+    }
+    if (__builtin_expect(!step_ok || !finite, 0)) {
+        // (the empty statement keeps this a branch: the compiler otherwise evaluates the
+        // divisions for every lane and selects)
+        asm volatile("");
+        return quant8_fp8_div<Fmt>(f, step);
+    }
+    u32x2 o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) q[j] = __builtin_amdgcn_fmed3f(q[j], -lim, lim);
+    // (the converter writes the half of its destination word that the last operand names)
+    if constexpr (Fmt) {
+        o.x = (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(q[2], q[3], __builtin_amdgcn_cvt_pk_bf8_f32(q[0], q[1], 0, false), true);
+        o.y = (uint32_t)__builtin_amdgcn_cvt_pk_bf8_f32(q[6], q[7], __builtin_amdgcn_cvt_pk_bf8_f32(q[4], q[5], 0, false), true);
+    } else {
+        o.x = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false), true);
+        o.y = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(q[6], q[7], __builtin_amdgcn_cvt_pk_fp8_f32(q[4], q[5], 0, false), true);
+    }
     return o;
 }
 
@@ -66,7 +119,9 @@ __global__ __launch_bounds__(kThreads) void quantize_fp8_kernel(
             float f[8];
             unpack8(raw[u], f);
             local = fmaxf(local, amax8(f));
-            *reinterpret_cast<u32x2*>(x8 + (v0 + u * stride) * 8) = quant8_fp8<Fmt>(f, step);
+            // streamed out: the codes' next reader is another kernel, and leaving them out of this
+            // kernel's cache footprint is worth 1.5-3 us at 4096 x 4096
+            __builtin_nontemporal_store(quant8_fp8<Fmt>(f, step), reinterpret_cast<u32x2*>(x8 + (v0 + u * stride) * 8));
         }
     };
     if (v + (kUnroll - 1) * stride < nvec) {

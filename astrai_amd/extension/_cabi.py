@@ -32,6 +32,7 @@ _F32 = ctypes.c_float
 PROTOTYPES = {
     "astrai_w8a8_abi_version": ([], _INT),
     "astrai_w8a8_last_error": ([], ctypes.c_char_p),
+    "astrai_w8a8_last_kernel": ([], ctypes.c_char_p),
     "astrai_w8a8_quantize_bf16_fp8": ([_P, _P, _P, _P, _I64, _INT, _P], _INT),
     "astrai_w8a8_amax_bf16": ([_P, _P, _I64, _P], _INT),
     "astrai_w8a8_amax_ring_push": ([_P, _INT, _INT, _P, _P, _F32, _F32, _P], _INT),
@@ -1163,6 +1164,12 @@ def mm_int8_resid(a: torch.Tensor, b: torch.Tensor, sa: torch.Tensor, sb: torch.
                     a_c.data_ptr(), b_c.data_ptr(), _ptr(sa), _ptr(sb), _ptr(bias), resid_c.data_ptr(),
                     out.data_ptr(), m, n, k, _stream(a)), lib)
     return out
+
+
+def last_kernel() -> str:
+    """Family name of the kernel the most recent GEMM entry of this thread launched
+    (diagnostic; ``astrai_w8a8_last_kernel``)."""
+    return _require().astrai_w8a8_last_kernel().decode()
 
 
 def mfma_probe(kind: int, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:

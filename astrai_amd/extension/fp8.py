@@ -203,12 +203,14 @@ class FP8State:
         self.fp8_format: FP8Format = FP8Format.HYBRID
         self._metas: Dict[Tuple, FP8TensorMeta] = {}
         self._last_device: Optional[torch.device] = None
-        # Opt-in (fp8_cache_weights): keep each weight's fp8 codes between calls for as
-        # long as the tensor's version counter stands still, instead of measuring and
-        # quantizing the weight again in every forward (fp8.py:291-299 does). Outputs
-        # are unchanged; writes that bypass the version counter (``w.data`` tricks)
-        # are not seen, hence opt-in.
-        self.cache_weights = False
+        # Weight-code cache (fp8_cache_weights): keep each weight's fp8 codes between calls
+        # for as long as the tensor's version counter stands still, instead of measuring
+        # and quantizing the weight again in every forward (fp8.py:291-299 does). Outputs
+        # and ring state are unchanged. None (the default) decides per call: on where no
+        # optimizer can be rewriting the weight between forwards -- autograd is off, or the
+        # weight takes no gradient --, off in a training step, where a write that bypasses
+        # the version counter (``w.data`` tricks of some optimizers) would go unseen.
+        self.cache_weights: Optional[bool] = None
         self._dyn_w: Dict[Tuple, Tuple] = {}
 
     def get_weight_meta(self, w: torch.Tensor) -> FP8TensorMeta:
@@ -237,9 +239,14 @@ class FP8State:
         self._dyn_w[key] = (weakref.ref(w), w._version, sw, w8)
         return sw, w8
 
+    def caches_weight(self, w: torch.Tensor) -> bool:
+        if self.cache_weights is not None:
+            return self.cache_weights
+        return not (torch.is_grad_enabled() and w.requires_grad)
+
     def reset(self) -> None:
         self.enabled = False
-        self.cache_weights = False
+        self.cache_weights = None
         self._metas.clear()
         self._dyn_w.clear()
         self._last_device = None
@@ -305,7 +312,7 @@ def fp8_linear_forward(x: torch.Tensor, w: torch.Tensor, bias=None):
         x2 = x.reshape(-1, w.size(1))
         sx = _dynamic_scale(x2, st.recipe, fmt)
         x8, _ = quantize_bf16(x2, sx, fmt)
-        if st.cache_weights:
+        if st.caches_weight(w):
             sw, w8 = st.dynamic_weight(w, fmt)
         else:
             sw = _dynamic_scale(w, st.recipe, fmt)
@@ -316,7 +323,7 @@ def fp8_linear_forward(x: torch.Tensor, w: torch.Tensor, bias=None):
         return out
     if not meta.x_init:
         meta.init_x(x, fmt)
-    if st.cache_weights and meta.w_settled(w):
+    if st.caches_weight(w) and meta.w_settled(w):
         # The weight ring already holds this weight's amax in every slot: pushing it
         # again would leave ring and step as they are, so codes made with that step
         # stay valid until the weight is written to.
@@ -363,13 +370,15 @@ def fp8_linear_enable(enabled: bool = True) -> None:
     fp8_state().enabled = enabled
 
 
-def fp8_cache_weights(enabled: bool = True) -> None:
+def fp8_cache_weights(enabled: Optional[bool] = True) -> None:
     """Keep each weight's fp8 codes between forwards while the weight is unmodified
-    (inference, or several micro-batches per optimizer step). Off by default: the
-    reference quantizes the weight in every call (fp8.py:291-299)."""
+    (inference, or several micro-batches per optimizer step): True / False force it on
+    or off for every Linear, None restores the default, which caches exactly where
+    autograd is off or the weight takes no gradient. The reference quantizes the weight
+    in every call (fp8.py:291-299); outputs and scaling state do not differ."""
     st = fp8_state()
     st.cache_weights = enabled
-    if not enabled:
+    if enabled is False:
         st._dyn_w.clear()
         for meta in st._metas.values():
             meta.w_cached = None

@@ -48,7 +48,8 @@ class AutoRegressiveLMConfig:
     num_key_value_heads: int = 4
     intermediate_size: int = 5632
     rms_norm_eps: float = 1e-5
-    rope_theta: float = 10000.0
+    rope_theta: Optional[float] = 10000.0
+    rope_scaling: Optional[dict] = None   # e.g. {"type": "ntk", "factor": 4.0}
     max_position_embeddings: int = 2048
     tie_word_embeddings: bool = False
 
@@ -99,6 +100,22 @@ def get_rotary_emb(dim: int, max_len: int, base: float = 10000.0) -> Tensor:
     t = torch.arange(0, max_len, dtype=torch.float64)
     freqs = torch.outer(t, theta).float()
     return torch.stack([torch.cos(freqs), torch.sin(freqs)], dim=-1)
+
+
+def ntk_base(base: float, dim: int, factor: float) -> float:
+    """NTK-aware stretching of the rotary base (components/rope.py:27-28)."""
+    return base * (factor ** (dim / (dim - 2)))
+
+
+def rotary_base(rope_theta: Optional[float], dim: int, rope_scaling: Optional[dict]) -> float:
+    """The base the rotary table is built from: ``rope_theta`` (10000 when absent,
+    transformer.py:41), stretched by :func:`ntk_base` when ``rope_scaling`` names the
+    type "ntk" (the default type); any other type leaves the base alone, as the
+    reference's ``RotaryEmbedding.__init__`` does (components/rope.py:44-50)."""
+    base = 10000.0 if rope_theta is None else rope_theta
+    if rope_scaling is not None and rope_scaling.get("type", "ntk") == "ntk":
+        base = ntk_base(base, dim, rope_scaling.get("factor", 1.0))
+    return base
 
 
 def apply_rotary_emb(x: Tensor, freqs_cis: Tensor) -> Tensor:
@@ -313,7 +330,8 @@ class AutoRegressiveLM(nn.Module):
         self.config = config
         rope_dim = config.hidden_size // config.num_attention_heads
         self.register_buffer(
-            "freqs_cis", get_rotary_emb(rope_dim, config.max_position_embeddings, config.rope_theta),
+            "freqs_cis", get_rotary_emb(rope_dim, config.max_position_embeddings,
+                                        rotary_base(config.rope_theta, rope_dim, getattr(config, "rope_scaling", None))),
             persistent=False)
         self.embed_tokens = Embedding(config.vocab_size, config.hidden_size)
         self.layers = nn.ModuleList(

@@ -560,7 +560,8 @@ int astrai_w8a8_gemm_int8_ptpc_tiled(const void* a, const void* b, const float* 
                                      void* stream);
 
 /*
- * Test hook: ONE MFMA instruction on a zero accumulator in a single 64-lane wave, for
+ * Diagnostic entry, not part of the path (the library's kernels never call it and no caller
+ * of the path needs it). ONE MFMA instruction on a zero accumulator in a single 64-lane wave, for
  * known-answer tests of the lane layouts the kernels assume (what the reference checks
  * with csrc/tests/fp8_mma_test.cu:81-145 for its mma.sync shape). Operands are row-major
  * [R][K] matrices a (first operand) and b (second); lane l loads row l % R and the K bytes
@@ -574,6 +575,16 @@ int astrai_w8a8_gemm_int8_ptpc_tiled(const void* a, const void* b, const float* 
  *     | 6 f32_16x16x32_bf16 ([16][32] bf16) | 7 f32_32x32x16_bf16 ([32][16] bf16)
  */
 int astrai_w8a8_mfma_probe(int kind, const void* a, const void* b, void* d_raw, void* stream);
+
+/* Diagnostic entry, not part of the path: the family name of the kernel that the calling
+ * thread's most recent GEMM entry launched ("wave128_q16", "wave128", "wave128_swiglu",
+ * "wave128_rope", "wave128_resid", "pingpong", "pingpong_block128", "mid128", "mid128_block128",
+ * "tiled_256", "tiled_128", "tiled_64", "generic", "gemv_dot", "gemv_rows", "gemv_rows_rope",
+ * "gemv_rows_fp8", "gemv_rows_fp8_block128"; "" before the first launch). A product sent out as
+ * whole 256-row tiles plus a ragged tail on the decode kernel reports the tile kernel. For tests
+ * and shape surveys that record which kernel a Linear of a given shape lands on; the static
+ * string lives as long as the library. No counterpart in the reference. */
+const char* astrai_w8a8_last_kernel(void);
 
 #ifdef __cplusplus
 }

@@ -31,6 +31,19 @@ def rotary_table(dim: int, max_len: int, base: float) -> torch.Tensor:
     return torch.stack([torch.cos(freqs), torch.sin(freqs)], dim=-1)
 
 
+def rotary_base_of(cfg) -> float:
+    """Base of the rotary table of a config: ``rope_theta`` (10000 when None,
+    astrai/model/transformer.py:41), times ``factor ** (dim / (dim - 2))`` under NTK
+    ``rope_scaling`` (astrai/model/components/rope.py:27-28,44-50; "ntk" is the default
+    type, other types change nothing there)."""
+    dim = cfg.hidden_size // cfg.num_attention_heads
+    base = 10000.0 if cfg.rope_theta is None else float(cfg.rope_theta)
+    scaling = getattr(cfg, "rope_scaling", None)
+    if scaling is not None and scaling.get("type", "ntk") == "ntk":
+        base = base * float(scaling.get("factor", 1.0)) ** (dim / (dim - 2))
+    return base
+
+
 def apply_rotary(x: torch.Tensor, freqs_cis: torch.Tensor) -> torch.Tensor:
     cos, sin = freqs_cis[..., 0], freqs_cis[..., 1]
     xc = torch.view_as_complex(x.float().reshape(*x.shape[:-1], -1, 2))
@@ -230,7 +243,7 @@ def forward(sd: Dict[str, torch.Tensor], cfg, input_ids: torch.Tensor,
     nh, nkv = cfg.num_attention_heads, cfg.num_key_value_heads
     hd = cfg.hidden_size // nh
     x = F.embedding(input_ids, sd["embed_tokens.weight"])
-    fc = rotary_table(hd, s, cfg.rope_theta).unsqueeze(0)  # [1, S, hd/2, 2]
+    fc = rotary_table(hd, s, rotary_base_of(cfg)).unsqueeze(0)  # [1, S, hd/2, 2]
     for i in range(cfg.num_hidden_layers):
         p = f"layers.{i}."
         h = F.rms_norm(x, (cfg.hidden_size,), sd[p + "input_norm.weight"], cfg.rms_norm_eps)
@@ -263,7 +276,7 @@ def forward_cached(sd: Dict[str, torch.Tensor], cfg, input_ids: torch.Tensor,
     nh, nkv = cfg.num_attention_heads, cfg.num_key_value_heads
     hd = cfg.hidden_size // nh
     x = F.embedding(input_ids, sd["embed_tokens.weight"])
-    table = rotary_table(hd, int(positions.max()) + 1, cfg.rope_theta)
+    table = rotary_table(hd, int(positions.max()) + 1, rotary_base_of(cfg))
     fc = table.index_select(0, positions).unsqueeze(0)      # [1, S, hd/2, 2]
     for i in range(cfg.num_hidden_layers):
         p = f"layers.{i}."

@@ -297,11 +297,11 @@ def test_four_wave_kernel_both_mfma_instances_whole_output(ops, m, n, k, fmt):
     bias = torch.randn(n, generator=g).to(torch.bfloat16)
     sa, sb = torch.tensor([0.37]), torch.tensor([0.011])
     ad, bd = a8.to(DEV), b8.to(DEV)
-    out = _cabi.mm_fp8(ad, bd, sa.to(DEV), sb.to(DEV), fmt, None, bias.to(DEV))
+    out = _cabi.mm_fp8(ad, bd, sa.to(DEV), sb.to(DEV), 0, None, bias.to(DEV))   # (format: the operands' dtype)
     assert_bf16_close(out, O.fp8_gemm_bias(a8, b8, sa, sb, bias), what="per tensor + bias")
     sa_r = torch.exp2(torch.rand(m, 1, generator=g) * 6.0 - 3.0)
     sb_r = torch.exp2(torch.rand(n, generator=g) * 6.0 - 3.0)
-    out = _cabi.mm_fp8(ad, bd, sa_r.to(DEV), sb_r.to(DEV), fmt, None, None)
+    out = _cabi.mm_fp8(ad, bd, sa_r.to(DEV), sb_r.to(DEV), 0, None, None)
     assert_bf16_close(out, O.fp8_gemm_bias(a8, b8, sa_r, sb_r, None), what="row/column steps")
 
 

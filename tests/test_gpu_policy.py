@@ -111,12 +111,41 @@ def test_weight_code_cache_changes_no_output(recipe_name):
         return outs, state
 
     plain, plain_state = run(False)
-    cached, cached_state = run(True)
-    for i, (a, c) in enumerate(zip(plain, cached)):
-        assert torch.equal(a, c), f"step {i}"
-    if recipe_name == "delayed":
-        for a, c in zip(plain_state, cached_state):
-            assert torch.equal(a, c)
+    for mode in (True, None):   # None: the default, which caches here (the weight takes no gradient)
+        cached, cached_state = run(mode)
+        for i, (a, c) in enumerate(zip(plain, cached)):
+            assert torch.equal(a, c), f"mode {mode} step {i}"
+        if recipe_name == "delayed":
+            for a, c in zip(plain_state, cached_state):
+                assert torch.equal(a, c)
+
+
+def test_weight_code_cache_default_follows_autograd():
+    """By default a weight's codes are kept exactly where nothing can be training it:
+    autograd off, or a weight without gradient; a weight under training is quantized in
+    every forward, as the reference does (fp8.py:291-299)."""
+    from astrai_amd.extension import fp8 as P
+    st = P.fp8_state()
+    st.reset()
+    w = torch.randn(40, 96).to(torch.bfloat16).to(DEV)
+    wp = torch.nn.Parameter(w.clone())
+    assert st.cache_weights is None
+    assert st.caches_weight(w) and not st.caches_weight(wp)
+    with torch.no_grad():
+        assert st.caches_weight(wp)
+    x = torch.randn(8, 96).to(torch.bfloat16).to(DEV)
+    with P.fp8_autocast(True, recipe=P.DynamicScaling(), fp8_format="e4m3"):
+        F.linear(x, wp)
+        assert not st._dyn_w                      # training: nothing kept
+        with torch.no_grad():
+            y0 = F.linear(x, wp)
+            assert len(st._dyn_w) == 1            # inference: codes kept ...
+            wp.mul_(2.0)
+            y1 = F.linear(x, wp)                  # ... and remade after a write
+        P.fp8_cache_weights(False)
+        with torch.no_grad():
+            assert torch.equal(F.linear(x, wp), y1) and not torch.equal(y0, y1)
+    st.reset()
 
 
 def test_int8_autocast_linear_matches_oracle_and_caches_weights():

@@ -40,6 +40,34 @@ def test_fp8_quantize_every_bf16_value(C, fmt, scale):
     assert amax.shape == (1,) and amax.item() == want_amax.item()
 
 
+@pytest.mark.parametrize("fmt", [0, 1])
+def test_fp8_quantize_every_bf16_value_many_steps(C, fmt):
+    """The quantizer forms its quotients from a reciprocal, an exact remainder and a correction,
+    and falls back to the IEEE division only near a rounding point of the conversion: all 65536
+    bf16 patterns -- infinities (saturate) and NaNs (stay NaN) included -- under 60 steps: random
+    ones, powers of two (every quotient exact, ties everywhere), steps whose reciprocal rounds
+    badly (mantissa all ones, just above a power of two), tiny and huge ones (the division path
+    throughout), the 1e-12 floor of the scaling policy."""
+    bits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    x = torch.from_numpy(bits.view(np.int16).copy()).view(torch.bfloat16)
+    nan = torch.isnan(x.float())
+    g = torch.Generator().manual_seed(77 + fmt)
+    steps = torch.exp2(torch.rand(40, generator=g) * 30.0 - 20.0).tolist()
+    ones = np.array([0x3fffffff, 0x3f800001, 0x3effffff, 0x40000001, 0x3a7fffff], dtype=np.uint32).view(np.float32)
+    steps += [1.0, 0.25, 2.0 ** -9, 64.0, 448.0, 1.0 / 448.0, 57344.0, 1e-12, 2.0 ** -70, 2.0 ** 70,
+              2.0 ** -61, 2.0 ** 61, 3.0, 0.1, 7.0 / 448.0] + [float(v) for v in ones]
+    xd = x.to(DEV)
+    for step in steps:
+        s = torch.tensor([step], dtype=torch.float32)
+        want, _ = O.fp8_quantize_saturating(torch.where(nan, torch.zeros_like(x), x), s, fmt)
+        got, _ = C.quantize_bf16(xd, s.to(DEV), fmt)
+        gc, wc = _codes(got), _codes(want)
+        bad = (gc != wc) & ~nan
+        assert not bad.any(), (f"step {step!r} fmt {fmt}: {int(bad.sum())} codes differ, first at bf16 pattern "
+                               f"{int(bad.nonzero()[0])}: got {int(gc[bad][0])} want {int(wc[bad][0])}")
+        assert torch.isnan(got.cpu().float()[nan]).all(), f"step {step!r}: a NaN became a number"
+
+
 def test_fp8_quantize_reference_vector_scale_half(C, golden):
     # tests/extension/test_fp8_mma.py:65-77
     torch.manual_seed(3)

@@ -31,6 +31,51 @@ def test_rotary_is_a_rotation_with_relative_position_property():
     torch.testing.assert_close(y[0, 1, 0, :2], torch.tensor([torch.cos(torch.tensor(1.0)), torch.sin(torch.tensor(1.0))]))
 
 
+def test_ntk_rope_scaling_stretches_the_base_by_the_closed_form():
+    """rope_scaling {"type": "ntk", "factor": f} multiplies the base by f^(d/(d-2))
+    (components/rope.py:27-54): the model's table and the oracle's against angles computed from
+    that closed form with Python floats; factor 1, no scaling and a non-NTK type give the plain
+    table; the scaled model follows the oracle end to end."""
+    import math
+    from astrai_amd.model import AutoRegressiveLM, AutoRegressiveLMConfig
+    from astrai_amd.model.decoder import get_rotary_emb, ntk_base, rotary_base
+    d, theta, factor = 64, 10000.0, 4.0
+    assert ntk_base(theta, d, factor) == theta * factor ** (d / (d - 2))
+    assert rotary_base(None, d, None) == 10000.0 and rotary_base(5e5, d, None) == 5e5
+    assert rotary_base(theta, d, {"factor": factor}) == ntk_base(theta, d, factor)          # default type
+    assert rotary_base(theta, d, {"type": "linear", "factor": factor}) == theta             # rope.py:47-50
+    assert rotary_base(theta, d, {"type": "ntk", "factor": 1.0}) == theta
+    table = get_rotary_emb(d, 40, rotary_base(theta, d, {"type": "ntk", "factor": factor}))
+    base = theta * factor ** (d / (d - 2))
+    for pos, pair in ((0, 0), (1, 0), (7, 3), (39, 31), (23, 17)):
+        ang = pos * base ** (-2 * pair / d)
+        want = torch.tensor([math.cos(ang), math.sin(ang)])
+        # the table rounds the angle to fp32 before cos / sin (reference: freqs.float())
+        assert torch.allclose(table[pos, pair], want, atol=2e-6 * max(1.0, ang)), (pos, pair)
+    # the highest frequency is stretched least, the lowest by the whole factor^(d/(d-2)) ... ^((d-2)/d) = factor
+    plain = get_rotary_emb(d, 40, theta)
+    assert torch.equal(table[:, 0], plain[:, 0])                  # pair 0: angle = position, base-free
+    ratio = (theta ** (-(d - 2) / d)) / (base ** (-(d - 2) / d))  # slowest pair's wavelength grows by `factor`
+    assert abs(ratio - factor) < 1e-9
+    cfg = AutoRegressiveLMConfig(vocab_size=97, hidden_size=128, num_hidden_layers=2, num_attention_heads=2,
+                                 num_key_value_heads=1, intermediate_size=192, max_position_embeddings=64,
+                                 rope_scaling={"type": "ntk", "factor": factor})
+    torch.manual_seed(5)
+    model = AutoRegressiveLM(cfg).to(torch.bfloat16).eval()
+    # (casting the model casts the table, as in the reference, where it is a float buffer too)
+    assert torch.equal(model.freqs_cis, get_rotary_emb(64, 64, ntk_base(10000.0, 64, factor)).to(torch.bfloat16))
+    assert not torch.equal(model.freqs_cis, get_rotary_emb(64, 64, 10000.0).to(torch.bfloat16))
+    ids = torch.randint(0, 97, (2, 24), generator=torch.Generator().manual_seed(6))
+    sd = {k: v.detach() for k, v in model.state_dict().items()}
+    with torch.no_grad():
+        got = model(ids)["logits"]
+        want = D.forward(sd, cfg, ids, D.bf16_linear_fn(sd))
+        cfg.rope_scaling = None
+        unscaled = D.forward(sd, cfg, ids, D.bf16_linear_fn(sd))
+    torch.testing.assert_close(got.float(), want.float(), atol=2e-2, rtol=2e-2)
+    assert not torch.equal(want, unscaled)   # the scaling is not a no-op at 24 positions
+
+
 def test_repeat_kv_repeats_each_head_in_place():
     x = torch.arange(2 * 3).float().reshape(1, 1, 2, 3)
     y = D.repeat_kv(x, 2)
