@@ -117,8 +117,42 @@ int astrai_w8a8_quantize_bf16_fp8(const void* x, void* x8, const float* scale, f
     if (!aligned16(x) || !aligned16(x8))
         return fail(ASTRAI_W8A8_BAD_ARG, "quantize_bf16_fp8: pointers must be 16-byte aligned");
     if (total == 0) return ASTRAI_W8A8_OK;
-    w8a8::launch_quantize_fp8(x, x8, scale, amax, total, fmt, static_cast<hipStream_t>(stream));
+    w8a8::launch_quantize_fp8(x, x8, scale, amax, nullptr, total, fmt, static_cast<hipStream_t>(stream));
     return check_launch("quantize_bf16_fp8");
+}
+
+int astrai_w8a8_quantize_bf16_fp8_partials(const void* x, void* x8, const float* scale, float* partials,
+                                           int64_t total, int fmt, void* stream) {
+    if (!x || !x8 || !scale || !partials)
+        return fail(ASTRAI_W8A8_BAD_ARG, "quantize_bf16_fp8_partials: null pointer");
+    if (total <= 0) return fail(ASTRAI_W8A8_BAD_ARG, "quantize_bf16_fp8_partials: size must be positive");
+    if (fmt != ASTRAI_W8A8_E4M3 && fmt != ASTRAI_W8A8_E5M2)
+        return fail(ASTRAI_W8A8_BAD_ARG, "quantize_bf16_fp8_partials: fmt must be 0 (e4m3) or 1 (e5m2)");
+    if (!aligned16(x) || !aligned16(x8))
+        return fail(ASTRAI_W8A8_BAD_ARG, "quantize_bf16_fp8_partials: pointers must be 16-byte aligned");
+    w8a8::launch_quantize_fp8(x, x8, scale, nullptr, partials, total, fmt, static_cast<hipStream_t>(stream));
+    return check_launch("quantize_bf16_fp8_partials");
+}
+
+int astrai_w8a8_amax_bf16_partials(const void* x, float* partials, int64_t total, void* stream) {
+    if (!x || !partials) return fail(ASTRAI_W8A8_BAD_ARG, "amax_bf16_partials: null pointer");
+    if (total <= 0) return fail(ASTRAI_W8A8_BAD_ARG, "amax_bf16_partials: size must be positive");
+    if (!aligned16(x)) return fail(ASTRAI_W8A8_BAD_ARG, "amax_bf16_partials: x must be 16-byte aligned");
+    w8a8::launch_amax_bf16(x, nullptr, partials, total, static_cast<hipStream_t>(stream));
+    return check_launch("amax_bf16_partials");
+}
+
+int astrai_w8a8_amax_ring_push_partials(float* hist, int n, int idx, const float* partials, float* amax_out,
+                                        float* scale, float fmax, float pow2_margin, void* stream) {
+    if (!hist || !partials || !scale)
+        return fail(ASTRAI_W8A8_BAD_ARG, "amax_ring_push_partials: null pointer");
+    if (n <= 0 || idx < 0 || idx >= n)
+        return fail(ASTRAI_W8A8_BAD_ARG, "amax_ring_push_partials: idx must lie in [0, n)");
+    if (!(fmax > 0.0f) || !(pow2_margin > 0.0f))
+        return fail(ASTRAI_W8A8_BAD_ARG, "amax_ring_push_partials: fmax and pow2_margin must be positive");
+    w8a8::launch_amax_ring_push(hist, n, idx, nullptr, partials, amax_out, scale, fmax, pow2_margin,
+                                static_cast<hipStream_t>(stream));
+    return check_launch("amax_ring_push_partials");
 }
 
 int astrai_w8a8_amax_bf16(const void* x, float* amax, int64_t total, void* stream) {
@@ -126,7 +160,7 @@ int astrai_w8a8_amax_bf16(const void* x, float* amax, int64_t total, void* strea
     if (total < 0) return fail(ASTRAI_W8A8_BAD_ARG, "amax_bf16: negative size");
     if (!aligned16(x)) return fail(ASTRAI_W8A8_BAD_ARG, "amax_bf16: x must be 16-byte aligned");
     if (total == 0) return ASTRAI_W8A8_OK;
-    w8a8::launch_amax_bf16(x, amax, total, static_cast<hipStream_t>(stream));
+    w8a8::launch_amax_bf16(x, amax, nullptr, total, static_cast<hipStream_t>(stream));
     return check_launch("amax_bf16");
 }
 
@@ -137,7 +171,7 @@ int astrai_w8a8_amax_ring_push(float* hist, int n, int idx, const float* amax, f
         return fail(ASTRAI_W8A8_BAD_ARG, "amax_ring_push: idx must lie in [0, n)");
     if (!(fmax > 0.0f) || !(pow2_margin > 0.0f))
         return fail(ASTRAI_W8A8_BAD_ARG, "amax_ring_push: fmax and pow2_margin must be positive");
-    w8a8::launch_amax_ring_push(hist, n, idx, amax, scale, fmax, pow2_margin,
+    w8a8::launch_amax_ring_push(hist, n, idx, amax, nullptr, nullptr, scale, fmax, pow2_margin,
                                 static_cast<hipStream_t>(stream));
     return check_launch("amax_ring_push");
 }

@@ -47,13 +47,18 @@ struct GemmArgs {
 };
 
 // quantize.hip
-void launch_quantize_fp8(const void* x, void* x8, const float* scale, float* amax,
+// The maximum of |x| leaves a quantizer either by atomic max into *amax or, when `partials` is
+// given, as kAmaxPartials per-workgroup maxima (every slot written) for the ring push to reduce.
+constexpr int kAmaxPartials = 1024;
+void launch_quantize_fp8(const void* x, void* x8, const float* scale, float* amax, float* partials,
                          int64_t total, int fmt, hipStream_t stream);
-// hist[idx] = *amax; *scale = max((max(hist) / fmax) / pow2_margin, 1e-12)
-void launch_amax_ring_push(float* hist, int n, int idx, const float* amax, float* scale,
-                           float fmax, float pow2_margin, hipStream_t stream);
-// *amax = max(*amax, max |x|)
-void launch_amax_bf16(const void* x, float* amax, int64_t total, hipStream_t stream);
+// hist[idx] = fresh; *scale = max((max(hist) / fmax) / pow2_margin, 1e-12), with fresh = *amax or
+// the maximum of the kAmaxPartials partials (then also stored to *amax_out when that is given)
+void launch_amax_ring_push(float* hist, int n, int idx, const float* amax, const float* partials,
+                           float* amax_out, float* scale, float fmax, float pow2_margin,
+                           hipStream_t stream);
+// *amax = max(*amax, max |x|), or the partial maxima
+void launch_amax_bf16(const void* x, float* amax, float* partials, int64_t total, hipStream_t stream);
 // codes of a [rows, cols] matrix row-major (x8, may be null) and transposed (x8t, [cols, rows])
 void launch_quantize_transpose_fp8(const void* x, void* x8, void* x8t, const float* scale,
                                    float* amax, int64_t rows, int64_t cols, int fmt,

@@ -90,9 +90,21 @@ __device__ __forceinline__ uint32_t quant1_int8(float f, float step) {
 // dozen atomics that have drained long before the tensor has streamed -- and at the
 // end a workgroup touches the slot only if its share has outgrown what the slot
 // holds by then, which a few dozen out of a thousand do on unsorted data.
-constexpr int kAmaxBlocks = 1024;  // grid cap: the workgroups stride over the tensor
+constexpr int kAmaxBlocks = kAmaxPartials;  // grid cap: the workgroups stride over the tensor
 constexpr int kUnroll = 4;         // independent 16-byte loads in flight per thread
 constexpr int kEarlyEvery = 16;
+
+// The other way to report the maximum: every workgroup stores its own into slot blockIdx.x of
+// a kAmaxBlocks-wide array (workgroup 0 zeroes the slots no workgroup owns) and the kernel
+// that consumes the maximum -- the ring push, one wave -- reduces the array. No atomics, no
+// slot to clear beforehand, nothing that waits at the end of the kernel: 3-4 us less than
+// the atomic form on a 4096 x 4096 tensor, and the cleared slot's fill launch besides.
+__device__ __forceinline__ void store_partial(float* partials, float local, float* slots) {
+    const float m = block_max(local, slots);
+    if (threadIdx.x == 0) partials[blockIdx.x] = m;
+    if (blockIdx.x == 0)
+        for (int i = gridDim.x + threadIdx.x; i < kAmaxBlocks; i += kThreads) partials[i] = 0.0f;
+}
 
 __device__ __forceinline__ void publish_early(float* amax, float local, float* slots) {
     const float m = block_max(local, slots);
@@ -103,7 +115,7 @@ __device__ __forceinline__ void publish_early(float* amax, float local, float* s
 template <int Fmt>
 __global__ __launch_bounds__(kThreads) void quantize_fp8_kernel(
     const uint16_t* __restrict__ x, uint8_t* __restrict__ x8, const float* __restrict__ scale,
-    float* __restrict__ amax, int64_t total) {
+    float* __restrict__ amax, float* __restrict__ partials, int64_t total) {
     __shared__ float slots[kThreads / kWave];
     const float step = *scale;
     float local = 0.0f;
@@ -128,7 +140,7 @@ __global__ __launch_bounds__(kThreads) void quantize_fp8_kernel(
         group(v);
         v += kUnroll * stride;
     }
-    if (amax && gridDim.x >= 64 && blockIdx.x % kEarlyEvery == 0) publish_early(amax, local, slots);
+    if (amax && !partials && gridDim.x >= 64 && blockIdx.x % kEarlyEvery == 0) publish_early(amax, local, slots);
     for (; v + (kUnroll - 1) * stride < nvec; v += kUnroll * stride) group(v);
     for (; v < nvec; v += stride) {
         float f[8];
@@ -144,7 +156,9 @@ __global__ __launch_bounds__(kThreads) void quantize_fp8_kernel(
             x8[i] = (uint8_t)cvt_pk_fp8<Fmt>(f / step, 0.0f);
         }
     }
-    if (amax) {
+    if (partials) {
+        store_partial(partials, local, slots);
+    } else if (amax) {
         const float m = block_max(local, slots);
         if (threadIdx.x == 0) atomic_max_nonneg(amax, m);
     }
@@ -155,7 +169,7 @@ __global__ __launch_bounds__(kThreads) void quantize_fp8_kernel(
 // (astrai/extension/fp8.py:289-292: t.abs().amax()); this is that reduction as one
 // read of the tensor, without the intermediate |x| tensor.
 __global__ __launch_bounds__(kThreads) void amax_bf16_kernel(
-    const uint16_t* __restrict__ x, float* __restrict__ amax, int64_t total) {
+    const uint16_t* __restrict__ x, float* __restrict__ amax, float* __restrict__ partials, int64_t total) {
     __shared__ float slots[kThreads / kWave];
     float local = 0.0f;
     const int64_t nvec = total >> 3;
@@ -176,7 +190,7 @@ __global__ __launch_bounds__(kThreads) void amax_bf16_kernel(
         group(v);
         v += kUnroll * stride;
     }
-    if (gridDim.x >= 64 && blockIdx.x % kEarlyEvery == 0) publish_early(amax, local, slots);
+    if (amax && gridDim.x >= 64 && blockIdx.x % kEarlyEvery == 0) publish_early(amax, local, slots);
     for (; v + (kUnroll - 1) * stride < nvec; v += kUnroll * stride) group(v);
     for (; v < nvec; v += stride) {
         float f[8];
@@ -187,6 +201,10 @@ __global__ __launch_bounds__(kThreads) void amax_bf16_kernel(
         const int64_t i = nvec * 8 + threadIdx.x;
         if (i < total) local = fmaxf(local, fabsf(bf16_to_f32(x[i])));
     }
+    if (partials) {
+        store_partial(partials, local, slots);
+        return;
+    }
     const float m = block_max(local, slots);
     if (threadIdx.x == 0) atomic_max_nonneg(amax, m);
 }
@@ -196,9 +214,21 @@ __global__ __launch_bounds__(kThreads) void amax_bf16_kernel(
 // record-then-refresh of FP8TensorMeta (astrai/extension/fp8.py:147-173, formula
 // :87-89) as one single-wave launch instead of six tiny ones.
 // (amax may be the ring's own slot: dynamic scaling is a ring of length one)
+// (partials: the fresh value is the maximum of a quantizer's kAmaxBlocks per-workgroup maxima
+// instead of *amax; amax_out, when given, receives it)
 __global__ __launch_bounds__(kWave) void amax_ring_push_kernel(
-    float* hist, int n, int idx, const float* amax, float* scale, float fmax, float pow2_margin) {
-    const float fresh = *amax;
+    float* hist, int n, int idx, const float* amax, const float* partials, float* amax_out,
+    float* scale, float fmax, float pow2_margin) {
+    float fresh;
+    if (partials) {
+        float m = 0.0f;
+#pragma unroll
+        for (int i = 0; i < kAmaxBlocks / kWave; ++i) m = fmaxf(m, partials[i * kWave + threadIdx.x]);
+        fresh = wave_max(m);
+        if (amax_out && threadIdx.x == 0) *amax_out = fresh;
+    } else {
+        fresh = *amax;
+    }
     float peak = 0.0f;
     for (int i = threadIdx.x; i < n; i += kWave) {
         float h = hist[i];
@@ -469,9 +499,8 @@ __global__ __launch_bounds__(kThreads) void add_rmsnorm_quantize_int8_rows_kerne
 // per row and a barrier after each reduction the kernel is bound by the latency of its
 // load -> reduce -> store chain (16,384 x 2048: 32 us for 100 MB), not by memory bandwidth.
 // NORM: y = bf16(w * (rstd * x)), rstd = rsqrt(mean(x^2) + eps), then the per-row int8
-// quantizer on y; otherwise the quantizer on x itself. The sum of squares is taken in another
-// order than in the one-workgroup-per-row kernel (a wave's tree over per-lane sums), which
-// is inside the fp32 rounding of that sum; the maxima and codes follow from it exactly.
+// quantizer on y; otherwise the quantizer on x itself. The sum of squares is taken in the
+// order of the one-workgroup-per-row kernel, so both kernels give a row the same bits.
 template <int KC, bool NORM>
 __global__ __launch_bounds__(kThreads) void wave_rows_int8_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, float eps,
@@ -506,15 +535,26 @@ __global__ __launch_bounds__(kThreads) void wave_rows_int8_kernel(
         float v[KC][8];
         float local = 0.0f;
         if constexpr (NORM) {
-            float ss = 0.0f;
+            // The sum of squares in the order of the one-workgroup-per-row kernel, so that a row's
+            // rstd -- and with it y and every code -- does not depend on how many rows a launch
+            // holds: there thread t = i mod 256 sums the pieces i = t, t + 256, ... as they come,
+            // each of the four waves reduces its 64 threads by the same butterfly, and the four
+            // results are added in wave order. Lane l holds the pieces of threads l, l + 64,
+            // l + 128, l + 192: four running sums, four butterflies, the same three additions.
+            float ssw[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int c = 0; c < KC; ++c) {
                 unpack8(cur[c], v[c]);
 #pragma unroll
-                for (int j = 0; j < 8; ++j) ss += v[c][j] * v[c][j];
+                for (int j = 0; j < 8; ++j) ssw[c & 3] += v[c][j] * v[c][j];
             }
 #pragma unroll
-            for (int off = 32; off; off >>= 1) ss += __shfl_xor(ss, off, kWave);
+            for (int wv = 0; wv < 4; ++wv)
+#pragma unroll
+                for (int off = 32; off; off >>= 1) ssw[wv] += __shfl_xor(ssw[wv], off, kWave);
+            float ss = ssw[0];
+#pragma unroll
+            for (int wv = 1; wv < 4; ++wv) ss += ssw[wv];
             const float rstd = rsqrtf(ss / (float)k + eps);
 #pragma unroll
             for (int c = 0; c < KC; ++c) {
@@ -792,7 +832,7 @@ __global__ __launch_bounds__(kThreads) void quantize_fp8_weight128_kernel(
 
 }  // namespace
 
-void launch_quantize_fp8(const void* x, void* x8, const float* scale, float* amax,
+void launch_quantize_fp8(const void* x, void* x8, const float* scale, float* amax, float* partials,
                          int64_t total, int fmt, hipStream_t stream) {
     if (total <= 0) return;
     const int64_t nvec = (total + 7) / 8;
@@ -803,24 +843,25 @@ void launch_quantize_fp8(const void* x, void* x8, const float* scale, float* ama
     auto xo = static_cast<uint8_t*>(x8);
     if (fmt)
         quantize_fp8_kernel<1><<<dim3((unsigned)blocks), dim3(kThreads), 0, stream>>>(
-            xs, xo, scale, amax, total);
+            xs, xo, scale, amax, partials, total);
     else
         quantize_fp8_kernel<0><<<dim3((unsigned)blocks), dim3(kThreads), 0, stream>>>(
-            xs, xo, scale, amax, total);
+            xs, xo, scale, amax, partials, total);
 }
 
-void launch_amax_ring_push(float* hist, int n, int idx, const float* amax, float* scale,
-                           float fmax, float pow2_margin, hipStream_t stream) {
-    amax_ring_push_kernel<<<dim3(1), dim3(kWave), 0, stream>>>(hist, n, idx, amax, scale, fmax,
-                                                               pow2_margin);
+void launch_amax_ring_push(float* hist, int n, int idx, const float* amax, const float* partials,
+                           float* amax_out, float* scale, float fmax, float pow2_margin,
+                           hipStream_t stream) {
+    amax_ring_push_kernel<<<dim3(1), dim3(kWave), 0, stream>>>(hist, n, idx, amax, partials, amax_out,
+                                                               scale, fmax, pow2_margin);
 }
 
-void launch_amax_bf16(const void* x, float* amax, int64_t total, hipStream_t stream) {
+void launch_amax_bf16(const void* x, float* amax, float* partials, int64_t total, hipStream_t stream) {
     if (total <= 0) return;
     int64_t blocks = ((total + 7) / 8 + 2 * kUnroll * kThreads - 1) / (2 * kUnroll * kThreads);
     if (blocks > kAmaxBlocks) blocks = kAmaxBlocks;
     amax_bf16_kernel<<<dim3((unsigned)blocks), dim3(kThreads), 0, stream>>>(
-        static_cast<const uint16_t*>(x), amax, total);
+        static_cast<const uint16_t*>(x), amax, partials, total);
 }
 
 void launch_quantize_transpose_fp8(const void* x, void* x8, void* x8t, const float* scale,

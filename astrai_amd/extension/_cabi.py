@@ -36,6 +36,9 @@ PROTOTYPES = {
     "astrai_w8a8_quantize_bf16_fp8": ([_P, _P, _P, _P, _I64, _INT, _P], _INT),
     "astrai_w8a8_amax_bf16": ([_P, _P, _I64, _P], _INT),
     "astrai_w8a8_amax_ring_push": ([_P, _INT, _INT, _P, _P, _F32, _F32, _P], _INT),
+    "astrai_w8a8_quantize_bf16_fp8_partials": ([_P, _P, _P, _P, _I64, _INT, _P], _INT),
+    "astrai_w8a8_amax_bf16_partials": ([_P, _P, _I64, _P], _INT),
+    "astrai_w8a8_amax_ring_push_partials": ([_P, _INT, _INT, _P, _P, _P, _F32, _F32, _P], _INT),
     "astrai_w8a8_quantize_transpose_bf16_fp8": ([_P, _P, _P, _P, _P, _I64, _I64, _INT, _P], _INT),
     "astrai_w8a8_quantize_bf16_int8_rows": ([_P, _P, _P, _I64, _I64, _P], _INT),
     "astrai_w8a8_add_rmsnorm_quantize_int8_rows": (
@@ -400,6 +403,75 @@ def amax_ring_push(hist: torch.Tensor, idx: int, amax: torch.Tensor, scale: torc
         _check(lib.astrai_w8a8_amax_ring_push(hist.data_ptr(), hist.numel(), int(idx),
                                              amax.data_ptr(), scale.data_ptr(), float(fmax),
                                              float(pow2_margin), _stream(hist)), lib)
+
+
+AMAX_PARTIALS = 1024   # ASTRAI_W8A8_AMAX_PARTIALS
+
+
+def new_amax_partials(device) -> torch.Tensor:
+    """A zeroed array for the per-workgroup maxima of :func:`quantize_bf16_partials` /
+    :func:`amax_bf16_partials` (producer and consumer must run on one stream)."""
+    return torch.zeros(AMAX_PARTIALS, device=device, dtype=torch.float32)
+
+
+def _check_partials(partials: torch.Tensor, ref: torch.Tensor) -> None:
+    if not (partials.is_cuda and partials.device == ref.device and partials.dtype == torch.float32
+            and partials.numel() == AMAX_PARTIALS and partials.is_contiguous()):
+        raise RuntimeError(f"partials must be a contiguous float32 tensor of {AMAX_PARTIALS} elements on the input device")
+
+
+def quantize_bf16_partials(x: torch.Tensor, scale: torch.Tensor, fmt: int, partials: torch.Tensor) -> torch.Tensor:
+    """:func:`quantize_bf16` with max |x| left as per-workgroup maxima in ``partials`` (every
+    slot written) for :func:`amax_ring_push_partials`; returns the codes."""
+    lib = _require()
+    _gpu(x, "quantize_bf16_partials")
+    if x.dtype != torch.bfloat16:
+        raise RuntimeError("x must be bf16")
+    _check_scale(scale, x, "scale")
+    _check_partials(partials, x)
+    x_c = x.contiguous()
+    with _on_device(x.device):
+        x8 = torch.empty_like(x_c, dtype=torch.float8_e5m2 if fmt else torch.float8_e4m3fn)
+        if x_c.numel():
+            _check(lib.astrai_w8a8_quantize_bf16_fp8_partials(
+                x_c.data_ptr(), x8.data_ptr(), scale.data_ptr(), partials.data_ptr(),
+                x_c.numel(), 1 if fmt else 0, _stream(x)), lib)
+        else:
+            partials.zero_()
+    return x8
+
+
+def amax_bf16_partials(x: torch.Tensor, partials: torch.Tensor) -> None:
+    """max |x| of a bf16 tensor as per-workgroup maxima in ``partials`` (every slot written)."""
+    lib = _require()
+    _gpu(x, "amax_bf16_partials")
+    if x.dtype != torch.bfloat16:
+        raise RuntimeError("x must be bf16")
+    _check_partials(partials, x)
+    x_c = x.contiguous()
+    with _on_device(x.device):
+        if x_c.numel():
+            _check(lib.astrai_w8a8_amax_bf16_partials(x_c.data_ptr(), partials.data_ptr(), x_c.numel(),
+                                                     _stream(x)), lib)
+        else:
+            partials.zero_()
+
+
+def amax_ring_push_partials(hist: torch.Tensor, idx: int, partials: torch.Tensor, scale: torch.Tensor,
+                            fmax: float, pow2_margin: float, amax_out: Optional[torch.Tensor] = None) -> None:
+    """:func:`amax_ring_push` with the fresh amax taken as the maximum of ``partials``."""
+    lib = _require()
+    _gpu(hist, "amax_ring_push_partials")
+    for t, name in ((hist, "hist"), (scale, "scale")) + (((amax_out, "amax_out"),) if amax_out is not None else ()):
+        if not (t.is_cuda and t.device == hist.device and t.dtype == torch.float32 and t.is_contiguous()):
+            raise RuntimeError(f"{name} must be a contiguous float32 tensor on the ring's device")
+    _check_partials(partials, hist)
+    if scale.numel() != 1 or (amax_out is not None and amax_out.numel() != 1):
+        raise RuntimeError("scale and amax_out must have one element")
+    with _on_device(hist.device):
+        _check(lib.astrai_w8a8_amax_ring_push_partials(
+            hist.data_ptr(), hist.numel(), int(idx), partials.data_ptr(), _ptr(amax_out), scale.data_ptr(),
+            float(fmax), float(pow2_margin), _stream(hist)), lib)
 
 
 def quantize_transpose_bf16(x: torch.Tensor, scale: torch.Tensor, fmt: int,

@@ -29,12 +29,16 @@ import torch
 from astrai_amd.extension import dispatch
 from astrai_amd.extension.ops.fp8 import (
     amax_bf16,
+    amax_bf16_partials,
     amax_ring_push,
+    amax_ring_push_partials,
     linear_backward_fp8,
     linear_forward_fp8,
     mm_fp8,
     mm_fp8_bias,
+    new_amax_partials,
     quantize_bf16,
+    quantize_bf16_partials,
 )
 
 FP8_MAX = {"e4m3": 448.0, "e5m2": 57344.0}
@@ -95,13 +99,33 @@ class DynamicScaling(FP8Recipe):
 class _AmaxRing:
     """One operand's amax history, write cursor, derived step and seeded flag."""
 
-    __slots__ = ("hist", "idx", "scale", "seeded")
+    __slots__ = ("hist", "idx", "scale", "seeded", "_partials")
 
     def __init__(self, device: torch.device, n: int):
         self.hist = torch.ones(n, device=device, dtype=torch.float32)
         self.scale = torch.ones(1, device=device, dtype=torch.float32)
         self.idx = 0
         self.seeded = False
+        self._partials = None
+
+    def takes_partials(self, recipe: FP8Recipe) -> bool:
+        """The fast bookkeeping applies: device ring, a stock recipe (both take the window's
+        maximum)."""
+        return self.hist.is_cuda and type(recipe) in (DelayedScaling, DynamicScaling)
+
+    @property
+    def partials(self) -> torch.Tensor:
+        """Scratch through which a quantizer hands this ring the amax it saw, as one maximum
+        per workgroup (no slot to clear, no atomics); made on first use."""
+        if self._partials is None:
+            self._partials = new_amax_partials(self.hist.device)
+        return self._partials
+
+    def push_partials(self, recipe: FP8Recipe, fmt: str) -> None:
+        """:meth:`push` of the amax a quantizer has just left in :attr:`partials`."""
+        amax_ring_push_partials(self.hist, self.idx, self.partials, self.scale, FP8_MAX[fmt],
+                                float(2 ** recipe.margin))
+        self.idx = (self.idx + 1) % self.hist.numel()
 
     def push(self, amax: torch.Tensor, recipe: FP8Recipe, fmt: str) -> None:
         # record first, then refresh: the step used next reflects amax seen so far
@@ -212,6 +236,7 @@ class FP8State:
         # the version counter (``w.data`` tricks of some optimizers) would go unseen.
         self.cache_weights: Optional[bool] = None
         self._dyn_w: Dict[Tuple, Tuple] = {}
+        self._scratch: Dict[Tuple, Tuple] = {}
 
     def get_weight_meta(self, w: torch.Tensor) -> FP8TensorMeta:
         key = (w.data_ptr(), w.shape, w.dtype)
@@ -239,6 +264,17 @@ class FP8State:
         self._dyn_w[key] = (weakref.ref(w), w._version, sw, w8)
         return sw, w8
 
+    def scratch(self, device: torch.device):
+        """``(partials, slot)`` of dynamic scaling on ``device`` and the current stream: the
+        per-workgroup maxima of the tensor being measured and a ring of one to push them
+        through. Per stream, because a measurement and its push are ordered by the stream only."""
+        key = (device, torch.cuda.current_stream(device).cuda_stream)
+        hit = self._scratch.get(key)
+        if hit is None:
+            hit = self._scratch[key] = (new_amax_partials(device),
+                                        torch.zeros(1, device=device, dtype=torch.float32))
+        return hit
+
     def caches_weight(self, w: torch.Tensor) -> bool:
         if self.cache_weights is not None:
             return self.cache_weights
@@ -249,6 +285,7 @@ class FP8State:
         self.cache_weights = None
         self._metas.clear()
         self._dyn_w.clear()
+        self._scratch.clear()
         self._last_device = None
 
 
@@ -283,14 +320,17 @@ def fp8_autocast(
 
 def _dynamic_scale(t: torch.Tensor, recipe: FP8Recipe, fmt: str) -> torch.Tensor:
     if t.is_cuda and t.dtype == torch.bfloat16:
-        amax = amax_bf16(t)  # one read, no |t| temporary
-        if type(recipe) in (DelayedScaling, DynamicScaling):
-            # a window of one: max((amax / FP8_MAX) / 2^margin, floor) in one launch
+        if type(recipe) in (DelayedScaling, DynamicScaling) and t.numel():
+            # one read of t (no |t| temporary) leaves one maximum per workgroup; a window of
+            # one then turns them into max((amax / FP8_MAX) / 2^margin, floor) in one launch
             # (flooring amax first, as the host formula does, cannot change that)
-            scale = torch.empty_like(amax)
-            amax_ring_push(amax, 0, amax, scale, FP8_MAX[fmt], float(2 ** recipe.margin))
+            st = fp8_state()
+            partials, slot = st.scratch(t.device)
+            scale = torch.empty(1, device=t.device, dtype=torch.float32)
+            amax_bf16_partials(t, partials)
+            amax_ring_push_partials(slot, 0, partials, scale, FP8_MAX[fmt], float(2 ** recipe.margin))
             return scale
-        amax = amax.reshape(()).clamp_min(_FLOOR)
+        amax = amax_bf16(t).reshape(()).clamp_min(_FLOOR)
     else:
         amax = t.abs().amax().to(torch.float32).clamp_min(_FLOOR)
     return recipe.scale_from_history(amax, fmt)
@@ -332,11 +372,31 @@ def fp8_linear_forward(x: torch.Tensor, w: torch.Tensor, bias=None):
             w8, amax_w = quantize_bf16(w, meta.w_scale, "e4m3")
             meta.w_cached = (weakref.ref(w), w._version, w8, amax_w)
         x2 = x.reshape(-1, w.size(1))
-        x8, amax_x = quantize_bf16(x2, meta.x_scale, "e4m3")
         has_bias = bias is not None and bias.numel() > 0
+        if meta._x.takes_partials(meta.recipe) and x2.numel():
+            x8 = quantize_bf16_partials(x2, meta.x_scale, "e4m3", meta._x.partials)
+            out = mm_fp8_bias(x8, meta.w_cached[2], meta.x_scale, meta.w_scale,
+                              bias if has_bias else None).reshape(*x.shape[:-1], w.size(0))
+            meta._x.push_partials(meta.recipe, fmt)
+            return out
+        x8, amax_x = quantize_bf16(x2, meta.x_scale, "e4m3")
         out = mm_fp8_bias(x8, meta.w_cached[2], meta.x_scale, meta.w_scale,
                           bias if has_bias else None).reshape(*x.shape[:-1], w.size(0))
         meta.update_x(amax_x, fmt)
+        return out
+    if meta._x.takes_partials(meta.recipe) and meta._w.takes_partials(meta.recipe) and x.numel() and w.numel():
+        # the fused forward's arithmetic (both operands quantized with the rings' current steps,
+        # GEMM with the bias in its epilogue), the two amax values going to their rings as
+        # per-workgroup maxima
+        x2 = x.reshape(-1, w.size(1))
+        has_bias = bias is not None and bias.numel() > 0
+        x8 = quantize_bf16_partials(x2, meta.x_scale, "e4m3", meta._x.partials)
+        w8 = quantize_bf16_partials(w, meta.w_scale, "e4m3", meta._w.partials)
+        out = mm_fp8_bias(x8, w8, meta.x_scale, meta.w_scale,
+                          bias if has_bias else None).reshape(*x.shape[:-1], w.size(0))
+        meta._x.push_partials(meta.recipe, fmt)
+        meta._w.push_partials(meta.recipe, fmt)
+        meta.note_w_push(w)
         return out
     out, amax_x, amax_w = linear_forward_fp8(x, w, bias, meta.x_scale, meta.w_scale)
     meta.update_x(amax_x, fmt)

@@ -32,6 +32,10 @@ def _fp8_mm_module() -> SimpleNamespace:
         quantize_transpose_bf16=_cabi.quantize_transpose_bf16,
         amax_bf16=_cabi.amax_bf16,
         amax_ring_push=_cabi.amax_ring_push,
+        new_amax_partials=_cabi.new_amax_partials,
+        quantize_bf16_partials=_cabi.quantize_bf16_partials,
+        amax_bf16_partials=_cabi.amax_bf16_partials,
+        amax_ring_push_partials=_cabi.amax_ring_push_partials,
         add_rmsnorm_quantize_fp8=_cabi.add_rmsnorm_quantize_fp8,
         silu_mul_quantize_fp8=_cabi.silu_mul_quantize_fp8,
     )

@@ -186,6 +186,32 @@ def amax_bf16(x: Tensor) -> Tensor:
     return _Kernels.get().amax_bf16(x)
 
 
+def new_amax_partials(device) -> Tensor:
+    """Scratch for the three ``*_partials`` primitives below: max |x| travels from the pass
+    that sees the tensor to the ring push as one maximum per workgroup, not through one
+    atomically updated (and beforehand cleared) slot. Producer and consumer share a stream."""
+    return _Kernels.get().new_amax_partials(device)
+
+
+def quantize_bf16_partials(x: Tensor, scale: Tensor, fmt: str, partials: Tensor) -> Tensor:
+    """``quantize_bf16`` that leaves max |x| in ``partials`` and returns the codes alone."""
+    _all_bf16("quantize_bf16_partials", x)
+    return _Kernels.get().quantize_bf16_partials(x, scale, _position(fmt, _FORMATS, "fmt"), partials)
+
+
+def amax_bf16_partials(x: Tensor, partials: Tensor) -> None:
+    """``amax_bf16`` that leaves max |x| in ``partials``."""
+    _all_bf16("amax_bf16_partials", x)
+    _Kernels.get().amax_bf16_partials(x, partials)
+
+
+def amax_ring_push_partials(hist: Tensor, idx: int, partials: Tensor, scale: Tensor, fmax: float,
+                            pow2_margin: float, amax_out: Optional[Tensor] = None) -> None:
+    """``amax_ring_push`` whose new amax is the maximum of ``partials`` (also written to
+    ``amax_out`` when given)."""
+    _Kernels.get().amax_ring_push_partials(hist, idx, partials, scale, fmax, pow2_margin, amax_out)
+
+
 def amax_ring_push(hist: Tensor, idx: int, amax: Tensor, scale: Tensor, fmax: float,
                    pow2_margin: float) -> None:
     """Delayed scaling's bookkeeping for one tensor in one launch, in place: the new amax

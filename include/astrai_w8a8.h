@@ -85,6 +85,26 @@ int astrai_w8a8_amax_ring_push(float* hist, int n, int idx, const float* amax, f
                                float fmax, float pow2_margin, void* stream);
 
 /*
+ * The three entries above with the maximum handed over as per-workgroup partial maxima
+ * instead of one atomically updated slot: the producer (the quantizer of
+ * csrc/kernels/fp8/mm.cu:99-126, or the amax pass) writes every one of the
+ * ASTRAI_W8A8_AMAX_PARTIALS fp32 slots of `partials` (unused ones zero), and the ring push
+ * reduces them -- max is order-free, so ring and step come out as with
+ * astrai_w8a8_quantize_bf16_fp8 + astrai_w8a8_amax_ring_push, bit for bit. No slot to clear
+ * before the producer, no atomics and nothing that waits at the producer's end: at 4096 x 4096
+ * the quantizer takes 10 us against 13.8 us, and the fill launch of the slot disappears. The
+ * forward of a Linear under delayed / dynamic scaling (astrai/extension/fp8.py:275-305) runs on
+ * these. amax_out (may be NULL) receives the reduced maximum. total must be positive.
+ */
+#define ASTRAI_W8A8_AMAX_PARTIALS 1024
+int astrai_w8a8_quantize_bf16_fp8_partials(const void* x_bf16, void* x8, const float* scale,
+                                           float* partials, int64_t total, int fmt, void* stream);
+int astrai_w8a8_amax_bf16_partials(const void* x_bf16, float* partials, int64_t total, void* stream);
+int astrai_w8a8_amax_ring_push_partials(float* hist, int n, int idx, const float* partials,
+                                        float* amax_out, float* scale, float fmax,
+                                        float pow2_margin, void* stream);
+
+/*
  * The same quantizer on a [rows, cols] matrix, writing the codes transposed
  * ([cols, rows], x8t) and, when x8 is not NULL, row-major as well, from one read
  * of x. Replaces the transposed-contiguous copies followed by quantize_bf16 in

@@ -55,6 +55,22 @@ def test_add_rmsnorm_quantize(C, rows, k, with_res):
     _codes_close(xq, wq, s, ws)
 
 
+@pytest.mark.parametrize("rows,k", [(2048, 2048), (513, 4096), (1000, 264), (600, 1024), (4099, 512), (700, 3080)])
+def test_rmsnorm_producer_bits_do_not_depend_on_the_launch_size(C, rows, k):
+    """A block of at least 512 rows runs one wave per row, fewer rows one workgroup per row;
+    both take the sum of squares in the same order, so a token's y, step and codes are the
+    same bits whether it is normalised in a prefill block or in a decode step."""
+    print(f"case rows={rows} k={k}", flush=True)
+    g = torch.Generator().manual_seed(rows * 7 + k)
+    x = (torch.randn(rows, k, generator=g) * torch.exp2(torch.randn(rows, 1, generator=g))).to(torch.bfloat16).to(DEV)
+    w = (1.0 + 0.1 * torch.randn(k, generator=g)).to(torch.bfloat16).to(DEV)
+    xq, s, _, y = C.add_rmsnorm_quantize_int8(x, w, 1e-5, None, want_y=True)          # one wave per row
+    for lo in range(0, rows, 300):                                                   # one workgroup per row
+        pq, ps, _, py = C.add_rmsnorm_quantize_int8(x[lo:lo + 300], w, 1e-5, None, want_y=True)
+        assert torch.equal(py.view(torch.int16), y[lo:lo + 300].view(torch.int16)), lo
+        assert torch.equal(ps, s[lo:lo + 300]) and torch.equal(pq, xq[lo:lo + 300]), lo
+
+
 @pytest.mark.parametrize("rows,width,fused_buffer", [(32, 5632, True), (32, 5632, False), (1, 5632, True),
                                                      (7, 8, False), (3, 8192, True)])
 def test_silu_mul_quantize(C, rows, width, fused_buffer):

@@ -75,3 +75,53 @@ def test_static_scratch_entry_rejects_what_does_not_fit():
     rc = lib.astrai_w8a8_attn_decode_bf16_static_scratch(16, 16, 16, 16, 16, None, None, b, 1, hkv, hkv, 128,
                                                          64, nsplit, 1.0, None)
     assert rc == 2 and b"scratch" in lib.astrai_w8a8_last_error()
+
+
+def test_static_scratch_entry_allocates_nothing_and_replays_in_a_graph():
+    """What the entry exists for: with the outputs brought by the caller, a call changes
+    neither torch's allocator counters nor the free device memory the driver reports, and it
+    can be recorded into a HIP graph whose replays (with eager work and synchronisations
+    between them, on fresh inputs written into the captured buffers) equal the workspace
+    entry's eager result."""
+    from astrai_amd.extension import _cabi
+    lib = _cabi.load()
+    b, h, hkv, s, max_len, newest, nsplit = 8, 16, 4, 1, 256, 200, 4
+    q, kc, vc, pos = _inputs(b, h, hkv, s, max_len, newest, seed=11)
+    d = 128
+    out = torch.zeros(b, s, h * d, dtype=torch.bfloat16, device=DEV)
+    oq = torch.zeros(b * s, h * d, dtype=torch.int8, device=DEV)
+    osc = torch.zeros(b * s, dtype=torch.float32, device=DEV)
+
+    def call():
+        rc = lib.astrai_w8a8_attn_decode_bf16_static_scratch(
+            q.data_ptr(), kc.data_ptr(), vc.data_ptr(), pos.data_ptr(), out.data_ptr(), oq.data_ptr(),
+            osc.data_ptr(), b, s, h, hkv, d, max_len, nsplit, d ** -0.5, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, lib.astrai_w8a8_last_error()
+
+    call()                      # (the first call on a device looks the array's address up)
+    torch.cuda.synchronize()
+    before = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), torch.cuda.mem_get_info()[0])
+    call()
+    torch.cuda.synchronize()
+    after = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved(), torch.cuda.mem_get_info()[0])
+    assert after == before, (before, after)
+    want = _cabi.attn_decode(q, kc, vc, pos, nsplit=nsplit)
+    assert torch.equal(out, want)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        call()
+    for rep in range(4):
+        gen = torch.Generator().manual_seed(100 + rep)
+        q.copy_(torch.randn(q.shape, generator=gen).to(torch.bfloat16))
+        kc[:, :, : newest + 1].copy_(torch.randn(b, hkv, newest + 1, d, generator=gen).to(torch.bfloat16))
+        want = _cabi.attn_decode(q, kc, vc, pos, nsplit=nsplit)      # eager, its own workspace
+        wq = torch.empty_like(oq)
+        torch.cuda.synchronize()
+        out.zero_(); oq.zero_(); osc.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"replay {rep}"
+        assert oq.abs().max() > 0 and torch.isfinite(osc).all()
