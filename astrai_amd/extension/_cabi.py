@@ -12,6 +12,7 @@ anywhere in this module: without the HIP library every call raises.
 from __future__ import annotations
 
 import ctypes
+import weakref
 import os
 from typing import Optional
 
@@ -179,21 +180,37 @@ def _on_device(dev: torch.device):
 _PAD_K_MIN_MACS = 1 << 24
 
 
+# padded forms of weight-side operands: key -> (weakref to the operand, its version, padded copy).
+# A Linear's codes are one long-lived tensor (Int8State, the fp8 weight metas), so its padded form
+# is made once, not on every call; an entry dies with its tensor or with a write to it.
+_padded_weights: dict = {}
+
+
+def _padded_weight(b_c: torch.Tensor, kp: int) -> torch.Tensor:
+    key = (b_c.data_ptr(), tuple(b_c.shape), b_c.dtype, kp)
+    hit = _padded_weights.get(key)
+    if hit is not None and hit[0]() is b_c and hit[1] == b_c._version:
+        return hit[2]
+    for dead in [k_ for k_, e in _padded_weights.items() if e[0]() is None]:
+        del _padded_weights[dead]
+    padded = torch.nn.functional.pad(b_c.view(torch.uint8), (0, kp - b_c.size(1))).view(b_c.dtype)
+    _padded_weights[key] = (weakref.ref(b_c), b_c._version, padded)
+    return padded
+
+
 def _pad_k(a_c: torch.Tensor, b_c: torch.Tensor):
     """``(a, b, k)`` with K padded by zero codes to the next multiple the tuned kernels take (256 for
     at most 128 activation rows, the decode kernels' item; 128 otherwise), when K % 16 != 0 and the
-    product is large enough to repay two copies; else the operands as they are."""
+    product is large enough to repay the copies; else the operands as they are. The activation is
+    padded per call; the weight-side operand's padded form is kept while that tensor lives unmodified."""
     m, k = a_c.shape
     n = b_c.size(0)
     if k % 16 == 0 or m * n * k < _PAD_K_MIN_MACS:
         return a_c, b_c, k
     q = 256 if m <= 128 else 128
     kp = -(-k // q) * q
-
-    def pad(t):
-        return torch.nn.functional.pad(t.view(torch.uint8), (0, kp - k)).view(t.dtype)
-
-    return pad(a_c), pad(b_c), kp
+    a_p = torch.nn.functional.pad(a_c.view(torch.uint8), (0, kp - k)).view(a_c.dtype)
+    return a_p, _padded_weight(b_c, kp), kp
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
@@ -1561,6 +1578,14 @@ def attn_cache_rows_supported(n_heads: int, n_kv_heads: int, head_dim: int) -> b
     return head_dim in (32, 64, 128, 256) and n_heads % n_kv_heads == 0 and n_heads // n_kv_heads <= 16
 
 
+def cache_context_len(positions: torch.Tensor, max_len: int) -> torch.Tensor:
+    """Number of cache positions a block of new tokens at ``positions`` can attend to: newest
+    position + 1, never more than the cache holds (rotary / cache-write kernels skip positions
+    at or past ``max_len``, so a model that runs past its cache must not read past it either).
+    An int32 scalar on ``positions``' device; nothing is read on the host."""
+    return torch.clamp(positions.max() + 1, min=0, max=max_len).to(torch.int32)
+
+
 def attn_cache_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                     positions: torch.Tensor) -> torch.Tensor:
     """Attention of new tokens ``q [batch, n_heads, seq, head_dim]`` at ``positions [seq]``
@@ -1585,7 +1610,7 @@ def attn_cache_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         key = ("ramp", pairs, str(q.device))
         if key not in _index_cache:
             _index_cache[key] = torch.arange(pairs + 1, dtype=torch.int32, device=q.device)
-        kv_indptr = _index_cache[key] * (positions.max() + 1).to(torch.int32)
+        kv_indptr = _index_cache[key] * cache_context_len(positions, max_len)
         k_pool, v_pool = k_cache.view(pairs * max_len, 1, d), v_cache.view(pairs * max_len, 1, d)
         if s == 1:
             out = attn_paged_decode(q.reshape(pairs, n_rep, d), k_pool, v_pool, table, rows, kv_indptr)

@@ -43,6 +43,24 @@ def test_attn_cache_rows_against_oracle(b, h, hkv, d, s, max_len, start):
     _close(got, want, "cache rows")
 
 
+def test_attn_cache_rows_position_past_the_cache_reads_the_cache_and_nothing_else():
+    """A model that runs past its cache hands over positions >= max_len (the cache-write kernels
+    skip those): the context is clamped to the cache, so the newest token then sees exactly the
+    max_len cached keys -- the output of position max_len - 1 -- and no key of the neighbouring
+    (sequence, KV head) pair, which directly follows in memory."""
+    from astrai_amd.extension import _cabi
+    g = torch.Generator().manual_seed(5)
+    b, h, hkv, d, max_len = 3, 4, 2, 64, 48
+    q = torch.randn(b, h, 1, d, generator=g).to(torch.bfloat16).to(DEV)
+    kc = torch.randn(b, hkv, max_len, d, generator=g).to(torch.bfloat16).to(DEV)
+    vc = torch.randn(b, hkv, max_len, d, generator=g).to(torch.bfloat16).to(DEV)
+    at_end = _cabi.attn_cache_rows(q, kc, vc, torch.tensor([max_len - 1], device=DEV))
+    for past in (max_len, max_len + 5, 10 * max_len):
+        got = _cabi.attn_cache_rows(q, kc, vc, torch.tensor([past], device=DEV))
+        assert torch.equal(got, at_end), past
+    _close(at_end, D.attn_cached(q.cpu(), kc.cpu(), vc.cpu(), torch.tensor([max_len - 1])), "full cache")
+
+
 def test_attn_cache_rows_scattered_positions():
     """Positions need not be consecutive: every row sees the keys at positions <= its own."""
     from astrai_amd.extension import _cabi

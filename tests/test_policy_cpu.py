@@ -261,3 +261,32 @@ def test_int8_weight_cache_is_tied_to_the_tensor_object(monkeypatch):
     del w3
     st.put_weight(w1, torch.ones(4, 8, dtype=torch.int8), torch.ones(4))
     assert all(e[0]() is not None for e in st._weights.values())
+
+
+def test_cache_context_len_is_clamped_to_the_cache():
+    """attn_cache_rows never addresses more keys than the cache holds, whatever the positions say."""
+    from astrai_amd.extension._cabi import cache_context_len
+    for pos, max_len, want in (([0], 8, 1), ([3, 4, 5], 8, 6), ([7], 8, 8), ([8], 8, 8), ([100, 3], 8, 8), ([2, 9], 16, 10)):
+        got = cache_context_len(torch.tensor(pos), max_len)
+        assert got.dtype == torch.int32 and got.item() == want, (pos, max_len)
+
+
+def test_weight_side_padding_is_made_once_and_follows_writes():
+    """K % 16 != 0 products pad both operands with zero codes; the weight's padded form is kept while
+    that tensor lives unmodified (a Linear's codes are one long-lived tensor), not rebuilt per call."""
+    from astrai_amd.extension import _cabi
+    a = torch.randint(-5, 5, (200, 1000), dtype=torch.int8)
+    w = torch.randint(-5, 5, (300, 1000), dtype=torch.int8)
+    a1, w1, k1 = _cabi._pad_k(a, w)
+    a2, w2, k2 = _cabi._pad_k(a, w)
+    assert k1 == k2 == 1024 and w1 is w2 and a1 is not a2
+    assert torch.equal(w1[:, :1000], w) and not w1[:, 1000:].any() and not a1[:, 1000:].any()
+    w[0, 0] += 1                                   # a write: the kept form is stale
+    _, w3, _ = _cabi._pad_k(a, w)
+    assert w3 is not w1 and torch.equal(w3[:, :1000], w)
+    n = len(_cabi._padded_weights)
+    del w, w1, w2, w3
+    _cabi._pad_k(a, torch.zeros(300, 1000, dtype=torch.int8))   # a new weight: dead entries are dropped
+    assert len(_cabi._padded_weights) <= n
+    small, ws, ks = _cabi._pad_k(a[:2, :40], a[:3, :40])        # too small to repay a copy
+    assert ks == 40 and small.shape == (2, 40)
