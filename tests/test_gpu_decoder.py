@@ -322,3 +322,120 @@ def test_config4_dimensions_fused_cached_graph_properties(monkeypatch):
     assert torch.equal(eager, graph)
     # the first generated token is the argmax of the prefill's last logits
     assert (eager[:, 0] == inc_tail[:, 0].argmax(-1)).float().mean().item() >= 0.9
+
+
+def test_config4_dimensions_layer_tensors_over_128_decode_positions(monkeypatch):
+    """The config-4 layer at its real dimensions and batch (32 sequences, 512-token prompt, then
+    the 128 decode positions 512 .. 639, where the decode attention's context is split four ways):
+    the tensors of the fused cached path that exist before any later requantization -- q after
+    rotary, the k and v cache rows, the attention output, the residual stream the layer hands on --
+    against the same quantities formed with tensor ops (stock norm, int8 Linear, fp32 rotary, fp32
+    softmax attention), head by head and position by position. Measured: q, k, v within 0.07% (the
+    two norms differ in a last bf16 bit here and there, which flips a few int8 codes), the decode
+    attention output within 1% (it leaves the kernel in per-token int8 form), the layer output
+    within 4.3% (two more per-token quantizations in the MLP). A wrong rotary phase, cache slot,
+    head mapping or context split is an error of order one on the heads or positions it hits: the
+    gates are per head and per position, 0.5% / 1% / 2% / 8%."""
+    from astrai_amd.extension import _cabi, w8a8
+    from astrai_amd.model import DenseKVCache, fuse_int8_weights
+    from astrai_amd.model.decoder import apply_rotary_emb
+    cfg, model = _model(4, vocab_size=32000, hidden_size=2048, num_hidden_layers=1, num_attention_heads=16,
+                        num_key_value_heads=4, intermediate_size=5632, max_position_embeddings=1024)
+    b, p, steps, nh, nkv, hd = 32, 512, 128, 16, 4, 128
+    total = p + steps
+    gm = model.to(DEV)
+    ids = torch.randint(0, cfg.vocab_size, (b, total), generator=torch.Generator().manual_seed(4)).to(DEV)
+    layer, att = gm.layers[0], gm.layers[0].attention
+    w8a8.int8_state().reset()
+
+    def rel_rms(got, want, dims):
+        return ((got.float() - want.float()).pow(2).mean(dims).sqrt() / want.float().pow(2).mean(dims).sqrt())
+
+    with torch.no_grad():
+        # ---- the layer's tensors from tensor ops (the modular arithmetic), all 640 positions at once
+        x0 = gm.embed_tokens(ids)
+        hn = layer.input_norm(x0)
+        with w8a8.int8_autocast(True):
+            q = att.q_proj(hn).view(b, total, nh, hd)
+            k = att.k_proj(hn).view(b, total, nkv, hd)
+            v = att.v_proj(hn).view(b, total, nkv, hd)
+        table = gm.freqs_cis[:total].unsqueeze(0).float()
+        q_ref, k_ref = apply_rotary_emb(q, table), apply_rotary_emb(k, table)      # [b, pos, heads, hd]
+        # fp32 causal attention for the decode positions and a sample of prompt positions
+        rows = torch.cat([torch.tensor([0, 1, 63, 64, 255, 256, 511]), torch.arange(p, total)]).to(DEV)
+        kx = k_ref.float().repeat_interleave(nh // nkv, dim=2).permute(0, 2, 1, 3)   # [b, nh, pos, hd]
+        vx = v.float().repeat_interleave(nh // nkv, dim=2).permute(0, 2, 1, 3)
+        qs = q_ref.float().permute(0, 2, 1, 3)[:, :, rows]                           # [b, nh, R, hd]
+        scores = qs @ kx.transpose(-1, -2) * hd ** -0.5
+        scores = scores.masked_fill(torch.arange(total, device=DEV)[None, None, None, :] > rows[None, None, :, None],
+                                    float("-inf"))
+        attn_ref = (torch.softmax(scores, -1) @ vx).permute(0, 2, 1, 3)              # [b, R, nh, hd]
+        del scores, kx, vx, qs
+        with w8a8.int8_autocast(True):
+            ao = att.o_proj(attn_ref.reshape(b, len(rows), nh * hd).to(torch.bfloat16)) + x0[:, rows]
+            resid_ref = layer.mlp(layer.post_attention_norm(ao)) + ao                # [b, R, hidden]
+        w8a8.int8_state().reset()
+
+        # ---- the fused cached path: prefill of 512, then 128 single-token steps
+        fuse_int8_weights(gm)
+        got_q, got_attn = {}, {}
+        real_rc, real_dec, real_pre = _cabi.mm_int8_rope_cache, _cabi.attn_decode, _cabi.attn_prefill
+
+        def rc(xq, w, sx, sw, fr, positions, *a, **kw):
+            out = real_rc(xq, w, sx, sw, fr, positions, *a, **kw)
+            got_q[int(positions[0])] = out.clone()        # [b, nh, s, hd]
+            return out
+
+        def dec(qq, kc, vc, positions, **kw):
+            out = real_dec(qq, kc, vc, positions, **kw)
+            got_attn[int(positions[0])] = (out[0].clone(), out[1].clone())   # per-token int8 form
+            return out
+
+        def pre(qq, kc, vc, positions, **kw):
+            out = real_pre(qq, kc, vc, positions, **kw)
+            got_attn[int(positions[0])] = out.clone()     # bf16 [b, s, nh * hd]
+            return out
+
+        monkeypatch.setattr(_cabi, "mm_int8_rope_cache", rc)
+        monkeypatch.setattr(_cabi, "attn_decode", dec)
+        monkeypatch.setattr(_cabi, "attn_prefill", pre)
+        cache = DenseKVCache(cfg, b, total, DEV, torch.bfloat16)
+        hidden = []
+        with w8a8.int8_autocast(True):
+            hidden.append(gm(ids[:, :p], cache, torch.arange(p, device=DEV))["hidden_states"][:, rows[:7]])
+            for t in range(p, total):
+                hidden.append(gm(ids[:, t:t + 1], cache, torch.tensor([t], device=DEV))["hidden_states"])
+        assert len(got_q) == 1 + steps and len(got_attn) == 1 + steps
+        assert _cabi.decode_nsplit(b * nkv, total) == 4      # the four-split plan of the last positions
+
+        # k / v rows of every position as the cache holds them, per KV head and position
+        kc, vc = cache.k[0][:, :, :total], cache.v[0][:, :, :total]                    # [b, nkv, pos, hd]
+        ek = rel_rms(kc, k_ref.permute(0, 2, 1, 3), (0, 3))                           # [nkv, pos]
+        ev = rel_rms(vc, v.permute(0, 2, 1, 3), (0, 3))
+        print(f"worst per-(KV head, position) error of the cache rows: k {ek.max().item():.4f} v {ev.max().item():.4f}", flush=True)
+        assert ek.max().item() <= 5e-3 and ev.max().item() <= 5e-3, (ek.max().item(), ev.max().item())
+        # q after rotary: the prompt block and every decode step, per head and position
+        eq = rel_rms(got_q[0], q_ref[:, :p].permute(0, 2, 1, 3), (0, 3))
+        print(f"worst per-(head, position) error of q over the prompt: {eq.max().item():.4f}", flush=True)
+        assert eq.max().item() <= 5e-3, eq.max().item()
+        for t in range(p, total):
+            eq = rel_rms(got_q[t], q_ref[:, t:t + 1].permute(0, 2, 1, 3), (0, 2, 3))  # [nh]
+            assert eq.max().item() <= 5e-3, (t, eq)
+        # attention output per head: sampled prompt positions, every decode position
+        pre_out = got_attn[0].view(b, p, nh, hd)
+        ea = rel_rms(pre_out[:, rows[:7]], attn_ref[:, :7], (0, 3))                   # [7, nh]
+        assert ea.max().item() <= 1e-2, ea            # bf16 output of the block kernel
+        worst = 0.0
+        for i, t in enumerate(range(p, total)):
+            aq, sa = got_attn[t]
+            a = (aq.float() * sa.reshape(-1, 1)).view(b, nh, hd)
+            e = rel_rms(a, attn_ref[:, 7 + i], (0, 2))                                # [nh]
+            worst = max(worst, e.max().item())
+            assert e.max().item() <= 2e-2, (t, e)     # per-token int8 form of the output: its own ~1%
+        print(f"worst per-head attention error over the decode positions: {worst:.4f}", flush=True)
+        # what the layer hands on (here: through the final norm), per sequence and position; this one
+        # has passed two more per-token quantizations (the MLP's), hence the wider gate
+        eh = rel_rms(torch.cat(hidden, 1), gm.norm(resid_ref), (2,))                  # [b, R]
+        print(f"worst per-(sequence, position) error of the layer output: {eh.max().item():.4f}", flush=True)
+        assert eh.max().item() <= 0.08, eh.max().item()
+    w8a8.int8_state().reset()
