@@ -26,8 +26,11 @@ PEAK_FP8_TFLOPS = 5000.0   # MI355X dense fp8 MFMA
 PEAK_INT8_TOPS = 5000.0    # MI355X dense int8 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM-side bytes per launch of the headline kernel from two counter passes
-# (reads 101.0 MB + writes 33.6 MB); algorithmic bytes are 67.1 MB
-HEADLINE_TRAFFIC_MB = 134.5
+# (reads 101.7 MB + writes 34.4 MB); algorithmic bytes are 67.1 MB
+HEADLINE_TRAFFIC_MB = 136.1
+# share of the q|k|v, output, gate|up and down GEMV kernels in the kernel time of one fused
+# config-4 decode layer (profiles/decoder_config4_int8_kernel_shares.txt)
+DECODE_GEMV_SHARE = 0.49
 
 
 LAUNCHES_PER_BATCH = 50   # event-timed launches per batch
@@ -179,6 +182,46 @@ def _bench_decoder(dev):
         t_pre_f = (time.perf_counter() - t0) / 3
         res["fused_prefill_ms"] = round(t_pre_f * 1e3, 2)
         res["fused_prefill_tokens_per_s"] = round(batch * prompt / t_pre_f)
+        # GEMM share of the fused prefill, measured live: HIP events around every int8 product
+        # (the four GEMM entries of a fused layer, their fused epilogues included, and the lm_head)
+        from astrai_amd.extension import _cabi
+        gemm_names = ("mm_int8", "mm_int8_resid", "mm_int8_swiglu", "mm_int8_rope_cache")
+        real = {n: getattr(_cabi, n) for n in gemm_names}
+        spans = []
+
+        def timed(fn):
+            def call(*a, **kw):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                out = fn(*a, **kw)
+                e1.record()
+                spans.append((e0, e1))
+                return out
+            return call
+
+        for n in gemm_names:
+            setattr(_cabi, n, timed(real[n]))
+        try:
+            w0, w1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            w0.record()
+            prefill()
+            w1.record()
+            torch.cuda.synchronize()
+        finally:
+            for n in gemm_names:
+                setattr(_cabi, n, real[n])
+        in_gemm = sum(a.elapsed_time(b) for a, b in spans)
+        res["gemm_share_of_gpu_time"] = {
+            "fused_prefill": round(in_gemm / w0.elapsed_time(w1), 3),
+            "fused_prefill_what": f"measured in this run: HIP events around the {len(spans)} int8 GEMM calls of one "
+                                  "32 x 512-token prefill (q|k|v + rotary epilogue, output + residual, gate|up + "
+                                  "SwiGLU epilogue and its one-read quantizer, down + residual, lm_head) over the "
+                                  "events around the whole prefill",
+            "fused_decode_step": DECODE_GEMV_SHARE,
+            "fused_decode_step_what": "NOT measured in this run: share of the four weight-streaming GEMV kernels in "
+                                      "the kernel time of a decode layer, from the rocprofv3 kernel trace in "
+                                      "profiles/decoder_config4_int8_kernel_shares.txt (graph replays are not "
+                                      "traced per kernel)"}
         decode_legs("fused_", t_pre_f)
         unfuse_int8_weights(model)
         # the same model with the stock bf16 kernels, for scale
@@ -320,6 +363,7 @@ def _measured_ceilings():
         return {}
     res = {}
     for key, pat in (("mfma_fp8_random_TFLOPs", r"mfma fp8 32x32x64\s+operands random:\s*([0-9.]+) Tops/s"),
+                     ("mfma_fp8_16x16x128_random_TFLOPs", r"mfma fp8 16x16x128\s+operands random:\s*([0-9.]+) Tops/s"),
                      ("mfma_i8_random_TOPs", r"mfma i8 32x32x32\s+operands random:\s*([0-9.]+) Tops/s"),
                      ("hbm_stream_45MB_GBs", r"hbm read, 45.1 MB per launch[^:]*:\s*[0-9.]+ us per launch, ([0-9.]+) GB/s")):
         m = re.search(pat, out)
@@ -587,18 +631,19 @@ def main():
                 "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP8_TFLOPS, 4),
                 "traffic": HEADLINE_TRAFFIC_MB, "traffic_unit": "MB per launch; NOT measured in this run: "
                 "rocprofv3 FETCH_SIZE + WRITE_SIZE of this kernel, calibrated on a plain copy, from "
-                "profiles/gemm_fp8_wave128_4096cubed.txt",
-                "kernel": "gemm_wave128_kernel<Op32F8<e4m3>,per-tensor> (256x256x128, 4 waves)",
+                "profiles/gemm_fp8_wave128_q16_4096cubed.txt",
+                "kernel": "gemm_wave128_q16_kernel<e4m3,per-tensor> (256x256x128 tiles, 4 waves, v_mfma_f32_16x16x128_f8f6f4)",
                 "avg_launch_us": round(kern_us, 2),
                 "timing": {"what": "HIP events on the launch stream; median of batch averages after a warm-up "
                                    "that ends when two consecutive batches agree within 2%; independent of "
                                    "--steps / --warmup, and run before them", **proto}}
-    if "mfma_fp8_random_TFLOPs" in ceilings:
+    if "mfma_fp8_16x16x128_random_TFLOPs" in ceilings:
         # the same kernel against what this GPU's MFMA pipe sustains on random operand bits
         roofline["measured_ceiling"] = {
-            "value": ceilings["mfma_fp8_random_TFLOPs"], "unit": "TFLOP/s",
-            "frac": round(achieved / ceilings["mfma_fp8_random_TFLOPs"], 4),
-            "what": "register-resident v_mfma_f32_32x32x64_f8f6f4 loop, random operand bits, measured in this run"}
+            "value": ceilings["mfma_fp8_16x16x128_random_TFLOPs"], "unit": "TFLOP/s",
+            "frac": round(achieved / ceilings["mfma_fp8_16x16x128_random_TFLOPs"], 4),
+            "what": "register-resident v_mfma_f32_16x16x128_f8f6f4 loop (the kernel's instruction), random "
+                    "operand bits, measured in this run"}
 
     # ---------------- CPU baseline: the oracle on this host ----------------
     cpu_baseline = None
