@@ -258,7 +258,7 @@ def _cpu_decoder_baseline(layers=1, prefill_batch=8, decode_steps=8):
     torch.manual_seed(4)
     model = AutoRegressiveLM(cfg).to(torch.bfloat16).eval()
     sd = {k: v.detach() for k, v in model.state_dict().items()}
-    lin = D.int8_linear_fn(sd)
+    lin = D.int8_linear_fn(sd, fast=True)
     batch, prompt = 32, 512
     ids = torch.randint(0, cfg.vocab_size, (batch, prompt), generator=torch.Generator().manual_seed(4))
     ids = ids[:prefill_batch]
@@ -907,7 +907,7 @@ def main():
                                 if "hbm_stream_45MB_GBs" in ceilings else {}),
                              "single_buffer_cache_resident_us": round(us1, 2)}
             if not args.no_cpu:
-                cms = cpu_median_ms(lambda: O2.int8_gemm(xq2c, wq2, sx2c, sw2c), trials=5)
+                cms = cpu_median_ms(lambda: O2.int8_gemm(xq2c, wq2, sx2c, sw2c, fast=True), trials=5)
                 cpu_c2[f"M{m}"] = {"ms": round(cms, 2), "GB/s": round(nbytes / (cms * 1e-3) / 1e9, 1)}
         extra["int8_gemv_11008x4096_hbm_ring"] = {"data": "BASELINE config 2 (seed 2)", **gemv}
         if cpu_c2:
@@ -960,7 +960,7 @@ def main():
         extra["int8_config0_16x2048x2048"] = {"data": "BASELINE config 0 (seed 0)",
                                               "us": round(_graph_us(launch0), 2)}
         if not args.no_cpu:
-            cms = cpu_median_ms(lambda: O2.int8_linear(xc, wq0c, sw0c), trials=5)
+            cms = cpu_median_ms(lambda: O2.int8_linear(xc, wq0c, sw0c, fast=True), trials=5)
             extra["int8_config0_16x2048x2048"]["cpu_oracle_ms"] = round(cms, 3)
             cpu_more["config0_int8_linear"] = {
                 "value": round(cms, 3), "unit": "ms", "cores": _cpu_threads(), "kind": "port",

@@ -220,14 +220,15 @@ def repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:
     return x.unsqueeze(-2).expand(*x.shape[:-2], h, n_rep, d).reshape(*x.shape[:-2], h * n_rep, d)
 
 
-def int8_linear_fn(sd: Dict[str, torch.Tensor]) -> Callable[[torch.Tensor, str], torch.Tensor]:
-    """Quantize every 2-D projection weight per output channel once; activations per token per call."""
+def int8_linear_fn(sd: Dict[str, torch.Tensor], fast: bool = False) -> Callable[[torch.Tensor, str], torch.Tensor]:
+    """Quantize every 2-D projection weight per output channel once; activations per token per call.
+    ``fast``: the library int8 routine with its sampled self-check (timing legs only)."""
     q = {k: O.int8_quantize_rows(v) for k, v in sd.items()
          if v.dim() == 2 and not k.startswith("embed_tokens")}
 
     def lin(x: torch.Tensor, name: str) -> torch.Tensor:
         wq, sw = q[name]
-        return O.int8_linear(x, wq, sw)
+        return O.int8_linear(x, wq, sw, fast=fast)
 
     return lin
 

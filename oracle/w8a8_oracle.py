@@ -182,21 +182,21 @@ def int8_acc(xq: torch.Tensor, wq: torch.Tensor, fast: bool = False) -> torch.Te
     return (xq.double() @ wq.double().t()).to(torch.int32)
 
 
-def int8_gemm(xq, wq, sx, sw, bias=None):
+def int8_gemm(xq, wq, sx, sw, bias=None, fast: bool = False):
     """``bf16(acc * sx[m] * sw[n] (+ bias[n]))`` with the broadcast-scale form of
     astrai/extension/ops/fp8.py:118 and the single-rounding epilogue of
-    csrc/kernels/fp8/gemm.cuh:405-435."""
-    acc = int8_acc(xq, wq).float() * sx.reshape(-1, 1).float() * sw.reshape(1, -1).float()
+    csrc/kernels/fp8/gemm.cuh:405-435. ``fast``: see :func:`int8_acc` (timing legs)."""
+    acc = int8_acc(xq, wq, fast=fast).float() * sx.reshape(-1, 1).float() * sw.reshape(1, -1).float()
     if bias is not None and bias.numel():
         acc = acc + bias.float()
     return acc.to(torch.bfloat16)
 
 
-def int8_linear(x, wq, sw, bias=None):
+def int8_linear(x, wq, sw, bias=None, fast: bool = False):
     """W8A8 linear: per-token quantize ``x`` then :func:`int8_gemm`."""
     k = wq.size(1)
     xq, sx = int8_quantize_rows(x.reshape(-1, k))
-    out = int8_gemm(xq, wq, sx, sw, bias)
+    out = int8_gemm(xq, wq, sx, sw, bias, fast=fast)
     return out.reshape(*x.shape[:-1], wq.size(0))
 
 
