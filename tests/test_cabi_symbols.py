@@ -49,6 +49,22 @@ def test_argument_validation_needs_no_gpu():
     assert rc == 1 and b"out_scale" in lib.astrai_w8a8_last_error()
     rc = lib.astrai_w8a8_gemm_fp8_pt(8, 16, 16, 16, None, None, 16, 4, 4, 64, 0, 0, None)
     assert rc == 1 and b"aligned" in lib.astrai_w8a8_last_error()
+    # the per-workgroup-maxima forms of the quantizer, the amax pass and the ring push
+    rc = lib.astrai_w8a8_quantize_bf16_fp8_partials(16, 16, 16, None, 64, 0, None)
+    assert rc == 1 and b"null" in lib.astrai_w8a8_last_error()
+    rc = lib.astrai_w8a8_quantize_bf16_fp8_partials(16, 16, 16, 16, 0, 0, None)
+    assert rc == 1 and b"positive" in lib.astrai_w8a8_last_error()
+    rc = lib.astrai_w8a8_quantize_bf16_fp8_partials(16, 24, 16, 16, 64, 0, None)
+    assert rc == 1 and b"aligned" in lib.astrai_w8a8_last_error()
+    rc = lib.astrai_w8a8_amax_bf16_partials(16, None, 64, None)
+    assert rc == 1 and b"null" in lib.astrai_w8a8_last_error()
+    rc = lib.astrai_w8a8_amax_ring_push_partials(16, 4, 4, 16, None, 16, 448.0, 1.0, None)
+    assert rc == 1 and b"idx" in lib.astrai_w8a8_last_error()
+    rc = lib.astrai_w8a8_amax_ring_push_partials(16, 4, 0, 16, None, 16, 0.0, 1.0, None)
+    assert rc == 1 and b"positive" in lib.astrai_w8a8_last_error()
+    assert _cabi.AMAX_PARTIALS == int(re.search(r"#define ASTRAI_W8A8_AMAX_PARTIALS\s+(\d+)", open(
+        os.path.join(ROOT, "include", "astrai_w8a8.h")).read()).group(1))
+    assert isinstance(lib.astrai_w8a8_last_kernel(), bytes)
     # the residual entry: residual required, aligned, and apart from the output
     rc = lib.astrai_w8a8_gemm_int8_ptpc_resid(16, 16, 16, 16, None, None, 4096, 4, 4, 64, None)
     assert rc == 1 and b"residual" in lib.astrai_w8a8_last_error()
