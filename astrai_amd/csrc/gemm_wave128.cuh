@@ -67,7 +67,7 @@ enum : int { EPI_PLAIN = 0, EPI_SWIGLU = 1, EPI_ROPE = 2, EPI_RESID = 3 };
 // class of instructions so that its share of the kernel's time -- issue slots and, under the
 // power cap, clock -- can be read off a timing. The library instantiates KO = 0 only; a
 // knocked-out kernel computes nothing meaningful.
-enum : int { KO_LDS_READS = 1, KO_LOADS = 2, KO_MFMA = 4, KO_STORES = 8 };
+enum : int { KO_LDS_READS = 1, KO_LOADS = 2, KO_MFMA = 4, KO_STORES = 8, KO_BARRIER = 16, KO_WAITS = 32 };
 
 template <class Op, int ScaleKind, int Epi = EPI_PLAIN, int KO = 0>
 __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_kernel(GemmArgs g, RopeCacheArgs rc) {

@@ -216,9 +216,11 @@ __global__ __launch_bounds__(Wave128Cfg::THREADS) void gemm_wave128_q16_kernel(G
         }
         // Slab k+1 has landed for this wave -- all but this half's eight loads are older --
         // and this wave is done reading slab k; after the barrier both hold for every wave.
-        wait_vmcnt<LOADS ? 8 : 0>();
-        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
-        phase_barrier();
+        if constexpr (!(KO & KO_WAITS)) {
+            wait_vmcnt<LOADS ? 8 : 0>();
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+        }
+        if constexpr (!(KO & KO_BARRIER)) phase_barrier();
         // (after the last slab the reads below fetch stale bytes that are never used)
         if constexpr (!ODD) {
             phase(xb, wb, 1, 1, [&](int r) __attribute__((always_inline)) { read_x(r, xs1, 0, xa); }, ldw(0));

@@ -169,6 +169,25 @@ __global__ __launch_bounds__(512) void l2_stream(const unsigned char* A, const u
     if (s == 0x12345678u) out[0] = s;
 }
 
+// The GEMM epilogue's store pattern with nothing before it: workgroup b owns a 256 x 256 bf16 tile
+// of a 4096 x 4096 matrix (tile map as above), each of its four waves a 128 x 128 quadrant, a store
+// instruction = four rows x 256 bytes, 16 bytes a lane. AUX: the cache-policy bits of the store.
+template <int AUX>
+__global__ __launch_bounds__(256) void tile_write(unsigned short* out, int ld) {
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int b = blockIdx.x, pid = (b & 7) * 32 + (b >> 3);
+    const int tm = (pid / 64) * 4 + pid % 4, tn = (pid % 64) / 4;
+    const unsigned row_bytes = (unsigned)ld * 2u;
+    __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(out + (size_t)tm * 256 * ld), 0, 256u * row_bytes, 0x00020000);
+    const unsigned off = (unsigned)((wave & 1) * 128 + (lane >> 4)) * row_bytes +
+                         (unsigned)(tn * 256 + (wave >> 1) * 128 + (lane & 15) * 8) * 2u;
+    const u32x4 v = {(unsigned)lane, (unsigned)b, 3u, 4u};
+#pragma unroll
+    for (int i = 0; i < 32; ++i)
+        __builtin_amdgcn_raw_buffer_store_b128(v, r, off + (unsigned)(i * 4) * row_bytes, 0, AUX);
+}
+
 template <class F>
 float time_ms(F f, int iters) {
     hipEvent_t e0, e1;
@@ -213,6 +232,16 @@ int main() {
     printf("hbm read, 1 GiB per launch: %.1f us, %.0f GB/s\n", ms * 1e3, big / ms / 1e6);
     ms = time_ms([&] { hbm_read<4><<<1, 256>>>((const u32x4*)buf, 1, o2); }, 500);
     printf("back-to-back launch of an empty kernel: %.2f us\n", ms * 1e3);
+
+    {
+        unsigned short* o16 = (unsigned short*)buf;
+        const float gap = ms;
+        ms = time_ms([&] { tile_write<0><<<256, 256>>>(o16, 4096); }, 500);
+        const float ms_nt = time_ms([&] { tile_write<2><<<256, 256>>>(o16, 4096); }, 500);
+        printf("GEMM epilogue store pattern alone (33.5 MB, 256 workgroups x 128 KiB): %.2f us per launch with default "
+               "stores, %.2f us non-temporal (launch gap %.2f us included) -> %.1f / %.1f TB/s net of the gap\n",
+               ms * 1e3, ms_nt * 1e3, gap * 1e3, 33.554432 / ((ms - gap) * 1e3), 33.554432 / ((ms_nt - gap) * 1e3));
+    }
 
     CK(hipFuncSetAttribute((const void*)l2_stream, hipFuncAttributeMaxDynamicSharedMemorySize, 131072));
     const int ld = 4096, ksteps = 32;

@@ -189,6 +189,11 @@ static void knockouts_q16(const char* what, const GemmArgs& g) {
     printf("  without either                 %.2f us\n", time_q16_us<SK, KO_LDS_READS | KO_LOADS>(g));
     printf("  without output stores          %.2f us\n", time_q16_us<SK, KO_STORES>(g));
     printf("  without MFMAs                  %.2f us\n", time_q16_us<SK, KO_MFMA>(g));
+    printf("  without the per-slab barrier   %.2f us\n", time_q16_us<SK, KO_BARRIER>(g));
+    printf("  without the per-slab waits     %.2f us\n", time_q16_us<SK, KO_WAITS>(g));
+    printf("  without barrier and waits      %.2f us\n", time_q16_us<SK, KO_BARRIER | KO_WAITS>(g));
+    printf("  without barrier, waits, loads and LDS reads %.2f us\n",
+           time_q16_us<SK, KO_BARRIER | KO_WAITS | KO_LOADS | KO_LDS_READS>(g));
 }
 
 int main(int argc, char** argv) {
