@@ -339,8 +339,9 @@ __global__ __launch_bounds__(Cfg::THREADS) void gemm_pingpong_kernel(GemmArgs g)
         make_rsrc(g.sa, kBlk ? (uint32_t)g.m * (uint32_t)kblocks * 4u : 0u);
     [[maybe_unused]] const uint32_t sa_off =
         (uint32_t)(m0 + wave_m * Cfg::WAVE_M + lane) * (uint32_t)kblocks * 4u;
+    // (a wave whose columns all lie past N clamps to the last block: its outputs are dropped)
     [[maybe_unused]] const float* const sb_row =
-        kBlk ? g.sb + (size_t)((n0 + wave_n * Cfg::WAVE_N) >> 7) * kblocks : nullptr;
+        kBlk ? g.sb + (size_t)min((n0 + wave_n * Cfg::WAVE_N) >> 7, ((g.n + 127) >> 7) - 1) * kblocks : nullptr;
     [[maybe_unused]] float blk_sa_ld = 1.0f, blk_sb_ld = 1.0f;  // scales in flight
     [[maybe_unused]] auto load_block_scales = [&](int kb) {
         if constexpr (kBlk) {
