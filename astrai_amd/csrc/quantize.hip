@@ -266,6 +266,17 @@ __global__ __launch_bounds__(kThreads) void quantize_transpose_fp8_kernel(
     for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
         const int64_t r0 = (t / tiles_x) * kTrRows, c0 = (t % tiles_x) * kTrCols;
         const int64_t c = c0 + cc * 8;
+        // all eight 16-byte pieces of the thread requested before the first is converted
+        u32x4 raw[2][4];
+        const bool col_in = vec && c < cols;
+#pragma unroll
+        for (int pass = 0; pass < 2; ++pass)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int64_t r = r0 + pass * 64 + r4 * 4 + i;
+                raw[pass][i] = u32x4{0u, 0u, 0u, 0u};
+                if (col_in && r < rows) raw[pass][i] = *reinterpret_cast<const u32x4*>(x + r * cols + c);
+            }
 #pragma unroll
         for (int pass = 0; pass < 2; ++pass) {
             u32x2 q[4];
@@ -273,9 +284,9 @@ __global__ __launch_bounds__(kThreads) void quantize_transpose_fp8_kernel(
             for (int i = 0; i < 4; ++i) {
                 const int64_t r = r0 + pass * 64 + r4 * 4 + i;
                 float f[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-                const bool whole = vec && r < rows && c < cols;
+                const bool whole = col_in && r < rows;
                 if (whole) {
-                    unpack8(*reinterpret_cast<const u32x4*>(x + r * cols + c), f);
+                    unpack8(raw[pass][i], f);
                 } else if (r < rows) {
 #pragma unroll
                     for (int j = 0; j < 8; ++j)
@@ -285,7 +296,7 @@ __global__ __launch_bounds__(kThreads) void quantize_transpose_fp8_kernel(
                 q[i] = quant8_fp8<Fmt>(f, step);
                 if (x8) {
                     if (whole) {
-                        *reinterpret_cast<u32x2*>(x8 + r * cols + c) = q[i];
+                        __builtin_nontemporal_store(q[i], reinterpret_cast<u32x2*>(x8 + r * cols + c));
                     } else if (r < rows) {
 #pragma unroll
                         for (int j = 0; j < 8; ++j)
@@ -295,13 +306,19 @@ __global__ __launch_bounds__(kThreads) void quantize_transpose_fp8_kernel(
                     }
                 }
             }
+            // 4 rows x 8 columns of bytes -> 8 dwords of one column each: two 4 x 4 byte
+            // transposes of two v_perm_b32 stages (byte selectors: 0-3 second source, 4-7 first)
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                uint32_t d = 0;
+            for (int half = 0; half < 2; ++half) {
+                const uint32_t a0 = half ? q[0].y : q[0].x, a1 = half ? q[1].y : q[1].x;
+                const uint32_t a2 = half ? q[2].y : q[2].x, a3 = half ? q[3].y : q[3].x;
+                const uint32_t lo01 = __builtin_amdgcn_perm(a1, a0, 0x05010400u), hi01 = __builtin_amdgcn_perm(a1, a0, 0x07030602u);
+                const uint32_t lo23 = __builtin_amdgcn_perm(a3, a2, 0x05010400u), hi23 = __builtin_amdgcn_perm(a3, a2, 0x07030602u);
+                const uint32_t d[4] = {__builtin_amdgcn_perm(lo23, lo01, 0x05040100u), __builtin_amdgcn_perm(lo23, lo01, 0x07060302u),
+                                       __builtin_amdgcn_perm(hi23, hi01, 0x05040100u), __builtin_amdgcn_perm(hi23, hi01, 0x07060302u)};
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    d |= (((j < 4 ? q[i].x : q[i].y) >> ((j & 3) * 8)) & 0xffu) << (8 * i);
-                *reinterpret_cast<uint32_t*>(tile + (cc * 8 + j) * kTrPitch + pass * 64 + r4 * 4) = d;
+                for (int j = 0; j < 4; ++j)
+                    *reinterpret_cast<uint32_t*>(tile + (cc * 8 + half * 4 + j) * kTrPitch + pass * 64 + r4 * 4) = d[j];
             }
         }
         __syncthreads();
@@ -317,7 +334,7 @@ __global__ __launch_bounds__(kThreads) void quantize_transpose_fp8_kernel(
             v.z = *reinterpret_cast<const uint32_t*>(src + 8);
             v.w = *reinterpret_cast<const uint32_t*>(src + 12);
             if (runs) {
-                *reinterpret_cast<u32x4*>(x8t + ct * rows + rt) = v;
+                __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(x8t + ct * rows + rt));
             } else {
                 const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
@@ -868,9 +885,9 @@ void launch_quantize_transpose_fp8(const void* x, void* x8, void* x8t, const flo
                                    float* amax, int64_t rows, int64_t cols, int fmt,
                                    hipStream_t stream) {
     if (rows <= 0 || cols <= 0) return;
-    // two or more tiles per workgroup once there are enough tiles to fill the chip
+    // a workgroup per tile while they are all resident at once (eight per compute unit)
     const int64_t ntiles = ((cols + kTrCols - 1) / kTrCols) * ((rows + kTrRows - 1) / kTrRows);
-    const dim3 grid((unsigned)(ntiles <= 256 ? ntiles : (ntiles < 1024 ? (ntiles + 1) / 2 : 512)));
+    const dim3 grid((unsigned)(ntiles <= 2048 ? ntiles : 2048));
     auto* xi = static_cast<const uint16_t*>(x);
     auto* o = static_cast<uint8_t*>(x8);
     auto* ot = static_cast<uint8_t*>(x8t);
