@@ -493,9 +493,10 @@ def amax_ring_push_partials(hist: torch.Tensor, idx: int, partials: torch.Tensor
 
 def quantize_transpose_bf16(x: torch.Tensor, scale: torch.Tensor, fmt: int,
                             want_rowmajor: bool = False, want_amax: bool = False):
-    """One pass over a bf16 ``[R, C]`` matrix -> ``(x8 [R,C] or None, x8t [C,R], amax [1])``:
+    """One pass over a bf16 ``[R, C]`` matrix -> ``(x8 [R,C] or None, x8t [C,R], amax [1] or None)``:
     the codes ``quantize_bf16`` gives for ``x`` and for ``x.t().contiguous()``
-    (mm.cu:276-312 makes that copy first). ``amax`` stays zero unless asked for."""
+    (mm.cu:276-312 makes that copy first). ``amax`` is measured (and its slot allocated and
+    cleared: one more launch) only when asked for."""
     lib = _require()
     _gpu(x, "quantize_transpose_bf16")
     if x.dtype != torch.bfloat16 or x.dim() != 2:
@@ -507,12 +508,11 @@ def quantize_transpose_bf16(x: torch.Tensor, scale: torch.Tensor, fmt: int,
     with _on_device(x.device):
         x8 = torch.empty((rows, cols), device=x.device, dtype=f8) if want_rowmajor else None
         x8t = torch.empty((cols, rows), device=x.device, dtype=f8)
-        amax = torch.zeros(1, device=x.device, dtype=torch.float32)
+        amax = torch.zeros(1, device=x.device, dtype=torch.float32) if want_amax else None
         if rows and cols:
             _check(lib.astrai_w8a8_quantize_transpose_bf16_fp8(
                 x_c.data_ptr(), _ptr(x8), x8t.data_ptr(), scale.data_ptr(),
-                amax.data_ptr() if want_amax else None, rows, cols, 1 if fmt else 0,
-                _stream(x)), lib)
+                _ptr(amax), rows, cols, 1 if fmt else 0, _stream(x)), lib)
     return x8, x8t, amax
 
 
@@ -556,7 +556,7 @@ def linear_backward_fp8(g, x, w, masks, sg, sw, sx, fmt: int):
         grad_input = torch.empty(x.shape, device=x.device, dtype=x.dtype)
         grad_weight = torch.empty((n, k), device=w.device, dtype=w.dtype)
         grad_bias = torch.empty(0, device=g.device, dtype=g.dtype)
-        amax_g = torch.zeros(1, device=g.device, dtype=torch.float32)
+        amax_g = None
         g8 = g8_t = None
         if masks[1]:
             # amax_g is measured only on the dX branch (mm.cu:293-296)
@@ -576,6 +576,8 @@ def linear_backward_fp8(g, x, w, masks, sg, sw, sx, fmt: int):
             amax_g = g_c.abs().amax().to(torch.float32).reshape(1)
         if masks[2]:
             grad_bias = g_c.sum(0).to(g.dtype)
+        if amax_g is None:
+            amax_g = torch.zeros(1, device=g.device, dtype=torch.float32)
     return grad_input, grad_weight, grad_bias, amax_g
 
 
