@@ -110,7 +110,8 @@ def test_fp8_quantize_noncontiguous_input(C):
 @pytest.mark.parametrize("fmt", [0, 1])
 @pytest.mark.parametrize("shape", [(1, 1), (1, 33), (33, 1), (17, 9), (128, 64), (130, 72), (16, 8),
                                    (48, 20), (129, 65), (256, 7), (19, 128), (1000, 520), (0, 8),
-                                   (2048, 4096)])
+                                   (2048, 4096),
+                                   (6016, 5896)])   # 47 x 47 tiles: more than one tile per workgroup
 def test_fp8_quantize_transposed_codes(C, shape, fmt):
     """One pass gives the codes of x and of x.t().contiguous() (the copies
     csrc/kernels/fp8/mm.cu:298-311 quantizes) and the amax, bit-exact, for
