@@ -8,6 +8,7 @@
 #include "gemm_wave128.cuh"
 #include "gemm_wave128_q16.cuh"
 #include "gemm_mid128.cuh"
+#include "gemm_small64.cuh"
 #include "gemm_tile.cuh"
 
 namespace w8a8 {
@@ -36,6 +37,7 @@ void launch_for(const GemmArgs& g, hipStream_t stream) {
 #endif
     if (pingpong_shape_ok(g)) return launch_pingpong<Op32F8<Fmt>, ScaleKind>(g, stream);
     if (mid128_shape_ok(g)) return launch_mid128<Op32F8<Fmt>, ScaleKind>(g, stream);
+    if (small64_shape_ok(g)) return launch_small64<Op32F8<Fmt>, ScaleKind>(g, stream);
     launch_tiled_auto<OpF8<Fmt>, ScaleKind>(g, stream);
 }
 }  // namespace

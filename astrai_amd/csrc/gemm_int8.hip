@@ -5,6 +5,7 @@
 // tiles of the same instruction; the generic tiled kernel takes everything else.
 #include "gemm_wave128.cuh"
 #include "gemm_mid128.cuh"
+#include "gemm_small64.cuh"
 #include "gemm_tile.cuh"
 
 namespace w8a8 {
@@ -28,6 +29,8 @@ bool launch_gemm_int8_tiled(const GemmArgs& g, hipStream_t stream, bool tail_on_
         launch_pingpong<Op32I8, SCALE_ROWCOL>(g, stream);
     else if (mid128_shape_ok(g))
         launch_mid128<Op32I8, SCALE_ROWCOL>(g, stream);
+    else if (small64_shape_ok(g))
+        launch_small64<Op32I8, SCALE_ROWCOL>(g, stream);
     else
         launch_tiled_auto<OpI8, SCALE_ROWCOL>(g, stream);
     return true;

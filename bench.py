@@ -875,6 +875,23 @@ def main():
             del mx, mw, my
         extra["int8_gemm_token_blocks_128x128_tiles"] = mid
 
+        # ---- a few hundred tokens against the config-4 projections (a short prompt, a large decode
+        # batch): too few 128 x 128 tiles as well; 64 x 64 tiles behind a ring of direct-to-LDS stages
+        few = {}
+        for (mm, nn, kk) in ((256, 3072, 2048), (256, 2048, 5632), (384, 2048, 5632), (256, 4096, 4096)):
+            mx = (torch.randn(mm, kk, device=dev) * 32).clamp(-127, 127).round().to(torch.int8)
+            mw = (torch.randn(nn, kk, device=dev) * 32).clamp(-127, 127).round().to(torch.int8)
+            msx, msw = torch.rand(mm, device=dev) + 0.5, torch.rand(nn, device=dev) + 0.5
+            my = torch.empty(mm, nn, device=dev, dtype=torch.bfloat16)
+            ms_few = ms_of(lambda: check(lib.astrai_w8a8_gemm_int8_ptpc(
+                mx.data_ptr(), mw.data_ptr(), msx.data_ptr(), msw.data_ptr(), None, my.data_ptr(), mm, nn, kk, 0,
+                stream)))
+            few[f"{mm}x{nn}x{kk}"] = {"us": round(ms_few * 1e3, 2),
+                                      "TOP/s": round(2.0 * mm * nn * kk / (ms_few * 1e-3) / 1e12, 1),
+                                      "kernel": _cabi.last_kernel()}
+            del mx, mw, my
+        extra["int8_gemm_few_hundred_tokens_64x64_tiles"] = few
+
         # ---- config 2: decode GEMV on the seed-2 tensors (activation and weight quantized per
         # token / per channel by the oracle's quantizer on the host), weights rotated through a
         # ring of ten copies (451 MB) so that the 256 MB Infinity Cache cannot serve them

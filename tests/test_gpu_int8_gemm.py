@@ -269,3 +269,43 @@ def test_large_ragged_tiles_with_guard_rows(C, m, n, k, out_dtype):
     else:
         assert torch.equal(out[rows].cpu(), O.int8_gemm(a[rows], b, sa[rows], sb))
         assert torch.equal(out[:m, cols].cpu(), O.int8_gemm(a, b[cols], sa, sb[cols]))
+
+
+SMALL_TILE_SHAPES = [(64, 64, 128),        # one tile, one slab
+                     (130, 200, 384),      # three slabs: fewer than the ring's stages
+                     (129, 257, 512),      # ragged rows and columns in the edge tiles
+                     (256, 4096, 4096),    # one workgroup per compute unit, 32 slabs
+                     (384, 2048, 5632),    # 44 slabs
+                     (300, 778, 1152),     # odd slab count, N % 4 != 0: scalar stores
+                     (1000, 2048, 2048),   # two workgroups per compute unit
+                     (64, 2048, 2176)]     # few rows with a K the decode kernels do not take
+
+
+@pytest.mark.parametrize("m,n,k", SMALL_TILE_SHAPES)
+def test_small_tile_kernel_int8_and_fp8(C, m, n, k):
+    """Shapes with too few 128 x 128 tiles for the mid-size kernel and K in whole 128-byte slabs run
+    64 x 64 tiles fed by a ring of direct-to-LDS stages: bf16 output of the int8 path bit-equal to
+    the oracle (with bias), per-tensor fp8 with bias and row / column fp8 within the 1e-2 gate, both
+    fp8 formats; the kernel each call landed on is checked."""
+    print(f"case m={m} n={n} k={k}", flush=True)
+    g = torch.Generator().manual_seed(m * 5 + n * 3 + k)
+    a, b = _rand_i8(g, m, k), _rand_i8(g, n, k)
+    sx = torch.rand(m, 1, generator=g) * 0.05 + 0.01
+    sw = torch.rand(n, generator=g) * 0.01 + 0.001
+    bias = torch.randn(n, generator=g).to(torch.bfloat16)
+    got = C.mm_int8(a.to(DEV), b.to(DEV), sx.to(DEV), sw.to(DEV), bias.to(DEV), 0)
+    assert C.last_kernel() == "small64", C.last_kernel()
+    want = O.int8_gemm(a, b, sx, sw, bias)
+    assert torch.equal(got.cpu().view(torch.int16), want.view(torch.int16))
+    for fmt, dt in ((0, torch.float8_e4m3fn), (1, torch.float8_e5m2)):
+        a8 = (torch.randn(m, k, generator=g) * 1.5).to(dt)
+        b8 = (torch.randn(n, k, generator=g) * 1.5).to(dt)
+        sa, sb = torch.tensor([0.37]), torch.tensor([0.011])
+        out = C.mm_fp8(a8.to(DEV), b8.to(DEV), sa.to(DEV), sb.to(DEV), 0, None, bias.to(DEV))
+        assert C.last_kernel() == "small64", C.last_kernel()
+        assert_bf16_close(out, O.fp8_gemm_bias(a8, b8, sa, sb, bias), what=f"small tiles, fmt {fmt}, per tensor + bias")
+        sa_r = torch.exp2(torch.rand(m, 1, generator=g) * 6.0 - 3.0)
+        sb_r = torch.exp2(torch.rand(n, generator=g) * 6.0 - 3.0)
+        out = C.mm_fp8(a8.to(DEV), b8.to(DEV), sa_r.to(DEV), sb_r.to(DEV), 0, None, None)
+        assert C.last_kernel() == "small64", C.last_kernel()
+        assert_bf16_close(out, O.fp8_gemm_bias(a8, b8, sa_r, sb_r, None), what=f"small tiles, fmt {fmt}, row/column steps")
