@@ -6,6 +6,7 @@
 // block, partial product promoted with sa[m,kb] * sb[n/128,kb]).
 #include "gemm_pingpong.cuh"
 #include "gemm_mid128.cuh"
+#include "gemm_small64.cuh"
 #include "gemm_tile.cuh"
 
 namespace w8a8 {
@@ -21,6 +22,8 @@ bool launch_gemm_fp8_block128_tiled(const GemmArgs& g, hipStream_t stream) {
     const int64_t tiles128 = (int64_t)((g.m + 127) / 128) * ((g.n + 127) / 128);
     if (mid128_shape_ok(g))   // blocks of a few hundred to a few thousand tokens: 128 x 128 tiles of the 32x32x64 MFMA
         launch_mid128<Op32F8<0>, SCALE_BLOCK128>(g, stream);
+    else if (small64_shape_ok(g))   // fewer tokens: 64 x 64 tiles behind a ring of stages
+        launch_small64<Op32F8<0>, SCALE_BLOCK128>(g, stream);
     else if (tiles128 >= 192)
         launch_tiled<OpF8<0>, CfgMid, SCALE_BLOCK128>(g, stream);
     else

@@ -33,7 +33,6 @@ struct Small64Cfg {
 
 template <class Op, int ScaleKind, int S>
 __global__ __launch_bounds__(256) void gemm_small64_kernel(GemmArgs g) {
-    static_assert(ScaleKind == SCALE_TENSOR || ScaleKind == SCALE_ROWCOL, "per-tensor or row x column scales");
     using Cfg = Small64Cfg<S>;
     using Acc = typename Op::Acc;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
@@ -70,7 +69,9 @@ __global__ __launch_bounds__(256) void gemm_small64_kernel(GemmArgs g) {
             b4[q][j] = 0.0f;
             if (n < g.n) {
                 if constexpr (ScaleKind == SCALE_ROWCOL) sw4[q][j] = g.sb[n];
-                if (bias) b4[q][j] = bf16_to_f32(bias[n]);
+                // (the block-scaled instance fetches the bias at the end: its loop counts its own loads)
+                if constexpr (ScaleKind != SCALE_BLOCK128)
+                    if (bias) b4[q][j] = bf16_to_f32(bias[n]);
             }
         }
 
@@ -125,7 +126,25 @@ __global__ __launch_bounds__(256) void gemm_small64_kernel(GemmArgs g) {
     for (int j = 0; j < 16; ++j) acc[j] = 0;
     u32x4 xa[4], wa[4], xb[4], wb[4];
 
+    // ---- 128-block scales: a slab is exactly one K-block and the tile's 64 columns lie in one
+    // weight block. The slab's product is formed in a temporary and joins the accumulator scaled by
+    // the row's and the block's steps, requested one slab ahead -- two loads an iteration, issued
+    // BEFORE the iteration's four slab loads, so that "all but the four youngest" below still means
+    // slab k + 1 has landed, and the steps with it.
+    [[maybe_unused]] float blk_sa_next = 0.0f, blk_sb_next = 0.0f;
+    [[maybe_unused]] const int kblocks = ksteps;
+    auto request_steps = [&](int kb) __attribute__((always_inline)) {
+        if constexpr (ScaleKind == SCALE_BLOCK128) {
+            static_assert(S == 4, "the wait counts of the block-scaled loop are written for four stages");
+            const int mrow = mw + lrow;
+            const int kc = min(kb, kblocks - 1);   // past the end: a harmless re-read
+            blk_sa_next = (mrow < g.m) ? g.sa[(size_t)mrow * kblocks + kc] : 0.0f;
+            blk_sb_next = g.sb[(size_t)(n0 >> 7) * kblocks + kc];
+        }
+    };
+
     // ---- prologue: slabs 0 .. S-2 in flight; slab 0 visible and in the first register set
+    request_steps(0);
 #pragma unroll
     for (int s = 0; s < S - 1; ++s) issue(s, s);
     wait_vmcnt<4 * (S - 2)>();
@@ -139,10 +158,22 @@ __global__ __launch_bounds__(256) void gemm_small64_kernel(GemmArgs g) {
         wait_vmcnt<4 * (S - 3)>();   // own loads of slab k + 1 (younger: slabs k + 2 .. k + S - 2)
         wait_lgkmcnt0();             // own reads of slab k
         phase_barrier();
+        [[maybe_unused]] const float sc = blk_sa_next * blk_sb_next;   // slab k's steps
+        request_steps(k + 1);
         issue(wr_stage, k + S - 1);
         read(rd_stage, xn, wn);
+        if constexpr (ScaleKind == SCALE_BLOCK128) {
+            Acc part;
 #pragma unroll
-        for (int q = 0; q < Op::STEPS; ++q) acc = Op::mma_step(q, wc, xc, acc);
+            for (int j = 0; j < 16; ++j) part[j] = 0;
+#pragma unroll
+            for (int q = 0; q < Op::STEPS; ++q) part = Op::mma_step(q, wc, xc, part);
+#pragma unroll
+            for (int j = 0; j < 16; ++j) acc[j] += part[j] * sc;
+        } else {
+#pragma unroll
+            for (int q = 0; q < Op::STEPS; ++q) acc = Op::mma_step(q, wc, xc, acc);
+        }
         rd_stage = (rd_stage == S - 1) ? 0 : rd_stage + 1;
         wr_stage = (wr_stage == S - 1) ? 0 : wr_stage + 1;
     };
@@ -166,7 +197,9 @@ __global__ __launch_bounds__(256) void gemm_small64_kernel(GemmArgs g) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const float f = (float)acc[4 * q + j];
-            if constexpr (ScaleKind == SCALE_TENSOR) {
+            if constexpr (ScaleKind == SCALE_BLOCK128) {
+                v[j] = f + ((bias && n + j < g.n) ? bf16_to_f32(bias[n + j]) : 0.0f);
+            } else if constexpr (ScaleKind == SCALE_TENSOR) {
                 v[j] = f * s_tensor + b4[q][j];
             } else {
 #pragma clang fp contract(off)

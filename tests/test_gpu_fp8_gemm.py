@@ -480,6 +480,23 @@ def test_block128_mid_size_tiles(m, n, k, bias):
     assert_bf16_close(out, O.fp8_gemm_blockscaled(x8, w8, sa, sb, b if bias else None), what="block128 mid-size")
 
 
+@pytest.mark.parametrize("m,n,k,bias", [(130, 200, 384, True), (300, 520, 1152, False), (256, 2048, 5632, True),
+                                        (65, 778, 128, False), (1000, 1024, 2048, True)])
+def test_block128_small_tiles(m, n, k, bias):
+    """Fewer than 140 tiles of 128 x 128 (and more rows than the decode kernel takes): the block-scaled
+    instance of the 64 x 64-tile kernel (ring of stages, a slab = one K-block scaled before it joins the
+    accumulator, its steps requested a slab ahead); ragged rows and columns, one to 44 slabs, wide scale range."""
+    from astrai_amd.extension import _cabi
+    from astrai_amd.extension.ops import fp8_block as blk
+    print(f"case m={m} n={n} k={k} bias={bias}", flush=True)
+    x, w, b = O.make_inputs(3, m, n, k, outlier_p=0.01, bias=bias)
+    x8, sa = O.fp8_quantize_act_block128(x)
+    w8, sb = O.fp8_quantize_weight_block128(w)
+    out = blk.mm_fp8_blockscaled(x8.to(DEV), w8.to(DEV), sa.to(DEV), sb.to(DEV), b.to(DEV) if bias else None)
+    assert _cabi.last_kernel() == "small64", _cabi.last_kernel()
+    assert_bf16_close(out, O.fp8_gemm_blockscaled(x8, w8, sa, sb, b if bias else None), what="block128 small tiles")
+
+
 def test_block128_golden_exact_rationals(golden):
     from astrai_amd.extension.ops import fp8_block as blk
     for c in golden("fp8_gemm_small.json")["block128"]:
