@@ -539,12 +539,24 @@ def main():
                                                     None, y3.data_ptr(), 16, 2048, 7168, stream))
             check(lib.astrai_w8a8_gemm_int8_ptpc(xt.data_ptr(), wq.data_ptr(), sxt.data_ptr(), sw.data_ptr(), None,
                                                  yt.data_ptr(), 4100, 4096, 4096, 0, stream))
+        # a few hundred tokens: 64 x 64 tiles behind a ring of stages (int8, two shapes in turn)
+        fews = []
+        for (mm, nn, kk) in ((256, 4096, 4096), (384, 2048, 5632)):
+            mx = (torch.randn(mm, kk, device=dev) * 32).clamp(-127, 127).round().to(torch.int8)
+            mw = (torch.randn(nn, kk, device=dev) * 32).clamp(-127, 127).round().to(torch.int8)
+            fews.append((mx, mw, torch.rand(mm, device=dev) + 0.5, torch.rand(nn, device=dev) + 0.5,
+                         torch.empty(mm, nn, device=dev, dtype=torch.bfloat16), mm, nn, kk))
+        for _ in range(20):
+            for (mx, mw, msx, msw, my, mm, nn, kk) in fews:
+                check(lib.astrai_w8a8_gemm_int8_ptpc(mx.data_ptr(), mw.data_ptr(), msx.data_ptr(), msw.data_ptr(),
+                                                     None, my.data_ptr(), mm, nn, kk, 0, stream))
         torch.cuda.synchronize()
         print(json.dumps({"trace_gemms": "20 launches each: int8 4096^3 per-token x per-channel (bf16 out), fp8 "
                                          "128-block 8192x2048x7168 on config-3 data, fp8 4096^3 with e4m3 output; "
                                          "then int8 2048x3072x2048, 2048x2048x5632, 1024x11264x2048 (mid-size kernel); "
                                          "then block-scaled 1024x11008x4096 (mid-size kernel) and 16x2048x7168 "
-                                         "(row-range kernel), and int8 4100x4096x4096 (large tiles + a four-row tail)"}))
+                                         "(row-range kernel), and int8 4100x4096x4096 (large tiles + a four-row tail); "
+                                         "then int8 256x4096x4096 and 384x2048x5632 (small-tile kernel)"}))
         return
 
     # ---------------- headline: config 1, fp8 per-tensor 4096^3 ----------------
